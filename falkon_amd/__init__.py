@@ -1,0 +1,6 @@
+"""falkon_amd: MI355X-native Gaussian kernel-vector products behind Falkon's kernel API."""
+from .options import FalkonOptions  # noqa: F401
+from .kernels import GaussianKernel  # noqa: F401
+from .mmv_ops import fdmmv, fmmv  # noqa: F401
+
+__version__ = "0.1.0"

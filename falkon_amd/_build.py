@@ -1,0 +1,65 @@
+"""Compile the HIP sources under ``falkon_amd/csrc`` into ``falkon_amd/lib/libfalkon_amd.so``.
+
+The library is built for gfx950 only, with plain ``hipcc`` (no torch headers: the
+C ABI takes raw pointers), one object per source compiled in parallel.
+"""
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_HERE, "csrc")
+LIB_DIR = os.path.join(_HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libfalkon_amd.so")
+OBJ_DIR = os.path.join(_HERE, "build")
+
+SOURCES = ["api.hip", "pack.hip", "mmv_small_f32.hip", "mmv_small_f64.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    # packed fp32 VALU ops are kept out of the generated code on purpose
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # keep MFMA accumulators in VGPRs: the epilogue reads every accumulator with VALU ops
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found; the falkon_amd native library needs ROCm's hipcc to build")
+
+
+def _compile(src: str) -> str:
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{res.stderr}")
+    return obj
+
+
+def build(verbose: bool = True, jobs: int = 0) -> str:
+    """Compile every source (always, also when a library is already there) and link."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    os.makedirs(LIB_DIR, exist_ok=True)
+    jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(_compile, SOURCES))
+    tmp = LIB_PATH + ".tmp"
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", tmp]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print(f"[falkon_amd] built {LIB_PATH}", file=sys.stderr)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()

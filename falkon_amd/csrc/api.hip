@@ -1,0 +1,291 @@
+// extern "C" entry points of libfalkon_amd: argument checks, workspace carving, launch plans.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "flk_common.h"
+
+namespace flk {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+constexpr int kColChunk = 4;          // right-hand sides handled per pass of the product kernel
+constexpr int64_t kTargetWgs = 2048;  // workgroups wanted per launch (256 CUs x 2 resident x 4 rounds)
+constexpr int64_t kMinChunkBlocks = 8;
+constexpr int kMaxSplits = 1024;
+
+struct Plan {
+    int64_t chunk_blocks;
+    int splits;
+};
+
+template <typename T>
+static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t dpad) {
+    const int64_t per_wg = mmv_small_b_blocks_per_wg<T>(dpad);
+    const int64_t b_tiles = (nb_blocks + per_wg - 1) / per_wg;
+    int64_t splits = (kTargetWgs + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
+    int64_t max_splits = na_blocks / kMinChunkBlocks;
+    if (max_splits < 1) max_splits = 1;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    if (splits < 1) splits = 1;
+    Plan p;
+    p.chunk_blocks = (na_blocks + splits - 1) / splits;
+    if (p.chunk_blocks < 1) p.chunk_blocks = 1;
+    p.splits = (int)((na_blocks + p.chunk_blocks - 1) / p.chunk_blocks);
+    if (p.splits < 1) p.splits = 1;
+    return p;
+}
+
+template <typename T>
+static size_t partial_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t) {
+    PackedView A = packed_view<T>(nullptr, n_a, d), B = packed_view<T>(nullptr, n_b, d);
+    Plan p = make_plan<T>(A.nblk, B.nblk, A.dpad);
+    int64_t tc = t < kColChunk ? t : kColChunk;
+    return align256((size_t)p.splits * tc * B.npad * sizeof(T));
+}
+
+static int check_matrix(const char *name, const void *p, int64_t rows, int64_t cols, int64_t rs, int64_t cs) {
+    if (rows < 0 || cols < 0) return fail(FLK_EINVAL, "%s: negative shape", name);
+    if (rows > 0 && cols > 0 && p == nullptr) return fail(FLK_EINVAL, "%s: null pointer", name);
+    if (rows > 1 && cols > 1 && rs != 1 && cs != 1)
+        return fail(FLK_EINVAL, "%s: neither stride is one (row stride %lld, column stride %lld)", name, (long long)rs,
+                    (long long)cs);
+    return FLK_OK;
+}
+
+// out[b,t] = sum_a K(A_a,B_b) vecp[t][a] (+ addend).  vecp is planar [t][A.npad].
+template <typename T>
+static int mmv_packed_planar(const PackedView &A, const PackedView &B, const T *vecp, int64_t t, const T *addend,
+                             int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
+                             T *partial, size_t partial_avail, hipStream_t st) {
+    if (B.n == 0 || t == 0) return FLK_OK;
+    if (A.d > mmv_small_max_d<T>())
+        return fail(FLK_EUNSUPPORTED, "feature dimension %lld exceeds the %lld the compiled kernels cover",
+                    (long long)A.d, (long long)mmv_small_max_d<T>());
+    Plan p = make_plan<T>(A.nblk, B.nblk, A.dpad);
+    for (int64_t t0 = 0; t0 < t; t0 += kColChunk) {
+        int tc = (int)(t - t0 < kColChunk ? t - t0 : kColChunk);
+        if ((size_t)p.splits * tc * B.npad * sizeof(T) > partial_avail)
+            return fail(FLK_ENOMEM, "workspace too small for %d partial sums of %lld x %d", p.splits,
+                        (long long)B.npad, tc);
+        int splits = p.splits;
+        if (A.nblk == 0) {
+            splits = 0;  // empty reduction: finalize sums nothing and writes the addend (or zero)
+        } else {
+            int rc = launch_mmv_small<T>(A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk_blocks, p.splits, partial, st);
+            if (rc != FLK_OK) return rc;
+        }
+        int rc = launch_finalize<T>(partial, splits, tc, B.n, B.npad, addend ? addend + t0 * add_cs : nullptr, add_rs,
+                                    add_cs, out + t0 * out_cs, out_rs, out_cs, zero_pad, st);
+        if (rc != FLK_OK) return rc;
+    }
+    return FLK_OK;
+}
+
+template <typename T>
+static int pack_impl(const void *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const void *sigma, int64_t n_sigma,
+                     void *packed, size_t bytes, hipStream_t st) {
+    int rc = check_matrix("X", X, n, d, rs, cs);
+    if (rc) return rc;
+    if (d < 1) return fail(FLK_EINVAL, "feature dimension must be positive");
+    if (sigma == nullptr) return fail(FLK_EINVAL, "sigma: null pointer");
+    if (n_sigma != 1 && n_sigma != d)
+        return fail(FLK_EINVAL, "The size of sigma (%lld) must match the number of features (%lld) or be 1",
+                    (long long)n_sigma, (long long)d);
+    if (bytes < packed_bytes<T>(n, d)) return fail(FLK_ENOMEM, "packed buffer too small");
+    if (n > 0 && packed == nullptr) return fail(FLK_EINVAL, "packed: null pointer");
+    PackedView v = packed_view<T>(packed, n, d);
+    return launch_pack<T>((const T *)X, n, d, rs, cs, (const T *)sigma, n_sigma, (T *)v.data, (T *)v.hnorm, v.dpad,
+                          v.nblk, st);
+}
+
+template <typename T>
+static int mmv_packed_impl(const void *pa, int64_t n_a, const void *pb, int64_t n_b, int64_t d, const void *vec,
+                           int64_t vec_rs, int64_t vec_cs, int64_t t, const void *addend, int64_t add_rs,
+                           int64_t add_cs, void *out, int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes,
+                           hipStream_t st) {
+    if (n_a < 0 || n_b < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
+    if (n_b == 0 || t == 0) return FLK_OK;
+    if (out == nullptr) return fail(FLK_EINVAL, "out: null pointer");
+    if (n_a > 0 && vec == nullptr) return fail(FLK_EINVAL, "vec: null pointer");
+    PackedView A = packed_view<T>(pa, n_a, d), B = packed_view<T>(pb, n_b, d);
+    size_t vec_bytes = align256((size_t)t * A.npad * sizeof(T));
+    size_t need = vec_bytes + partial_bytes<T>(n_a, n_b, d, t);
+    if (ws_bytes < need || (need > 0 && ws == nullptr))
+        return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+    T *vecp = (T *)ws;
+    T *partial = (T *)((char *)ws + vec_bytes);
+    int rc = launch_vec_planar<T>((const T *)vec, n_a, t, vec_rs, vec_cs, vecp, A.npad, st);
+    if (rc) return rc;
+    return mmv_packed_planar<T>(A, B, vecp, t, (const T *)addend, add_rs, add_cs, (T *)out, out_rs, out_cs, false,
+                                partial, ws_bytes - vec_bytes, st);
+}
+
+template <typename T>
+static size_t fmmv_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {
+    PackedView A = packed_view<T>(nullptr, m, d);
+    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + align256((size_t)t * A.npad * sizeof(T)) +
+           partial_bytes<T>(m, n, d, t);
+}
+
+template <typename T>
+static size_t fdmmv_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {
+    PackedView X = packed_view<T>(nullptr, n, d), C = packed_view<T>(nullptr, m, d);
+    size_t p1 = partial_bytes<T>(m, n, d, t), p2 = partial_bytes<T>(n, m, d, t);
+    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + align256((size_t)t * C.npad * sizeof(T)) +
+           align256((size_t)t * X.npad * sizeof(T)) + (p1 > p2 ? p1 : p2);
+}
+
+template <typename T>
+static int fmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
+                     int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v, int64_t v_rs,
+                     int64_t v_cs, int64_t t, void *out, int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes,
+                     hipStream_t st) {
+    if (n < 0 || m < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
+    int rc;
+    if ((rc = check_matrix("v", v, m, t, v_rs, v_cs))) return rc;
+    if ((rc = check_matrix("out", out, n, t, out_rs, out_cs))) return rc;
+    size_t need = fmmv_ws_bytes<T>(n, m, d, t);
+    if (ws_bytes < need || (need > 0 && ws == nullptr))
+        return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+    char *p = (char *)ws;
+    void *px = p; p += packed_bytes<T>(n, d);
+    void *pc = p; p += packed_bytes<T>(m, d);
+    if ((rc = pack_impl<T>(X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
+    if ((rc = pack_impl<T>(X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, packed_bytes<T>(m, d), st))) return rc;
+    return mmv_packed_impl<T>(pc, m, px, n, d, v, v_rs, v_cs, t, nullptr, 0, 0, out, out_rs, out_cs, p,
+                              ws_bytes - (size_t)(p - (char *)ws), st);
+}
+
+template <typename T>
+static int fdmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
+                      int64_t x2_rs, int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v,
+                      int64_t v_rs, int64_t v_cs, const void *w, int64_t w_rs, int64_t w_cs, int64_t t, void *out,
+                      int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes, hipStream_t st) {
+    if (n < 0 || m < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
+    int rc;
+    if (v == nullptr && m > 0 && t > 0) return fail(FLK_EINVAL, "v: null pointer (v is required)");
+    if ((rc = check_matrix("v", v, m, t, v_rs, v_cs))) return rc;
+    if (w && (rc = check_matrix("w", w, n, t, w_rs, w_cs))) return rc;
+    if ((rc = check_matrix("out", out, m, t, out_rs, out_cs))) return rc;
+    size_t need = fdmmv_ws_bytes<T>(n, m, d, t);
+    if (ws_bytes < need || (need > 0 && ws == nullptr))
+        return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+    PackedView X = packed_view<T>(nullptr, n, d), C = packed_view<T>(nullptr, m, d);
+    char *p = (char *)ws;
+    void *px = p; p += packed_bytes<T>(n, d);
+    void *pc = p; p += packed_bytes<T>(m, d);
+    T *vp = (T *)p; p += align256((size_t)t * C.npad * sizeof(T));
+    T *up = (T *)p; p += align256((size_t)t * X.npad * sizeof(T));
+    T *partial = (T *)p;
+    size_t partial_avail = ws_bytes - (size_t)(p - (char *)ws);
+    if ((rc = pack_impl<T>(X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
+    if ((rc = pack_impl<T>(X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, packed_bytes<T>(m, d), st))) return rc;
+    if ((rc = launch_vec_planar<T>((const T *)v, m, t, v_rs, v_cs, vp, C.npad, st))) return rc;
+    X = packed_view<T>(px, n, d);
+    C = packed_view<T>(pc, m, d);
+    // u = K v + w, planar [t][X.npad] with zeroed padding so it can feed the second product directly
+    if ((rc = mmv_packed_planar<T>(C, X, vp, t, (const T *)w, w_rs, w_cs, up, 1, X.npad, true, partial, partial_avail,
+                                   st)))
+        return rc;
+    // out = K^T u
+    return mmv_packed_planar<T>(X, C, up, t, nullptr, 0, 0, (T *)out, out_rs, out_cs, false, partial, partial_avail,
+                                st);
+}
+
+}  // namespace flk
+
+using namespace flk;
+
+extern "C" {
+
+int flk_version(void) { return 100; }
+const char *flk_last_error(void) { return g_err; }
+int64_t flk_max_d(int dtype) { return dtype == FLK_F64 ? mmv_small_max_d<double>() : mmv_small_max_d<float>(); }
+int64_t flk_max_t(void) { return 65535; }
+
+size_t flk_gauss_packed_bytes(int64_t n, int64_t d, int dtype) {
+    if (n < 0 || d < 1) return 0;
+    return dtype == FLK_F64 ? packed_bytes<double>(n, d) : packed_bytes<float>(n, d);
+}
+
+int flk_gauss_pack(const void *X, int64_t n, int64_t d, int64_t x_rs, int64_t x_cs, const void *sigma,
+                   int64_t n_sigma, int dtype, void *packed, size_t packed_bytes_, void *stream) {
+    g_err[0] = 0;
+    if (dtype == FLK_F32) return pack_impl<float>(X, n, d, x_rs, x_cs, sigma, n_sigma, packed, packed_bytes_, (hipStream_t)stream);
+    if (dtype == FLK_F64) return pack_impl<double>(X, n, d, x_rs, x_cs, sigma, n_sigma, packed, packed_bytes_, (hipStream_t)stream);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
+size_t flk_gauss_mmv_packed_workspace_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t, int dtype) {
+    if (n_a < 0 || n_b < 0 || d < 1 || t < 0) return 0;
+    if (dtype == FLK_F64)
+        return align256((size_t)t * packed_view<double>(nullptr, n_a, d).npad * 8) + partial_bytes<double>(n_a, n_b, d, t);
+    return align256((size_t)t * packed_view<float>(nullptr, n_a, d).npad * 4) + partial_bytes<float>(n_a, n_b, d, t);
+}
+
+int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b, int64_t n_b, int64_t d,
+                         const void *vec, int64_t vec_rs, int64_t vec_cs, int64_t t, const void *addend,
+                         int64_t add_rs, int64_t add_cs, void *out, int64_t out_rs, int64_t out_cs, int dtype,
+                         void *workspace, size_t workspace_bytes, void *stream) {
+    g_err[0] = 0;
+    if (dtype == FLK_F32)
+        return mmv_packed_impl<float>(packed_a, n_a, packed_b, n_b, d, vec, vec_rs, vec_cs, t, addend, add_rs, add_cs,
+                                      out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    if (dtype == FLK_F64)
+        return mmv_packed_impl<double>(packed_a, n_a, packed_b, n_b, d, vec, vec_rs, vec_cs, t, addend, add_rs, add_cs,
+                                       out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
+size_t flk_gauss_fmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
+    if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
+    return dtype == FLK_F64 ? fmmv_ws_bytes<double>(n, m, d, t) : fmmv_ws_bytes<float>(n, m, d, t);
+}
+
+int flk_gauss_fmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
+                   int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v, int64_t v_rs,
+                   int64_t v_cs, int64_t t, void *out, int64_t out_rs, int64_t out_cs, int dtype, void *workspace,
+                   size_t workspace_bytes, void *stream) {
+    g_err[0] = 0;
+    if (dtype == FLK_F32)
+        return fmmv_impl<float>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t, out,
+                                out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    if (dtype == FLK_F64)
+        return fmmv_impl<double>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t, out,
+                                 out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
+size_t flk_gauss_fdmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
+    if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
+    return dtype == FLK_F64 ? fdmmv_ws_bytes<double>(n, m, d, t) : fdmmv_ws_bytes<float>(n, m, d, t);
+}
+
+int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
+                    int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v, int64_t v_rs,
+                    int64_t v_cs, const void *w, int64_t w_rs, int64_t w_cs, int64_t t, void *out, int64_t out_rs,
+                    int64_t out_cs, int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+    g_err[0] = 0;
+    if (dtype == FLK_F32)
+        return fdmmv_impl<float>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w, w_rs,
+                                 w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    if (dtype == FLK_F64)
+        return fdmmv_impl<double>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w, w_rs,
+                                  w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
+}  // extern "C"

@@ -1,0 +1,84 @@
+// Shared declarations of the falkon_amd native library (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/falkon_amd.h"
+
+namespace flk {
+
+// sqrt(log2(e)): rows are scaled by this over sigma so that
+// exp(-1/2 |x/s - c/s|^2) == exp2(x~.c~ - 1/2|x~|^2 - 1/2|c~|^2) with a bare v_exp_f32.
+constexpr double kSqrtLog2e = 1.2011224087864498;
+
+// Packed-operand geometry.  f32: blocks of 32 rows, features split over the two
+// lane halves of a wave (MFMA 32x32x2).  f64: blocks of 16 rows, features split
+// over the four lane quarters (MFMA 16x16x4).
+template <typename T> struct Geo;
+template <> struct Geo<float>  { static constexpr int BLK = 32; static constexpr int KG = 2; };
+template <> struct Geo<double> { static constexpr int BLK = 16; static constexpr int KG = 4; };
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
+
+struct PackedView {
+    const void *data;   // [nblk][dpad][BLK]
+    const void *hnorm;  // [npad]  -1/2 * |x~|^2, zero on padding rows
+    int64_t n, d, dpad, nblk, npad;
+};
+
+template <typename T>
+inline PackedView packed_view(const void *buf, int64_t n, int64_t d) {
+    PackedView v;
+    v.n = n; v.d = d;
+    v.dpad = round_up(d, Geo<T>::KG);
+    v.nblk = (n + Geo<T>::BLK - 1) / Geo<T>::BLK;
+    v.npad = v.nblk * Geo<T>::BLK;
+    v.data = buf;
+    v.hnorm = (const char *)buf + align256((size_t)v.nblk * v.dpad * Geo<T>::BLK * sizeof(T));
+    return v;
+}
+template <typename T>
+inline size_t packed_bytes(int64_t n, int64_t d) {
+    int64_t dpad = round_up(d, Geo<T>::KG);
+    int64_t nblk = (n + Geo<T>::BLK - 1) / Geo<T>::BLK;
+    return align256((size_t)nblk * dpad * Geo<T>::BLK * sizeof(T)) + align256((size_t)nblk * Geo<T>::BLK * sizeof(T));
+}
+
+// error plumbing -------------------------------------------------------------
+int fail(int code, const char *fmt, ...);
+#define FLK_HIP(expr)                                                                      \
+    do {                                                                                   \
+        hipError_t e__ = (expr);                                                           \
+        if (e__ != hipSuccess)                                                             \
+            return ::flk::fail(FLK_EHIP, "%s failed: %s", #expr, hipGetErrorString(e__));  \
+    } while (0)
+#define FLK_LAUNCH_CHECK(name)                                                              \
+    do {                                                                                   \
+        hipError_t e__ = hipGetLastError();                                                \
+        if (e__ != hipSuccess)                                                             \
+            return ::flk::fail(FLK_EHIP, "launch of %s failed: %s", name, hipGetErrorString(e__)); \
+    } while (0)
+
+// launchers implemented in the .hip files -------------------------------------
+template <typename T>
+int launch_pack(const T *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const T *sigma, int64_t n_sigma,
+                T *pdata, T *hnorm, int64_t dpad, int64_t nblk, hipStream_t st);
+
+template <typename T>
+int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad, hipStream_t st);
+
+template <typename T>
+int launch_finalize(const T *partial, int splits, int64_t t, int64_t nb, int64_t nb_pad, const T *addend,
+                    int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
+                    hipStream_t st);
+
+// Register-resident ("small d") product kernel.  Returns FLK_EUNSUPPORTED if dpad is out of its range.
+template <typename T>
+int launch_mmv_small(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tt,
+                     int64_t a_chunk_blocks, int splits, T *partial, hipStream_t st);
+template <typename T> int64_t mmv_small_max_d();
+template <typename T> int mmv_small_b_blocks_per_wg(int64_t dpad);
+
+}  // namespace flk

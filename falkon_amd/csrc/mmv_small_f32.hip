@@ -1,0 +1,197 @@
+// Register-resident Gaussian kernel-vector product, fp32, gfx950.
+//
+//   partial[split][t][b] = sum_{a in chunk(split)} exp2(A~_a . B~_b + hA_a + hB_b) * vec[a,t]
+//
+// The kernel matrix is never stored.  A wave owns FR blocks of 32 output rows
+// (the "B side") whose packed features stay in registers for the whole kernel,
+// and streams blocks of 32 reduction rows (the "A side") straight from L2/HBM
+// into registers (the packed layout makes every load a contiguous 128-byte run
+// per half wave).  For every (A block, B block) pair the 32x32 cross term is
+// v_mfma_f32_32x32x2_f32 accumulated over the features, started from the two
+// half norms, so the accumulator holds the base-2 exponent directly; then
+// clamp-at-zero, v_exp_f32 and T FMAs per entry contract it against vec.
+// Accumulator layout of the 32x32x2 MFMA: lane l, register r holds
+//   column j = l % 32 (B row), row i = 8*(r/4) + 4*(l/32) + r%4 (A row),
+// so a lane sums over A rows privately and needs no cross-lane traffic until
+// the very end (one xor-32 shuffle to join the two lane halves).
+#include "flk_common.h"
+
+namespace flk {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWavesPerWg = 4;
+constexpr int kFlushEvery = 16;  // A blocks between flushes of the short accumulator
+
+__device__ __forceinline__ float kexp2_clamped(float x) {
+    // min(exp2(x), 1) == exp2(min(x, 0)): the reference clamps the squared distance at
+    // 1e-20 before exp (distance_kernel.py:100,157-158), i.e. K <= 1.  The median-of-three
+    // with 0 and 1 folds into the clamp bit of v_exp_f32, so the clamp costs no instruction.
+    return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(x), 0.0f, 1.0f);
+}
+
+template <int DP, int TT>
+struct AFrag {
+    float a[DP];        // features h*DP + s of row j of the A block
+    floatx4 hn[4];      // half norms of the 16 A rows this lane accumulates over
+    floatx4 vec[TT][4]; // right-hand side entries of those rows
+};
+
+template <int DP, int TT>
+__device__ __forceinline__ void load_afrag(AFrag<DP, TT> &f, const float *__restrict__ PA,
+                                           const float *__restrict__ hA, const float *__restrict__ vecp,
+                                           int64_t vec_ld, int64_t ab, int j, int h) {
+    const float *p = PA + (ab * (2 * DP) + (int64_t)h * DP) * 32 + j;
+#pragma unroll
+    for (int s = 0; s < DP; s++) f.a[s] = p[s * 32];
+    const int64_t r0 = ab * 32 + 4 * h;
+#pragma unroll
+    for (int g = 0; g < 4; g++) f.hn[g] = *(const floatx4 *)(hA + r0 + 8 * g);
+#pragma unroll
+    for (int t = 0; t < TT; t++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) f.vec[t][g] = *(const floatx4 *)(vecp + t * vec_ld + r0 + 8 * g);
+}
+
+template <int DP, int FR, int TT>
+__device__ __forceinline__ void tile_step(const AFrag<DP, TT> &f, const float (&breg)[FR][DP], const float (&hb)[FR],
+                                          float (&o1)[FR][TT]) {
+    floatx16 acc[FR];
+#pragma unroll
+    for (int q = 0; q < FR; q++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[q][r] = f.hn[r >> 2][r & 3] + hb[q];
+#pragma unroll
+    for (int s = 0; s < DP; s++)
+#pragma unroll
+        for (int q = 0; q < FR; q++) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[s], breg[q][s], acc[q], 0, 0, 0);
+#pragma unroll
+    for (int q = 0; q < FR; q++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            float k = kexp2_clamped(acc[q][r]);
+#pragma unroll
+            for (int t = 0; t < TT; t++) o1[q][t] = __builtin_fmaf(k, f.vec[t][r >> 2][r & 3], o1[q][t]);
+        }
+}
+
+template <int DP, int FR, int TT>
+__global__ void __launch_bounds__(256)
+    mmv_small_f32_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
+                         int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB, int64_t na_blocks,
+                         int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial, int64_t nb_pad) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int j = lane & 31, h = lane >> 5;
+    const int64_t bb0 = ((int64_t)blockIdx.x * kWavesPerWg + wave) * FR;
+    if (bb0 >= nb_blocks) return;  // whole wave idle; no barriers in this kernel
+    const int64_t a0 = (int64_t)blockIdx.y * a_chunk_blocks;
+    int64_t a1 = a0 + a_chunk_blocks;
+    if (a1 > na_blocks) a1 = na_blocks;
+
+    // resident B fragments (blocks past the end re-read the last block; their results are not stored)
+    float breg[FR][DP];
+    float hb[FR];
+#pragma unroll
+    for (int q = 0; q < FR; q++) {
+        int64_t bb = bb0 + q < nb_blocks ? bb0 + q : nb_blocks - 1;
+        const float *p = PB + (bb * (2 * DP) + (int64_t)h * DP) * 32 + j;
+#pragma unroll
+        for (int s = 0; s < DP; s++) breg[q][s] = p[s * 32];
+        hb[q] = hB[bb * 32 + j];
+    }
+
+    float o1[FR][TT], o2[FR][TT];
+#pragma unroll
+    for (int q = 0; q < FR; q++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) { o1[q][t] = 0.f; o2[q][t] = 0.f; }
+
+    AFrag<DP, TT> f0, f1;
+    if (a0 < a1) load_afrag<DP, TT>(f0, PA, hA, vecp, vec_ld, a0, j, h);
+    int since_flush = 0;
+    for (int64_t ab = a0; ab < a1; ab += 2) {
+        const bool has1 = ab + 1 < a1;
+        if (has1) load_afrag<DP, TT>(f1, PA, hA, vecp, vec_ld, ab + 1, j, h);
+        tile_step<DP, FR, TT>(f0, breg, hb, o1);
+        if (has1) {
+            if (ab + 2 < a1) load_afrag<DP, TT>(f0, PA, hA, vecp, vec_ld, ab + 2, j, h);
+            tile_step<DP, FR, TT>(f1, breg, hb, o1);
+        }
+        since_flush += 2;
+        if (since_flush >= kFlushEvery) {
+            since_flush = 0;
+#pragma unroll
+            for (int q = 0; q < FR; q++)
+#pragma unroll
+                for (int t = 0; t < TT; t++) { o2[q][t] += o1[q][t]; o1[q][t] = 0.f; }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < FR; q++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            float s = o2[q][t] + o1[q][t];
+            s += __shfl_xor(s, 32, 64);
+            if (h == 0 && bb0 + q < nb_blocks)
+                partial[((int64_t)blockIdx.y * TT + t) * nb_pad + (bb0 + q) * 32 + j] = s;
+        }
+}
+
+// ---------------------------------------------------------------------------
+// dispatch
+// ---------------------------------------------------------------------------
+constexpr int kMaxDpFr4 = 16;  // dpad <= 32: four resident B blocks per wave
+constexpr int kMaxDpFr2 = 32;  // dpad <= 64: two
+
+template <> int64_t mmv_small_max_d<float>() { return 2 * kMaxDpFr2; }
+template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad) {
+    return kWavesPerWg * ((dpad / 2) <= kMaxDpFr4 ? 4 : 2);
+}
+
+template <int DP, int FR, int TT>
+static int launch_one(const PackedView &A, const PackedView &B, const float *vecp, int64_t vec_ld,
+                      int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
+    const int64_t per_wg = kWavesPerWg * FR;
+    dim3 grid((unsigned)((B.nblk + per_wg - 1) / per_wg), (unsigned)splits);
+    hipLaunchKernelGGL((mmv_small_f32_kernel<DP, FR, TT>), grid, dim3(256), 0, st, (const float *)A.data,
+                       (const float *)A.hnorm, vecp, vec_ld, (const float *)B.data, (const float *)B.hnorm, A.nblk,
+                       B.nblk, a_chunk_blocks, partial, B.npad);
+    FLK_LAUNCH_CHECK("mmv_small_f32_kernel");
+    return FLK_OK;
+}
+
+template <int DP, int FR>
+static int launch_tt(int tt, const PackedView &A, const PackedView &B, const float *vecp, int64_t vec_ld,
+                     int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
+    switch (tt) {
+        case 1: return launch_one<DP, FR, 1>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 2: return launch_one<DP, FR, 2>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 3: return launch_one<DP, FR, 3>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 4: return launch_one<DP, FR, 4>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+    }
+    return fail(FLK_EINVAL, "mmv_small: column chunk %d not in 1..4", tt);
+}
+
+template <>
+int launch_mmv_small<float>(const PackedView &A, const PackedView &B, const float *vecp, int64_t vec_ld, int tt,
+                            int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
+    if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_small: operands packed with different feature counts");
+    const int dp = (int)(A.dpad / 2);
+#define FLK_CASE4(DPV) \
+    case DPV: return launch_tt<DPV, 4>(tt, A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+#define FLK_CASE2(DPV) \
+    case DPV: return launch_tt<DPV, 2>(tt, A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+    switch (dp) {
+        FLK_CASE4(1) FLK_CASE4(2) FLK_CASE4(3) FLK_CASE4(4) FLK_CASE4(5) FLK_CASE4(6) FLK_CASE4(7) FLK_CASE4(8)
+        FLK_CASE4(9) FLK_CASE4(10) FLK_CASE4(11) FLK_CASE4(12) FLK_CASE4(13) FLK_CASE4(14) FLK_CASE4(15) FLK_CASE4(16)
+        FLK_CASE2(17) FLK_CASE2(18) FLK_CASE2(19) FLK_CASE2(20) FLK_CASE2(21) FLK_CASE2(22) FLK_CASE2(23) FLK_CASE2(24)
+        FLK_CASE2(25) FLK_CASE2(26) FLK_CASE2(27) FLK_CASE2(28) FLK_CASE2(29) FLK_CASE2(30) FLK_CASE2(31) FLK_CASE2(32)
+    }
+#undef FLK_CASE4
+#undef FLK_CASE2
+    return fail(FLK_EUNSUPPORTED, "mmv_small<f32>: padded feature count %lld not in 2..64", (long long)A.dpad);
+}
+
+}  // namespace flk

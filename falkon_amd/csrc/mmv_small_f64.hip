@@ -1,0 +1,183 @@
+// Register-resident Gaussian kernel-vector product, fp64, gfx950.
+//
+// Same structure as the fp32 kernel with the 16x16x4 fp64 MFMA: a wave keeps FR
+// blocks of 16 output rows (B side) in registers and streams blocks of 16
+// reduction rows (A side).  Lane l supplies features q*DP + s (q = l / 16) of
+// block position l % 16.  Accumulator register r of lane l holds
+//   column j = l % 16 (B position), row 4*r + q (A position);
+// positions map to matrix rows through the packing order pos(row) =
+// 4*(row%4) + row/4, so a lane's four accumulator rows are the consecutive
+// matrix rows 4*q .. 4*q+3 of the A block.
+#include "flk_common.h"
+
+namespace flk {
+
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWavesPerWg64 = 4;
+constexpr int kFlushEvery64 = 16;
+
+__device__ __forceinline__ double kexp2_clamped(double x) {
+    // exp2(min(x, 0)): the reference clamps the squared distance at 1e-20 before exp
+    // (distance_kernel.py:100,157-158), i.e. K <= 1.
+    return exp2(fmin(x, 0.0));
+}
+
+template <int DP, int TT>
+struct AFrag64 {
+    double a[DP];
+    doublex4 hn;
+    doublex4 vec[TT];
+};
+
+template <int DP, int TT>
+__device__ __forceinline__ void load_afrag64(AFrag64<DP, TT> &f, const double *__restrict__ PA,
+                                             const double *__restrict__ hA, const double *__restrict__ vecp,
+                                             int64_t vec_ld, int64_t ab, int j, int q) {
+    const double *p = PA + (ab * (4 * DP) + (int64_t)q * DP) * 16 + j;
+#pragma unroll
+    for (int s = 0; s < DP; s++) f.a[s] = p[s * 16];
+    const int64_t r0 = ab * 16 + 4 * q;
+    f.hn = *(const doublex4 *)(hA + r0);
+#pragma unroll
+    for (int t = 0; t < TT; t++) f.vec[t] = *(const doublex4 *)(vecp + t * vec_ld + r0);
+}
+
+template <int DP, int FR, int TT>
+__device__ __forceinline__ void tile_step64(const AFrag64<DP, TT> &f, const double (&breg)[FR][DP],
+                                            const double (&hb)[FR], double (&o1)[FR][TT]) {
+    doublex4 acc[FR];
+#pragma unroll
+    for (int c = 0; c < FR; c++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[c][r] = f.hn[r] + hb[c];
+#pragma unroll
+    for (int s = 0; s < DP; s++)
+#pragma unroll
+        for (int c = 0; c < FR; c++) acc[c] = __builtin_amdgcn_mfma_f64_16x16x4f64(f.a[s], breg[c][s], acc[c], 0, 0, 0);
+#pragma unroll
+    for (int c = 0; c < FR; c++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            double k = kexp2_clamped(acc[c][r]);
+#pragma unroll
+            for (int t = 0; t < TT; t++) o1[c][t] = __builtin_fma(k, f.vec[t][r], o1[c][t]);
+        }
+}
+
+template <int DP, int FR, int TT>
+__global__ void __launch_bounds__(256)
+    mmv_small_f64_kernel(const double *__restrict__ PA, const double *__restrict__ hA, const double *__restrict__ vecp,
+                         int64_t vec_ld, const double *__restrict__ PB, const double *__restrict__ hB,
+                         int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks, double *__restrict__ partial,
+                         int64_t nb_pad) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int j = lane & 15, q = lane >> 4;
+    const int jrow = 4 * (j & 3) + (j >> 2);  // matrix row (within its block) held at position j
+    const int64_t bb0 = ((int64_t)blockIdx.x * kWavesPerWg64 + wave) * FR;
+    if (bb0 >= nb_blocks) return;
+    const int64_t a0 = (int64_t)blockIdx.y * a_chunk_blocks;
+    int64_t a1 = a0 + a_chunk_blocks;
+    if (a1 > na_blocks) a1 = na_blocks;
+
+    double breg[FR][DP];
+    double hb[FR];
+#pragma unroll
+    for (int c = 0; c < FR; c++) {
+        int64_t bb = bb0 + c < nb_blocks ? bb0 + c : nb_blocks - 1;
+        const double *p = PB + (bb * (4 * DP) + (int64_t)q * DP) * 16 + j;
+#pragma unroll
+        for (int s = 0; s < DP; s++) breg[c][s] = p[s * 16];
+        hb[c] = hB[bb * 16 + jrow];
+    }
+
+    double o1[FR][TT], o2[FR][TT];
+#pragma unroll
+    for (int c = 0; c < FR; c++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) { o1[c][t] = 0.0; o2[c][t] = 0.0; }
+
+    AFrag64<DP, TT> f0, f1;
+    if (a0 < a1) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, a0, j, q);
+    int since_flush = 0;
+    for (int64_t ab = a0; ab < a1; ab += 2) {
+        const bool has1 = ab + 1 < a1;
+        if (has1) load_afrag64<DP, TT>(f1, PA, hA, vecp, vec_ld, ab + 1, j, q);
+        tile_step64<DP, FR, TT>(f0, breg, hb, o1);
+        if (has1) {
+            if (ab + 2 < a1) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, ab + 2, j, q);
+            tile_step64<DP, FR, TT>(f1, breg, hb, o1);
+        }
+        since_flush += 2;
+        if (since_flush >= kFlushEvery64) {
+            since_flush = 0;
+#pragma unroll
+            for (int c = 0; c < FR; c++)
+#pragma unroll
+                for (int t = 0; t < TT; t++) { o2[c][t] += o1[c][t]; o1[c][t] = 0.0; }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < FR; c++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            double s = o2[c][t] + o1[c][t];
+            s += __shfl_xor(s, 16, 64);
+            s += __shfl_xor(s, 32, 64);
+            if (q == 0 && bb0 + c < nb_blocks)
+                partial[((int64_t)blockIdx.y * TT + t) * nb_pad + (bb0 + c) * 16 + jrow] = s;
+        }
+}
+
+constexpr int kMaxDp64Fr4 = 8;   // dpad <= 32
+constexpr int kMaxDp64Fr2 = 16;  // dpad <= 64
+
+template <> int64_t mmv_small_max_d<double>() { return 4 * kMaxDp64Fr2; }
+template <> int mmv_small_b_blocks_per_wg<double>(int64_t dpad) {
+    return kWavesPerWg64 * ((dpad / 4) <= kMaxDp64Fr4 ? 4 : 2);
+}
+
+template <int DP, int FR, int TT>
+static int launch_one64(const PackedView &A, const PackedView &B, const double *vecp, int64_t vec_ld,
+                        int64_t a_chunk_blocks, int splits, double *partial, hipStream_t st) {
+    const int64_t per_wg = kWavesPerWg64 * FR;
+    dim3 grid((unsigned)((B.nblk + per_wg - 1) / per_wg), (unsigned)splits);
+    hipLaunchKernelGGL((mmv_small_f64_kernel<DP, FR, TT>), grid, dim3(256), 0, st, (const double *)A.data,
+                       (const double *)A.hnorm, vecp, vec_ld, (const double *)B.data, (const double *)B.hnorm, A.nblk,
+                       B.nblk, a_chunk_blocks, partial, B.npad);
+    FLK_LAUNCH_CHECK("mmv_small_f64_kernel");
+    return FLK_OK;
+}
+
+template <int DP, int FR>
+static int launch_tt64(int tt, const PackedView &A, const PackedView &B, const double *vecp, int64_t vec_ld,
+                       int64_t a_chunk_blocks, int splits, double *partial, hipStream_t st) {
+    switch (tt) {
+        case 1: return launch_one64<DP, FR, 1>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 2: return launch_one64<DP, FR, 2>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 3: return launch_one64<DP, FR, 3>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 4: return launch_one64<DP, FR, 4>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+    }
+    return fail(FLK_EINVAL, "mmv_small: column chunk %d not in 1..4", tt);
+}
+
+template <>
+int launch_mmv_small<double>(const PackedView &A, const PackedView &B, const double *vecp, int64_t vec_ld, int tt,
+                             int64_t a_chunk_blocks, int splits, double *partial, hipStream_t st) {
+    if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_small: operands packed with different feature counts");
+    const int dp = (int)(A.dpad / 4);
+#define FLK_CASE4(DPV) \
+    case DPV: return launch_tt64<DPV, 4>(tt, A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+#define FLK_CASE2(DPV) \
+    case DPV: return launch_tt64<DPV, 2>(tt, A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+    switch (dp) {
+        FLK_CASE4(1) FLK_CASE4(2) FLK_CASE4(3) FLK_CASE4(4) FLK_CASE4(5) FLK_CASE4(6) FLK_CASE4(7) FLK_CASE4(8)
+        FLK_CASE2(9) FLK_CASE2(10) FLK_CASE2(11) FLK_CASE2(12) FLK_CASE2(13) FLK_CASE2(14) FLK_CASE2(15) FLK_CASE2(16)
+    }
+#undef FLK_CASE4
+#undef FLK_CASE2
+    return fail(FLK_EUNSUPPORTED, "mmv_small<f64>: padded feature count %lld not in 4..64", (long long)A.dpad);
+}
+
+}  // namespace flk

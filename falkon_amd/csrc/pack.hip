@@ -1,0 +1,136 @@
+// Prologue / epilogue kernels: operand packing, planar right-hand sides, split reduction.
+#include "flk_common.h"
+
+namespace flk {
+
+// ---------------------------------------------------------------------------
+// pack: X[n,d] (any unit-stride order) -> [nblk][dpad][BLK] scaled by sqrt(log2 e)/sigma,
+// plus hnorm[row] = -1/2 |x~|^2.  One workgroup per block of BLK rows; a
+// BLK x 32 tile goes through LDS so that both the read (along the unit stride
+// of X) and the write (along rows of the block) are coalesced.
+// Row r of an f64 block is stored at position 4*(r%4) + r/4: the 16x16x4 MFMA
+// hands lane quarter q the accumulator rows q, q+4, q+8, q+12, and with this
+// order those are four consecutive rows of the matrix.
+// ---------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ int block_pos(int r);
+template <> __device__ __forceinline__ int block_pos<float>(int r) { return r; }
+template <> __device__ __forceinline__ int block_pos<double>(int r) { return 4 * (r & 3) + (r >> 2); }
+
+template <typename T>
+__global__ void __launch_bounds__(256) pack_kernel(const T *__restrict__ X, int64_t n, int64_t d, int64_t rs,
+                                                   int64_t cs, const T *__restrict__ sigma, int64_t n_sigma,
+                                                   T *__restrict__ pdata, T *__restrict__ hnorm, int64_t dpad) {
+    constexpr int BLK = Geo<T>::BLK;
+    constexpr int KT = 32;                       // features per LDS tile
+    __shared__ T tile[BLK][KT + 1];
+    __shared__ double nrm[BLK];
+    const int tid = threadIdx.x;
+    const int64_t blk = blockIdx.x;
+    const int64_t row0 = blk * BLK;
+    if (tid < BLK) nrm[tid] = 0.0;
+    const bool row_major = (cs == 1);
+    for (int64_t k0 = 0; k0 < dpad; k0 += KT) {
+        __syncthreads();
+        // load + scale
+        for (int e = tid; e < BLK * KT; e += 256) {
+            int r, k;
+            if (row_major) { r = e / KT; k = e % KT; } else { k = e / BLK; r = e % BLK; }
+            int64_t row = row0 + r, kk = k0 + k;
+            T val = T(0);
+            if (row < n && kk < d) {
+                double s = kSqrtLog2e / (double)sigma[n_sigma == 1 ? 0 : kk];
+                val = (T)((double)X[row * rs + kk * cs] * s);
+            }
+            tile[r][k] = val;
+        }
+        __syncthreads();
+        // store feature-major
+        for (int e = tid; e < BLK * KT; e += 256) {
+            int k = e / BLK, r = e % BLK;
+            int64_t kk = k0 + k;
+            if (kk < dpad) pdata[(blk * dpad + kk) * BLK + block_pos<T>(r)] = tile[r][k];
+        }
+        if (tid < BLK) {
+            double s = 0.0;
+            int kmax = (int)((dpad - k0) < KT ? (dpad - k0) : KT);
+            for (int k = 0; k < kmax; k++) { double x = (double)tile[tid][k]; s += x * x; }
+            nrm[tid] += s;
+        }
+    }
+    if (tid < BLK) hnorm[row0 + tid] = (T)(-0.5 * nrm[tid]);
+}
+
+template <typename T>
+int launch_pack(const T *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const T *sigma, int64_t n_sigma,
+                T *pdata, T *hnorm, int64_t dpad, int64_t nblk, hipStream_t st) {
+    if (nblk == 0) return FLK_OK;
+    hipLaunchKernelGGL(pack_kernel<T>, dim3((unsigned)nblk), dim3(256), 0, st, X, n, d, rs, cs, sigma, n_sigma, pdata,
+                       hnorm, dpad);
+    FLK_LAUNCH_CHECK("pack_kernel");
+    return FLK_OK;
+}
+template int launch_pack<float>(const float *, int64_t, int64_t, int64_t, int64_t, const float *, int64_t, float *,
+                                float *, int64_t, int64_t, hipStream_t);
+template int launch_pack<double>(const double *, int64_t, int64_t, int64_t, int64_t, const double *, int64_t, double *,
+                                 double *, int64_t, int64_t, hipStream_t);
+
+// ---------------------------------------------------------------------------
+// vec_planar: v[n,t] with element strides (rs, cs) -> vp[t][npad], zero padded.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) vec_planar_kernel(const T *__restrict__ v, int64_t n, int64_t rs, int64_t cs,
+                                                         T *__restrict__ vp, int64_t npad) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    int64_t t = blockIdx.y;
+    if (i < npad) vp[t * npad + i] = (i < n) ? v[i * rs + t * cs] : T(0);
+}
+template <typename T>
+int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad, hipStream_t st) {
+    if (npad == 0 || t == 0) return FLK_OK;
+    hipLaunchKernelGGL(vec_planar_kernel<T>, dim3((unsigned)((npad + 255) / 256), (unsigned)t), dim3(256), 0, st, v, n,
+                       rs, cs, vp, npad);
+    FLK_LAUNCH_CHECK("vec_planar_kernel");
+    return FLK_OK;
+}
+template int launch_vec_planar<float>(const float *, int64_t, int64_t, int64_t, int64_t, float *, int64_t, hipStream_t);
+template int launch_vec_planar<double>(const double *, int64_t, int64_t, int64_t, int64_t, double *, int64_t,
+                                       hipStream_t);
+
+// ---------------------------------------------------------------------------
+// finalize: out[b,t] = sum_s partial[s][t][b] (+ addend[b,t]); fixed summation
+// order, so results are reproducible run to run (no atomics anywhere).
+// With zero_pad the rows n_b..nb_pad of a planar output are cleared as well.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) finalize_kernel(const T *__restrict__ partial, int splits, int64_t tt,
+                                                       int64_t nb, int64_t nb_pad, const T *__restrict__ addend,
+                                                       int64_t add_rs, int64_t add_cs, T *__restrict__ out,
+                                                       int64_t out_rs, int64_t out_cs, bool zero_pad) {
+    int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    int64_t t = blockIdx.y;
+    if (b >= nb_pad) return;
+    if (b >= nb) {
+        if (zero_pad) out[b * out_rs + t * out_cs] = T(0);
+        return;
+    }
+    double s = 0.0;
+    for (int sp = 0; sp < splits; sp++) s += (double)partial[((int64_t)sp * tt + t) * nb_pad + b];
+    if (addend) s += (double)addend[b * add_rs + t * add_cs];
+    out[b * out_rs + t * out_cs] = (T)s;
+}
+template <typename T>
+int launch_finalize(const T *partial, int splits, int64_t t, int64_t nb, int64_t nb_pad, const T *addend,
+                    int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
+                    hipStream_t st) {
+    if (nb_pad == 0 || t == 0) return FLK_OK;
+    hipLaunchKernelGGL(finalize_kernel<T>, dim3((unsigned)((nb_pad + 255) / 256), (unsigned)t), dim3(256), 0, st,
+                       partial, splits, t, nb, nb_pad, addend, add_rs, add_cs, out, out_rs, out_cs, zero_pad);
+    FLK_LAUNCH_CHECK("finalize_kernel");
+    return FLK_OK;
+}
+template int launch_finalize<float>(const float *, int, int64_t, int64_t, int64_t, const float *, int64_t, int64_t,
+                                    float *, int64_t, int64_t, bool, hipStream_t);
+template int launch_finalize<double>(const double *, int, int64_t, int64_t, int64_t, const double *, int64_t, int64_t,
+                                     double *, int64_t, int64_t, bool, hipStream_t);
+
+}  // namespace flk

@@ -1,0 +1,136 @@
+"""Kernel base class: the plugin API whose ``mmv`` / ``dmmv`` this build sits behind.
+
+Same public surface as falkon/kernels/kernel.py:14-577: argument validation, per-call option
+override by ``dataclasses.replace``, and the ``_decide_*_impl`` hooks that pick the backend
+callable.  The hooks return this build's ``fmmv`` / ``fdmmv`` (MI355X only).
+"""
+import dataclasses
+from abc import ABC, abstractmethod
+from typing import Dict, Optional
+
+import torch
+
+from ..mmv_ops.fmmv import fdmmv, fmmv
+from ..options import FalkonOptions
+from ..utils.helpers import check_same_device, check_same_dtype
+
+__all__ = ("Kernel",)
+
+
+class Kernel(torch.nn.Module, ABC):
+    def __init__(self, name: str, opt: Optional[FalkonOptions]):
+        super().__init__()
+        self.name = name
+        self.params: FalkonOptions = opt if opt is not None else FalkonOptions()
+
+    # -- validation (falkon/kernels/kernel.py:44-127) ---------------------------------------
+    @staticmethod
+    def _check_dmmv_dimensions(X1, X2, v, w, out):
+        if v is None and w is None:
+            raise ValueError("One of v and w must be specified to run fdMMV.")
+        if X1.dim() != 2:
+            raise ValueError("Matrix X1 must be 2D.")
+        if X2.dim() != 2:
+            raise ValueError("Matrix X2 must be 2D.")
+        if v is not None and v.dim() == 1:
+            v = v.reshape((-1, 1))
+        if v is not None and v.dim() != 2:
+            raise ValueError(f"v must be a vector or a 2D matrix. Found {len(v.shape)}D.")
+        if w is not None and w.dim() == 1:
+            w = w.reshape((-1, 1))
+        if w is not None and w.dim() != 2:
+            raise ValueError(f"w must be a vector or a 2D matrix. Found {len(w.shape)}D.")
+        T = v.size(1) if v is not None else w.size(1)
+        M = X2.size(0)
+        if out is not None and out.shape != (M, T):
+            raise ValueError(f"Output dimension is incorrect. Expected ({M}, {T}) found {out.shape}")
+        if v is not None and v.shape != (X2.size(0), T):
+            raise ValueError(f"Dimensions of matrix v are incorrect: Expected ({M}, {T}) found {v.shape}")
+        if w is not None and w.shape != (X1.size(0), T):
+            raise ValueError(f"Dimensions of matrix w are incorrect: Expected ({X1.size(0)}, {T}) found {w.shape}")
+        if not check_same_dtype(X1, X2, v, w, out):
+            raise TypeError("Data types of input matrices must be equal.")
+        return X1, X2, v, w, out
+
+    @staticmethod
+    def _check_mmv_dimensions(X1, X2, v, out):
+        if X1.dim() != 2:
+            raise ValueError("Matrix X1 must be 2D.")
+        if X2.dim() != 2:
+            raise ValueError("Matrix X2 must be 2D.")
+        if v.dim() == 1:
+            v = v.reshape((-1, 1))
+        if v.dim() != 2:
+            raise ValueError(f"v must be a vector or a 2D matrix. Found {len(v.shape)}D.")
+        if out is not None and out.shape != (X1.size(0), v.size(1)):
+            raise ValueError(f"Output dimension is incorrect. Expected ({X1.size(0)}, {v.size(1)}) found {out.shape}")
+        if v.shape != (X2.size(0), v.size(1)):
+            raise ValueError(
+                f"Dimensions of matrix v are incorrect: Expected ({X2.size(0)}, {v.size(1)}) found {v.shape}")
+        if not check_same_dtype(X1, X2, v, out):
+            raise TypeError("Data types of input matrices must be equal.")
+        return X1, X2, v, out
+
+    @staticmethod
+    def _check_mm_dimensions(X1, X2, diag, out):
+        if X1.dim() != 2:
+            raise ValueError("Matrix X1 must be 2D.")
+        if X2.dim() != 2:
+            raise ValueError("Matrix X2 must be 2D.")
+        N, M = X1.size(0), X2.size(0)
+        if not diag:
+            if out is not None and out.shape != (N, M):
+                raise ValueError(f"Output dimension is incorrect. Expected ({N}, {M}) found {out.shape}.")
+        else:
+            if N != M:
+                raise ValueError(f"Cannot compute the kernel diagonal between matrices with {N} and {M} samples.")
+            if out is not None and out.reshape(-1).shape[0] != N:
+                raise ValueError(f"Output dimension is incorrect. Expected ({N}) found {out.shape}.")
+        if not check_same_dtype(X1, X2, out):
+            raise TypeError("Data types of input matrices must be equal.")
+        return X1, X2, out
+
+    @staticmethod
+    def _check_device_properties(*args, fn_name: str, opt):
+        if not check_same_device(*args):
+            raise RuntimeError(f"All input arguments to {fn_name} must be on the same device")
+
+    def _merged(self, opt: Optional[FalkonOptions]) -> FalkonOptions:
+        """Per-call options override the kernel's own (falkon/kernels/kernel.py:283-285)."""
+        if opt is None:
+            return self.params
+        return dataclasses.replace(self.params, **dataclasses.asdict(opt))
+
+    # -- products (falkon/kernels/kernel.py:226-459) --------------------------------------------
+    def mmv(self, X1, X2, v, out=None, opt: Optional[FalkonOptions] = None,
+            kwargs_m1: Optional[Dict[str, torch.Tensor]] = None, kwargs_m2: Optional[Dict[str, torch.Tensor]] = None):
+        """``K(X1, X2) @ v``: X1 (N x D), X2 (M x D), v (M x T) or (M,), result (N x T)."""
+        X1, X2, v, out = self._check_mmv_dimensions(X1, X2, v, out)
+        params = self._merged(opt)
+        mmv_impl = self._decide_mmv_impl(X1, X2, v, params)
+        return mmv_impl(X1=X1, X2=X2, v=v, kernel=self, out=out, opt=params, kwargs_m1=kwargs_m1, kwargs_m2=kwargs_m2)
+
+    def _decide_mmv_impl(self, X1, X2, v, opt: FalkonOptions):
+        return fmmv
+
+    def dmmv(self, X1, X2, v, w, out=None, opt: Optional[FalkonOptions] = None,
+             kwargs_m1: Optional[Dict[str, torch.Tensor]] = None, kwargs_m2: Optional[Dict[str, torch.Tensor]] = None):
+        """``K(X1, X2).T @ (K(X1, X2) @ v + w)``: v (M x T), w (N x T) or None, result (M x T)."""
+        X1, X2, v, w, out = self._check_dmmv_dimensions(X1, X2, v, w, out)
+        params = self._merged(opt)
+        dmmv_impl = self._decide_dmmv_impl(X1, X2, v, w, params)
+        return dmmv_impl(X1=X1, X2=X2, v=v, w=w, kernel=self, out=out, differentiable=False, opt=params,
+                         kwargs_m1=kwargs_m1, kwargs_m2=kwargs_m2)
+
+    def _decide_dmmv_impl(self, X1, X2, v, w, opt: FalkonOptions):
+        return fdmmv
+
+    @abstractmethod
+    def compute(self, X1: torch.Tensor, X2: torch.Tensor, out: torch.Tensor, diag: bool, **kwargs) -> torch.Tensor:
+        """Fill ``out`` with the kernel matrix of ``X1`` and ``X2`` (falkon/kernels/kernel.py:461-497)."""
+
+    def extra_mem(self, is_differentiable, is_sparse, dtype, density1=None, density2=None) -> Dict[str, float]:
+        return {}
+
+    def __str__(self):
+        return f"<{self.name} kernel>"

@@ -1,0 +1,236 @@
+"""Gaussian kernel-vector products on the MI355X: ``fmmv`` and ``fdmmv``.
+
+Drop-in for the two callables the reference's kernels dispatch to
+(falkon/mmv_ops/fmmv.py:960-973 ``fmmv`` and :976-1131 ``fdmmv``): same
+signatures, same validation, same ``out`` semantics, same exception types.
+The work itself is done by ``libfalkon_amd.so`` through its C ABI; the kernel
+matrix is never materialised, so the reference's memory-driven blocking over
+rows and columns (fmmv.py:60-114,488-544) reduces to "keep the whole problem
+resident; split the rows of X1 only if the packed operands do not fit".
+There is no CPU computation in this module.
+"""
+import math
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from .. import _backend
+from ..options import BaseOptions
+from ..utils.helpers import sizeof_dtype
+from .utils import check_contiguity, create_output_mat, usable_gpu_memory
+
+__all__ = ("fmmv", "fdmmv", "gauss_fmmv_native", "gauss_fdmmv_native")
+
+_DTYPE_CODE = {torch.float32: _backend.FLK_F32, torch.float64: _backend.FLK_F64}
+
+
+def _mat(t: torch.Tensor) -> Tuple[int, int, int, int]:
+    """(ptr, rows, row_stride, col_stride) of a 2-D tensor, strides in elements."""
+    return t.data_ptr(), t.shape[0], t.stride(0), t.stride(1)
+
+
+def _stream_handle(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def gauss_fmmv_native(X1, X2, sigma_dev, v, out) -> None:
+    """out[n,t] = K(X1,X2) @ v through ``flk_gauss_fmmv``.  All tensors on one GPU, 2-D, same dtype."""
+    lib = _backend.load()
+    code = _DTYPE_CODE[X1.dtype]
+    n, d = X1.shape
+    m, t = v.shape
+    ws_bytes = lib.flk_gauss_fmmv_workspace_bytes(n, m, d, t, code)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=X1.device)
+    p1, _, r1, c1 = _mat(X1)
+    p2, _, r2, c2 = _mat(X2)
+    pv, _, rv, cv = _mat(v)
+    po, _, ro, co = _mat(out)
+    with torch.cuda.device(X1.device):
+        rc = lib.flk_gauss_fmmv(p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
+                                pv, rv, cv, t, po, ro, co, code, ws.data_ptr(), ws_bytes, _stream_handle(X1.device))
+    _backend.raise_for_status(rc, "flk_gauss_fmmv")
+
+
+def gauss_fdmmv_native(X1, X2, sigma_dev, v, w, out) -> None:
+    """out[m,t] = K^T (K v + w) through ``flk_gauss_fdmmv``.  ``w`` may be None."""
+    lib = _backend.load()
+    code = _DTYPE_CODE[X1.dtype]
+    n, d = X1.shape
+    m, t = v.shape
+    ws_bytes = lib.flk_gauss_fdmmv_workspace_bytes(n, m, d, t, code)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=X1.device)
+    p1, _, r1, c1 = _mat(X1)
+    p2, _, r2, c2 = _mat(X2)
+    pv, _, rv, cv = _mat(v)
+    pw, rw, cw = (w.data_ptr(), w.stride(0), w.stride(1)) if w is not None else (None, 0, 0)
+    po, _, ro, co = _mat(out)
+    with torch.cuda.device(X1.device):
+        rc = lib.flk_gauss_fdmmv(p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
+                                 pv, rv, cv, pw, rw, cw, t, po, ro, co, code, ws.data_ptr(), ws_bytes,
+                                 _stream_handle(X1.device))
+    _backend.raise_for_status(rc, "flk_gauss_fdmmv")
+
+
+# ---------------------------------------------------------------------------
+# host-side planning
+# ---------------------------------------------------------------------------
+def _require_gaussian(kernel):
+    if getattr(kernel, "kernel_name", None) != "gaussian" or not hasattr(kernel, "sigma"):
+        raise NotImplementedError(
+            "falkon_amd accelerates the Gaussian kernel only; "
+            f"kernel '{getattr(kernel, 'name', type(kernel).__name__)}' has no MI355X kernel-vector path")
+
+
+def _reject_block_kwargs(kwargs_m1, kwargs_m2):
+    if kwargs_m1 or kwargs_m2:
+        # the reference forwards these to the kernel's core function, and the Gaussian core takes none
+        # (falkon/kernels/diff_kernel.py:90-91, distance_kernel.py:140-142)
+        raise TypeError("The Gaussian kernel takes no per-block keyword tensors (kwargs_m1 / kwargs_m2)")
+
+
+def _compute_device(opt: BaseOptions, data_devs) -> torch.device:
+    """The GPU to compute on; mirrors the reference's device choice (fmmv.py:906,1038) minus its CPU branch."""
+    if opt.use_cpu:
+        raise RuntimeError("falkon_amd has no CPU compute path: `use_cpu=True` cannot be honoured "
+                           "(the MI355X kernels are the only implementation)")
+    if not torch.cuda.is_available():
+        raise RuntimeError("falkon_amd needs a ROCm GPU (MI355X); torch.cuda.is_available() is False")
+    cuda_devs = {d for d in data_devs if d.type == "cuda"}
+    if len(cuda_devs) > 1:
+        raise RuntimeError("All GPU-resident inputs must be on the same device")
+    if cuda_devs:
+        return next(iter(cuda_devs))
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _rows_that_fit(n: int, bytes_for_rows, usable: float) -> int:
+    """Largest row count r <= n with bytes_for_rows(r) <= usable (bytes_for_rows is non-decreasing)."""
+    if bytes_for_rows(n) <= usable:
+        return n
+    lo, hi = 0, n
+    while hi - lo > 1:
+        mid = (lo + hi) // 2
+        if bytes_for_rows(mid) <= usable:
+            lo = mid
+        else:
+            hi = mid
+    if lo < 1:
+        raise MemoryError("Available memory %.2fMB is not enough." % (usable / 2**20))
+    return lo
+
+
+def _on(t: Optional[torch.Tensor], dev: torch.device) -> Optional[torch.Tensor]:
+    if t is None or t.device == dev:
+        return t
+    return t.to(dev, non_blocking=True)
+
+
+def _check_dtype(dtype):
+    if dtype not in _DTYPE_CODE:
+        raise TypeError(f"Dtype {dtype} not valid")
+
+
+def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optional[torch.Tensor] = None,
+         opt: Optional[BaseOptions] = None, kwargs_m1: Optional[Dict[str, torch.Tensor]] = None,
+         kwargs_m2: Optional[Dict[str, torch.Tensor]] = None) -> torch.Tensor:
+    """``out = K(X1, X2) @ v`` (N x T), same contract as falkon/mmv_ops/fmmv.py:960-973 / :887-932."""
+    opt = opt if opt is not None else BaseOptions()
+    _require_gaussian(kernel)
+    _reject_block_kwargs(kwargs_m1, kwargs_m2)
+    check_contiguity((X1, "X1"), (X2, "X2"), (v, "v"), (out, "out"))
+    if any(t.requires_grad for t in [X1, X2, v] + list(kernel.diff_params.values())):
+        raise NotImplementedError("falkon_amd.fmmv does not implement the autograd backward pass; "
+                                  "detach the inputs and the kernel parameters")
+    _check_dtype(X1.dtype)
+    data_devs = (X1.device, X2.device, v.device)
+    dev = _compute_device(opt, data_devs)
+    N, D = X1.shape
+    M, T = v.shape
+    out = create_output_mat(out, data_devs, shape=(N, T), dtype=v.dtype, other_mat=X1)
+    lib = _backend.load()
+    code, sz = _DTYPE_CODE[X1.dtype], sizeof_dtype(X1.dtype)
+    x1_in, out_in = X1.device == dev, out.device == dev
+
+    with torch.inference_mode():
+        sigma_dev = kernel._sigma_on(dev, X1.dtype)
+        usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack)
+        fixed = (0 if X2.device == dev else M * D * sz) + (0 if v.device == dev else M * T * sz)
+
+        def need(rows: int) -> float:
+            stage = (0 if x1_in else rows * D * sz) + (0 if out_in else rows * T * sz)
+            return lib.flk_gauss_fmmv_workspace_bytes(rows, M, D, T, code) + stage + fixed
+
+        blk = _rows_that_fit(N, need, usable) if N > 0 else 0
+        X2d, vd = _on(X2, dev), _on(v, dev)
+        if blk == N:
+            X1d = _on(X1, dev)
+            outd = out if out_in else torch.empty((N, T), dtype=out.dtype, device=dev)
+            gauss_fmmv_native(X1d, X2d, sigma_dev, vd, outd)
+            if not out_in:
+                out.copy_(outd)
+        else:
+            for i in range(0, N, blk):
+                li = min(blk, N - i)
+                X1d = _on(X1[i:i + li], dev)
+                outd = out[i:i + li] if out_in else torch.empty((li, T), dtype=out.dtype, device=dev)
+                gauss_fmmv_native(X1d, X2d, sigma_dev, vd, outd)
+                if not out_in:
+                    out[i:i + li].copy_(outd)
+    return out
+
+
+def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch.Tensor], kernel,
+          out: Optional[torch.Tensor] = None, differentiable: bool = False, opt: Optional[BaseOptions] = None,
+          kwargs_m1: Optional[Dict[str, torch.Tensor]] = None,
+          kwargs_m2: Optional[Dict[str, torch.Tensor]] = None) -> torch.Tensor:
+    """``out = K(X1, X2).T @ (K(X1, X2) @ v + w)`` (M x T), same contract as falkon/mmv_ops/fmmv.py:976-1131.
+
+    ``v`` is required (the reference reads ``v.shape`` unconditionally, fmmv.py:1035-1041); ``w`` may be None.
+    """
+    opt = opt if opt is not None else BaseOptions()
+    if differentiable:
+        raise NotImplementedError(
+            "Manual D-MMV is not implemented for differentiable inputs. Try using the KeOps version instead.")
+    _require_gaussian(kernel)
+    _reject_block_kwargs(kwargs_m1, kwargs_m2)
+    check_contiguity((X1, "X1"), (X2, "X2"), (v, "v"), (out, "out"))
+    if v is None:
+        raise ValueError("fdmmv needs `v`; to compute K.T @ w alone call mmv(X2, X1, w)")
+    _check_dtype(X1.dtype)
+    data_devs = [X1.device, X2.device, v.device] + ([w.device] if w is not None else [])
+    dev = _compute_device(opt, data_devs)
+    N, D = X1.shape[-2:]
+    M, T = v.shape[-2:]
+    lib = _backend.load()
+    code, sz = _DTYPE_CODE[X1.dtype], sizeof_dtype(X1.dtype)
+
+    with torch.inference_mode():
+        out = create_output_mat(out, data_devs, shape=(M, T), dtype=v.dtype, other_mat=X1)
+        x1_in, out_in = X1.device == dev, out.device == dev
+        w_in = w is None or w.device == dev
+        sigma_dev = kernel._sigma_on(dev, X1.dtype)
+        usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack)
+        fixed = ((0 if X2.device == dev else M * D * sz) + (0 if v.device == dev else M * T * sz)
+                 + (0 if out_in else M * T * sz))
+
+        def need(rows: int) -> float:
+            stage = (0 if x1_in else rows * D * sz) + (0 if w_in else rows * T * sz)
+            extra = M * T * sz if rows < N else 0          # per-block result that is added into out
+            return lib.flk_gauss_fdmmv_workspace_bytes(rows, M, D, T, code) + stage + fixed + extra
+
+        blk = _rows_that_fit(N, need, usable) if N > 0 else 0
+        X2d, vd = _on(X2, dev), _on(v, dev)
+        outd = out if out_in else torch.empty((M, T), dtype=out.dtype, device=dev)
+        if blk == N:
+            gauss_fdmmv_native(_on(X1, dev), X2d, sigma_dev, vd, _on(w, dev), outd)
+        else:
+            tmp = torch.empty((M, T), dtype=out.dtype, device=dev)
+            for bi, i in enumerate(range(0, N, blk)):
+                li = min(blk, N - i)
+                wd = _on(w[i:i + li], dev) if w is not None else None
+                gauss_fdmmv_native(_on(X1[i:i + li], dev), X2d, sigma_dev, vd, wd, outd if bi == 0 else tmp)
+                if bi > 0:
+                    outd.add_(tmp)
+        if not out_in:
+            out.copy_(outd)
+    return out

@@ -1,0 +1,51 @@
+"""Validation, output allocation and device-memory budget for the kernel-vector drivers.
+
+Same rules as falkon/mmv_ops/utils.py:36-58,124-155.
+"""
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from ..utils.tensor_helpers import create_C, create_fortran, create_same_stride, is_contig
+
+__all__ = ("check_contiguity", "create_output_mat", "usable_gpu_memory")
+
+
+def check_contiguity(*args: Tuple[Optional[torch.Tensor], str]) -> None:
+    """Every given tensor needs a unit stride (falkon/mmv_ops/utils.py:36-39)."""
+    for tensor, name in args:
+        if tensor is not None and not is_contig(tensor):
+            raise ValueError(f"Tensor '{name}' must be memory contiguous")
+
+
+def create_output_mat(out: Optional[torch.Tensor], data_devs: Sequence[torch.device], shape: Tuple[int, int],
+                      dtype: torch.dtype, other_mat: torch.Tensor, output_stride: Optional[str] = None) -> torch.Tensor:
+    """Return ``out`` if given, else a new matrix on the first GPU the data lives on (the host,
+    pinned, if all data is on the host) laid out like ``other_mat``
+    (falkon/mmv_ops/utils.py:124-155)."""
+    if out is not None:
+        return out
+    out_dev = torch.device("cpu")
+    for ddev in data_devs:
+        if ddev.type == "cuda":
+            out_dev = ddev
+            break
+    pin = out_dev.type != "cuda"
+    if output_stride is None:
+        return create_same_stride(shape, other_mat, dtype, device=out_dev, pin_memory=pin)
+    if output_stride == "F":
+        return create_fortran(shape, dtype, device=out_dev, pin_memory=pin)
+    return create_C(shape, dtype, device=out_dev, pin_memory=pin)
+
+
+def usable_gpu_memory(dev: torch.device, max_gpu_mem: float, slack: float) -> float:
+    """Bytes a call may use on ``dev``: ``slack * min(free, max_gpu_mem)``
+    (falkon/mmv_ops/utils.py:47-58; free memory counts what torch's allocator holds cached,
+    falkon/utils/devices.py:84-96).  Raises MemoryError when nothing is left."""
+    free, _total = torch.cuda.mem_get_info(dev)
+    cached = torch.cuda.memory_reserved(dev) - torch.cuda.memory_allocated(dev)
+    usable = min((free + cached) * slack, max_gpu_mem * slack)
+    if usable < 0:
+        raise MemoryError(f"Usable memory on device {dev} is less than 0. Either there is no free memory "
+                          f"available, or the `max_gpu_mem` setting is too low.")
+    return usable

@@ -1,0 +1,117 @@
+/*
+ * falkon_amd -- C ABI of the MI355X (gfx950) Gaussian kernel-vector products.
+ *
+ * Every entry point is plain C: device pointers, sizes, element strides and a
+ * HIP stream handle (passed as void*).  No torch types cross this boundary.
+ * All functions return 0 on success or a negative FLK_E* code; the message of
+ * the last failure on the calling thread is available from flk_last_error().
+ * Nothing here synchronises the device or allocates device memory: work is
+ * enqueued on `stream`, scratch space comes from the caller (`workspace`).
+ *
+ * Matrices are described as (pointer, rows, cols, row_stride, col_stride) with
+ * strides in ELEMENTS, so both C-ordered (col_stride == 1) and Fortran-ordered
+ * (row_stride == 1) operands of the reference are accepted as they are
+ * (falkon/mmv_ops/utils.py:36-39 requires only that some stride equals one).
+ *
+ * dtype: FLK_F32 (0) or FLK_F64 (1); all operands of a call share it
+ * (falkon/kernels/kernel.py:78-79,102-103).
+ */
+#ifndef FALKON_AMD_H
+#define FALKON_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLK_F32 0
+#define FLK_F64 1
+
+#define FLK_OK          0
+#define FLK_EINVAL     -1   /* bad argument (shape, stride, dtype, null pointer)      */
+#define FLK_ENOMEM     -2   /* workspace too small                                    */
+#define FLK_EUNSUPPORTED -3 /* shape outside what the compiled kernels cover          */
+#define FLK_EHIP       -4   /* a HIP runtime call or kernel launch failed             */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int flk_version(void);
+
+/* Message describing the last non-zero return on this thread ("" if none). */
+const char *flk_last_error(void);
+
+/* Largest feature dimension and number of right-hand sides the kernels cover. */
+int64_t flk_max_d(int dtype);
+int64_t flk_max_t(void);
+
+/* ---- packed operands ------------------------------------------------------
+ * The kernels consume each data matrix in a "packed" form: rows are scaled by
+ * sqrt(log2 e)/sigma, regrouped in blocks of 32 (f32) or 16 (f64) rows stored
+ * feature-major, zero padded, and followed by the vector -1/2*||row||^2.
+ * This replaces the reference's per-block `mat / sigma` and `square_norm`
+ * prologue of rbf_core (falkon/kernels/distance_kernel.py:148-154;
+ * falkon/c_ext/ops/cuda/cuda_square_norm.cu:15-68).
+ */
+
+/* Bytes needed for the packed form of an n x d matrix. */
+size_t flk_gauss_packed_bytes(int64_t n, int64_t d, int dtype);
+
+/* Pack X[n,d].  sigma is a DEVICE array of n_sigma (1 or d) lengthscales in the
+ * data dtype (the reference moves sigma to the data's device and dtype,
+ * distance_kernel.py:148).  Any other n_sigma is FLK_EINVAL, which the host
+ * layer turns into the RuntimeError the reference raises
+ * (falkon/tests/test_kernels.py:338-358). */
+int flk_gauss_pack(const void *X, int64_t n, int64_t d, int64_t x_rs, int64_t x_cs,
+                   const void *sigma, int64_t n_sigma, int dtype,
+                   void *packed, size_t packed_bytes, void *stream);
+
+/* ---- products on packed operands -------------------------------------------
+ * out[b,t] = sum_a K(A_a, B_b) * vec[a,t]  (+ addend[b,t] if addend != NULL)
+ * with A = n_a packed rows (the reduction side) and B = n_b packed rows (the
+ * output side).  K(X1,X2) @ v is (A=X2, B=X1, vec=v); K(X1,X2)^T @ u is
+ * (A=X1, B=X2, vec=u).  out is overwritten, never accumulated into
+ * (falkon/mmv_ops/fmmv.py:369,732).
+ */
+size_t flk_gauss_mmv_packed_workspace_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t, int dtype);
+
+int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b, int64_t n_b, int64_t d,
+                         const void *vec, int64_t vec_rs, int64_t vec_cs, int64_t t,
+                         const void *addend, int64_t add_rs, int64_t add_cs,
+                         void *out, int64_t out_rs, int64_t out_cs, int dtype,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- one-call products on plain matrices ----------------------------------
+ * flk_gauss_fmmv  replaces falkon.mmv_ops.fmmv.fmmv for the dense Gaussian case
+ *   (falkon/mmv_ops/fmmv.py:960-973 -> :309-402 -> distance_kernel.py:140-159):
+ *   out[n,t] = K(X1[n,d], X2[m,d]) @ v[m,t].
+ * flk_gauss_fdmmv replaces falkon.mmv_ops.fmmv.fdmmv
+ *   (falkon/mmv_ops/fmmv.py:976-1131 -> :683-767):
+ *   out[m,t] = K^T @ (K @ v + w), v[m,t] required, w[n,t] may be NULL.
+ * Both pack X1 and X2 into the workspace, never materialise K, and leave the
+ * inputs untouched.  The workspace must hold at least the number of bytes the
+ * matching *_workspace_bytes call returns.
+ */
+size_t flk_gauss_fmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype);
+
+int flk_gauss_fmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
+                   const void *X2, int64_t m, int64_t x2_rs, int64_t x2_cs, int64_t d,
+                   const void *sigma, int64_t n_sigma,
+                   const void *v, int64_t v_rs, int64_t v_cs, int64_t t,
+                   void *out, int64_t out_rs, int64_t out_cs, int dtype,
+                   void *workspace, size_t workspace_bytes, void *stream);
+
+size_t flk_gauss_fdmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype);
+
+int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
+                    const void *X2, int64_t m, int64_t x2_rs, int64_t x2_cs, int64_t d,
+                    const void *sigma, int64_t n_sigma,
+                    const void *v, int64_t v_rs, int64_t v_cs,
+                    const void *w, int64_t w_rs, int64_t w_cs, int64_t t,
+                    void *out, int64_t out_rs, int64_t out_cs, int dtype,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FALKON_AMD_H */

@@ -1,0 +1,162 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs.
+
+Tolerances are the ones the task states: relative error (norm-wise per output column)
+1e-5 in fp32 and 1e-11 in fp64 against the reference-equivalent CPU path (``oracle.mmv_ref``).
+"""
+import numpy as np
+import pytest
+import torch
+
+from falkon_amd import FalkonOptions, GaussianKernel
+from oracle import brute, inputs, mmv_ref
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.float64: 1e-11}
+
+
+def _rand(n, d, m, t, dtype, seed, scale=1.0):
+    g = np.random.default_rng(seed)
+    np_dt = np.float32 if dtype == torch.float32 else np.float64
+    X = torch.from_numpy((g.standard_normal((n, d)) * scale).astype(np_dt))
+    C = torch.from_numpy((g.standard_normal((m, d)) * scale).astype(np_dt))
+    v = torch.from_numpy(g.standard_normal((m, t)).astype(np_dt))
+    w = torch.from_numpy(g.standard_normal((n, t)).astype(np_dt))
+    return X, C, v, w
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("n,m,d,t", [
+    (20, 5, 3, 2),          # the reference's basic test shape (tests/test_kernels.py:32-35)
+    (1500, 250, 3, 2),      # its multi-block shape (:529-535)
+    (100, 250, 28, 1),
+    (1000, 333, 9, 1),
+    (777, 129, 1, 3),
+    (515, 1031, 17, 4),
+    (300, 200, 33, 5),
+    (257, 100, 64, 1),
+    (64, 64, 2, 7),
+])
+def test_mmv_dmmv_vs_oracle(dev, dtype, n, m, d, t):
+    X, C, v, w = _rand(n, d, m, t, dtype, seed=n * 7 + m)
+    sigma = 1.0 + 0.5 * np.sqrt(d)
+    k = GaussianKernel(sigma)
+    exp_mmv = mmv_ref.fmmv_ref(X, C, v, sigma)
+    exp_dmmv = mmv_ref.fdmmv_ref(X, C, v, w, sigma)
+    exp_dmmv_now = mmv_ref.fdmmv_ref(X, C, v, None, sigma)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    got_mmv = k.mmv(Xg, Cg, vg)
+    got_dmmv = k.dmmv(Xg, Cg, vg, wg)
+    got_dmmv_now = k.dmmv(Xg, Cg, vg, None)
+    assert got_mmv.shape == (n, t) and got_dmmv.shape == (m, t)
+    assert rel_err(got_mmv, exp_mmv) < TOL[dtype]
+    assert rel_err(got_dmmv, exp_dmmv) < TOL[dtype]
+    assert rel_err(got_dmmv_now, exp_dmmv_now) < TOL[dtype]
+    # and against the closed form, which does not share the expanded-norm route
+    assert rel_err(got_mmv, brute.mmv_brute(X, C, sigma, v)) < 5 * TOL[dtype]
+    assert rel_err(got_dmmv, brute.dmmv_brute(X, C, sigma, v, w)) < 5 * TOL[dtype]
+
+
+@pytest.mark.parametrize("order", ["C", "F"])
+@pytest.mark.parametrize("sig", ["single", "vec"])
+def test_reference_fixture_fp64(dev, order, sig):
+    """Reference TestGaussianKernel.test_dense_kernel: seeds 92..95, n=20 m=5 d=3 t=2, fp64,
+    sigma 3.0 and [3,3,3], C and F order, rtol=atol=1e-8 (tests/test_kernels.py:299-319)."""
+    A, B, v, w = inputs.reference_test_mats(20, 5, 3, 2, np.float64, order)
+    sigma = torch.tensor([3.0]) if sig == "single" else torch.tensor([3.0] * 3)
+    k = GaussianKernel(sigma)
+    K = torch.from_numpy(brute.gaussian_brute(A, B, sigma))
+    Ag, Bg, vg, wg = (a.to(dev) for a in (A, B, v, w))
+    if order == "F":
+        Ag, Bg, vg, wg = (torch.empty_strided(a.shape, (1, a.shape[0]), dtype=a.dtype, device=dev).copy_(a) for a in (Ag, Bg, vg, wg))
+    out = torch.empty(20, 2, dtype=torch.float64, device=dev)
+    got = k.mmv(Ag, Bg, vg, out=out)
+    assert got.data_ptr() == out.data_ptr(), "MMV output tensor was not used"
+    torch.testing.assert_close(got.cpu(), K @ v, rtol=1e-8, atol=1e-8)
+    torch.testing.assert_close(k.mmv(Ag, Bg, vg).cpu(), K @ v, rtol=1e-8, atol=1e-8)
+    dout = torch.empty(5, 2, dtype=torch.float64, device=dev)
+    dgot = k.dmmv(Ag, Bg, vg, wg, out=dout)
+    assert dgot.data_ptr() == dout.data_ptr(), "D-MMV output tensor was not used"
+    torch.testing.assert_close(dgot.cpu(), K.T @ (K @ v + w), rtol=1e-8, atol=1e-8)
+    torch.testing.assert_close(k.dmmv(Ag, Bg, vg, wg).cpu(), K.T @ (K @ v + w), rtol=1e-8, atol=1e-8)
+    # output follows X1's memory order (mmv_ops/utils.py:124-155)
+    assert (k.mmv(Ag, Bg, vg).stride(0) == 1) == (order == "F")
+
+
+def test_per_dimension_sigma_fp32(dev):
+    g = np.random.default_rng(5)
+    X = torch.from_numpy(g.uniform(-1, 1, (4000, 9)).astype(np.float32))
+    C = X[g.choice(4000, 500, replace=False)].clone()
+    sigma = torch.from_numpy(g.uniform(0.5, 2.0, 9))
+    v = torch.from_numpy(g.standard_normal((500, 1)).astype(np.float32))
+    k = GaussianKernel(sigma)
+    got = k.dmmv(X.to(dev), C.to(dev), v.to(dev), None)
+    assert rel_err(got, mmv_ref.fdmmv_ref(X, C, v, None, sigma)) < 1e-5
+    # per-dimension sigma == isotropic sigma=1 on pre-divided data (distance_kernel.py:151-152)
+    k1 = GaussianKernel(1.0)
+    s32 = sigma.float()
+    got1 = k1.dmmv((X / s32).to(dev), (C / s32).to(dev), v.to(dev), None)
+    assert rel_err(got, got1) < 1e-5
+
+
+def test_wrong_sigma_length_raises(dev):
+    X, C, v, w = _rand(20, 3, 5, 2, torch.float64, 1)
+    k = GaussianKernel(torch.tensor([2.0, 2.0], dtype=torch.float64))
+    with pytest.raises(RuntimeError):
+        k.mmv(X.to(dev), C.to(dev), v.to(dev))
+
+
+def test_host_data_round_trip(dev):
+    """CPU-resident inputs are computed on the GPU and returned on the host, as the reference's
+    CPU-data / GPU-compute mode does (fmmv.py:797-839)."""
+    X, C, v, w = _rand(3000, 10, 400, 2, torch.float32, 3)
+    k = GaussianKernel(2.5)
+    got = k.mmv(X, C, v)
+    assert got.device.type == "cpu"
+    assert rel_err(got, mmv_ref.fmmv_ref(X, C, v, 2.5)) < 1e-5
+    got = k.dmmv(X, C, v, w)
+    assert got.device.type == "cpu"
+    assert rel_err(got, mmv_ref.fdmmv_ref(X, C, v, w, 2.5)) < 1e-5
+
+
+def test_row_blocking_under_memory_budget(dev):
+    """A small max_gpu_mem forces several row blocks; results equal the unblocked ones
+    (the reference's TestLargeComputations idea, tests/test_kernels.py:529-573)."""
+    X, C, v, w = _rand(20000, 8, 300, 2, torch.float32, 4)
+    k = GaussianKernel(2.0)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    full_m, full_d = k.mmv(Xg, Cg, vg), k.dmmv(Xg, Cg, vg, wg)
+    opt = FalkonOptions(max_gpu_mem=400 * 2**10)
+    blk_m, blk_d = k.mmv(Xg, Cg, vg, opt=opt), k.dmmv(Xg, Cg, vg, wg, opt=opt)
+    assert rel_err(blk_m, full_m) < 1e-6
+    assert rel_err(blk_d, full_d) < 1e-5
+    with pytest.raises(MemoryError):
+        k.mmv(Xg, Cg, vg, opt=FalkonOptions(max_gpu_mem=1024))
+
+
+def test_determinism(dev):
+    X, C, v, w = _rand(50000, 28, 2000, 1, torch.float32, 6)
+    k = GaussianKernel(3.8)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    a = k.dmmv(Xg, Cg, vg, wg).clone()
+    b = k.dmmv(Xg, Cg, vg, wg)
+    assert torch.equal(a, b)
+
+
+def test_config2_shape_reduced(dev):
+    """Config 2 (d=28, sigma=3.8, fp32 dfmmv) at N=100k, M=5k against the blocked CPU oracle."""
+    X, C, sigma, v, w = inputs.make_config("C2", N=100_000, M=5_000)
+    k = GaussianKernel(sigma)
+    got = k.dmmv(X.to(dev), C.to(dev), v.to(dev), w.to(dev))
+    exp = mmv_ref.fdmmv_ref(X, C, v, w, sigma, max_cpu_mem=2 * 2**30)
+    assert rel_err(got, exp) < 1e-5
+
+
+def test_config1_full(dev):
+    """Config 1 at full size: fp64 fmmv, N=20000 d=8 M=1000, sigma=2, tolerance 1e-11."""
+    X, C, sigma, v, _ = inputs.make_config("C1")
+    k = GaussianKernel(sigma)
+    got = k.mmv(X.to(dev), C.to(dev), v.to(dev))
+    exp = mmv_ref.fmmv_ref(X, C, v, sigma, max_cpu_mem=2 * 2**30)
+    assert rel_err(got, exp) < 1e-11

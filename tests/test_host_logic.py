@@ -1,0 +1,158 @@
+"""Host-side behaviour that needs no GPU: the C ABI surface, argument validation, options."""
+import ctypes
+import dataclasses
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import falkon_amd
+from falkon_amd import FalkonOptions, GaussianKernel, _backend
+from falkon_amd.kernels.distance_kernel import validate_sigma
+from falkon_amd.utils.tensor_helpers import create_same_stride, is_contig, is_f_contig
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "falkon_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(flk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_backend.library_path()) if os.path.exists(_backend.library_path()) else _backend.load()
+    names = _declared_symbols()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/falkon_amd.h but not exported"
+    assert set(names) == set(_backend._SIGNATURES), "ctypes signature table and header disagree"
+
+
+def test_size_queries_need_no_gpu():
+    lib = _backend.load()
+    assert lib.flk_version() >= 100
+    assert lib.flk_max_d(_backend.FLK_F32) >= 28 and lib.flk_max_d(_backend.FLK_F64) >= 28
+    # packed fp32: 32-row blocks, features padded to a multiple of 2, plus half norms, 256-byte aligned parts
+    assert lib.flk_gauss_packed_bytes(33, 3, _backend.FLK_F32) == 2 * 4 * 32 * 4 + 256
+    assert lib.flk_gauss_packed_bytes(16, 5, _backend.FLK_F64) == 8 * 16 * 8 + 256
+    small = lib.flk_gauss_fdmmv_workspace_bytes(1000, 100, 8, 1, _backend.FLK_F32)
+    big = lib.flk_gauss_fdmmv_workspace_bytes(100000, 100, 8, 1, _backend.FLK_F32)
+    assert 0 < small < big
+    # config 2 stays far below 288 GB: nothing of size N x M is ever allocated
+    assert lib.flk_gauss_fdmmv_workspace_bytes(1_000_000, 20_000, 28, 1, _backend.FLK_F32) < 512 * 2**20
+
+
+def test_bad_arguments_rejected_on_host_before_any_launch():
+    lib = _backend.load()
+    rc = lib.flk_gauss_pack(None, 10, 3, 3, 1, None, 1, _backend.FLK_F32, None, 0, None)
+    assert rc == _backend.FLK_EINVAL and "null" in _backend.last_error()
+    rc = lib.flk_gauss_pack(4096, 10, 3, 3, 1, 4096, 2, _backend.FLK_F32, 4096, 1 << 20, None)
+    assert rc == _backend.FLK_EINVAL and "sigma" in _backend.last_error()
+    rc = lib.flk_gauss_pack(4096, 10, 3, 6, 2, 4096, 1, _backend.FLK_F32, 4096, 1 << 20, None)
+    assert rc == _backend.FLK_EINVAL and "stride" in _backend.last_error()
+    rc = lib.flk_gauss_pack(4096, 10, 3, 3, 1, 4096, 1, 7, 4096, 1 << 20, None)
+    assert rc == _backend.FLK_EINVAL
+    rc = lib.flk_gauss_fmmv(4096, 10, 3, 1, 4096, 5, 3, 1, 3, 4096, 1, 4096, 1, 1, 1, 4096, 1, 1, _backend.FLK_F32,
+                            4096, 16, None)
+    assert rc == _backend.FLK_ENOMEM
+    with pytest.raises(MemoryError):
+        _backend.raise_for_status(rc, "flk_gauss_fmmv")
+    rc = lib.flk_gauss_fdmmv(4096, 10, 3, 1, 4096, 5, 3, 1, 3, 4096, 1, None, 1, 1, None, 0, 0, 1, 4096, 1, 1,
+                             _backend.FLK_F32, 4096, 1 << 30, None)
+    assert rc == _backend.FLK_EINVAL and "v" in _backend.last_error()
+
+
+def test_validate_sigma_and_kernel_object():
+    assert validate_sigma(2).dtype == torch.float64 and validate_sigma(2).shape == (1,)
+    assert validate_sigma(torch.ones(5, 1)).shape == (5,)
+    with pytest.raises(ValueError):
+        validate_sigma(torch.ones(2, 2))
+    with pytest.raises(TypeError):
+        validate_sigma(None)
+    k = GaussianKernel(torch.tensor([1.0, 2.0]))
+    assert list(k.diff_params) == ["sigma"] and not k.sigma.requires_grad
+    assert k.kernel_name == "gaussian" and "GaussianKernel" in repr(k)
+    assert isinstance(k.detach(), GaussianKernel)
+    # compute() is the explicit kernel block (not on the mmv path) and follows the closed form
+    X, C = torch.randn(6, 2, dtype=torch.float64), torch.randn(4, 2, dtype=torch.float64)
+    K = k.compute(X, C, torch.empty(6, 4, dtype=torch.float64), diag=False)
+    s = torch.tensor([1.0, 2.0], dtype=torch.float64)
+    torch.testing.assert_close(K, torch.exp(-0.5 * torch.cdist(X / s, C / s) ** 2), rtol=1e-10, atol=1e-12)
+
+
+def test_dimension_and_dtype_checks_match_reference():
+    """falkon/kernels/kernel.py:44-105."""
+    k = GaussianKernel(1.0)
+    X, C, v, w = torch.randn(8, 3), torch.randn(4, 3), torch.randn(4, 2), torch.randn(8, 2)
+    with pytest.raises(ValueError, match="X1 must be 2D"):
+        k.mmv(X[0], C, v)
+    with pytest.raises(ValueError, match="X2 must be 2D"):
+        k.dmmv(X, C[0], v, w)
+    with pytest.raises(ValueError, match="Dimensions of matrix v"):
+        k.mmv(X, C, v[:3])
+    with pytest.raises(ValueError, match="Dimensions of matrix w"):
+        k.dmmv(X, C, v, w[:5])
+    with pytest.raises(ValueError, match="Output dimension"):
+        k.mmv(X, C, v, out=torch.empty(8, 3))
+    with pytest.raises(ValueError, match="One of v and w"):
+        k.dmmv(X, C, None, None)
+    with pytest.raises(TypeError, match="Data types"):
+        k.mmv(X, C.double(), v)
+    with pytest.raises(ValueError, match="memory contiguous"):
+        k.mmv(torch.randn(16, 6)[::2, ::2], C, v)
+    with pytest.raises(NotImplementedError):
+        k.dmmv(X.clone().requires_grad_(), C, v, w)
+    # 1-D v is reshaped to a column before reaching the backend
+    seen = {}
+    k._decide_mmv_impl = lambda *a: (lambda **kw: seen.update(kw) or "ok")
+    assert k.mmv(X, C, torch.randn(4)) == "ok" and seen["v"].shape == (4, 1) and seen["kernel"] is k
+
+
+def test_no_cpu_fallback():
+    k = GaussianKernel(1.0)
+    X, C, v = torch.randn(8, 3), torch.randn(4, 3), torch.randn(4, 2)
+    with pytest.raises(RuntimeError, match="no CPU compute path"):
+        k.mmv(X, C, v, opt=FalkonOptions(use_cpu=True))
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="needs a ROCm GPU"):
+            k.dmmv(X, C, v, None)
+
+
+def test_options_merge_like_reference():
+    """Per-call options replace the kernel's (falkon/kernels/kernel.py:283-285)."""
+    k = GaussianKernel(1.0, opt=FalkonOptions(max_gpu_mem=123.0))
+    assert k._merged(None).max_gpu_mem == 123.0
+    assert k._merged(FalkonOptions(use_cpu=True)).use_cpu is True
+    fields = {f.name for f in dataclasses.fields(FalkonOptions)}
+    for name in ("use_cpu", "max_gpu_mem", "max_cpu_mem", "memory_slack", "keops_active", "cg_tolerance",
+                 "cg_full_gradient_every", "pc_epsilon_32", "no_single_kernel", "num_fmm_streams"):
+        assert name in fields
+    assert FalkonOptions().cg_epsilon(torch.float32) == 1e-7 and FalkonOptions().pc_epsilon(torch.float64) == 1e-13
+
+
+def test_stride_helpers():
+    """falkon/utils/tensor_helpers.py:128-213."""
+    c, f = torch.empty(5, 3), torch.empty(3, 5).T
+    assert is_contig(c) and is_contig(f) and not is_contig(torch.empty(10, 6)[::2, ::2])
+    assert is_f_contig(f) and not is_f_contig(c)
+    # (n,1) columns: non-strict accepts them as column-major, strict wants stride(1) >= n
+    col = torch.empty(5, 1)
+    assert is_f_contig(col, strict=False) and not is_f_contig(col, strict=True)
+    assert is_f_contig(torch.empty_strided((5, 1), (1, 5)), strict=True)
+    assert create_same_stride((7, 2), f, torch.float32, "cpu").stride() == (1, 7)
+    assert create_same_stride((7, 2), c, torch.float32, "cpu").stride() == (2, 1)
+    with pytest.raises(ValueError):
+        create_same_stride((7, 2), torch.empty(10, 6)[::2, ::2], torch.float32, "cpu")
+
+
+def test_product_code_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "falkon_amd")
+    for base, _, files in os.walk(pkg):
+        for fn in files:
+            if fn.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(base, fn)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), fn
+                assert "/root/reference" not in text, fn
