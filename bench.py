@@ -1,0 +1,160 @@
+#!/usr/bin/env python3
+"""Benchmark of the Gaussian dfmmv hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3] [--no-cpu-baseline]
+
+A step is one ``GaussianKernel.dmmv`` call (K^T (K v + w)) on inputs that are already
+resident in HBM; packing of X and C is part of every step.  The default workload is
+configuration 2 of BASELINE.json: N=1,000,000 x d=28 standard-normal rows, M=20,000
+centres drawn from them, sigma=3.8, fp32, one right-hand side.  One JSON line goes to stdout.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 matrix peak = fp32 vector peak (vendor figure)
+
+WORKLOADS = {
+    # name: (seed, N, d, M, T, has_w)
+    "C2": (1002, 1_000_000, 28, 20_000, 1, True),
+    "C3": (1003, 10_000_000, 9, 50_000, 1, False),
+}
+
+# HBM bytes per launch of the product kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
+# (profiles/), keyed by workload; None where it has not been measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def make_inputs(name):
+    """Synthetic inputs of the named configuration (draw order X, idx, sigma, v, w)."""
+    seed, N, d, M, T, has_w = WORKLOADS[name]
+    rng = np.random.default_rng(seed)
+    if name == "C2":
+        X = rng.standard_normal((N, d), dtype=np.float32)
+    else:
+        X = rng.random((N, d), dtype=np.float32) * 2.0 - 1.0
+    idx = rng.choice(N, size=M, replace=False)
+    sigma = torch.tensor([3.8], dtype=torch.float64) if name == "C2" else torch.from_numpy(rng.uniform(0.5, 2.0, d))
+    v = rng.standard_normal((M, T)).astype(np.float32)
+    w = rng.standard_normal((N, T)).astype(np.float32) if has_w else None
+    C = np.ascontiguousarray(X[idx])
+    return (torch.from_numpy(X), torch.from_numpy(C), sigma, torch.from_numpy(v),
+            torch.from_numpy(w) if w is not None else None)
+
+
+def cpu_baseline(X, C, sigma, v, w, gpu_out_fn, rows):
+    """Reference-equivalent CPU path (the oracle restatement, torch CPU ops) on the first `rows` rows."""
+    from oracle import mmv_ref                      # checker only; never on the product path
+    Xs = X[:rows].contiguous()
+    ws = w[:rows].contiguous() if w is not None else None
+    mmv_ref.fdmmv_ref(Xs[:2000], C, v, ws[:2000] if ws is not None else None, sigma, max_cpu_mem=4 * 2**30)  # warm-up
+    t0 = time.perf_counter()
+    exp = mmv_ref.fdmmv_ref(Xs, C, v, ws, sigma, max_cpu_mem=4 * 2**30)
+    dt = time.perf_counter() - t0
+    got = gpu_out_fn(Xs, ws).double().cpu()
+    rel = float(((got - exp.double()).norm(dim=0) / exp.double().norm(dim=0)).max())
+    M, T = v.shape
+    return {"value": rows * M * T / dt, "unit": "kernel entries/s", "cores": torch.get_num_threads(),
+            "kind": "port", "host_cpus": os.cpu_count(),
+            "sample": f"first {rows} rows of X with the full M={M} (dfmmv is linear in N), "
+                      f"max_cpu_mem=4GiB, {dt:.2f} s", "gpu_vs_cpu_rel_err_on_sample": rel}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=0)
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
+                    help="only run a plain device copy of BYTES bytes five times (reference point for the "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only; --gpus must be 1 "
+              "(sharding over rows of X with one M x T all-reduce is described in DESIGN.md, not built)",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+
+    if args.copy_calibration:
+        src = torch.ones(args.copy_calibration // 4, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes": src.numel() * 4, "copies": 5}))
+        return
+
+    from falkon_amd import GaussianKernel, _backend
+    lib = _backend.load()                            # raises if the HIP library is missing
+    dev = torch.device("cuda:0")
+    seed, N, d, M, T, has_w = WORKLOADS[args.workload]
+    X, C, sigma, v, w = make_inputs(args.workload)
+    Xg, Cg, vg = X.to(dev), C.to(dev), v.to(dev)
+    wg = w.to(dev) if w is not None else None
+    kernel = GaussianKernel(sigma)
+    out = torch.empty(M, T, dtype=torch.float32, device=dev)
+
+    def step():
+        kernel.dmmv(Xg, Cg, vg, wg, out=out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.flk_kernel_timing_enable(1)                  # HIP events around each product-kernel launch, on its stream
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    tot_ms, launches = ctypes.c_double(), ctypes.c_int64()
+    rc = lib.flk_kernel_timing_read(ctypes.byref(tot_ms), ctypes.byref(launches))
+    _backend.raise_for_status(rc, "flk_kernel_timing_read")
+    lib.flk_kernel_timing_enable(0)
+
+    ms_per_step = elapsed / args.steps * 1e3
+    value = N * M * T / (elapsed / args.steps)
+    # one launch of the product kernel evaluates all N*M pairs once: (2d+4) flop per kernel value + 2T to contract
+    flop_per_launch = N * M * (2 * d + 4 + 2 * T)
+    kern_ms = tot_ms.value / max(launches.value, 1)
+    achieved = flop_per_launch / (kern_ms * 1e-3) / 1e12
+    res = {
+        "metric": "dfmmv kernel-entries/sec (N*M*T/s) fp32, 1 MI355X",
+        "value": value, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: Gaussian dfmmv K^T(Kv+w), N={N}, d={d}, M={M}, T={T}, "
+                               f"{'sigma=3.8' if args.workload == 'C2' else 'per-dimension sigma'}, fp32, "
+                               f"inputs resident in HBM, packing included in every step"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / FP32_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel": "mmv_small_f32_kernel", "launches_per_step": launches.value / args.steps,
+                     "avg_launch_ms": kern_ms, "flop_per_launch": flop_per_launch},
+        "whole_step_flop_frac": (N * M * (2 * (2 * d + 4) + 4 * T)) / (elapsed / args.steps) / 1e12 / FP32_PEAK_TFLOPS,
+    }
+    if not args.no_cpu_baseline:
+        rows = args.cpu_rows or (N if args.workload == "C2" else 400_000)
+
+        def gpu_on(Xs, ws):
+            return kernel.dmmv(Xs.to(dev), Cg, vg, ws.to(dev) if ws is not None else None)
+
+        res["cpu_baseline"] = cpu_baseline(X, C, sigma, v, w, gpu_on, rows)
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -24,6 +24,8 @@ _SIGNATURES = {
     "flk_last_error": (c_char_p, []),
     "flk_max_d": (c_int64, [c_int]),
     "flk_max_t": (c_int64, []),
+    "flk_kernel_timing_enable": (c_int, [c_int]),
+    "flk_kernel_timing_read": (c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_int64)]),
     "flk_gauss_packed_bytes": (c_size_t, [c_int64, c_int64, c_int]),
     "flk_gauss_pack": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_int, c_void_p,
                                c_size_t, c_void_p]),

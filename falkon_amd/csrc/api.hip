@@ -2,6 +2,9 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <utility>
+#include <vector>
 
 #include "flk_common.h"
 
@@ -17,9 +20,42 @@ int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+// Optional instrumentation: HIP events around every launch of the product kernel, recorded on
+// the stream the kernel runs on.  Off by default; a benchmark switches it on to obtain the
+// kernel's own duration without an external profiler.
+static std::mutex g_timing_mu;
+static bool g_timing_on = false;
+static std::vector<std::pair<hipEvent_t, hipEvent_t>> g_timing_events;
+
+static void timing_clear_locked() {
+    for (auto &e : g_timing_events) {
+        (void)hipEventDestroy(e.first);
+        (void)hipEventDestroy(e.second);
+    }
+    g_timing_events.clear();
+}
+
+struct ScopedKernelTimer {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipStream_t st;
+    explicit ScopedKernelTimer(hipStream_t s) : st(s) {
+        std::lock_guard<std::mutex> g(g_timing_mu);
+        if (!g_timing_on) return;
+        if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { e0 = e1 = nullptr; return; }
+        (void)hipEventRecord(e0, st);
+    }
+    ~ScopedKernelTimer() {
+        if (!e0) return;
+        (void)hipEventRecord(e1, st);
+        std::lock_guard<std::mutex> g(g_timing_mu);
+        g_timing_events.emplace_back(e0, e1);
+    }
+};
+
 constexpr int kColChunk = 4;          // right-hand sides handled per pass of the product kernel
-constexpr int64_t kTargetWgs = 2048;  // workgroups wanted per launch (256 CUs x 2 resident x 4 rounds)
-constexpr int64_t kMinChunkBlocks = 8;
+constexpr int64_t kTargetWgs = 8192;  // workgroups wanted per launch: 256 CUs x 2 resident x 16 rounds, so that
+                                      // the partly filled last round costs a few percent at most
+constexpr int64_t kMinChunkBlocks = 16;
 constexpr int kMaxSplits = 1024;
 
 struct Plan {
@@ -81,6 +117,7 @@ static int mmv_packed_planar(const PackedView &A, const PackedView &B, const T *
         if (A.nblk == 0) {
             splits = 0;  // empty reduction: finalize sums nothing and writes the addend (or zero)
         } else {
+            ScopedKernelTimer timer(st);
             int rc = launch_mmv_small<T>(A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk_blocks, p.splits, partial, st);
             if (rc != FLK_OK) return rc;
         }
@@ -215,6 +252,30 @@ int flk_version(void) { return 100; }
 const char *flk_last_error(void) { return g_err; }
 int64_t flk_max_d(int dtype) { return dtype == FLK_F64 ? mmv_small_max_d<double>() : mmv_small_max_d<float>(); }
 int64_t flk_max_t(void) { return 65535; }
+
+int flk_kernel_timing_enable(int on) {
+    std::lock_guard<std::mutex> g(g_timing_mu);
+    timing_clear_locked();
+    g_timing_on = on != 0;
+    return FLK_OK;
+}
+
+int flk_kernel_timing_read(double *total_ms, int64_t *launches) {
+    g_err[0] = 0;
+    if (!total_ms || !launches) return fail(FLK_EINVAL, "null output pointer");
+    std::lock_guard<std::mutex> g(g_timing_mu);
+    double tot = 0.0;
+    for (auto &e : g_timing_events) {
+        FLK_HIP(hipEventSynchronize(e.second));
+        float ms = 0.f;
+        FLK_HIP(hipEventElapsedTime(&ms, e.first, e.second));
+        tot += ms;
+    }
+    *total_ms = tot;
+    *launches = (int64_t)g_timing_events.size();
+    timing_clear_locked();
+    return FLK_OK;
+}
 
 size_t flk_gauss_packed_bytes(int64_t n, int64_t d, int dtype) {
     if (n < 0 || d < 1) return 0;

@@ -31,48 +31,71 @@ __device__ __forceinline__ float kexp2_clamped(float x) {
     return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(x), 0.0f, 1.0f);
 }
 
-template <int DP, int TT>
-struct AFrag {
-    float a[DP];        // features h*DP + s of row j of the A block
-    floatx4 hn[4];      // half norms of the 16 A rows this lane accumulates over
-    floatx4 vec[TT][4]; // right-hand side entries of those rows
+// Per-row quantities of an A block (half norms and right-hand side entries) reach the lanes through
+// a small wave-private LDS buffer: each lane fetches ONE dword from global memory, the wave writes the
+// 32*(1+TT) values to LDS and every lane reads back the 16 rows it accumulates over with broadcast
+// ds_read_b128.  Loading those 16 values per lane straight from global memory costs the texture
+// addresser a full 64-lane x 16-byte pass per instruction although only 128 distinct bytes are
+// touched, which measurably throttles the kernel.  No workgroup barrier is involved: a wave only
+// ever reads what it wrote itself.
+template <int TT> struct RowVals {
+    static constexpr int N = 32 * (1 + TT);       // floats staged per A block
+    static constexpr int C = (N + 63) / 64;       // dwords fetched per lane
+    float x[C];
 };
 
-template <int DP, int TT>
-__device__ __forceinline__ void load_afrag(AFrag<DP, TT> &f, const float *__restrict__ PA,
-                                           const float *__restrict__ hA, const float *__restrict__ vecp,
-                                           int64_t vec_ld, int64_t ab, int j, int h) {
+template <int TT>
+__device__ __forceinline__ void fetch_rowvals(RowVals<TT> &rv, const float *const (&src)[RowVals<TT>::C], int64_t ab) {
+#pragma unroll
+    for (int c = 0; c < RowVals<TT>::C; c++) rv.x[c] = src[c][ab * 32];
+}
+
+template <int TT>
+__device__ __forceinline__ void stage_rowvals(const RowVals<TT> &rv, float *lds, int lane) {
+#pragma unroll
+    for (int c = 0; c < RowVals<TT>::C; c++) {
+        int e = lane + 64 * c;
+        if (e < RowVals<TT>::N) lds[e] = rv.x[c];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+template <int DP>
+__device__ __forceinline__ void load_a(float (&a)[DP], const float *__restrict__ PA, int64_t ab, int j, int h) {
     const float *p = PA + (ab * (2 * DP) + (int64_t)h * DP) * 32 + j;
 #pragma unroll
-    for (int s = 0; s < DP; s++) f.a[s] = p[s * 32];
-    const int64_t r0 = ab * 32 + 4 * h;
-#pragma unroll
-    for (int g = 0; g < 4; g++) f.hn[g] = *(const floatx4 *)(hA + r0 + 8 * g);
-#pragma unroll
-    for (int t = 0; t < TT; t++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) f.vec[t][g] = *(const floatx4 *)(vecp + t * vec_ld + r0 + 8 * g);
+    for (int s = 0; s < DP; s++) a[s] = p[s * 32];
 }
 
 template <int DP, int FR, int TT>
-__device__ __forceinline__ void tile_step(const AFrag<DP, TT> &f, const float (&breg)[FR][DP], const float (&hb)[FR],
-                                          float (&o1)[FR][TT]) {
+__device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds, int h, const float (&breg)[FR][DP],
+                                          const float (&hb)[FR], float (&o1)[FR][TT]) {
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    floatx4 hn[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) hn[g] = *(const floatx4 *)(lds + 8 * g + 4 * h);
     floatx16 acc[FR];
 #pragma unroll
     for (int q = 0; q < FR; q++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[q][r] = f.hn[r >> 2][r & 3] + hb[q];
+        for (int r = 0; r < 16; r++) acc[q][r] = hn[r >> 2][r & 3] + hb[q];
+    floatx4 vec[TT][4];
+#pragma unroll
+    for (int t = 0; t < TT; t++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) vec[t][g] = *(const floatx4 *)(lds + 32 + 32 * t + 8 * g + 4 * h);
 #pragma unroll
     for (int s = 0; s < DP; s++)
 #pragma unroll
-        for (int q = 0; q < FR; q++) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[s], breg[q][s], acc[q], 0, 0, 0);
+        for (int q = 0; q < FR; q++) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], breg[q][s], acc[q], 0, 0, 0);
 #pragma unroll
     for (int q = 0; q < FR; q++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             float k = kexp2_clamped(acc[q][r]);
 #pragma unroll
-            for (int t = 0; t < TT; t++) o1[q][t] = __builtin_fmaf(k, f.vec[t][r >> 2][r & 3], o1[q][t]);
+            for (int t = 0; t < TT; t++) o1[q][t] = __builtin_fmaf(k, vec[t][r >> 2][r & 3], o1[q][t]);
         }
 }
 
@@ -81,6 +104,8 @@ __global__ void __launch_bounds__(256)
     mmv_small_f32_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
                          int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB, int64_t na_blocks,
                          int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial, int64_t nb_pad) {
+    using RV = RowVals<TT>;
+    __shared__ __attribute__((aligned(16))) float stage[kWavesPerWg][2][RV::N];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int j = lane & 31, h = lane >> 5;
@@ -96,10 +121,15 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int q = 0; q < FR; q++) {
         int64_t bb = bb0 + q < nb_blocks ? bb0 + q : nb_blocks - 1;
-        const float *p = PB + (bb * (2 * DP) + (int64_t)h * DP) * 32 + j;
-#pragma unroll
-        for (int s = 0; s < DP; s++) breg[q][s] = p[s * 32];
+        load_a<DP>(breg[q], PB, bb, j, h);
         hb[q] = hB[bb * 32 + j];
+    }
+    // where this lane's staged dwords come from: element e = lane + 64c of [hn(32) | vec_0(32) | vec_1(32) ...]
+    const float *src[RV::C];
+#pragma unroll
+    for (int c = 0; c < RV::C; c++) {
+        int e = lane + 64 * c;
+        src[c] = (e < 32 || e >= RV::N) ? hA + (e & 31) : vecp + (int64_t)((e - 32) >> 5) * vec_ld + (e & 31);
     }
 
     float o1[FR][TT], o2[FR][TT];
@@ -108,16 +138,25 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
         for (int t = 0; t < TT; t++) { o1[q][t] = 0.f; o2[q][t] = 0.f; }
 
-    AFrag<DP, TT> f0, f1;
-    if (a0 < a1) load_afrag<DP, TT>(f0, PA, hA, vecp, vec_ld, a0, j, h);
+    float fa0[DP], fa1[DP];
+    RV rv;
+    float *lds0 = stage[wave][0], *lds1 = stage[wave][1];
+    if (a0 < a1) {
+        load_a<DP>(fa0, PA, a0, j, h);
+        fetch_rowvals<TT>(rv, src, a0);
+        stage_rowvals<TT>(rv, lds0, lane);
+    }
     int since_flush = 0;
     for (int64_t ab = a0; ab < a1; ab += 2) {
         const bool has1 = ab + 1 < a1;
-        if (has1) load_afrag<DP, TT>(f1, PA, hA, vecp, vec_ld, ab + 1, j, h);
-        tile_step<DP, FR, TT>(f0, breg, hb, o1);
+        if (has1) { load_a<DP>(fa1, PA, ab + 1, j, h); fetch_rowvals<TT>(rv, src, ab + 1); }
+        tile_step<DP, FR, TT>(fa0, lds0, h, breg, hb, o1);
         if (has1) {
-            if (ab + 2 < a1) load_afrag<DP, TT>(f0, PA, hA, vecp, vec_ld, ab + 2, j, h);
-            tile_step<DP, FR, TT>(f1, breg, hb, o1);
+            stage_rowvals<TT>(rv, lds1, lane);
+            const bool has2 = ab + 2 < a1;
+            if (has2) { load_a<DP>(fa0, PA, ab + 2, j, h); fetch_rowvals<TT>(rv, src, ab + 2); }
+            tile_step<DP, FR, TT>(fa1, lds1, h, breg, hb, o1);
+            if (has2) stage_rowvals<TT>(rv, lds0, lane);
         }
         since_flush += 2;
         if (since_flush >= kFlushEvery) {

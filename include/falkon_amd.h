@@ -45,6 +45,14 @@ const char *flk_last_error(void);
 int64_t flk_max_d(int dtype);
 int64_t flk_max_t(void);
 
+/* Instrumentation (no counterpart in the reference, which times whole calls with
+ * falkon/utils/tictoc.py:19-63): when enabled, the library brackets every launch of the
+ * product kernel with HIP events on the launch stream.  flk_kernel_timing_read waits for
+ * the recorded events, returns the summed kernel time and the number of launches since
+ * the last read/enable, and clears the records. */
+int flk_kernel_timing_enable(int on);
+int flk_kernel_timing_read(double *total_ms, int64_t *launches);
+
 /* ---- packed operands ------------------------------------------------------
  * The kernels consume each data matrix in a "packed" form: rows are scaled by
  * sqrt(log2 e)/sigma, regrouped in blocks of 32 (f32) or 16 (f64) rows stored
