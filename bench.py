@@ -60,13 +60,20 @@ def cpu_baseline(X, C, sigma, v, w, gpu_out_fn, rows):
     t0 = time.perf_counter()
     exp = mmv_ref.fdmmv_ref(Xs, C, v, ws, sigma, max_cpu_mem=4 * 2**30)
     dt = time.perf_counter() - t0
-    got = gpu_out_fn(Xs, ws).double().cpu()
-    rel = float(((got - exp.double()).norm(dim=0) / exp.double().norm(dim=0)).max())
+    got, got64 = gpu_out_fn(Xs, ws)
+    got, got64, exp = got.double().cpu(), got64.double().cpu(), exp.double()
+
+    def rel(a, b):
+        return float(((a - b).norm(dim=0) / b.norm(dim=0)).max())
+
     M, T = v.shape
     return {"value": rows * M * T / dt, "unit": "kernel entries/s", "cores": torch.get_num_threads(),
             "kind": "port", "host_cpus": os.cpu_count(),
             "sample": f"first {rows} rows of X with the full M={M} (dfmmv is linear in N), "
-                      f"max_cpu_mem=4GiB, {dt:.2f} s", "gpu_vs_cpu_rel_err_on_sample": rel}
+                      f"max_cpu_mem=4GiB, {dt:.2f} s",
+            # fp64 anchor = the same product in fp64 on the same fp32-valued inputs (GPU fp64 kernel)
+            "rel_err_gpu_f32_vs_cpu_f32": rel(got, exp), "rel_err_gpu_f32_vs_f64": rel(got, got64),
+            "rel_err_cpu_f32_vs_f64": rel(exp, got64)}
 
 
 def main():
@@ -150,7 +157,11 @@ def main():
         rows = args.cpu_rows or (N if args.workload == "C2" else 400_000)
 
         def gpu_on(Xs, ws):
-            return kernel.dmmv(Xs.to(dev), Cg, vg, ws.to(dev) if ws is not None else None)
+            Xd = Xs.to(dev)
+            wd = ws.to(dev) if ws is not None else None
+            r32 = kernel.dmmv(Xd, Cg, vg, wd)
+            r64 = kernel.dmmv(Xd.double(), Cg.double(), vg.double(), wd.double() if wd is not None else None)
+            return r32, r64
 
         res["cpu_baseline"] = cpu_baseline(X, C, sigma, v, w, gpu_on, rows)
     print(json.dumps(res), flush=True)

@@ -2,5 +2,6 @@
 from .options import FalkonOptions  # noqa: F401
 from .kernels import GaussianKernel  # noqa: F401
 from .mmv_ops import fdmmv, fmmv  # noqa: F401
+from .models import Falkon, InCoreFalkon  # noqa: F401
 
 __version__ = "0.1.0"

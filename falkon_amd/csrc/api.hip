@@ -59,34 +59,57 @@ constexpr int64_t kMinChunkBlocks = 16;
 constexpr int kMaxSplits = 1024;
 
 struct Plan {
-    int64_t chunk_blocks;
-    int splits;
+    bool large;            // LDS-tiled kernel (d beyond the register-resident kernel's range)
+    int64_t chunk;         // reduction-side work per workgroup: A blocks (small) or A tiles (large)
+    int splits;            // grid.y
+    int partials;          // partial results the finalize kernel sums (= splits x partials per split)
+    int col_chunk;         // right-hand sides per pass
 };
 
+constexpr int64_t kTargetWgsLarge = 2048;  // one 512-thread workgroup per CU: 8 rounds
+
 template <typename T>
-static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t dpad) {
-    const int64_t per_wg = mmv_small_b_blocks_per_wg<T>(dpad);
-    const int64_t b_tiles = (nb_blocks + per_wg - 1) / per_wg;
-    int64_t splits = (kTargetWgs + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
-    int64_t max_splits = na_blocks / kMinChunkBlocks;
-    if (max_splits < 1) max_splits = 1;
-    if (splits > max_splits) splits = max_splits;
-    if (splits > kMaxSplits) splits = kMaxSplits;
-    if (splits < 1) splits = 1;
+static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t dpad) {
     Plan p;
-    p.chunk_blocks = (na_blocks + splits - 1) / splits;
-    if (p.chunk_blocks < 1) p.chunk_blocks = 1;
-    p.splits = (int)((na_blocks + p.chunk_blocks - 1) / p.chunk_blocks);
-    if (p.splits < 1) p.splits = 1;
+    p.large = d > mmv_small_max_d<T>();
+    if (!p.large) {
+        const int64_t per_wg = mmv_small_b_blocks_per_wg<T>(dpad);
+        const int64_t b_tiles = (nb_blocks + per_wg - 1) / per_wg;
+        int64_t splits = (kTargetWgs + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
+        int64_t max_splits = na_blocks / kMinChunkBlocks;
+        if (max_splits < 1) max_splits = 1;
+        if (splits > max_splits) splits = max_splits;
+        if (splits > kMaxSplits) splits = kMaxSplits;
+        if (splits < 1) splits = 1;
+        p.chunk = (na_blocks + splits - 1) / splits;
+        if (p.chunk < 1) p.chunk = 1;
+        p.splits = (int)((na_blocks + p.chunk - 1) / p.chunk);
+        if (p.splits < 1) p.splits = 1;
+        p.partials = p.splits;
+        p.col_chunk = kColChunk;
+    } else {
+        const int64_t a_tiles = (na_blocks + mmv_large_a_tile_blocks<T>() - 1) / mmv_large_a_tile_blocks<T>();
+        const int64_t b_tiles = (nb_blocks + mmv_large_b_tile_blocks<T>() - 1) / mmv_large_b_tile_blocks<T>();
+        int64_t splits = (kTargetWgsLarge + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
+        if (splits > a_tiles) splits = a_tiles;
+        if (splits > kMaxSplits) splits = kMaxSplits;
+        if (splits < 1) splits = 1;
+        p.chunk = (a_tiles + splits - 1) / splits;
+        if (p.chunk < 1) p.chunk = 1;
+        p.splits = (int)((a_tiles + p.chunk - 1) / p.chunk);
+        if (p.splits < 1) p.splits = 1;
+        p.partials = p.splits * mmv_large_partials_per_split<T>();
+        p.col_chunk = mmv_large_max_cols<T>();
+    }
     return p;
 }
 
 template <typename T>
 static size_t partial_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t) {
     PackedView A = packed_view<T>(nullptr, n_a, d), B = packed_view<T>(nullptr, n_b, d);
-    Plan p = make_plan<T>(A.nblk, B.nblk, A.dpad);
-    int64_t tc = t < kColChunk ? t : kColChunk;
-    return align256((size_t)p.splits * tc * B.npad * sizeof(T));
+    Plan p = make_plan<T>(A.nblk, B.nblk, d, A.dpad);
+    int64_t tc = t < p.col_chunk ? t : p.col_chunk;
+    return align256((size_t)p.partials * tc * B.npad * sizeof(T));
 }
 
 static int check_matrix(const char *name, const void *p, int64_t rows, int64_t cols, int64_t rs, int64_t cs) {
@@ -104,25 +127,23 @@ static int mmv_packed_planar(const PackedView &A, const PackedView &B, const T *
                              int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
                              T *partial, size_t partial_avail, hipStream_t st) {
     if (B.n == 0 || t == 0) return FLK_OK;
-    if (A.d > mmv_small_max_d<T>())
-        return fail(FLK_EUNSUPPORTED, "feature dimension %lld exceeds the %lld the compiled kernels cover",
-                    (long long)A.d, (long long)mmv_small_max_d<T>());
-    Plan p = make_plan<T>(A.nblk, B.nblk, A.dpad);
-    for (int64_t t0 = 0; t0 < t; t0 += kColChunk) {
-        int tc = (int)(t - t0 < kColChunk ? t - t0 : kColChunk);
-        if ((size_t)p.splits * tc * B.npad * sizeof(T) > partial_avail)
-            return fail(FLK_ENOMEM, "workspace too small for %d partial sums of %lld x %d", p.splits,
+    Plan p = make_plan<T>(A.nblk, B.nblk, A.d, A.dpad);
+    for (int64_t t0 = 0; t0 < t; t0 += p.col_chunk) {
+        int tc = (int)(t - t0 < p.col_chunk ? t - t0 : p.col_chunk);
+        if ((size_t)p.partials * tc * B.npad * sizeof(T) > partial_avail)
+            return fail(FLK_ENOMEM, "workspace too small for %d partial sums of %lld x %d", p.partials,
                         (long long)B.npad, tc);
-        int splits = p.splits;
+        int partials = p.partials;
         if (A.nblk == 0) {
-            splits = 0;  // empty reduction: finalize sums nothing and writes the addend (or zero)
+            partials = 0;  // empty reduction: finalize sums nothing and writes the addend (or zero)
         } else {
             ScopedKernelTimer timer(st);
-            int rc = launch_mmv_small<T>(A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk_blocks, p.splits, partial, st);
+            int rc = p.large ? launch_mmv_large<T>(A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st)
+                             : launch_mmv_small<T>(A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st);
             if (rc != FLK_OK) return rc;
         }
-        int rc = launch_finalize<T>(partial, splits, tc, B.n, B.npad, addend ? addend + t0 * add_cs : nullptr, add_rs,
-                                    add_cs, out + t0 * out_cs, out_rs, out_cs, zero_pad, st);
+        int rc = launch_finalize<T>(partial, partials, tc, B.n, B.npad, addend ? addend + t0 * add_cs : nullptr,
+                                    add_rs, add_cs, out + t0 * out_cs, out_rs, out_cs, zero_pad, st);
         if (rc != FLK_OK) return rc;
     }
     return FLK_OK;
@@ -250,7 +271,7 @@ extern "C" {
 
 int flk_version(void) { return 100; }
 const char *flk_last_error(void) { return g_err; }
-int64_t flk_max_d(int dtype) { return dtype == FLK_F64 ? mmv_small_max_d<double>() : mmv_small_max_d<float>(); }
+int64_t flk_max_d(int dtype) { (void)dtype; return (int64_t)1 << 20; }
 int64_t flk_max_t(void) { return 65535; }
 
 int flk_kernel_timing_enable(int on) {

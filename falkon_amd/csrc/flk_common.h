@@ -81,4 +81,14 @@ int launch_mmv_small(const PackedView &A, const PackedView &B, const T *vecp, in
 template <typename T> int64_t mmv_small_max_d();
 template <typename T> int mmv_small_b_blocks_per_wg(int64_t dpad);
 
+// LDS-tiled ("large d") product kernel: any padded feature count, up to mmv_large_max_cols columns per pass.
+// Writes splits * mmv_large_partials_per_split partial results.
+template <typename T>
+int launch_mmv_large(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
+                     int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st);
+template <typename T> int mmv_large_a_tile_blocks();
+template <typename T> int mmv_large_b_tile_blocks();
+template <typename T> int mmv_large_partials_per_split();
+template <typename T> int mmv_large_max_cols();
+
 }  // namespace flk

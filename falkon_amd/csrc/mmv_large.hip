@@ -1,0 +1,311 @@
+// LDS-tiled Gaussian kernel-vector product for large feature counts (d > 64), fp32 and fp64, gfx950.
+//
+//   partial[split'][t][b] = sum_{a in chunk} exp2(A~_a . B~_b + hA_a + hB_b) * vec[a,t]
+//
+// A workgroup of 8 waves owns one tile of output rows (B side) and walks over the tiles of
+// reduction rows (A side) of its chunk.  For every (A tile, B tile) the cross term is a GEMM over
+// the features: feature chunks of both tiles are staged in LDS (double buffered, one barrier per
+// chunk, 16-byte global loads straight from the packed layout, which is already in operand order),
+// every wave keeps a WA_FR x WB_FR grid of MFMA accumulators in registers.  After the last feature
+// chunk the accumulators hold x~.c~; the epilogue adds the half norms, applies exp2 with the clamp,
+// and contracts the tile against vec into per-lane output accumulators that live in registers for
+// the whole kernel.  K is never written anywhere.
+//
+// Waves are arranged 2 (A) x 4 (B); waves with the same wb produce partial sums for the same
+// output rows and simply write separate partials (they count as extra splits for the reduction).
+#include "flk_common.h"
+
+namespace flk {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+typedef double doublex2 __attribute__((ext_vector_type(2)));
+
+template <typename T> struct LTraits;
+
+template <> struct LTraits<float> {
+    static constexpr int BLK = 32, KG = 2, ACCN = 16, NG = 4, VPL = 4;  // VPL: elements per 16-byte vector
+    typedef floatx16 acc_t;
+    typedef floatx4 vec4_t;
+    static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+    }
+    // offset (within the block, in matrix rows) of the g-th group of 4 consecutive accumulator rows
+    static __device__ __forceinline__ int group_off(int g, int lg) { return 8 * g + 4 * lg; }
+    static __device__ __forceinline__ int out_row(int j) { return j; }
+    static __device__ __forceinline__ float kexp(float x) {
+        return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(x), 0.0f, 1.0f);
+    }
+};
+
+template <> struct LTraits<double> {
+    static constexpr int BLK = 16, KG = 4, ACCN = 4, NG = 1, VPL = 2;
+    typedef doublex4 acc_t;
+    typedef doublex4 vec4_t;
+    static __device__ __forceinline__ acc_t mfma(double a, double b, acc_t c) {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int group_off(int g, int lg) { return 4 * lg; }
+    static __device__ __forceinline__ int out_row(int j) { return 4 * (j & 3) + (j >> 2); }
+    static __device__ __forceinline__ double kexp(double x) { return exp2(fmin(x, 0.0)); }
+};
+
+constexpr int kLWavesA = 2, kLWavesB = 4, kLThreads = 64 * kLWavesA * kLWavesB;
+
+template <typename T, int WA_FR, int WB_FR, int KC> struct LGeo {
+    typedef LTraits<T> TR;
+    static constexpr int NAB = kLWavesA * WA_FR;             // A blocks per tile
+    static constexpr int NBB = kLWavesB * WB_FR;             // B blocks per tile
+    static constexpr int A_ROWS = NAB * TR::BLK, B_ROWS = NBB * TR::BLK;
+    static constexpr int A_ELEMS = NAB * KC * 64, B_ELEMS = NBB * KC * 64;   // per stage
+    static constexpr int A_VECS = A_ELEMS / TR::VPL, B_VECS = B_ELEMS / TR::VPL;
+    static constexpr int A_VPT = (A_VECS + kLThreads - 1) / kLThreads;      // 16-byte vectors per thread
+    static constexpr int B_VPT = (B_VECS + kLThreads - 1) / kLThreads;
+};
+
+// One 16-byte piece of a stage: vector index vi enumerates [block][step][lane group][row/VPL], which is
+// also the order in LDS, so the LDS side of the copy is linear.
+template <typename T, int KC>
+__device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t blk0, int64_t nblk, int64_t dpad,
+                                              int64_t DPsteps, int64_t s0, int vi, bool &valid) {
+    typedef LTraits<T> TR;
+    constexpr int VPB = TR::BLK / TR::VPL;
+    const int jv = vi % VPB;
+    const int lg = (vi / VPB) % TR::KG;
+    const int s = (vi / (VPB * TR::KG)) % KC;
+    const int blk = vi / (VPB * TR::KG * KC);
+    int64_t b = blk0 + blk;
+    if (b >= nblk) b = nblk - 1;                 // past the end: any valid block (its rows get zero weight / are not stored)
+    valid = (s0 + s) < DPsteps;                  // feature tail: zero fill
+    const int64_t ss = valid ? s0 + s : 0;
+    return P + (b * dpad + (int64_t)lg * DPsteps + ss) * TR::BLK + jv * TR::VPL;
+}
+
+template <typename T, int WA_FR, int WB_FR, int KC, int TT>
+__global__ void __launch_bounds__(kLThreads)
+    mmv_large_kernel(const T *__restrict__ PA, const T *__restrict__ hA, const T *__restrict__ vecp, int64_t vec_ld,
+                     int tcols, const T *__restrict__ PB, const T *__restrict__ hB, int64_t na_blocks,
+                     int64_t nb_blocks, int64_t dpad, int64_t a_tiles_per_chunk, T *__restrict__ partial,
+                     int64_t nb_pad) {
+    typedef LTraits<T> TR;
+    typedef LGeo<T, WA_FR, WB_FR, KC> G;
+    typedef typename TR::acc_t acc_t;
+    typedef typename TR::vec4_t vec4_t;
+    struct __attribute__((aligned(16))) V16 { T v[TR::VPL]; };
+
+    __shared__ __attribute__((aligned(16))) T ldsA[2][G::A_ELEMS];
+    __shared__ __attribute__((aligned(16))) T ldsB[2][G::B_ELEMS];
+    __shared__ __attribute__((aligned(32))) T ldsRow[(1 + TT) * G::A_ROWS];   // [hA | vec_0 | vec_1 ...] of the A tile
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wa = wave % kLWavesA, wb = wave / kLWavesA;
+    const int j = lane % TR::BLK, lg = lane / TR::BLK;
+    const int64_t DPsteps = dpad / TR::KG;
+    const int64_t bblk0 = (int64_t)blockIdx.x * G::NBB;
+    const int64_t a_tiles = (na_blocks + G::NAB - 1) / G::NAB;
+    const int64_t at0 = (int64_t)blockIdx.y * a_tiles_per_chunk;
+    int64_t at1 = at0 + a_tiles_per_chunk;
+    if (at1 > a_tiles) at1 = a_tiles;
+    const int64_t n_chunks = (DPsteps + KC - 1) / KC;
+
+    // half norms of this lane's output rows
+    T hb[WB_FR];
+#pragma unroll
+    for (int q = 0; q < WB_FR; q++) {
+        int64_t bb = bblk0 + wb * WB_FR + q;
+        if (bb >= nb_blocks) bb = nb_blocks - 1;
+        hb[q] = hB[bb * TR::BLK + TR::out_row(j)];
+    }
+    T out[WB_FR][TT];
+#pragma unroll
+    for (int q = 0; q < WB_FR; q++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) out[q][t] = T(0);
+
+    for (int64_t at = at0; at < at1; at++) {
+        const int64_t ablk0 = at * G::NAB;
+        acc_t acc[WA_FR][WB_FR];
+#pragma unroll
+        for (int p = 0; p < WA_FR; p++)
+#pragma unroll
+            for (int q = 0; q < WB_FR; q++)
+#pragma unroll
+                for (int r = 0; r < TR::ACCN; r++) acc[p][q][r] = T(0);
+
+        V16 ra[G::A_VPT], rb[G::B_VPT];
+        auto fetch = [&](int64_t chunk) {
+            const int64_t s0 = chunk * KC;
+#pragma unroll
+            for (int c = 0; c < G::A_VPT; c++) {
+                int vi = tid + c * kLThreads;
+                if (vi < G::A_VECS) {
+                    bool valid;
+                    const T *src = stage_src<T, KC>(PA, ablk0, na_blocks, dpad, DPsteps, s0, vi, valid);
+                    V16 x = *(const V16 *)src;
+                    if (!valid)
+#pragma unroll
+                        for (int e = 0; e < TR::VPL; e++) x.v[e] = T(0);
+                    ra[c] = x;
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < G::B_VPT; c++) {
+                int vi = tid + c * kLThreads;
+                if (vi < G::B_VECS) {
+                    bool valid;
+                    const T *src = stage_src<T, KC>(PB, bblk0, nb_blocks, dpad, DPsteps, s0, vi, valid);
+                    V16 x = *(const V16 *)src;
+                    if (!valid)
+#pragma unroll
+                        for (int e = 0; e < TR::VPL; e++) x.v[e] = T(0);
+                    rb[c] = x;
+                }
+            }
+        };
+        auto commit = [&](int buf) {
+#pragma unroll
+            for (int c = 0; c < G::A_VPT; c++) {
+                int vi = tid + c * kLThreads;
+                if (vi < G::A_VECS) *(V16 *)(&ldsA[buf][vi * TR::VPL]) = ra[c];
+            }
+#pragma unroll
+            for (int c = 0; c < G::B_VPT; c++) {
+                int vi = tid + c * kLThreads;
+                if (vi < G::B_VECS) *(V16 *)(&ldsB[buf][vi * TR::VPL]) = rb[c];
+            }
+        };
+
+        // previous tile's epilogue may still be reading ldsRow and the stage buffers
+        __syncthreads();
+        // per-row values of the A tile: rows past n_a carry zero weight
+        for (int e = tid; e < (1 + TT) * G::A_ROWS; e += kLThreads) {
+            const int which = e / G::A_ROWS, r = e % G::A_ROWS;
+            const int64_t row = ablk0 * TR::BLK + r;
+            T val = T(0);
+            if (row < na_blocks * TR::BLK) {
+                if (which == 0) val = hA[row];
+                else if (which - 1 < tcols) val = vecp[(int64_t)(which - 1) * vec_ld + row];
+            }
+            ldsRow[e] = val;
+        }
+        fetch(0);
+        commit(0);
+        __syncthreads();
+
+        for (int64_t ch = 0; ch < n_chunks; ch++) {
+            const int buf = (int)(ch & 1);
+            if (ch + 1 < n_chunks) fetch(ch + 1);
+            const T *la = &ldsA[buf][(wa * WA_FR) * KC * 64 + lane];
+            const T *lb = &ldsB[buf][(wb * WB_FR) * KC * 64 + lane];
+#pragma unroll
+            for (int s = 0; s < KC; s++) {
+                T av[WA_FR], bv[WB_FR];
+#pragma unroll
+                for (int p = 0; p < WA_FR; p++) av[p] = la[(p * KC + s) * 64];
+#pragma unroll
+                for (int q = 0; q < WB_FR; q++) bv[q] = lb[(q * KC + s) * 64];
+#pragma unroll
+                for (int p = 0; p < WA_FR; p++)
+#pragma unroll
+                    for (int q = 0; q < WB_FR; q++) acc[p][q] = TR::mfma(av[p], bv[q], acc[p][q]);
+            }
+            if (ch + 1 < n_chunks) commit(buf ^ 1);
+            __syncthreads();
+        }
+
+        // epilogue: exponent = acc + hA_i + hB_j ; K = exp2 clamped ; out[q][t] += K * vec[i][t]
+#pragma unroll
+        for (int p = 0; p < WA_FR; p++) {
+            const int rbase = (wa * WA_FR + p) * TR::BLK;
+#pragma unroll
+            for (int g = 0; g < TR::NG; g++) {
+                const int ro = rbase + TR::group_off(g, lg);
+                const vec4_t hn = *(const vec4_t *)(&ldsRow[ro]);
+#pragma unroll
+                for (int q = 0; q < WB_FR; q++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        T x = acc[p][q][4 * g + e] + (hn[e] + hb[q]);
+                        acc[p][q][4 * g + e] = TR::kexp(x);
+                    }
+#pragma unroll
+                for (int t = 0; t < TT; t++) {
+                    const vec4_t vv = *(const vec4_t *)(&ldsRow[(1 + t) * G::A_ROWS + ro]);
+#pragma unroll
+                    for (int q = 0; q < WB_FR; q++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) out[q][t] = __builtin_fma(acc[p][q][4 * g + e], vv[e], out[q][t]);
+                }
+            }
+        }
+    }
+
+    // join the lane groups that hold the same output row, then one partial per (split, wa)
+#pragma unroll
+    for (int q = 0; q < WB_FR; q++) {
+        const int64_t bb = bblk0 + wb * WB_FR + q;
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            T s = out[q][t];
+            if (TR::KG == 4) s += __shfl_xor(s, 16, 64);
+            s += __shfl_xor(s, 32, 64);
+            if (lg == 0 && bb < nb_blocks && t < tcols)
+                partial[(((int64_t)blockIdx.y * kLWavesA + wa) * tcols + t) * nb_pad + bb * TR::BLK + TR::out_row(j)] = s;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// dispatch
+// ---------------------------------------------------------------------------
+template <typename T> struct LCfg;
+template <> struct LCfg<float>  { static constexpr int WA_FR = 4, WB_FR = 2, KC = 8; };   // tile 256 (A) x 256 (B) rows
+template <> struct LCfg<double> { static constexpr int WA_FR = 4, WB_FR = 2, KC = 8; };   // tile 128 (A) x 128 (B) rows
+
+template <typename T> int mmv_large_max_cols();
+template <typename T> int mmv_large_a_tile_blocks() { return kLWavesA * LCfg<T>::WA_FR; }
+template <typename T> int mmv_large_b_tile_blocks() { return kLWavesB * LCfg<T>::WB_FR; }
+template <typename T> int mmv_large_partials_per_split() { return kLWavesA; }
+template <> int mmv_large_max_cols<float>() { return 16; }
+template <> int mmv_large_max_cols<double>() { return 16; }
+template int mmv_large_a_tile_blocks<float>();
+template int mmv_large_a_tile_blocks<double>();
+template int mmv_large_b_tile_blocks<float>();
+template int mmv_large_b_tile_blocks<double>();
+template int mmv_large_partials_per_split<float>();
+template int mmv_large_partials_per_split<double>();
+
+template <typename T, int TT>
+static int launch_large_tt(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
+                           int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
+    typedef LCfg<T> C;
+    const int64_t nbb = kLWavesB * C::WB_FR;
+    dim3 grid((unsigned)((B.nblk + nbb - 1) / nbb), (unsigned)splits);
+    hipLaunchKernelGGL((mmv_large_kernel<T, C::WA_FR, C::WB_FR, C::KC, TT>), grid, dim3(kLThreads), 0, st,
+                       (const T *)A.data, (const T *)A.hnorm, vecp, vec_ld, tcols, (const T *)B.data,
+                       (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, a_tiles_per_chunk, partial, B.npad);
+    FLK_LAUNCH_CHECK("mmv_large_kernel");
+    return FLK_OK;
+}
+
+template <typename T>
+int launch_mmv_large(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
+                     int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
+    if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_large: operands packed with different feature counts");
+    if (tcols < 1 || tcols > mmv_large_max_cols<T>())
+        return fail(FLK_EINVAL, "mmv_large: column chunk %d not in 1..%d", tcols, mmv_large_max_cols<T>());
+    if (tcols == 1) return launch_large_tt<T, 1>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    if (tcols == 2) return launch_large_tt<T, 2>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    if (tcols <= 4) return launch_large_tt<T, 4>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    if (tcols <= 8) return launch_large_tt<T, 8>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    if (tcols <= 12) return launch_large_tt<T, 12>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    return launch_large_tt<T, 16>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+}
+template int launch_mmv_large<float>(const PackedView &, const PackedView &, const float *, int64_t, int, int64_t,
+                                     int, float *, hipStream_t);
+template int launch_mmv_large<double>(const PackedView &, const PackedView &, const double *, int64_t, int, int64_t,
+                                      int, double *, hipStream_t);
+
+}  // namespace flk

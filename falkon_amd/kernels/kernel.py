@@ -10,6 +10,7 @@ from typing import Dict, Optional
 
 import torch
 
+from ..mmv_ops.fmm import fmm
 from ..mmv_ops.fmmv import fdmmv, fmmv
 from ..options import FalkonOptions
 from ..utils.helpers import check_same_device, check_same_dtype
@@ -100,6 +101,20 @@ class Kernel(torch.nn.Module, ABC):
         if opt is None:
             return self.params
         return dataclasses.replace(self.params, **dataclasses.asdict(opt))
+
+    # -- kernel matrix (falkon/kernels/kernel.py:135-224) ----------------------------------------
+    def __call__(self, X1, X2, diag: bool = False, out=None, opt: Optional[FalkonOptions] = None,
+                 kwargs_m1: Optional[Dict[str, torch.Tensor]] = None, kwargs_m2: Optional[Dict[str, torch.Tensor]] = None):
+        """The kernel matrix ``K(X1, X2)`` (N x M), or its diagonal when ``diag``."""
+        X1, X2, out = self._check_mm_dimensions(X1, X2, diag, out)
+        self._check_device_properties(X1, X2, out, fn_name="kernel", opt=opt)
+        params = self._merged(opt)
+        mm_impl = self._decide_mm_impl(X1, X2, diag, params)
+        return mm_impl(kernel=self, opt=params, out=out, diag=diag, X1=X1, X2=X2, kwargs_m1=kwargs_m1,
+                       kwargs_m2=kwargs_m2)
+
+    def _decide_mm_impl(self, X1, X2, diag: bool, opt: FalkonOptions):
+        return fmm
 
     # -- products (falkon/kernels/kernel.py:226-459) --------------------------------------------
     def mmv(self, X1, X2, v, out=None, opt: Optional[FalkonOptions] = None,

@@ -1,0 +1,122 @@
+"""sklearn-style estimator: ``Falkon(kernel, penalty, M).fit(X, Y).predict(X)``.
+
+Same constructor, attributes and flow as falkon/models/falkon.py:120-320 and
+falkon/models/model_utils.py:20-222 (centres -> preconditioner -> preconditioned CG ->
+``alpha_``; ``predict`` is one ``kernel.mmv``).  The whole problem is made resident on the GPU for
+the duration of ``fit`` (the reference's ``InCoreFalkon`` mode) whatever device the data came from;
+fitted attributes are returned on the data's device.
+"""
+import time
+from typing import Callable, Optional, Union
+
+import numpy as np
+import torch
+
+from .center_selection import CenterSelector, UniformSelector
+from .optim import FalkonConjugateGradient
+from .options import FalkonOptions
+from .preconditioner import FalkonPreconditioner
+from .utils.helpers import check_same_dtype
+
+__all__ = ("Falkon", "InCoreFalkon")
+
+try:                                    # keep sklearn's get_params / set_params / clone when it is there
+    from sklearn.base import BaseEstimator as _Base
+except Exception:                       # pragma: no cover
+    _Base = object
+
+
+class Falkon(_Base):
+    def __init__(self, kernel, penalty: float, M: Optional[int],
+                 center_selection: Union[str, CenterSelector] = "uniform", maxiter: int = 20,
+                 seed: Optional[int] = None, error_fn: Optional[Callable] = None, error_every: Optional[int] = 1,
+                 weight_fn: Optional[Callable] = None, options: Optional[FalkonOptions] = None):
+        if weight_fn is not None:
+            raise NotImplementedError("weighted least squares is not part of this build")
+        self.kernel, self.penalty, self.M, self.maxiter = kernel, penalty, M, maxiter
+        self.seed, self.error_fn, self.error_every, self.weight_fn = seed, error_fn, error_every, weight_fn
+        if seed is not None:
+            torch.manual_seed(seed)
+        self.random_state_ = np.random.default_rng(seed)
+        self.options = options or FalkonOptions()
+        if isinstance(center_selection, str):
+            if center_selection.lower() != "uniform":
+                raise ValueError(f'Center selection "{center_selection}" is not valid.')
+            if M is None:
+                raise ValueError("M must be specified when no `CenterSelector` object is provided. "
+                                 "Specify an integer value for `M` or a `CenterSelector` object.")
+            center_selection = UniformSelector(self.random_state_, num_centers=M)
+        self.center_selection = center_selection
+        self.alpha_ = self.beta_ = self.ny_points_ = self.precond = None
+        self.fit_times_ = self.val_errors_ = None
+
+    def _device(self) -> torch.device:
+        if self.options.use_cpu or not torch.cuda.is_available():
+            raise RuntimeError("falkon_amd.Falkon runs on the GPU only (no CPU solver in this build)")
+        return torch.device("cuda", torch.cuda.current_device())
+
+    def fit(self, X: torch.Tensor, Y: torch.Tensor, Xts: Optional[torch.Tensor] = None,
+            Yts: Optional[torch.Tensor] = None, warm_start: Optional[torch.Tensor] = None):
+        if X.shape[0] != Y.shape[0]:
+            raise ValueError(f"X and Y must have the same number of samples (found {X.shape[0]} and {Y.shape[0]})")
+        if Y.dim() == 1:
+            Y = Y.unsqueeze(1)
+        if Y.dim() != 2:
+            raise ValueError(f"Y is expected 1D or 2D. Found {Y.dim()}D.")
+        if not check_same_dtype(X, Y):
+            raise TypeError("X and Y must have the same data-type.")
+        dev = X.device if X.is_cuda else self._device()
+        self.alpha_ = self.beta_ = self.ny_points_ = self.precond = None
+        self.fit_times_, self.val_errors_ = [], []
+        t_s = time.time()
+        with torch.inference_mode():
+            ny_points = self.center_selection.select(X, None)
+            Xd, Yd, Cd = X.to(dev), Y.to(dev), ny_points.to(dev)
+            self.precond = FalkonPreconditioner(self.penalty, self.kernel, self.options)
+            self.precond.init(Cd)
+            self.fit_times_.append(time.time() - t_s)
+            cb = None
+            if self.error_fn is not None and self.error_every is not None:
+                cb = self._callback(Xd, Yd, Xts, Yts, Cd)
+            optim = FalkonConjugateGradient(self.kernel, self.precond, self.options)
+            ws = warm_start.to(dev) if warm_start is not None else None
+            beta = optim.solve(Xd, Cd, Yd, self.penalty, initial_solution=ws, max_iter=self.maxiter, callback=cb)
+            alpha = self.precond.apply(beta)
+            self.alpha_, self.beta_, self.ny_points_ = alpha.to(X.device), beta.to(X.device), ny_points
+        return self
+
+    def _callback(self, X, Y, Xts, Yts, ny_points):
+        def val_cback(it, beta, train_time):
+            self.fit_times_.append(self.fit_times_[0] + train_time)
+            if it % self.error_every != 0:
+                print(f"Iteration {it:3d} - Elapsed {self.fit_times_[-1]:.2f}s", flush=True)
+                return
+            alpha = self.precond.apply(beta)
+            on_val = Xts is not None and Yts is not None
+            pred = self._predict(Xts if on_val else X, ny_points, alpha)
+            err = self.error_fn((Yts if on_val else Y).to(pred.device), pred)
+            name = "error"
+            if isinstance(err, tuple) and len(err) == 2:
+                err, name = err
+            print(f"Iteration {it:3d} - Elapsed {self.fit_times_[-1]:.2f}s - "
+                  f"{'validation' if on_val else 'training'} {name}: {err}", flush=True)
+            self.val_errors_.append(err)
+        return val_cback
+
+    def _predict(self, X, ny_points, alpha):
+        with torch.inference_mode():
+            dev = alpha.device if alpha.is_cuda else (X.device if X.is_cuda else self._device())
+            return self.kernel.mmv(X.to(dev), ny_points.to(dev), alpha.to(dev), opt=self.options)
+
+    def predict(self, X: torch.Tensor) -> torch.Tensor:
+        if self.alpha_ is None or self.ny_points_ is None:
+            raise RuntimeError("Falkon has not been trained. `predict` must be called after `fit`.")
+        return self._predict(X, self.ny_points_, self.alpha_).to(X.device)
+
+    def to(self, device):
+        self.alpha_, self.ny_points_ = self.alpha_.to(device), self.ny_points_.to(device)
+        return self
+
+
+class InCoreFalkon(Falkon):
+    """Alias: every fit is in-core on the GPU in this build (falkon/models/incore_falkon.py:178-257)."""

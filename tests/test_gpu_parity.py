@@ -9,7 +9,7 @@ import torch
 
 from falkon_amd import FalkonOptions, GaussianKernel
 from oracle import brute, inputs, mmv_ref
-from conftest import rel_err
+from conftest import check_parity, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -82,6 +82,47 @@ def test_reference_fixture_fp64(dev, order, sig):
     torch.testing.assert_close(k.dmmv(Ag, Bg, vg, wg).cpu(), K.T @ (K @ v + w), rtol=1e-8, atol=1e-8)
     # output follows X1's memory order (mmv_ops/utils.py:124-155)
     assert (k.mmv(Ag, Bg, vg).stride(0) == 1) == (order == "F")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("n,m,d,t", [
+    (100, 250, 110, 2),     # the reference's large-d shape (tests/test_kernels.py:594-601)
+    (300, 257, 65, 1),      # first d beyond the register-resident kernel
+    (1000, 700, 200, 3),
+    (513, 300, 784, 10),    # configuration 4's d and T
+    (40, 1100, 131, 17),    # more columns than one pass holds, odd d
+    (700, 20, 1000, 5),
+])
+def test_large_d_vs_oracle(dev, dtype, n, m, d, t):
+    """d > 64 runs the LDS-tiled kernel; same tolerances against the blocked CPU oracle."""
+    X, C, v, w = _rand(n, d, m, t, dtype, seed=n + d, scale=0.5)
+    sigma = 0.6 * np.sqrt(d)
+    k = GaussianKernel(sigma)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    got_mmv = k.mmv(Xg, Cg, vg)
+    got_dmmv = k.dmmv(Xg, Cg, vg, wg)
+    assert rel_err(got_mmv, mmv_ref.fmmv_ref(X, C, v, sigma)) < TOL[dtype]
+    assert rel_err(got_dmmv, mmv_ref.fdmmv_ref(X, C, v, w, sigma)) < TOL[dtype]
+    assert rel_err(got_mmv, brute.mmv_brute(X, C, sigma, v)) < 5 * TOL[dtype]
+
+
+def test_config4_shape_reduced(dev):
+    """Config 4 (d=784, T=10, sigma=10, 80 % zeros) at N=20000, M=2000, fp32 and fp64, fmmv and dfmmv.
+
+    All kernel values lie in [0.53, 1] here, so a column of K v is close to mean(K) * sum(v[:, t]) and
+    columns whose sum(v) is small are ill-conditioned: the CPU fp32 path is itself 5e-6..5e-5 away from
+    its fp64 twin.  check_parity handles that case.
+    """
+    for dtype in (torch.float32, torch.float64):
+        X, C, sigma, v, w = inputs.make_config("C4", N=20_000, M=2_000, dtype=dtype)
+        k = GaussianKernel(sigma)
+        Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+        Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+        budget = 2 * 2**30
+        check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma, max_cpu_mem=budget),
+                     mmv_ref.fmmv_ref(Xd, Cd, vd, sigma, max_cpu_mem=budget), TOL[dtype])
+        check_parity(k.dmmv(Xg, Cg, vg, wg), mmv_ref.fdmmv_ref(X, C, v, w, sigma, max_cpu_mem=budget),
+                     mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma, max_cpu_mem=budget), TOL[dtype])
 
 
 def test_per_dimension_sigma_fp32(dev):
