@@ -1,0 +1,179 @@
+"""The callers of the hot path: conjugate gradient, preconditioner, Falkon estimator.
+
+CPU part: the oracle's restatement of the pipeline is pinned against the closed-form solution of the
+linear system (the reference's own check, falkon/tests/test_conjgrad.py:74-131), the product's CG and
+preconditioner algebra are checked without a GPU.  GPU part: ``Falkon.fit`` / ``predict`` with the HIP
+products against the CPU pipeline.
+"""
+import numpy as np
+import pytest
+import torch
+
+from falkon_amd import Falkon, FalkonOptions, GaussianKernel
+from falkon_amd.center_selection import FixedSelector, UniformSelector
+from falkon_amd.optim import ConjugateGradient
+from falkon_amd.preconditioner import FalkonPreconditioner
+from oracle import falkon_ref, gaussian_ref, inputs
+
+
+def _conjgrad_problem(dtype=np.float64):
+    """falkon/tests/test_conjgrad.py:74-99: N=500, M=10, D=1000, sigma=100, lambda=10; gen_random seeds 10 / 9,
+    centres chosen with default_rng(2)."""
+    N, M, D = 500, 10, 1000
+    X = torch.from_numpy(inputs.gen_random(N, D, dtype, F=False, seed=10))
+    Y = torch.from_numpy(inputs.gen_random(N, 1, dtype, F=False, seed=9))
+    idx = np.random.default_rng(2).choice(N, M, replace=False)
+    return X, Y, X[idx].clone(), 100.0, 10.0
+
+
+def test_oracle_pipeline_solves_the_normal_equations():
+    X, Y, C, sigma, lam = _conjgrad_problem()
+    alpha = falkon_ref.falkon_fit_ref(X, Y, C, sigma, lam, maxiter=200, cg_tolerance=1e-10)
+    expected = falkon_ref.nystrom_krr_direct(X, Y, C, sigma, lam)
+    np.testing.assert_allclose(alpha.numpy(), expected, rtol=1e-5)
+
+
+def test_oracle_pipeline_multiple_rhs_and_prediction():
+    X, Y, C, sigma, lam = _conjgrad_problem()
+    Y10 = torch.from_numpy(inputs.gen_random(500, 10, np.float64, seed=9))
+    alpha = falkon_ref.falkon_fit_ref(X, Y10, C, sigma, lam, maxiter=200, cg_tolerance=1e-10)
+    expected = falkon_ref.nystrom_krr_direct(X, Y10, C, sigma, lam)
+    np.testing.assert_allclose(alpha.numpy(), expected, rtol=1e-5)
+    Knm = gaussian_ref.rbf_core_ref(X, C, None, torch.tensor([sigma]))
+    torch.testing.assert_close(falkon_ref.falkon_predict_ref(X, C, alpha, sigma), Knm @ alpha, rtol=1e-10, atol=1e-12)
+
+
+def test_conjugate_gradient_on_dense_spd_system():
+    g = np.random.default_rng(0)
+    Q = g.standard_normal((30, 30))
+    A = torch.from_numpy(Q @ Q.T + 30 * np.eye(30))
+    B = torch.from_numpy(g.standard_normal((30, 3)))
+    cg = ConjugateGradient(FalkonOptions(cg_tolerance=1e-9))
+    X = cg.solve(None, B, lambda v: A @ v, max_iter=100)
+    torch.testing.assert_close(A @ X, B, rtol=1e-9, atol=1e-9)
+    assert cg.num_iter < 60
+    X2 = cg.solve(X.clone(), B, lambda v: A @ v, max_iter=5)          # warm start stays converged
+    torch.testing.assert_close(X2, X, rtol=1e-9, atol=1e-9)
+
+
+class _DenseKernel:
+    """Stands in for the GPU kernel object so the preconditioner algebra can run on the host."""
+
+    def __init__(self, sigma):
+        self.sigma = torch.tensor([float(sigma)])
+
+    def __call__(self, X1, X2, opt=None):
+        return gaussian_ref.rbf_core_ref(X1.double(), X2.double(), None, self.sigma).to(X1.dtype)
+
+
+def test_preconditioner_invariants():
+    """falkon/tests/test_chol_prec.py:17-67: T^T T = K + eps M I, A^T A = T T^T / M + lambda I, solves invert."""
+    g = np.random.default_rng(1)
+    C = torch.from_numpy(g.standard_normal((40, 5)))
+    lam, M = 1e-3, 40
+    pc = FalkonPreconditioner(lam, _DenseKernel(2.0), FalkonOptions())
+    with pytest.raises(RuntimeError):
+        pc.invA(torch.ones(40, 1, dtype=torch.float64))
+    pc.init(C)
+    K = _DenseKernel(2.0)(C, C)
+    T, A = pc.LT.T, pc.LA.T
+    torch.testing.assert_close(T.T @ T, K + 1e-13 * M * torch.eye(M, dtype=torch.float64), rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(A.T @ A, T @ T.T / M + lam * torch.eye(M, dtype=torch.float64), rtol=1e-10, atol=1e-10)
+    v = torch.from_numpy(g.standard_normal((40, 3)))
+    torch.testing.assert_close(A @ pc.invA(v), v, rtol=1e-8, atol=1e-8)
+    torch.testing.assert_close(A.T @ pc.invAt(v), v, rtol=1e-8, atol=1e-8)
+    torch.testing.assert_close(T @ pc.invT(v), v, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(T.T @ pc.invTt(v), v, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(pc.apply(v), pc.invT(pc.invA(v)), rtol=0, atol=0)
+    torch.testing.assert_close(pc.apply_t(v), pc.invAt(pc.invTt(v)), rtol=0, atol=0)
+    # and the oracle's scipy restatement builds the same factors
+    ref = falkon_ref.PrecondRef(C, torch.tensor([2.0]), lam)
+    np.testing.assert_allclose(ref.T, T.numpy(), rtol=1e-8, atol=1e-10)
+    np.testing.assert_allclose(ref.A, A.numpy(), rtol=1e-8, atol=1e-10)
+
+
+def test_center_selection_is_seeded_uniform_without_replacement():
+    X = torch.arange(200, dtype=torch.float32).reshape(100, 2)
+    sel = UniformSelector(np.random.default_rng(7), num_centers=10)
+    C, idx = sel.select_indices(X, None)
+    expect = np.random.default_rng(7).choice(100, size=10, replace=False)
+    assert np.array_equal(idx.numpy(), expect) and torch.equal(C, X[expect])
+    assert len(set(idx.tolist())) == 10
+    Xf = torch.empty_strided((100, 2), (1, 100)).copy_(X)
+    assert UniformSelector(0, 5).select(Xf, None).stride(0) == 1          # memory order is kept
+    with pytest.warns(UserWarning):
+        assert UniformSelector(0, 500).select(X, None).shape[0] == 100
+    fs = FixedSelector(X[:3])
+    assert fs.select(X, None) is not None
+    with pytest.raises(RuntimeError):
+        fs.select_indices(X, None)
+
+
+def test_falkon_constructor_errors():
+    k = GaussianKernel(1.0)
+    with pytest.raises(ValueError):
+        Falkon(k, 1e-3, None)
+    with pytest.raises(ValueError):
+        Falkon(k, 1e-3, 10, center_selection="kmeans")
+    f = Falkon(k, 1e-3, 10)
+    with pytest.raises(RuntimeError):
+        f.predict(torch.zeros(3, 2))
+    with pytest.raises(ValueError):
+        f.fit(torch.zeros(5, 2), torch.zeros(4))
+    with pytest.raises(TypeError):
+        f.fit(torch.zeros(5, 2), torch.zeros(5, dtype=torch.float64))
+    assert f.get_params()["M"] == 10                                       # sklearn surface
+
+
+# --------------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+def test_falkon_cg_matches_direct_solve_on_gpu(dev):
+    """The reference's conjugate-gradient test (tests/test_conjgrad.py:100-131) through the HIP products."""
+    X, Y, C, sigma, lam = _conjgrad_problem()
+    model = Falkon(GaussianKernel(sigma), lam, M=10, center_selection=FixedSelector(C), maxiter=200,
+                   options=FalkonOptions(cg_tolerance=1e-10))
+    model.fit(X.to(dev), Y.to(dev))
+    expected = falkon_ref.nystrom_krr_direct(X, Y, C, sigma, lam)
+    np.testing.assert_allclose(model.alpha_.cpu().numpy(), expected, rtol=1e-5)
+    Y10 = torch.from_numpy(inputs.gen_random(500, 10, np.float64, seed=9))
+    model.fit(X.to(dev), Y10.to(dev))
+    np.testing.assert_allclose(model.alpha_.cpu().numpy(), falkon_ref.nystrom_krr_direct(X, Y10, C, sigma, lam), rtol=1e-5)
+
+
+def _config5(N, Nts, seed=1005, d=28):
+    rng = np.random.default_rng(seed)
+    X = rng.standard_normal((N, d)).astype(np.float32)
+    Xts = rng.standard_normal((Nts, d)).astype(np.float32)
+    a = rng.standard_normal(d) / np.sqrt(d)
+    y = np.sign(np.sin(X @ a) + 0.3 * rng.standard_normal(N)).astype(np.float32)
+    yts = np.sign(np.sin(Xts @ a) + 0.3 * rng.standard_normal(Nts)).astype(np.float32)
+    return tuple(torch.from_numpy(t) for t in (X, y.reshape(-1, 1), Xts, yts.reshape(-1, 1)))
+
+
+@pytest.mark.gpu
+def test_config5_reduced_end_to_end(dev):
+    """Config 5 at N=40000, M=2000, test 8000: sigma=3.8, penalty=1e-6, 20 CG iterations, fp32.
+    Test MSE of the GPU fit must be within 0.1 % (relative) of the CPU pipeline's on the same centres."""
+    X, Y, Xts, Yts = _config5(40_000, 8_000)
+    M, sigma, lam = 2_000, 3.8, 1e-6
+    model = Falkon(GaussianKernel(sigma), lam, M=M, maxiter=20, seed=12)
+    model.fit(X, Y)                                                        # host data, GPU compute, host results
+    assert model.alpha_.device.type == "cpu" and model.alpha_.shape == (M, 1)
+    pred = model.predict(Xts)
+    mse_gpu = float(((pred - Yts) ** 2).mean())
+    C = model.ny_points_
+    alpha_ref = falkon_ref.falkon_fit_ref(X, Y, C, sigma, lam, maxiter=20)
+    mse_ref = float(((falkon_ref.falkon_predict_ref(Xts, C, alpha_ref, sigma) - Yts) ** 2).mean())
+    assert abs(mse_gpu - mse_ref) / mse_ref < 1e-3, (mse_gpu, mse_ref)
+    assert mse_gpu < 0.9                                                   # it learned something (labels are +-1)
+    # resident-data variant gives the same model
+    model2 = Falkon(GaussianKernel(sigma), lam, M=M, maxiter=20, center_selection=FixedSelector(C))
+    model2.fit(X.to(dev), Y.to(dev))
+    assert model2.alpha_.is_cuda
+    mse2 = float(((model2.predict(Xts.to(dev)).cpu() - Yts) ** 2).mean())
+    assert abs(mse2 - mse_gpu) / mse_gpu < 1e-3
+    # warm start from the preconditioned solution resumes instead of restarting
+    model3 = Falkon(GaussianKernel(sigma), lam, M=M, maxiter=2, center_selection=FixedSelector(C))
+    model3.fit(X.to(dev), Y.to(dev), warm_start=model2.beta_.clone())
+    mse3 = float(((model3.predict(Xts.to(dev)).cpu() - Yts) ** 2).mean())
+    assert abs(mse3 - mse_gpu) / mse_gpu < 5e-3
