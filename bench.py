@@ -22,11 +22,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 matrix peak = fp32 vector peak (vendor figure)
+FP64_PEAK_TFLOPS = 78.6    # MI355X fp64 matrix peak = fp64 vector peak
 
 WORKLOADS = {
     # name: (seed, N, d, M, T, has_w)
     "C2": (1002, 1_000_000, 28, 20_000, 1, True),
     "C3": (1003, 10_000_000, 9, 50_000, 1, False),
+    "C4": (1004, 500_000, 784, 10_000, 10, True),
 }
 
 # HBM bytes per launch of the product kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
@@ -40,10 +42,18 @@ def make_inputs(name):
     rng = np.random.default_rng(seed)
     if name == "C2":
         X = rng.standard_normal((N, d), dtype=np.float32)
-    else:
+    elif name == "C3":
         X = rng.random((N, d), dtype=np.float32) * 2.0 - 1.0
+    else:                                   # C4: uniform[0,1) with 80 % of the entries zeroed, stored dense
+        X = rng.random((N, d), dtype=np.float32)
+        X *= rng.random((N, d), dtype=np.float32) < 0.2
     idx = rng.choice(N, size=M, replace=False)
-    sigma = torch.tensor([3.8], dtype=torch.float64) if name == "C2" else torch.from_numpy(rng.uniform(0.5, 2.0, d))
+    if name == "C2":
+        sigma = torch.tensor([3.8], dtype=torch.float64)
+    elif name == "C3":
+        sigma = torch.from_numpy(rng.uniform(0.5, 2.0, d))
+    else:
+        sigma = torch.tensor([10.0], dtype=torch.float64)
     v = rng.standard_normal((M, T)).astype(np.float32)
     w = rng.standard_normal((N, T)).astype(np.float32) if has_w else None
     C = np.ascontiguousarray(X[idx])
@@ -82,6 +92,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f64"], help="arithmetic type (the headline is f32)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=0)
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
@@ -111,10 +122,14 @@ def main():
     dev = torch.device("cuda:0")
     seed, N, d, M, T, has_w = WORKLOADS[args.workload]
     X, C, sigma, v, w = make_inputs(args.workload)
+    tdt = torch.float32 if args.dtype == "f32" else torch.float64
+    X, C, v = X.to(tdt), C.to(tdt), v.to(tdt)
+    w = w.to(tdt) if w is not None else None
+    peak = FP32_PEAK_TFLOPS if args.dtype == "f32" else FP64_PEAK_TFLOPS
     Xg, Cg, vg = X.to(dev), C.to(dev), v.to(dev)
     wg = w.to(dev) if w is not None else None
     kernel = GaussianKernel(sigma)
-    out = torch.empty(M, T, dtype=torch.float32, device=dev)
+    out = torch.empty(M, T, dtype=tdt, device=dev)
 
     def step():
         kernel.dmmv(Xg, Cg, vg, wg, out=out)
@@ -140,27 +155,31 @@ def main():
     kern_ms = tot_ms.value / max(launches.value, 1)
     achieved = flop_per_launch / (kern_ms * 1e-3) / 1e12
     res = {
-        "metric": "dfmmv kernel-entries/sec (N*M*T/s) fp32, 1 MI355X",
+        "metric": f"dfmmv kernel-entries/sec (N*M*T/s) {'fp32' if args.dtype == 'f32' else 'fp64'}, 1 MI355X",
         "value": value, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": f"{args.workload}: Gaussian dfmmv K^T(Kv+w), N={N}, d={d}, M={M}, T={T}, "
-                               f"{'sigma=3.8' if args.workload == 'C2' else 'per-dimension sigma'}, fp32, "
+                               f"{ {'C2': 'sigma=3.8', 'C3': 'per-dimension sigma', 'C4': 'sigma=10'}[args.workload] }, "
+                               f"{'fp32' if args.dtype == 'f32' else 'fp64'}, "
                                f"inputs resident in HBM, packing included in every step"},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / FP32_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "kernel": "mmv_small_f32_kernel", "launches_per_step": launches.value / args.steps,
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                     "frac": achieved / peak,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.dtype == "f32" else None,
+                     "kernel": ("mmv_large_kernel" if d > 64 else "mmv_small_%s_kernel" % args.dtype),
+                     "launches_per_step": launches.value / args.steps,
                      "avg_launch_ms": kern_ms, "flop_per_launch": flop_per_launch},
-        "whole_step_flop_frac": (N * M * (2 * (2 * d + 4) + 4 * T)) / (elapsed / args.steps) / 1e12 / FP32_PEAK_TFLOPS,
+        "whole_step_flop_frac": (N * M * (2 * (2 * d + 4) + 4 * T)) / (elapsed / args.steps) / 1e12 / peak,
     }
     if not args.no_cpu_baseline:
-        rows = args.cpu_rows or (N if args.workload == "C2" else 400_000)
+        rows = args.cpu_rows or {"C2": N, "C3": 400_000, "C4": 100_000}[args.workload]
 
         def gpu_on(Xs, ws):
             Xd = Xs.to(dev)
             wd = ws.to(dev) if ws is not None else None
             r32 = kernel.dmmv(Xd, Cg, vg, wd)
-            r64 = kernel.dmmv(Xd.double(), Cg.double(), vg.double(), wd.double() if wd is not None else None)
+            r64 = r32 if tdt == torch.float64 else kernel.dmmv(Xd.double(), Cg.double(), vg.double(),
+                                                               wd.double() if wd is not None else None)
             return r32, r64
 
         res["cpu_baseline"] = cpu_baseline(X, C, sigma, v, w, gpu_on, rows)

@@ -162,8 +162,10 @@ static int pack_impl(const void *X, int64_t n, int64_t d, int64_t rs, int64_t cs
     if (bytes < packed_bytes<T>(n, d)) return fail(FLK_ENOMEM, "packed buffer too small");
     if (n > 0 && packed == nullptr) return fail(FLK_EINVAL, "packed: null pointer");
     PackedView v = packed_view<T>(packed, n, d);
+    // odd-d fp32 operands of the register-resident kernel carry 1.0 in their one padding feature
+    const bool one_pad = sizeof(T) == 4 && (d & 1) && d <= mmv_small_max_d<T>();
     return launch_pack<T>((const T *)X, n, d, rs, cs, (const T *)sigma, n_sigma, (T *)v.data, (T *)v.hnorm, v.dpad,
-                          v.nblk, st);
+                          v.nblk, one_pad, st);
 }
 
 template <typename T>

@@ -64,7 +64,7 @@ int fail(int code, const char *fmt, ...);
 // launchers implemented in the .hip files -------------------------------------
 template <typename T>
 int launch_pack(const T *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const T *sigma, int64_t n_sigma,
-                T *pdata, T *hnorm, int64_t dpad, int64_t nblk, hipStream_t st);
+                T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st);
 
 template <typename T>
 int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad, hipStream_t st);

@@ -19,7 +19,8 @@ template <> __device__ __forceinline__ int block_pos<double>(int r) { return 4 *
 template <typename T>
 __global__ void __launch_bounds__(256) pack_kernel(const T *__restrict__ X, int64_t n, int64_t d, int64_t rs,
                                                    int64_t cs, const T *__restrict__ sigma, int64_t n_sigma,
-                                                   T *__restrict__ pdata, T *__restrict__ hnorm, int64_t dpad) {
+                                                   T *__restrict__ pdata, T *__restrict__ hnorm, int64_t dpad,
+                                                   bool one_pad) {
     constexpr int BLK = Geo<T>::BLK;
     constexpr int KT = 32;                       // features per LDS tile
     __shared__ T tile[BLK][KT + 1];
@@ -40,6 +41,8 @@ __global__ void __launch_bounds__(256) pack_kernel(const T *__restrict__ X, int6
             if (row < n && kk < d) {
                 double s = kSqrtLog2e / (double)sigma[n_sigma == 1 ? 0 : kk];
                 val = (T)((double)X[row * rs + kk * cs] * s);
+            } else if (one_pad && kk == d) {
+                val = T(1);          // padding feature of odd-d fp32 operands: multiplies the folded half norm
             }
             tile[r][k] = val;
         }
@@ -52,7 +55,7 @@ __global__ void __launch_bounds__(256) pack_kernel(const T *__restrict__ X, int6
         }
         if (tid < BLK) {
             double s = 0.0;
-            int kmax = (int)((dpad - k0) < KT ? (dpad - k0) : KT);
+            int kmax = (int)((d - k0) < KT ? (d - k0) : KT);   // real features only
             for (int k = 0; k < kmax; k++) { double x = (double)tile[tid][k]; s += x * x; }
             nrm[tid] += s;
         }
@@ -62,17 +65,17 @@ __global__ void __launch_bounds__(256) pack_kernel(const T *__restrict__ X, int6
 
 template <typename T>
 int launch_pack(const T *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const T *sigma, int64_t n_sigma,
-                T *pdata, T *hnorm, int64_t dpad, int64_t nblk, hipStream_t st) {
+                T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st) {
     if (nblk == 0) return FLK_OK;
     hipLaunchKernelGGL(pack_kernel<T>, dim3((unsigned)nblk), dim3(256), 0, st, X, n, d, rs, cs, sigma, n_sigma, pdata,
-                       hnorm, dpad);
+                       hnorm, dpad, one_pad);
     FLK_LAUNCH_CHECK("pack_kernel");
     return FLK_OK;
 }
 template int launch_pack<float>(const float *, int64_t, int64_t, int64_t, int64_t, const float *, int64_t, float *,
-                                float *, int64_t, int64_t, hipStream_t);
+                                float *, int64_t, int64_t, bool, hipStream_t);
 template int launch_pack<double>(const double *, int64_t, int64_t, int64_t, int64_t, const double *, int64_t, double *,
-                                 double *, int64_t, int64_t, hipStream_t);
+                                 double *, int64_t, int64_t, bool, hipStream_t);
 
 // ---------------------------------------------------------------------------
 // vec_planar: v[n,t] with element strides (rs, cs) -> vp[t][npad], zero padded.
