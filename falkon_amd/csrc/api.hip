@@ -52,11 +52,11 @@ struct ScopedKernelTimer {
     }
 };
 
-constexpr int kColChunk = 4;          // right-hand sides handled per pass of the product kernel
 constexpr int64_t kTargetWgs = 8192;  // workgroups wanted per launch: 256 CUs x 2 resident x 16 rounds, so that
                                       // the partly filled last round costs a few percent at most
 constexpr int64_t kMinChunkBlocks = 16;
-constexpr int kMaxSplits = 1024;
+constexpr int kMaxSplits = 4096;
+constexpr int64_t kWideChunkBlocks = 64;  // column chunks wider than 4 accumulate in one fp32 level: keep the chunks short
 
 struct Plan {
     bool large;            // LDS-tiled kernel (d beyond the register-resident kernel's range)
@@ -69,7 +69,7 @@ struct Plan {
 constexpr int64_t kTargetWgsLarge = 2048;  // one 512-thread workgroup per CU: 8 rounds
 
 template <typename T>
-static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t dpad) {
+static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t dpad, int64_t t) {
     Plan p;
     p.large = d > mmv_small_max_d<T>();
     if (!p.large) {
@@ -79,6 +79,11 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
         int64_t max_splits = na_blocks / kMinChunkBlocks;
         if (max_splits < 1) max_splits = 1;
         if (splits > max_splits) splits = max_splits;
+        p.col_chunk = mmv_small_max_cols<T>(dpad);
+        if (t > 4 && p.col_chunk > 4) {
+            int64_t want = (na_blocks + kWideChunkBlocks - 1) / kWideChunkBlocks;
+            if (splits < want) splits = want;
+        }
         if (splits > kMaxSplits) splits = kMaxSplits;
         if (splits < 1) splits = 1;
         p.chunk = (na_blocks + splits - 1) / splits;
@@ -86,7 +91,6 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
         p.splits = (int)((na_blocks + p.chunk - 1) / p.chunk);
         if (p.splits < 1) p.splits = 1;
         p.partials = p.splits;
-        p.col_chunk = kColChunk;
     } else {
         const int64_t a_tiles = (na_blocks + mmv_large_a_tile_blocks<T>() - 1) / mmv_large_a_tile_blocks<T>();
         const int64_t b_tiles = (nb_blocks + mmv_large_b_tile_blocks<T>() - 1) / mmv_large_b_tile_blocks<T>();
@@ -107,7 +111,7 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
 template <typename T>
 static size_t partial_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t) {
     PackedView A = packed_view<T>(nullptr, n_a, d), B = packed_view<T>(nullptr, n_b, d);
-    Plan p = make_plan<T>(A.nblk, B.nblk, d, A.dpad);
+    Plan p = make_plan<T>(A.nblk, B.nblk, d, A.dpad, t);
     int64_t tc = t < p.col_chunk ? t : p.col_chunk;
     return align256((size_t)p.partials * tc * B.npad * sizeof(T));
 }
@@ -127,7 +131,7 @@ static int mmv_packed_planar(const PackedView &A, const PackedView &B, const T *
                              int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
                              T *partial, size_t partial_avail, hipStream_t st) {
     if (B.n == 0 || t == 0) return FLK_OK;
-    Plan p = make_plan<T>(A.nblk, B.nblk, A.d, A.dpad);
+    Plan p = make_plan<T>(A.nblk, B.nblk, A.d, A.dpad, t);
     for (int64_t t0 = 0; t0 < t; t0 += p.col_chunk) {
         int tc = (int)(t - t0 < p.col_chunk ? t - t0 : p.col_chunk);
         if ((size_t)p.partials * tc * B.npad * sizeof(T) > partial_avail)
@@ -179,7 +183,7 @@ static int mmv_packed_impl(const void *pa, int64_t n_a, const void *pb, int64_t 
     if (out == nullptr) return fail(FLK_EINVAL, "out: null pointer");
     if (n_a > 0 && vec == nullptr) return fail(FLK_EINVAL, "vec: null pointer");
     PackedView A = packed_view<T>(pa, n_a, d), B = packed_view<T>(pb, n_b, d);
-    size_t vec_bytes = align256((size_t)t * A.npad * sizeof(T));
+    size_t vec_bytes = align256((size_t)(t + kColPad) * A.npad * sizeof(T));
     size_t need = vec_bytes + partial_bytes<T>(n_a, n_b, d, t);
     if (ws_bytes < need || (need > 0 && ws == nullptr))
         return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
@@ -194,7 +198,7 @@ static int mmv_packed_impl(const void *pa, int64_t n_a, const void *pb, int64_t 
 template <typename T>
 static size_t fmmv_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {
     PackedView A = packed_view<T>(nullptr, m, d);
-    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + align256((size_t)t * A.npad * sizeof(T)) +
+    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + align256((size_t)(t + kColPad) * A.npad * sizeof(T)) +
            partial_bytes<T>(m, n, d, t);
 }
 
@@ -202,8 +206,8 @@ template <typename T>
 static size_t fdmmv_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {
     PackedView X = packed_view<T>(nullptr, n, d), C = packed_view<T>(nullptr, m, d);
     size_t p1 = partial_bytes<T>(m, n, d, t), p2 = partial_bytes<T>(n, m, d, t);
-    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + align256((size_t)t * C.npad * sizeof(T)) +
-           align256((size_t)t * X.npad * sizeof(T)) + (p1 > p2 ? p1 : p2);
+    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + align256((size_t)(t + kColPad) * C.npad * sizeof(T)) +
+           align256((size_t)(t + kColPad) * X.npad * sizeof(T)) + (p1 > p2 ? p1 : p2);
 }
 
 template <typename T>
@@ -247,8 +251,8 @@ static int fdmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, c
     char *p = (char *)ws;
     void *px = p; p += packed_bytes<T>(n, d);
     void *pc = p; p += packed_bytes<T>(m, d);
-    T *vp = (T *)p; p += align256((size_t)t * C.npad * sizeof(T));
-    T *up = (T *)p; p += align256((size_t)t * X.npad * sizeof(T));
+    T *vp = (T *)p; p += align256((size_t)(t + kColPad) * C.npad * sizeof(T));
+    T *up = (T *)p; p += align256((size_t)(t + kColPad) * X.npad * sizeof(T));
     T *partial = (T *)p;
     size_t partial_avail = ws_bytes - (size_t)(p - (char *)ws);
     if ((rc = pack_impl<T>(X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
@@ -256,7 +260,9 @@ static int fdmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, c
     if ((rc = launch_vec_planar<T>((const T *)v, m, t, v_rs, v_cs, vp, C.npad, st))) return rc;
     X = packed_view<T>(px, n, d);
     C = packed_view<T>(pc, m, d);
-    // u = K v + w, planar [t][X.npad] with zeroed padding so it can feed the second product directly
+    // u = K v + w, planar [t][X.npad] with zeroed padding (rows and the spare planes) so it can feed the
+    // second product directly
+    if ((rc = launch_zero_fill<T>(up + t * X.npad, kColPad * X.npad, st))) return rc;
     if ((rc = mmv_packed_planar<T>(C, X, vp, t, (const T *)w, w_rs, w_cs, up, 1, X.npad, true, partial, partial_avail,
                                    st)))
         return rc;
@@ -316,8 +322,10 @@ int flk_gauss_pack(const void *X, int64_t n, int64_t d, int64_t x_rs, int64_t x_
 size_t flk_gauss_mmv_packed_workspace_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t, int dtype) {
     if (n_a < 0 || n_b < 0 || d < 1 || t < 0) return 0;
     if (dtype == FLK_F64)
-        return align256((size_t)t * packed_view<double>(nullptr, n_a, d).npad * 8) + partial_bytes<double>(n_a, n_b, d, t);
-    return align256((size_t)t * packed_view<float>(nullptr, n_a, d).npad * 4) + partial_bytes<float>(n_a, n_b, d, t);
+        return align256((size_t)(t + kColPad) * packed_view<double>(nullptr, n_a, d).npad * 8) +
+               partial_bytes<double>(n_a, n_b, d, t);
+    return align256((size_t)(t + kColPad) * packed_view<float>(nullptr, n_a, d).npad * 4) +
+           partial_bytes<float>(n_a, n_b, d, t);
 }
 
 int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b, int64_t n_b, int64_t d,

@@ -67,7 +67,9 @@ int launch_pack(const T *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const 
                 T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st);
 
 template <typename T>
-int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad, hipStream_t st);
+int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad,
+                      hipStream_t st);   // also clears the kColPad planes after the t-th
+template <typename T> int launch_zero_fill(T *p, int64_t count, hipStream_t st);
 
 template <typename T>
 int launch_finalize(const T *partial, int splits, int64_t t, int64_t nb, int64_t nb_pad, const T *addend,
@@ -80,6 +82,11 @@ int launch_mmv_small(const PackedView &A, const PackedView &B, const T *vecp, in
                      int64_t a_chunk_blocks, int splits, T *partial, hipStream_t st);
 template <typename T> int64_t mmv_small_max_d();
 template <typename T> int mmv_small_b_blocks_per_wg(int64_t dpad);
+template <typename T> int mmv_small_max_cols(int64_t dpad);   // right-hand sides per pass
+
+// Planes a planar right-hand side buffer must hold for t columns: kernels compute whole column
+// chunks and read zero planes beyond the caller's columns.
+constexpr int64_t kColPad = 15;
 
 // LDS-tiled ("large d") product kernel: any padded feature count, up to mmv_large_max_cols columns per pass.
 // Writes splits * mmv_large_partials_per_split partial results.

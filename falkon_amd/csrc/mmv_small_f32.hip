@@ -13,6 +13,10 @@ template <> int64_t mmv_small_max_d<float>() { return 2 * kMaxDpFr2; }
 template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad) {
     return kWavesPerWg * ((dpad / 2) <= kMaxDpFr4 ? 4 : 2);
 }
+template <> int mmv_small_max_cols<float>(int64_t dpad) {
+    const int64_t dp = dpad / 2;   // must match the instantiations in launch_tt
+    return dp <= 7 ? 16 : dp <= 12 ? 12 : dp <= 16 ? 8 : 4;
+}
 
 template <>
 int launch_mmv_small<float>(const PackedView &A, const PackedView &B, const float *vecp, int64_t vec_ld, int tt,

@@ -81,34 +81,95 @@ __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds
     for (int q = 0; q < FR; q++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[q][r] = FOLD ? hn[r >> 2][r & 3] : hn[r >> 2][r & 3] + hb[q];
-    floatx4 vec[TT][4];
+    if constexpr (TT <= 4) {
+        // few right-hand sides: their entries are read before the MFMA chain and wait in registers
+        floatx4 vec[TT][4];
 #pragma unroll
-    for (int t = 0; t < TT; t++)
+        for (int t = 0; t < TT; t++)
 #pragma unroll
-        for (int g = 0; g < 4; g++) vec[t][g] = *(const floatx4 *)(lds + 32 + 32 * t + 8 * g + 4 * h);
+            for (int g = 0; g < 4; g++) vec[t][g] = *(const floatx4 *)(lds + 32 + 32 * t + 8 * g + 4 * h);
 #pragma unroll
-    for (int s = 0; s < DP; s++)
+        for (int s = 0; s < DP; s++)
 #pragma unroll
-        for (int q = 0; q < FR; q++) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], breg[q][s], acc[q], 0, 0, 0);
+            for (int q = 0; q < FR; q++)
+                acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], breg[q][s], acc[q], 0, 0, 0);
 #pragma unroll
-    for (int q = 0; q < FR; q++)
+        for (int q = 0; q < FR; q++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            float k = kexp2_clamped(acc[q][r]);
+            for (int r = 0; r < 16; r++) {
+                float k = kexp2_clamped(acc[q][r]);
 #pragma unroll
-            for (int t = 0; t < TT; t++) o1[q][t] = __builtin_fmaf(k, vec[t][r >> 2][r & 3], o1[q][t]);
+                for (int t = 0; t < TT; t++) o1[q][t] = __builtin_fmaf(k, vec[t][r >> 2][r & 3], o1[q][t]);
+            }
+    } else {
+        // many right-hand sides: kernel values replace the exponents in the accumulator registers,
+        // then each group of four rows is contracted against one broadcast LDS read per column
+#pragma unroll
+        for (int s = 0; s < DP; s++)
+#pragma unroll
+            for (int q = 0; q < FR; q++)
+                acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], breg[q][s], acc[q], 0, 0, 0);
+#pragma unroll
+        for (int q = 0; q < FR; q++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[q][r] = kexp2_clamped(acc[q][r]);
+        // Groups of up to four columns of one row group, software pipelined by hand: the reads of the
+        // next group are issued, then a compiler memory fence pins them there, then the FMAs of the
+        // current group run.  Without the fences the compiler moves all 4*TT LDS reads to the front
+        // (to hide their latency) and spills.
+        constexpr int NGRP = 4 * ((TT + 3) / 4);
+        floatx4 cur[4], nxt[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (u < TT) cur[u] = *(const floatx4 *)(lds + 32 + 32 * u + 4 * h);
+#pragma unroll
+        for (int grp = 0; grp < NGRP; grp++) {
+            const int g = grp / ((TT + 3) / 4), t0 = 4 * (grp % ((TT + 3) / 4));
+            if (grp + 1 < NGRP) {
+                const int g1 = (grp + 1) / ((TT + 3) / 4), t1 = 4 * ((grp + 1) % ((TT + 3) / 4));
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    if (t1 + u < TT) nxt[u] = *(const floatx4 *)(lds + 32 + 32 * (t1 + u) + 8 * g1 + 4 * h);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (t0 + u < TT) {
+#pragma unroll
+                    for (int q = 0; q < FR; q++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            o1[q][t0 + u] = __builtin_fmaf(acc[q][4 * g + e], cur[u][e], o1[q][t0 + u]);
+                }
+            // fence: the updated accumulators pass through it, so this group's FMAs stay above it and the
+            // next group's reads (ordered by the memory clobber) stay below the previous one
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (t0 + u < TT) {
+                    if constexpr (FR == 4)
+                        asm volatile("" : "+v"(o1[0][t0 + u]), "+v"(o1[1][t0 + u]), "+v"(o1[2][t0 + u]), "+v"(o1[3][t0 + u])
+                                     : "v"(lds) : "memory");
+                    else
+                        asm volatile("" : "+v"(o1[0][t0 + u]), "+v"(o1[1][t0 + u]) : "v"(lds) : "memory");
+                }
+#pragma unroll
+            for (int u = 0; u < 4; u++) cur[u] = nxt[u];
         }
+    }
 }
 
 // FOLD (odd feature counts only): the one padding feature of the packed rows carries 1.0, and the
 // resident B fragment puts hB_j into that slot, so the MFMA chain adds hB_j by itself and the
 // accumulators start from the A block's half norms without any VALU add.
 template <int DP, int FR, int TT, bool FOLD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 registers per lane
     mmv_small_f32_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
                          int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB, int64_t na_blocks,
-                         int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial, int64_t nb_pad) {
+                         int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial, int64_t nb_pad,
+                         int tcols) {
+    // TT columns are computed, the first tcols of them stored; vecp must hold TT planes (zeros beyond the
+    // caller's columns).
     using RV = RowVals<TT>;
+    constexpr bool kTwoLevel = TT <= 4;   // long accumulator only where registers allow; wider TT uses short chunks
     __shared__ __attribute__((aligned(16))) float stage[kWavesPerWg][2][RV::N];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -137,11 +198,11 @@ __global__ void __launch_bounds__(256)
         src[c] = (e < 32 || e >= RV::N) ? hA + (e & 31) : vecp + (int64_t)((e - 32) >> 5) * vec_ld + (e & 31);
     }
 
-    float o1[FR][TT], o2[FR][TT];
+    float o1[FR][TT], o2[FR][kTwoLevel ? TT : 1];
 #pragma unroll
     for (int q = 0; q < FR; q++)
 #pragma unroll
-        for (int t = 0; t < TT; t++) { o1[q][t] = 0.f; o2[q][t] = 0.f; }
+        for (int t = 0; t < TT; t++) { o1[q][t] = 0.f; if (kTwoLevel) o2[q][t] = 0.f; }
 
     float fa0[DP], fa1[DP];
     RV rv;
@@ -164,7 +225,7 @@ __global__ void __launch_bounds__(256)
             if (has2) stage_rowvals<TT>(rv, lds0, lane);
         }
         since_flush += 2;
-        if (since_flush >= kFlushEvery) {
+        if (kTwoLevel && since_flush >= kFlushEvery) {
             since_flush = 0;
 #pragma unroll
             for (int q = 0; q < FR; q++)
@@ -176,10 +237,10 @@ __global__ void __launch_bounds__(256)
     for (int q = 0; q < FR; q++)
 #pragma unroll
         for (int t = 0; t < TT; t++) {
-            float s = o2[q][t] + o1[q][t];
+            float s = kTwoLevel ? o2[q][t] + o1[q][t] : o1[q][t];
             s += __shfl_xor(s, 32, 64);
-            if (h == 0 && bb0 + q < nb_blocks)
-                partial[((int64_t)blockIdx.y * TT + t) * nb_pad + (bb0 + q) * 32 + j] = s;
+            if (h == 0 && bb0 + q < nb_blocks && t < tcols)
+                partial[((int64_t)blockIdx.y * tcols + t) * nb_pad + (bb0 + q) * 32 + j] = s;
         }
 }
 

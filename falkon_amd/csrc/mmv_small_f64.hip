@@ -134,6 +134,7 @@ constexpr int kMaxDp64Fr4 = 8;   // dpad <= 32
 constexpr int kMaxDp64Fr2 = 16;  // dpad <= 64
 
 template <> int64_t mmv_small_max_d<double>() { return 4 * kMaxDp64Fr2; }
+template <> int mmv_small_max_cols<double>(int64_t dpad) { (void)dpad; return 4; }
 template <> int mmv_small_b_blocks_per_wg<double>(int64_t dpad) {
     return kWavesPerWg64 * ((dpad / 4) <= kMaxDp64Fr4 ? 4 : 2);
 }

@@ -78,20 +78,36 @@ template int launch_pack<double>(const double *, int64_t, int64_t, int64_t, int6
                                  double *, int64_t, int64_t, bool, hipStream_t);
 
 // ---------------------------------------------------------------------------
-// vec_planar: v[n,t] with element strides (rs, cs) -> vp[t][npad], zero padded.
+// vec_planar: v[n,t] with element strides (rs, cs) -> vp[t + kColPad][npad]: rows past n and the
+// kColPad planes past t are zero.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256) vec_planar_kernel(const T *__restrict__ v, int64_t n, int64_t rs, int64_t cs,
-                                                         T *__restrict__ vp, int64_t npad) {
+                                                         T *__restrict__ vp, int64_t npad, int64_t tcols) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     int64_t t = blockIdx.y;
-    if (i < npad) vp[t * npad + i] = (i < n) ? v[i * rs + t * cs] : T(0);
+    if (i < npad) vp[t * npad + i] = (i < n && t < tcols) ? v[i * rs + t * cs] : T(0);
 }
+
+template <typename T>
+__global__ void __launch_bounds__(256) zero_fill_kernel(T *__restrict__ p, int64_t count) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) p[i] = T(0);
+}
+template <typename T>
+int launch_zero_fill(T *p, int64_t count, hipStream_t st) {
+    if (count <= 0) return FLK_OK;
+    hipLaunchKernelGGL(zero_fill_kernel<T>, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, p, count);
+    FLK_LAUNCH_CHECK("zero_fill_kernel");
+    return FLK_OK;
+}
+template int launch_zero_fill<float>(float *, int64_t, hipStream_t);
+template int launch_zero_fill<double>(double *, int64_t, hipStream_t);
 template <typename T>
 int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad, hipStream_t st) {
     if (npad == 0 || t == 0) return FLK_OK;
-    hipLaunchKernelGGL(vec_planar_kernel<T>, dim3((unsigned)((npad + 255) / 256), (unsigned)t), dim3(256), 0, st, v, n,
-                       rs, cs, vp, npad);
+    hipLaunchKernelGGL(vec_planar_kernel<T>, dim3((unsigned)((npad + 255) / 256), (unsigned)(t + kColPad)), dim3(256),
+                       0, st, v, n, rs, cs, vp, npad, t);
     FLK_LAUNCH_CHECK("vec_planar_kernel");
     return FLK_OK;
 }

@@ -37,6 +37,11 @@ def _rand(n, d, m, t, dtype, seed, scale=1.0):
     (300, 200, 33, 5),
     (257, 100, 64, 1),
     (64, 64, 2, 7),
+    (2000, 900, 10, 10),    # the reference's mmv benchmark columns (benchmarks/timing_benchmarks/mmv_timings.py:48-127)
+    (400, 3000, 9, 16),
+    (600, 500, 28, 6),
+    (500, 400, 31, 21),     # more columns than one pass holds
+    (300, 300, 40, 9),      # d > 32: column chunks of four
 ])
 def test_mmv_dmmv_vs_oracle(dev, dtype, n, m, d, t):
     X, C, v, w = _rand(n, d, m, t, dtype, seed=n * 7 + m)
