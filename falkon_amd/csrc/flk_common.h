@@ -20,6 +20,15 @@ template <> struct Geo<float>  { static constexpr int BLK = 32; static constexpr
 template <> struct Geo<double> { static constexpr int BLK = 16; static constexpr int KG = 4; };
 
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// Feature counts up to kSmallMaxD run the register-resident kernels and are padded to the MFMA's
+// K granularity only; larger ones run the LDS-tiled kernel, which consumes features in chunks of
+// kLargeKChunk MFMA steps, and are zero padded to whole chunks so that the kernel has no feature tail.
+constexpr int64_t kSmallMaxD = 64;
+constexpr int64_t kLargeKChunk = 8;
+template <typename T> inline int64_t padded_features(int64_t d) {
+    return d <= kSmallMaxD ? round_up(d, Geo<T>::KG) : round_up(d, Geo<T>::KG * kLargeKChunk);
+}
 inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 
 struct PackedView {
@@ -32,7 +41,7 @@ template <typename T>
 inline PackedView packed_view(const void *buf, int64_t n, int64_t d) {
     PackedView v;
     v.n = n; v.d = d;
-    v.dpad = round_up(d, Geo<T>::KG);
+    v.dpad = padded_features<T>(d);
     v.nblk = (n + Geo<T>::BLK - 1) / Geo<T>::BLK;
     v.npad = v.nblk * Geo<T>::BLK;
     v.data = buf;
@@ -41,7 +50,7 @@ inline PackedView packed_view(const void *buf, int64_t n, int64_t d) {
 }
 template <typename T>
 inline size_t packed_bytes(int64_t n, int64_t d) {
-    int64_t dpad = round_up(d, Geo<T>::KG);
+    int64_t dpad = padded_features<T>(d);
     int64_t nblk = (n + Geo<T>::BLK - 1) / Geo<T>::BLK;
     return align256((size_t)nblk * dpad * Geo<T>::BLK * sizeof(T)) + align256((size_t)nblk * Geo<T>::BLK * sizeof(T));
 }

@@ -2,7 +2,7 @@
 //
 //   partial[split'][t][b] = sum_{a in chunk} exp2(A~_a . B~_b + hA_a + hB_b) * vec[a,t]
 //
-// A workgroup of 8 waves owns one tile of output rows (B side) and walks over the tiles of
+// A workgroup owns one tile of output rows (B side) and walks over the tiles of
 // reduction rows (A side) of its chunk.  For every (A tile, B tile) the cross term is a GEMM over
 // the features: feature chunks of both tiles are staged in LDS (double buffered, one barrier per
 // chunk, 16-byte global loads straight from the packed layout, which is already in operand order),
@@ -11,7 +11,7 @@
 // and contracts the tile against vec into per-lane output accumulators that live in registers for
 // the whole kernel.  K is never written anywhere.
 //
-// Waves are arranged 2 (A) x 4 (B); waves with the same wb produce partial sums for the same
+// Waves are arranged WVA (A) x WVB (B); waves with the same wb produce partial sums for the same
 // output rows and simply write separate partials (they count as extra splits for the reduction).
 #include "flk_common.h"
 
@@ -28,6 +28,7 @@ template <> struct LTraits<float> {
     static constexpr int BLK = 32, KG = 2, ACCN = 16, NG = 4, VPL = 4;  // VPL: elements per 16-byte vector
     typedef floatx16 acc_t;
     typedef floatx4 vec4_t;
+    typedef floatx4 v16_t;     // one 16-byte load
     static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
     }
@@ -43,6 +44,7 @@ template <> struct LTraits<double> {
     static constexpr int BLK = 16, KG = 4, ACCN = 4, NG = 1, VPL = 2;
     typedef doublex4 acc_t;
     typedef doublex4 vec4_t;
+    typedef doublex2 v16_t;
     static __device__ __forceinline__ acc_t mfma(double a, double b, acc_t c) {
         return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
     }
@@ -51,24 +53,27 @@ template <> struct LTraits<double> {
     static __device__ __forceinline__ double kexp(double x) { return exp2(fmin(x, 0.0)); }
 };
 
-constexpr int kLWavesA = 2, kLWavesB = 4, kLThreads = 64 * kLWavesA * kLWavesB;
 
-template <typename T, int WA_FR, int WB_FR, int KC> struct LGeo {
+template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC> struct LGeo {
     typedef LTraits<T> TR;
+    static constexpr int kLWavesA = WVA, kLWavesB = WVB, kLThreads = 64 * WVA * WVB;
+    static_assert(kLargeKChunk % KC == 0, "packed features are padded to kLargeKChunk steps");
     static constexpr int NAB = kLWavesA * WA_FR;             // A blocks per tile
     static constexpr int NBB = kLWavesB * WB_FR;             // B blocks per tile
     static constexpr int A_ROWS = NAB * TR::BLK, B_ROWS = NBB * TR::BLK;
     static constexpr int A_ELEMS = NAB * KC * 64, B_ELEMS = NBB * KC * 64;   // per stage
     static constexpr int A_VECS = A_ELEMS / TR::VPL, B_VECS = B_ELEMS / TR::VPL;
-    static constexpr int A_VPT = (A_VECS + kLThreads - 1) / kLThreads;      // 16-byte vectors per thread
-    static constexpr int B_VPT = (B_VECS + kLThreads - 1) / kLThreads;
+    static constexpr int A_VPT = A_VECS / kLThreads;      // 16-byte vectors per thread
+    static constexpr int B_VPT = B_VECS / kLThreads;
+    static_assert(A_VECS % kLThreads == 0 && B_VECS % kLThreads == 0, "stage must split evenly over the threads");
 };
 
 // One 16-byte piece of a stage: vector index vi enumerates [block][step][lane group][row/VPL], which is
-// also the order in LDS, so the LDS side of the copy is linear.
+// also the order in LDS, so the LDS side of the copy is linear.  The packed feature count is a whole
+// number of chunks (padded_features), so there is no feature tail to mask.
 template <typename T, int KC>
 __device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t blk0, int64_t nblk, int64_t dpad,
-                                              int64_t DPsteps, int64_t s0, int vi, bool &valid) {
+                                              int64_t DPsteps, int64_t s0, int vi) {
     typedef LTraits<T> TR;
     constexpr int VPB = TR::BLK / TR::VPL;
     const int jv = vi % VPB;
@@ -77,22 +82,21 @@ __device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t b
     const int blk = vi / (VPB * TR::KG * KC);
     int64_t b = blk0 + blk;
     if (b >= nblk) b = nblk - 1;                 // past the end: any valid block (its rows get zero weight / are not stored)
-    valid = (s0 + s) < DPsteps;                  // feature tail: zero fill
-    const int64_t ss = valid ? s0 + s : 0;
-    return P + (b * dpad + (int64_t)lg * DPsteps + ss) * TR::BLK + jv * TR::VPL;
+    return P + (b * dpad + (int64_t)lg * DPsteps + s0 + s) * TR::BLK + jv * TR::VPL;
 }
 
-template <typename T, int WA_FR, int WB_FR, int KC, int TT>
-__global__ void __launch_bounds__(kLThreads)
+template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC, int TT>
+__global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   // two waves per SIMD either way
     mmv_large_kernel(const T *__restrict__ PA, const T *__restrict__ hA, const T *__restrict__ vecp, int64_t vec_ld,
                      int tcols, const T *__restrict__ PB, const T *__restrict__ hB, int64_t na_blocks,
                      int64_t nb_blocks, int64_t dpad, int64_t a_tiles_per_chunk, T *__restrict__ partial,
                      int64_t nb_pad) {
     typedef LTraits<T> TR;
-    typedef LGeo<T, WA_FR, WB_FR, KC> G;
+    typedef LGeo<T, WVA, WVB, WA_FR, WB_FR, KC> G;
+    constexpr int kLWavesA = WVA, kLWavesB = WVB, kLThreads = 64 * WVA * WVB;
     typedef typename TR::acc_t acc_t;
     typedef typename TR::vec4_t vec4_t;
-    struct __attribute__((aligned(16))) V16 { T v[TR::VPL]; };
+    typedef typename TR::v16_t V16;
 
     __shared__ __attribute__((aligned(16))) T ldsA[2][G::A_ELEMS];
     __shared__ __attribute__((aligned(16))) T ldsB[2][G::B_ELEMS];
@@ -108,7 +112,7 @@ __global__ void __launch_bounds__(kLThreads)
     const int64_t at0 = (int64_t)blockIdx.y * a_tiles_per_chunk;
     int64_t at1 = at0 + a_tiles_per_chunk;
     if (at1 > a_tiles) at1 = a_tiles;
-    const int64_t n_chunks = (DPsteps + KC - 1) / KC;
+    const int64_t n_chunks = DPsteps / KC;     // dpad is a whole number of chunks
 
     // half norms of this lane's output rows
     T hb[WB_FR];
@@ -138,43 +142,17 @@ __global__ void __launch_bounds__(kLThreads)
         auto fetch = [&](int64_t chunk) {
             const int64_t s0 = chunk * KC;
 #pragma unroll
-            for (int c = 0; c < G::A_VPT; c++) {
-                int vi = tid + c * kLThreads;
-                if (vi < G::A_VECS) {
-                    bool valid;
-                    const T *src = stage_src<T, KC>(PA, ablk0, na_blocks, dpad, DPsteps, s0, vi, valid);
-                    V16 x = *(const V16 *)src;
-                    if (!valid)
+            for (int c = 0; c < G::A_VPT; c++)
+                ra[c] = *(const V16 *)stage_src<T, KC>(PA, ablk0, na_blocks, dpad, DPsteps, s0, tid + c * kLThreads);
 #pragma unroll
-                        for (int e = 0; e < TR::VPL; e++) x.v[e] = T(0);
-                    ra[c] = x;
-                }
-            }
-#pragma unroll
-            for (int c = 0; c < G::B_VPT; c++) {
-                int vi = tid + c * kLThreads;
-                if (vi < G::B_VECS) {
-                    bool valid;
-                    const T *src = stage_src<T, KC>(PB, bblk0, nb_blocks, dpad, DPsteps, s0, vi, valid);
-                    V16 x = *(const V16 *)src;
-                    if (!valid)
-#pragma unroll
-                        for (int e = 0; e < TR::VPL; e++) x.v[e] = T(0);
-                    rb[c] = x;
-                }
-            }
+            for (int c = 0; c < G::B_VPT; c++)
+                rb[c] = *(const V16 *)stage_src<T, KC>(PB, bblk0, nb_blocks, dpad, DPsteps, s0, tid + c * kLThreads);
         };
         auto commit = [&](int buf) {
 #pragma unroll
-            for (int c = 0; c < G::A_VPT; c++) {
-                int vi = tid + c * kLThreads;
-                if (vi < G::A_VECS) *(V16 *)(&ldsA[buf][vi * TR::VPL]) = ra[c];
-            }
+            for (int c = 0; c < G::A_VPT; c++) *(V16 *)(&ldsA[buf][(tid + c * kLThreads) * TR::VPL]) = ra[c];
 #pragma unroll
-            for (int c = 0; c < G::B_VPT; c++) {
-                int vi = tid + c * kLThreads;
-                if (vi < G::B_VECS) *(V16 *)(&ldsB[buf][vi * TR::VPL]) = rb[c];
-            }
+            for (int c = 0; c < G::B_VPT; c++) *(V16 *)(&ldsB[buf][(tid + c * kLThreads) * TR::VPL]) = rb[c];
         };
 
         // previous tile's epilogue may still be reading ldsRow and the stage buffers
@@ -199,17 +177,35 @@ __global__ void __launch_bounds__(kLThreads)
             if (ch + 1 < n_chunks) fetch(ch + 1);
             const T *la = &ldsA[buf][(wa * WA_FR) * KC * 64 + lane];
             const T *lb = &ldsB[buf][(wb * WB_FR) * KC * 64 + lane];
+            // Operands are read one step ahead of the MFMAs that use them.  The empty asm after each step
+            // is a compiler fence: it redefines the operands just used (so that step's MFMAs stay above it)
+            // and clobbers memory through the LDS pointer (so the reads of later steps stay below it).
+            // Left alone the compiler hoists all KC steps' reads to the top of the chunk, which costs ~40
+            // registers and pushes the global prefetch registers around.
+            T av[WA_FR], bv[WB_FR], an[WA_FR], bn[WB_FR];
+#pragma unroll
+            for (int p = 0; p < WA_FR; p++) av[p] = la[(p * KC) * 64];
+#pragma unroll
+            for (int q = 0; q < WB_FR; q++) bv[q] = lb[(q * KC) * 64];
 #pragma unroll
             for (int s = 0; s < KC; s++) {
-                T av[WA_FR], bv[WB_FR];
+                if (s + 1 < KC) {
 #pragma unroll
-                for (int p = 0; p < WA_FR; p++) av[p] = la[(p * KC + s) * 64];
+                    for (int p = 0; p < WA_FR; p++) an[p] = la[(p * KC + s + 1) * 64];
 #pragma unroll
-                for (int q = 0; q < WB_FR; q++) bv[q] = lb[(q * KC + s) * 64];
+                    for (int q = 0; q < WB_FR; q++) bn[q] = lb[(q * KC + s + 1) * 64];
+                }
 #pragma unroll
                 for (int p = 0; p < WA_FR; p++)
 #pragma unroll
                     for (int q = 0; q < WB_FR; q++) acc[p][q] = TR::mfma(av[p], bv[q], acc[p][q]);
+                static_assert(WA_FR == 4 && WB_FR == 2, "the step fence lists its operands explicitly");
+                asm volatile("" : "+v"(av[0]), "+v"(av[1]), "+v"(av[2]), "+v"(av[3]), "+v"(bv[0]), "+v"(bv[1])
+                             : "v"(la), "v"(lb) : "memory");
+#pragma unroll
+                for (int p = 0; p < WA_FR; p++) av[p] = an[p];
+#pragma unroll
+                for (int q = 0; q < WB_FR; q++) bv[q] = bn[q];
             }
             if (ch + 1 < n_chunks) commit(buf ^ 1);
             __syncthreads();
@@ -261,13 +257,16 @@ __global__ void __launch_bounds__(kLThreads)
 // dispatch
 // ---------------------------------------------------------------------------
 template <typename T> struct LCfg;
-template <> struct LCfg<float>  { static constexpr int WA_FR = 4, WB_FR = 2, KC = 8; };   // tile 256 (A) x 256 (B) rows
-template <> struct LCfg<double> { static constexpr int WA_FR = 4, WB_FR = 2, KC = 8; };   // tile 128 (A) x 128 (B) rows
+// fp32: 4 waves (2 x 2), two workgroups per CU so that one workgroup's barrier and LDS latencies are covered
+// by the other; tile 256 (A) x 128 (B) rows.
+template <> struct LCfg<float>  { static constexpr int WVA = 2, WVB = 2, WA_FR = 4, WB_FR = 2, KC = 8; };
+// fp64: 8 waves (2 x 4), one workgroup per CU; tile 128 (A) x 128 (B) rows.
+template <> struct LCfg<double> { static constexpr int WVA = 2, WVB = 4, WA_FR = 4, WB_FR = 2, KC = 8; };
 
 template <typename T> int mmv_large_max_cols();
-template <typename T> int mmv_large_a_tile_blocks() { return kLWavesA * LCfg<T>::WA_FR; }
-template <typename T> int mmv_large_b_tile_blocks() { return kLWavesB * LCfg<T>::WB_FR; }
-template <typename T> int mmv_large_partials_per_split() { return kLWavesA; }
+template <typename T> int mmv_large_a_tile_blocks() { return LCfg<T>::WVA * LCfg<T>::WA_FR; }
+template <typename T> int mmv_large_b_tile_blocks() { return LCfg<T>::WVB * LCfg<T>::WB_FR; }
+template <typename T> int mmv_large_partials_per_split() { return LCfg<T>::WVA; }
 template <> int mmv_large_max_cols<float>() { return 16; }
 template <> int mmv_large_max_cols<double>() { return 16; }
 template int mmv_large_a_tile_blocks<float>();
@@ -281,9 +280,10 @@ template <typename T, int TT>
 static int launch_large_tt(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
                            int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
     typedef LCfg<T> C;
-    const int64_t nbb = kLWavesB * C::WB_FR;
+    const int64_t nbb = C::WVB * C::WB_FR;
     dim3 grid((unsigned)((B.nblk + nbb - 1) / nbb), (unsigned)splits);
-    hipLaunchKernelGGL((mmv_large_kernel<T, C::WA_FR, C::WB_FR, C::KC, TT>), grid, dim3(kLThreads), 0, st,
+    hipLaunchKernelGGL((mmv_large_kernel<T, C::WVA, C::WVB, C::WA_FR, C::WB_FR, C::KC, TT>), grid,
+                       dim3(64 * C::WVA * C::WVB), 0, st,
                        (const T *)A.data, (const T *)A.hnorm, vecp, vec_ld, tcols, (const T *)B.data,
                        (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, a_tiles_per_chunk, partial, B.npad);
     FLK_LAUNCH_CHECK("mmv_large_kernel");
