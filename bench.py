@@ -31,9 +31,14 @@ WORKLOADS = {
     "C4": (1004, 500_000, 784, 10_000, 10, True),
 }
 
-# HBM bytes per launch of the product kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
-# (profiles/), keyed by workload; None where it has not been measured.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch of the product kernel, keyed by workload: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# (KiB per dispatch, mean over the launches of the kernel) scaled by what the same counters read for a plain
+# 1 GiB device copy (FETCH_SIZE reads half the true bytes on this box: factor 2.0; WRITE_SIZE factor 1.0).
+# The summaries are under profiles/.  None where it has not been measured.
+MEASURED_TRAFFIC_BYTES = {
+    "C2": int((73418.8 * 2.0 + 17773.4 * 1.0) * 1024),     # 168.6 MB; algorithmic: packed X 112 MB + C + vectors
+    "C4": int((2.60826e7 * 2.0) * 1024),                   # 53.4 GB (reads only; tiles are re-read from L2/MALL/HBM)
+}
 
 
 def make_inputs(name):
@@ -93,6 +98,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"], help="arithmetic type (the headline is f32)")
+    ap.add_argument("--op", default="dmmv", choices=["dmmv", "mmv"],
+                    help="dmmv = K^T(Kv+w), the headline; mmv = K v only (one launch per step)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=0)
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
@@ -129,10 +136,13 @@ def main():
     Xg, Cg, vg = X.to(dev), C.to(dev), v.to(dev)
     wg = w.to(dev) if w is not None else None
     kernel = GaussianKernel(sigma)
-    out = torch.empty(M, T, dtype=tdt, device=dev)
+    out = torch.empty(M if args.op == "dmmv" else N, T, dtype=tdt, device=dev)
 
     def step():
-        kernel.dmmv(Xg, Cg, vg, wg, out=out)
+        if args.op == "dmmv":
+            kernel.dmmv(Xg, Cg, vg, wg, out=out)
+        else:
+            kernel.mmv(Xg, Cg, vg, out=out)
 
     for _ in range(args.warmup):
         step()
@@ -155,11 +165,11 @@ def main():
     kern_ms = tot_ms.value / max(launches.value, 1)
     achieved = flop_per_launch / (kern_ms * 1e-3) / 1e12
     res = {
-        "metric": f"dfmmv kernel-entries/sec (N*M*T/s) {'fp32' if args.dtype == 'f32' else 'fp64'}, 1 MI355X",
+        "metric": f"{'dfmmv' if args.op == 'dmmv' else 'fmmv'} kernel-entries/sec (N*M*T/s) {'fp32' if args.dtype == 'f32' else 'fp64'}, 1 MI355X",
         "value": value, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": f"{args.workload}: Gaussian dfmmv K^T(Kv+w), N={N}, d={d}, M={M}, T={T}, "
+        "config": {"workload": f"{args.workload}: Gaussian {'dfmmv K^T(Kv+w)' if args.op == 'dmmv' else 'fmmv K v'}, N={N}, d={d}, M={M}, T={T}, "
                                f"{ {'C2': 'sigma=3.8', 'C3': 'per-dimension sigma', 'C4': 'sigma=10'}[args.workload] }, "
                                f"{'fp32' if args.dtype == 'f32' else 'fp64'}, "
                                f"inputs resident in HBM, packing included in every step"},
@@ -169,9 +179,10 @@ def main():
                      "kernel": ("mmv_large_kernel" if d > 64 else "mmv_small_%s_kernel" % args.dtype),
                      "launches_per_step": launches.value / args.steps,
                      "avg_launch_ms": kern_ms, "flop_per_launch": flop_per_launch},
-        "whole_step_flop_frac": (N * M * (2 * (2 * d + 4) + 4 * T)) / (elapsed / args.steps) / 1e12 / peak,
+        "whole_step_flop_frac": (N * M * ((2 if args.op == "dmmv" else 1) * (2 * d + 4 + 2 * T)))
+                                / (elapsed / args.steps) / 1e12 / peak,
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.op == "dmmv":
         rows = args.cpu_rows or {"C2": N, "C3": 400_000, "C4": 100_000}[args.workload]
 
         def gpu_on(Xs, ws):

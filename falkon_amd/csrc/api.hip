@@ -108,6 +108,25 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
     return p;
 }
 
+// Width of the kernel instantiation that serves a column chunk of tc right-hand sides: the kernels read
+// that many planes of the planar right-hand side, so the planes past the caller's columns must be zero.
+template <typename T>
+static int instantiated_cols(const Plan &p, int tc) {
+    static const int small32[] = {1, 2, 3, 4, 6, 8, 12, 16}, large[] = {1, 2, 4, 8, 12, 16};
+    if (p.large) {
+        for (int w : large) if (tc <= w) return w;
+    } else if (sizeof(T) == 4) {
+        for (int w : small32) if (tc <= w) return w;
+    }
+    return tc;
+}
+template <typename T>
+static int64_t zero_planes_needed(const Plan &p, int64_t t) {
+    if (t <= 0) return 0;
+    int tc_last = (int)(t % p.col_chunk == 0 ? p.col_chunk : t % p.col_chunk);
+    return instantiated_cols<T>(p, tc_last) - tc_last;
+}
+
 template <typename T>
 static size_t partial_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t) {
     PackedView A = packed_view<T>(nullptr, n_a, d), B = packed_view<T>(nullptr, n_b, d);
@@ -189,7 +208,8 @@ static int mmv_packed_impl(const void *pa, int64_t n_a, const void *pb, int64_t 
         return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
     T *vecp = (T *)ws;
     T *partial = (T *)((char *)ws + vec_bytes);
-    int rc = launch_vec_planar<T>((const T *)vec, n_a, t, vec_rs, vec_cs, vecp, A.npad, st);
+    Plan plan = make_plan<T>(A.nblk, B.nblk, A.d, A.dpad, t);
+    int rc = launch_vec_planar<T>((const T *)vec, n_a, t, vec_rs, vec_cs, vecp, A.npad, zero_planes_needed<T>(plan, t), st);
     if (rc) return rc;
     return mmv_packed_planar<T>(A, B, vecp, t, (const T *)addend, add_rs, add_cs, (T *)out, out_rs, out_cs, false,
                                 partial, ws_bytes - vec_bytes, st);
@@ -257,12 +277,14 @@ static int fdmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, c
     size_t partial_avail = ws_bytes - (size_t)(p - (char *)ws);
     if ((rc = pack_impl<T>(X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
     if ((rc = pack_impl<T>(X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, packed_bytes<T>(m, d), st))) return rc;
-    if ((rc = launch_vec_planar<T>((const T *)v, m, t, v_rs, v_cs, vp, C.npad, st))) return rc;
     X = packed_view<T>(px, n, d);
     C = packed_view<T>(pc, m, d);
+    Plan plan1 = make_plan<T>(C.nblk, X.nblk, d, C.dpad, t), plan2 = make_plan<T>(X.nblk, C.nblk, d, X.dpad, t);
+    if ((rc = launch_vec_planar<T>((const T *)v, m, t, v_rs, v_cs, vp, C.npad, zero_planes_needed<T>(plan1, t), st)))
+        return rc;
     // u = K v + w, planar [t][X.npad] with zeroed padding (rows and the spare planes) so it can feed the
     // second product directly
-    if ((rc = launch_zero_fill<T>(up + t * X.npad, kColPad * X.npad, st))) return rc;
+    if ((rc = launch_zero_fill<T>(up + t * X.npad, zero_planes_needed<T>(plan2, t) * X.npad, st))) return rc;
     if ((rc = mmv_packed_planar<T>(C, X, vp, t, (const T *)w, w_rs, w_cs, up, 1, X.npad, true, partial, partial_avail,
                                    st)))
         return rc;

@@ -55,6 +55,29 @@ inline size_t packed_bytes(int64_t n, int64_t d) {
     return align256((size_t)nblk * dpad * Geo<T>::BLK * sizeof(T)) + align256((size_t)nblk * Geo<T>::BLK * sizeof(T));
 }
 
+// Workgroups are handed to the 8 XCDs round-robin by linear workgroup id, and each XCD has its own L2.
+// This remaps the id so that every XCD works on one contiguous range of logical ids: workgroups that
+// share a chunk of the reduction side (same logical y, neighbouring x) then share an L2 instead of
+// making all eight XCDs fetch that chunk from HBM.
+#if defined(__HIPCC__)
+// y_fastest picks which neighbours share an XCD: false -> same reduction chunk, neighbouring output tiles
+// (right when the reduction side is the big operand), true -> same output tile, all reduction chunks
+// (right when the output side is the big operand, whose tile is then fetched once instead of once per chunk).
+__device__ __forceinline__ void xcd_remap(unsigned &bx, unsigned &by, bool y_fastest) {
+    const unsigned gx = gridDim.x, gy = gridDim.y, total = gx * gy;
+    const unsigned id = blockIdx.y * gx + blockIdx.x;
+    const unsigned q = total / 8, r = total % 8, xcd = id % 8, local = id / 8;
+    const unsigned logical = xcd * q + (xcd < r ? xcd : r) + local;
+    if (y_fastest) {
+        by = logical % gy;
+        bx = logical / gy;
+    } else {
+        bx = logical % gx;
+        by = logical / gx;
+    }
+}
+#endif
+
 // error plumbing -------------------------------------------------------------
 int fail(int code, const char *fmt, ...);
 #define FLK_HIP(expr)                                                                      \
@@ -77,7 +100,7 @@ int launch_pack(const T *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const 
 
 template <typename T>
 int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad,
-                      hipStream_t st);   // also clears the kColPad planes after the t-th
+                      int64_t zero_planes, hipStream_t st);   // also clears zero_planes planes after the t-th
 template <typename T> int launch_zero_fill(T *p, int64_t count, hipStream_t st);
 
 template <typename T>

@@ -90,7 +90,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     mmv_large_kernel(const T *__restrict__ PA, const T *__restrict__ hA, const T *__restrict__ vecp, int64_t vec_ld,
                      int tcols, const T *__restrict__ PB, const T *__restrict__ hB, int64_t na_blocks,
                      int64_t nb_blocks, int64_t dpad, int64_t a_tiles_per_chunk, T *__restrict__ partial,
-                     int64_t nb_pad) {
+                     int64_t nb_pad, bool y_fastest) {
     typedef LTraits<T> TR;
     typedef LGeo<T, WVA, WVB, WA_FR, WB_FR, KC> G;
     constexpr int kLWavesA = WVA, kLWavesB = WVB, kLThreads = 64 * WVA * WVB;
@@ -102,14 +102,16 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     __shared__ __attribute__((aligned(16))) T ldsB[2][G::B_ELEMS];
     __shared__ __attribute__((aligned(32))) T ldsRow[(1 + TT) * G::A_ROWS];   // [hA | vec_0 | vec_1 ...] of the A tile
 
+    unsigned bx, by;
+    xcd_remap(bx, by, y_fastest);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wa = wave % kLWavesA, wb = wave / kLWavesA;
     const int j = lane % TR::BLK, lg = lane / TR::BLK;
     const int64_t DPsteps = dpad / TR::KG;
-    const int64_t bblk0 = (int64_t)blockIdx.x * G::NBB;
+    const int64_t bblk0 = (int64_t)bx * G::NBB;
     const int64_t a_tiles = (na_blocks + G::NAB - 1) / G::NAB;
-    const int64_t at0 = (int64_t)blockIdx.y * a_tiles_per_chunk;
+    const int64_t at0 = (int64_t)by * a_tiles_per_chunk;
     int64_t at1 = at0 + a_tiles_per_chunk;
     if (at1 > a_tiles) at1 = a_tiles;
     const int64_t n_chunks = DPsteps / KC;     // dpad is a whole number of chunks
@@ -248,7 +250,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             if (TR::KG == 4) s += __shfl_xor(s, 16, 64);
             s += __shfl_xor(s, 32, 64);
             if (lg == 0 && bb < nb_blocks && t < tcols)
-                partial[(((int64_t)blockIdx.y * kLWavesA + wa) * tcols + t) * nb_pad + bb * TR::BLK + TR::out_row(j)] = s;
+                partial[(((int64_t)by * kLWavesA + wa) * tcols + t) * nb_pad + bb * TR::BLK + TR::out_row(j)] = s;
         }
     }
 }
@@ -285,7 +287,7 @@ static int launch_large_tt(const PackedView &A, const PackedView &B, const T *ve
     hipLaunchKernelGGL((mmv_large_kernel<T, C::WVA, C::WVB, C::WA_FR, C::WB_FR, C::KC, TT>), grid,
                        dim3(64 * C::WVA * C::WVB), 0, st,
                        (const T *)A.data, (const T *)A.hnorm, vecp, vec_ld, tcols, (const T *)B.data,
-                       (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, a_tiles_per_chunk, partial, B.npad);
+                       (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, a_tiles_per_chunk, partial, B.npad, B.n > A.n);
     FLK_LAUNCH_CHECK("mmv_large_kernel");
     return FLK_OK;
 }

@@ -165,18 +165,20 @@ __global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 r
     mmv_small_f32_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
                          int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB, int64_t na_blocks,
                          int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial, int64_t nb_pad,
-                         int tcols) {
+                         int tcols, bool y_fastest) {
     // TT columns are computed, the first tcols of them stored; vecp must hold TT planes (zeros beyond the
     // caller's columns).
     using RV = RowVals<TT>;
     constexpr bool kTwoLevel = TT <= 4;   // long accumulator only where registers allow; wider TT uses short chunks
     __shared__ __attribute__((aligned(16))) float stage[kWavesPerWg][2][RV::N];
+    unsigned bx, by;
+    xcd_remap(bx, by, y_fastest);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int j = lane & 31, h = lane >> 5;
-    const int64_t bb0 = ((int64_t)blockIdx.x * kWavesPerWg + wave) * FR;
+    const int64_t bb0 = ((int64_t)bx * kWavesPerWg + wave) * FR;
     if (bb0 >= nb_blocks) return;  // whole wave idle; no barriers in this kernel
-    const int64_t a0 = (int64_t)blockIdx.y * a_chunk_blocks;
+    const int64_t a0 = (int64_t)by * a_chunk_blocks;
     int64_t a1 = a0 + a_chunk_blocks;
     if (a1 > na_blocks) a1 = na_blocks;
 
@@ -240,7 +242,7 @@ __global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 r
             float s = kTwoLevel ? o2[q][t] + o1[q][t] : o1[q][t];
             s += __shfl_xor(s, 32, 64);
             if (h == 0 && bb0 + q < nb_blocks && t < tcols)
-                partial[((int64_t)blockIdx.y * tcols + t) * nb_pad + (bb0 + q) * 32 + j] = s;
+                partial[((int64_t)by * tcols + t) * nb_pad + (bb0 + q) * 32 + j] = s;
         }
 }
 

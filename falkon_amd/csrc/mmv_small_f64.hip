@@ -70,14 +70,16 @@ __global__ void __launch_bounds__(256)
     mmv_small_f64_kernel(const double *__restrict__ PA, const double *__restrict__ hA, const double *__restrict__ vecp,
                          int64_t vec_ld, const double *__restrict__ PB, const double *__restrict__ hB,
                          int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks, double *__restrict__ partial,
-                         int64_t nb_pad) {
+                         int64_t nb_pad, bool y_fastest) {
+    unsigned bx, by;
+    xcd_remap(bx, by, y_fastest);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int j = lane & 15, q = lane >> 4;
     const int jrow = 4 * (j & 3) + (j >> 2);  // matrix row (within its block) held at position j
-    const int64_t bb0 = ((int64_t)blockIdx.x * kWavesPerWg64 + wave) * FR;
+    const int64_t bb0 = ((int64_t)bx * kWavesPerWg64 + wave) * FR;
     if (bb0 >= nb_blocks) return;
-    const int64_t a0 = (int64_t)blockIdx.y * a_chunk_blocks;
+    const int64_t a0 = (int64_t)by * a_chunk_blocks;
     int64_t a1 = a0 + a_chunk_blocks;
     if (a1 > na_blocks) a1 = na_blocks;
 
@@ -126,7 +128,7 @@ __global__ void __launch_bounds__(256)
             s += __shfl_xor(s, 16, 64);
             s += __shfl_xor(s, 32, 64);
             if (q == 0 && bb0 + c < nb_blocks)
-                partial[((int64_t)blockIdx.y * TT + t) * nb_pad + (bb0 + c) * 16 + jrow] = s;
+                partial[((int64_t)by * TT + t) * nb_pad + (bb0 + c) * 16 + jrow] = s;
         }
 }
 
@@ -146,7 +148,7 @@ static int launch_one64(const PackedView &A, const PackedView &B, const double *
     dim3 grid((unsigned)((B.nblk + per_wg - 1) / per_wg), (unsigned)splits);
     hipLaunchKernelGGL((mmv_small_f64_kernel<DP, FR, TT>), grid, dim3(256), 0, st, (const double *)A.data,
                        (const double *)A.hnorm, vecp, vec_ld, (const double *)B.data, (const double *)B.hnorm, A.nblk,
-                       B.nblk, a_chunk_blocks, partial, B.npad);
+                       B.nblk, a_chunk_blocks, partial, B.npad, B.n > A.n);
     FLK_LAUNCH_CHECK("mmv_small_f64_kernel");
     return FLK_OK;
 }

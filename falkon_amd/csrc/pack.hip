@@ -78,8 +78,8 @@ template int launch_pack<double>(const double *, int64_t, int64_t, int64_t, int6
                                  double *, int64_t, int64_t, bool, hipStream_t);
 
 // ---------------------------------------------------------------------------
-// vec_planar: v[n,t] with element strides (rs, cs) -> vp[t + kColPad][npad]: rows past n and the
-// kColPad planes past t are zero.
+// vec_planar: v[n,t] with element strides (rs, cs) -> vp[t + zero_planes][npad]: rows past n and the
+// zero_planes planes past t are zero.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256) vec_planar_kernel(const T *__restrict__ v, int64_t n, int64_t rs, int64_t cs,
@@ -104,15 +104,17 @@ int launch_zero_fill(T *p, int64_t count, hipStream_t st) {
 template int launch_zero_fill<float>(float *, int64_t, hipStream_t);
 template int launch_zero_fill<double>(double *, int64_t, hipStream_t);
 template <typename T>
-int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad, hipStream_t st) {
+int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad,
+                      int64_t zero_planes, hipStream_t st) {
     if (npad == 0 || t == 0) return FLK_OK;
-    hipLaunchKernelGGL(vec_planar_kernel<T>, dim3((unsigned)((npad + 255) / 256), (unsigned)(t + kColPad)), dim3(256),
-                       0, st, v, n, rs, cs, vp, npad, t);
+    hipLaunchKernelGGL(vec_planar_kernel<T>, dim3((unsigned)((npad + 255) / 256), (unsigned)(t + zero_planes)),
+                       dim3(256), 0, st, v, n, rs, cs, vp, npad, t);
     FLK_LAUNCH_CHECK("vec_planar_kernel");
     return FLK_OK;
 }
-template int launch_vec_planar<float>(const float *, int64_t, int64_t, int64_t, int64_t, float *, int64_t, hipStream_t);
-template int launch_vec_planar<double>(const double *, int64_t, int64_t, int64_t, int64_t, double *, int64_t,
+template int launch_vec_planar<float>(const float *, int64_t, int64_t, int64_t, int64_t, float *, int64_t, int64_t,
+                                      hipStream_t);
+template int launch_vec_planar<double>(const double *, int64_t, int64_t, int64_t, int64_t, double *, int64_t, int64_t,
                                        hipStream_t);
 
 // ---------------------------------------------------------------------------
