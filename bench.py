@@ -36,8 +36,8 @@ WORKLOADS = {
 # 1 GiB device copy (FETCH_SIZE reads half the true bytes on this box: factor 2.0; WRITE_SIZE factor 1.0).
 # The summaries are under profiles/.  None where it has not been measured.
 MEASURED_TRAFFIC_BYTES = {
-    "C2": int((73418.8 * 2.0 + 17773.4 * 1.0) * 1024),     # 168.6 MB; algorithmic: packed X 112 MB + C + vectors
-    "C4": int((2.60826e7 * 2.0) * 1024),                   # 53.4 GB (reads only; tiles are re-read from L2/MALL/HBM)
+    "C2": int((73470.7 * 2.0 + 17773.4 * 1.0) * 1024),     # 168.7 MB; algorithmic: packed X 112 MB + C + vectors
+    "C4": int((2.61207e7 * 2.0) * 1024),                   # 53.5 GB (reads only; tiles are re-read from L2/MALL/HBM)
 }
 
 
