@@ -5,7 +5,7 @@
 
 A step is one ``GaussianKernel.dmmv`` call (K^T (K v + w)) on inputs that are already
 resident in HBM; packing of X and C is part of every step.  The default workload is
-configuration 2 of BASELINE.json: N=1,000,000 x d=28 standard-normal rows, M=20,000
+the HIGGS-shaped configuration: N=1,000,000 x d=28 standard-normal rows, M=20,000
 centres drawn from them, sigma=3.8, fp32, one right-hand side.  One JSON line goes to stdout.
 """
 import argparse
@@ -108,7 +108,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only; --gpus must be 1 "
-              "(sharding over rows of X with one M x T all-reduce is described in DESIGN.md, not built)",
+              "(sharding would split the rows of X and end with one M x T all-reduce; it is not built)",
               file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():

@@ -112,7 +112,7 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
 // that many planes of the planar right-hand side, so the planes past the caller's columns must be zero.
 template <typename T>
 static int instantiated_cols(const Plan &p, int tc) {
-    static const int small32[] = {1, 2, 3, 4, 6, 8, 12, 16}, large[] = {1, 2, 4, 8, 12, 16};
+    static const int small32[] = {1, 2, 3, 4, 6, 8, 12, 16}, large[] = {1, 2, 4, 16};
     if (p.large) {
         for (int w : large) if (tc <= w) return w;
     } else if (sizeof(T) == 4) {

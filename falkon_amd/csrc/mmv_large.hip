@@ -35,6 +35,8 @@ template <> struct LTraits<float> {
     // offset (within the block, in matrix rows) of the g-th group of 4 consecutive accumulator rows
     static __device__ __forceinline__ int group_off(int g, int lg) { return 8 * g + 4 * lg; }
     static __device__ __forceinline__ int out_row(int j) { return j; }
+    // matrix row (within its block) of accumulator register r in lane group lg
+    static __device__ __forceinline__ int acc_row(int r, int lg) { return 8 * (r >> 2) + 4 * lg + (r & 3); }
     static __device__ __forceinline__ float kexp(float x) {
         return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(x), 0.0f, 1.0f);
     }
@@ -50,6 +52,7 @@ template <> struct LTraits<double> {
     }
     static __device__ __forceinline__ int group_off(int g, int lg) { return 4 * lg; }
     static __device__ __forceinline__ int out_row(int j) { return 4 * (j & 3) + (j >> 2); }
+    static __device__ __forceinline__ int acc_row(int r, int lg) { return 4 * lg + r; }
     static __device__ __forceinline__ double kexp(double x) { return exp2(fmin(x, 0.0)); }
 };
 
@@ -100,7 +103,13 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 
     __shared__ __attribute__((aligned(16))) T ldsA[2][G::A_ELEMS];
     __shared__ __attribute__((aligned(16))) T ldsB[2][G::B_ELEMS];
-    __shared__ __attribute__((aligned(32))) T ldsRow[(1 + TT) * G::A_ROWS];   // [hA | vec_0 | vec_1 ...] of the A tile
+    // More than four columns: the contraction against vec runs on the MFMA as well (a second, small GEMM whose
+    // A operand are the kernel values sitting in the accumulator registers, see the epilogue), with vec staged
+    // as [row][16 columns] at a stride of 17 elements.  Up to four columns: per-lane FMAs, vec staged planar.
+    constexpr bool kMfmaEpi = TT > 4;
+    constexpr int kVecStride = 17;
+    constexpr int kRowBuf = kMfmaEpi ? G::A_ROWS * (1 + kVecStride) : (1 + TT) * G::A_ROWS;
+    __shared__ __attribute__((aligned(32))) T ldsRow[kRowBuf];   // [hA | vec ...] of the A tile
 
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
@@ -124,11 +133,16 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         if (bb >= nb_blocks) bb = nb_blocks - 1;
         hb[q] = hB[bb * TR::BLK + TR::out_row(j)];
     }
-    T out[WB_FR][TT];
+    T out[WB_FR][kMfmaEpi ? 1 : TT];          // per-lane FMA path: out[q][t] for this lane's output row
+    acc_t out2[kMfmaEpi ? WB_FR : 1];         // MFMA path: lane = column t, registers = output rows
 #pragma unroll
     for (int q = 0; q < WB_FR; q++)
 #pragma unroll
-        for (int t = 0; t < TT; t++) out[q][t] = T(0);
+        for (int t = 0; t < (kMfmaEpi ? 1 : TT); t++) out[q][t] = T(0);
+#pragma unroll
+    for (int q = 0; q < (kMfmaEpi ? WB_FR : 1); q++)
+#pragma unroll
+        for (int r = 0; r < TR::ACCN; r++) out2[q][r] = T(0);
 
     for (int64_t at = at0; at < at1; at++) {
         const int64_t ablk0 = at * G::NAB;
@@ -160,7 +174,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         // previous tile's epilogue may still be reading ldsRow and the stage buffers
         __syncthreads();
         // per-row values of the A tile: rows past n_a carry zero weight
-        for (int e = tid; e < (1 + TT) * G::A_ROWS; e += kLThreads) {
+        for (int e = tid; e < (1 + (kMfmaEpi ? 16 : TT)) * G::A_ROWS; e += kLThreads) {
             const int which = e / G::A_ROWS, r = e % G::A_ROWS;
             const int64_t row = ablk0 * TR::BLK + r;
             T val = T(0);
@@ -168,7 +182,8 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                 if (which == 0) val = hA[row];
                 else if (which - 1 < tcols) val = vecp[(int64_t)(which - 1) * vec_ld + row];
             }
-            ldsRow[e] = val;
+            if (!kMfmaEpi || which == 0) ldsRow[e] = val;
+            else ldsRow[G::A_ROWS + r * kVecStride + (which - 1)] = val;
         }
         fetch(0);
         commit(0);
@@ -214,6 +229,12 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         }
 
         // epilogue: exponent = acc + hA_i + hB_j ; K = exp2 clamped ; out[q][t] += K * vec[i][t]
+        // Columns are contracted in groups of four whose LDS reads are issued one group ahead; the fence
+        // after each group (the updated accumulators pass through an empty asm that also clobbers memory
+        // through the LDS pointer) keeps the compiler from moving every read to the front and spilling.
+        static_assert(WB_FR == 2, "the epilogue fence lists its operands explicitly");
+        if constexpr (!kMfmaEpi) {
+        constexpr int NTG = (TT + 3) / 4;
 #pragma unroll
         for (int p = 0; p < WA_FR; p++) {
             const int rbase = (wa * WA_FR + p) * TR::BLK;
@@ -221,36 +242,107 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             for (int g = 0; g < TR::NG; g++) {
                 const int ro = rbase + TR::group_off(g, lg);
                 const vec4_t hn = *(const vec4_t *)(&ldsRow[ro]);
+                vec4_t cur[4], nxt[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    if (u < TT) cur[u] = *(const vec4_t *)(&ldsRow[(1 + u) * G::A_ROWS + ro]);
+                T kv[WB_FR][4];
 #pragma unroll
                 for (int q = 0; q < WB_FR; q++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        T x = acc[p][q][4 * g + e] + (hn[e] + hb[q]);
-                        acc[p][q][4 * g + e] = TR::kexp(x);
+                    for (int e = 0; e < 4; e++) kv[q][e] = TR::kexp(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
+#pragma unroll
+                for (int tg = 0; tg < NTG; tg++) {
+                    const int t0 = 4 * tg;
+                    if (tg + 1 < NTG) {
+#pragma unroll
+                        for (int u = 0; u < 4; u++)
+                            if (t0 + 4 + u < TT) nxt[u] = *(const vec4_t *)(&ldsRow[(1 + t0 + 4 + u) * G::A_ROWS + ro]);
                     }
 #pragma unroll
-                for (int t = 0; t < TT; t++) {
-                    const vec4_t vv = *(const vec4_t *)(&ldsRow[(1 + t) * G::A_ROWS + ro]);
+                    for (int u = 0; u < 4; u++)
+                        if (t0 + u < TT) {
+#pragma unroll
+                            for (int q = 0; q < WB_FR; q++)
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    out[q][t0 + u] = __builtin_fma(kv[q][e], cur[u][e], out[q][t0 + u]);
+                        }
+#pragma unroll
+                    for (int u = 0; u < 4; u++)
+                        if (t0 + u < TT)
+                            asm volatile("" : "+v"(out[0][t0 + u]), "+v"(out[1][t0 + u]) : "v"(&ldsRow[0]) : "memory");
+#pragma unroll
+                    for (int u = 0; u < 4; u++) cur[u] = nxt[u];
+                }
+            }
+        }
+        } else {
+            // kernel values in place of the exponents
+#pragma unroll
+            for (int p = 0; p < WA_FR; p++) {
+                const int rbase = (wa * WA_FR + p) * TR::BLK;
+#pragma unroll
+                for (int g = 0; g < TR::NG; g++) {
+                    const vec4_t hn = *(const vec4_t *)(&ldsRow[rbase + TR::group_off(g, lg)]);
 #pragma unroll
                     for (int q = 0; q < WB_FR; q++)
 #pragma unroll
-                        for (int e = 0; e < 4; e++) out[q][t] = __builtin_fma(acc[p][q][4 * g + e], vv[e], out[q][t]);
+                        for (int e = 0; e < 4; e++)
+                            acc[p][q][4 * g + e] = TR::kexp(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
+                }
+            }
+            // out2[q][j-rows][t] += sum_i K[i][j] vec[i][t]: accumulator register s of a lane is exactly the MFMA
+            // A operand of step s (row i = acc_row(s, lg), column j = lane), so K needs no data movement; the
+            // B operand is vec[acc_row(s, lg)][t] with t = lane % 16 (columns past 16 are never stored).
+            const int tl = j & 15;
+            const T *vb = &ldsRow[G::A_ROWS + tl];
+            // one read ahead, fenced like the feature loop (otherwise all reads are hoisted and spilled)
+            T bval = vb[((wa * WA_FR) * TR::BLK + TR::acc_row(0, lg)) * kVecStride], bnext = T(0);
+#pragma unroll
+            for (int p = 0; p < WA_FR; p++) {
+                const int rbase = (wa * WA_FR + p) * TR::BLK;
+#pragma unroll
+                for (int s2 = 0; s2 < TR::ACCN; s2++) {
+                    if (s2 + 1 < TR::ACCN) bnext = vb[(rbase + TR::acc_row(s2 + 1, lg)) * kVecStride];
+                    else if (p + 1 < WA_FR) bnext = vb[(rbase + TR::BLK + TR::acc_row(0, lg)) * kVecStride];
+#pragma unroll
+                    for (int q = 0; q < WB_FR; q++) out2[q] = TR::mfma(acc[p][q][s2], bval, out2[q]);
+                    asm volatile("" : "+v"(bval) : "v"(vb) : "memory");
+                    bval = bnext;
                 }
             }
         }
     }
 
-    // join the lane groups that hold the same output row, then one partial per (split, wa)
+    if constexpr (kMfmaEpi) {
+        // lane = column t (both lane groups hold different output rows): no cross-lane step
+        const int tl = j & 15;
+        if (j < 16 && tl < tcols) {
 #pragma unroll
-    for (int q = 0; q < WB_FR; q++) {
-        const int64_t bb = bblk0 + wb * WB_FR + q;
+            for (int q = 0; q < WB_FR; q++) {
+                const int64_t bb = bblk0 + wb * WB_FR + q;
+                if (bb < nb_blocks) {
 #pragma unroll
-        for (int t = 0; t < TT; t++) {
-            T s = out[q][t];
-            if (TR::KG == 4) s += __shfl_xor(s, 16, 64);
-            s += __shfl_xor(s, 32, 64);
-            if (lg == 0 && bb < nb_blocks && t < tcols)
-                partial[(((int64_t)by * kLWavesA + wa) * tcols + t) * nb_pad + bb * TR::BLK + TR::out_row(j)] = s;
+                    for (int r = 0; r < TR::ACCN; r++)
+                        partial[(((int64_t)by * kLWavesA + wa) * tcols + tl) * nb_pad + bb * TR::BLK +
+                                TR::acc_row(r, lg)] = out2[q][r];
+                }
+            }
+        }
+    } else {
+        // join the lane groups that hold the same output row, then one partial per (split, wa)
+#pragma unroll
+        for (int q = 0; q < WB_FR; q++) {
+            const int64_t bb = bblk0 + wb * WB_FR + q;
+#pragma unroll
+            for (int t = 0; t < TT; t++) {
+                T s = out[q][t];
+                if (TR::KG == 4) s += __shfl_xor(s, 16, 64);
+                s += __shfl_xor(s, 32, 64);
+                if (lg == 0 && bb < nb_blocks && t < tcols)
+                    partial[(((int64_t)by * kLWavesA + wa) * tcols + t) * nb_pad + bb * TR::BLK + TR::out_row(j)] = s;
+            }
         }
     }
 }
@@ -301,9 +393,7 @@ int launch_mmv_large(const PackedView &A, const PackedView &B, const T *vecp, in
     if (tcols == 1) return launch_large_tt<T, 1>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols == 2) return launch_large_tt<T, 2>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols <= 4) return launch_large_tt<T, 4>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
-    if (tcols <= 8) return launch_large_tt<T, 8>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
-    if (tcols <= 12) return launch_large_tt<T, 12>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
-    return launch_large_tt<T, 16>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    return launch_large_tt<T, 16>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);   // MFMA epilogue
 }
 template int launch_mmv_large<float>(const PackedView &, const PackedView &, const float *, int64_t, int, int64_t,
                                      int, float *, hipStream_t);

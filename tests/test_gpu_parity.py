@@ -97,6 +97,8 @@ def test_reference_fixture_fp64(dev, order, sig):
     (513, 300, 784, 10),    # configuration 4's d and T
     (40, 1100, 131, 17),    # more columns than one pass holds, odd d
     (700, 20, 1000, 5),
+    (600, 400, 96, 16),     # a full 16-column pass (the MFMA contraction of kernel values against v)
+    (333, 520, 300, 7),
 ])
 def test_large_d_vs_oracle(dev, dtype, n, m, d, t):
     """d > 64 runs the LDS-tiled kernel; same tolerances against the blocked CPU oracle."""
