@@ -46,6 +46,10 @@ _SIGNATURES = {
                                 c_void_p, c_int64, c_int64, c_int64,
                                 c_void_p, c_int64, c_int64, c_int,
                                 c_void_p, c_size_t, c_void_p]),
+    "flk_gauss_fmm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int, c_int]),
+    "flk_gauss_fmm": (c_int, [*_MAT, *_MAT, c_int64, c_void_p, c_int64,
+                              c_void_p, c_int64, c_int64, c_int, c_int,
+                              c_void_p, c_size_t, c_void_p]),
 }
 
 

@@ -15,7 +15,7 @@ LIB_DIR = os.path.join(_HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfalkon_amd.so")
 OBJ_DIR = os.path.join(_HERE, "build")
 
-SOURCES = ["api.hip", "pack.hip", "mmv_small_f32.hip", "mmv_small_f32_fold.hip", "mmv_small_f64.hip", "mmv_large.hip"]
+SOURCES = ["api.hip", "pack.hip", "mmv_small_f32.hip", "mmv_small_f32_fold.hip", "mmv_small_f64.hip", "mmv_large.hip", "fmm.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

@@ -187,7 +187,7 @@ static int pack_impl(const void *X, int64_t n, int64_t d, int64_t rs, int64_t cs
     PackedView v = packed_view<T>(packed, n, d);
     // odd-d fp32 operands of the register-resident kernel carry 1.0 in their one padding feature
     const bool one_pad = sizeof(T) == 4 && (d & 1) && d <= mmv_small_max_d<T>();
-    return launch_pack<T>((const T *)X, n, d, rs, cs, (const T *)sigma, n_sigma, (T *)v.data, (T *)v.hnorm, v.dpad,
+    return launch_pack<T, T>((const T *)X, n, d, rs, cs, (const T *)sigma, n_sigma, (T *)v.data, (T *)v.hnorm, v.dpad,
                           v.nblk, one_pad, st);
 }
 
@@ -291,6 +291,37 @@ static int fdmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, c
     // out = K^T u
     return mmv_packed_planar<T>(X, C, up, t, nullptr, 0, 0, (T *)out, out_rs, out_cs, false, partial, partial_avail,
                                 st);
+}
+
+// TI: element type of X1, X2, sigma and out; T: type the kernel values are computed in.
+template <typename TI, typename T>
+static int fmm_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
+                    int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, void *out, int64_t out_rs,
+                    int64_t out_cs, void *ws, size_t ws_bytes, hipStream_t st) {
+    if (n < 0 || m < 0 || d < 1) return fail(FLK_EINVAL, "bad shape");
+    int rc;
+    if ((rc = check_matrix("X1", X1, n, d, x1_rs, x1_cs))) return rc;
+    if ((rc = check_matrix("X2", X2, m, d, x2_rs, x2_cs))) return rc;
+    if ((rc = check_matrix("out", out, n, m, out_rs, out_cs))) return rc;
+    if (sigma == nullptr) return fail(FLK_EINVAL, "sigma: null pointer");
+    if (n_sigma != 1 && n_sigma != d)
+        return fail(FLK_EINVAL, "The size of sigma (%lld) must match the number of features (%lld) or be 1",
+                    (long long)n_sigma, (long long)d);
+    if (n == 0 || m == 0) return FLK_OK;
+    const size_t need = packed_bytes<T>(n, d) + packed_bytes<T>(m, d);
+    if (ws_bytes < need || ws == nullptr)
+        return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+    PackedView P1 = packed_view<T>(ws, n, d), P2 = packed_view<T>((char *)ws + packed_bytes<T>(n, d), m, d);
+    if ((rc = launch_pack<TI, T>((const TI *)X1, n, d, x1_rs, x1_cs, (const TI *)sigma, n_sigma, (T *)P1.data,
+                                 (T *)P1.hnorm, P1.dpad, P1.nblk, false, st)))
+        return rc;
+    if ((rc = launch_pack<TI, T>((const TI *)X2, m, d, x2_rs, x2_cs, (const TI *)sigma, n_sigma, (T *)P2.data,
+                                 (T *)P2.hnorm, P2.dpad, P2.nblk, false, st)))
+        return rc;
+    // lanes run along the B operand: make that the dimension of out with the unit stride (a dimension of
+    // extent one never has its stride applied, so it can take either role)
+    if (out_cs == 1 || m == 1) return launch_fmm<T, TI>(P1, P2, (TI *)out, out_rs, st);
+    return launch_fmm<T, TI>(P2, P1, (TI *)out, out_cs, st);
 }
 
 }  // namespace flk
@@ -399,6 +430,29 @@ int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, con
     if (dtype == FLK_F64)
         return fdmmv_impl<double>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w, w_rs,
                                   w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
+size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype, int compute_f64) {
+    if (n < 0 || m < 0 || d < 1) return 0;
+    if (dtype == FLK_F64 || compute_f64) return packed_bytes<double>(n, d) + packed_bytes<double>(m, d);
+    return packed_bytes<float>(n, d) + packed_bytes<float>(m, d);
+}
+
+int flk_gauss_fmm(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
+                  int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, void *out, int64_t out_rs,
+                  int64_t out_cs, int dtype, int compute_f64, void *workspace, size_t workspace_bytes, void *stream) {
+    g_err[0] = 0;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == FLK_F64)
+        return fmm_impl<double, double>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs, out_cs,
+                                        workspace, workspace_bytes, st);
+    if (dtype == FLK_F32 && compute_f64)
+        return fmm_impl<float, double>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs, out_cs,
+                                       workspace, workspace_bytes, st);
+    if (dtype == FLK_F32)
+        return fmm_impl<float, float>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs, out_cs,
+                                      workspace, workspace_bytes, st);
     return fail(FLK_EINVAL, "unknown dtype %d", dtype);
 }
 

@@ -94,9 +94,14 @@ int fail(int code, const char *fmt, ...);
     } while (0)
 
 // launchers implemented in the .hip files -------------------------------------
-template <typename T>
-int launch_pack(const T *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const T *sigma, int64_t n_sigma,
+template <typename TI, typename T>   // TI: caller's element type, T: type of the packed operand
+int launch_pack(const TI *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const TI *sigma, int64_t n_sigma,
                 T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st);
+
+// Explicit kernel matrix out[a][b] = K(A_a, B_b) from two packed operands; O is the element type of out,
+// whose rows (A side) are ld elements apart and whose columns (B side) are contiguous.
+template <typename T, typename O>
+int launch_fmm(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st);
 
 template <typename T>
 int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad,

@@ -16,9 +16,11 @@ template <typename T> __device__ __forceinline__ int block_pos(int r);
 template <> __device__ __forceinline__ int block_pos<float>(int r) { return r; }
 template <> __device__ __forceinline__ int block_pos<double>(int r) { return 4 * (r & 3) + (r >> 2); }
 
-template <typename T>
-__global__ void __launch_bounds__(256) pack_kernel(const T *__restrict__ X, int64_t n, int64_t d, int64_t rs,
-                                                   int64_t cs, const T *__restrict__ sigma, int64_t n_sigma,
+// TI is the caller's element type, T the type of the packed operand (T = double with TI = float serves
+// kernel matrices that are computed in double precision from single precision data).
+template <typename TI, typename T>
+__global__ void __launch_bounds__(256) pack_kernel(const TI *__restrict__ X, int64_t n, int64_t d, int64_t rs,
+                                                   int64_t cs, const TI *__restrict__ sigma, int64_t n_sigma,
                                                    T *__restrict__ pdata, T *__restrict__ hnorm, int64_t dpad,
                                                    bool one_pad) {
     constexpr int BLK = Geo<T>::BLK;
@@ -63,19 +65,21 @@ __global__ void __launch_bounds__(256) pack_kernel(const T *__restrict__ X, int6
     if (tid < BLK) hnorm[row0 + tid] = (T)(-0.5 * nrm[tid]);
 }
 
-template <typename T>
-int launch_pack(const T *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const T *sigma, int64_t n_sigma,
+template <typename TI, typename T>
+int launch_pack(const TI *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const TI *sigma, int64_t n_sigma,
                 T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st) {
     if (nblk == 0) return FLK_OK;
-    hipLaunchKernelGGL(pack_kernel<T>, dim3((unsigned)nblk), dim3(256), 0, st, X, n, d, rs, cs, sigma, n_sigma, pdata,
+    hipLaunchKernelGGL((pack_kernel<TI, T>), dim3((unsigned)nblk), dim3(256), 0, st, X, n, d, rs, cs, sigma, n_sigma, pdata,
                        hnorm, dpad, one_pad);
     FLK_LAUNCH_CHECK("pack_kernel");
     return FLK_OK;
 }
-template int launch_pack<float>(const float *, int64_t, int64_t, int64_t, int64_t, const float *, int64_t, float *,
-                                float *, int64_t, int64_t, bool, hipStream_t);
-template int launch_pack<double>(const double *, int64_t, int64_t, int64_t, int64_t, const double *, int64_t, double *,
-                                 double *, int64_t, int64_t, bool, hipStream_t);
+template int launch_pack<float, float>(const float *, int64_t, int64_t, int64_t, int64_t, const float *, int64_t,
+                                       float *, float *, int64_t, int64_t, bool, hipStream_t);
+template int launch_pack<double, double>(const double *, int64_t, int64_t, int64_t, int64_t, const double *, int64_t,
+                                         double *, double *, int64_t, int64_t, bool, hipStream_t);
+template int launch_pack<float, double>(const float *, int64_t, int64_t, int64_t, int64_t, const float *, int64_t,
+                                        double *, double *, int64_t, int64_t, bool, hipStream_t);
 
 // ---------------------------------------------------------------------------
 // vec_planar: v[n,t] with element strides (rs, cs) -> vp[t + zero_planes][npad]: rows past n and the

@@ -1,48 +1,86 @@
-"""Explicit kernel matrix K(X1, X2), needed once per fit for the preconditioner's K_MM.
+"""Explicit kernel matrix K(X1, X2): the K(C, C) the preconditioner factorises once per fit, and
+``kernel(X1, X2)``.
 
-Not on the kernel-vector hot path: the blocks are produced by the kernel's ``compute`` with stock
-torch-ROCm ops, as the reference's GPU path does (falkon/mmv_ops/fmm.py:298-388).  With
-``opt.no_single_kernel`` fp32 inputs are computed in fp64 and stored in fp32
-(falkon/mmv_ops/fmm.py:619-622).
+Drop-in for falkon/mmv_ops/fmm.py:298-388,530-640 in the dense, non-differentiable Gaussian case:
+``flk_gauss_fmm`` packs both operands and writes the matrix in one launch (cross term on MFMA, exp2 on
+the accumulators).  With ``opt.no_single_kernel`` fp32 inputs are evaluated in fp64 and rounded once
+when stored (falkon/mmv_ops/fmm.py:619-622).  Rows of X1 are split only when the result is wanted on
+the host or the operands do not fit.  The diagonal (``diag=True``) is O(N d) and stays on stock torch
+ops through the kernel's ``compute``.
 """
 from typing import Optional
 
 import torch
 
+from .. import _backend
 from ..options import BaseOptions
+from ..utils.helpers import sizeof_dtype
+from .fmmv import _DTYPE_CODE, _check_dtype, _compute_device, _mat, _on, _require_gaussian, _rows_that_fit, \
+    _stream_handle
 from .utils import check_contiguity, create_output_mat, usable_gpu_memory
 
-__all__ = ("fmm",)
+__all__ = ("fmm", "gauss_fmm_native")
+
+
+def gauss_fmm_native(X1, X2, sigma_dev, out, compute_f64: bool) -> None:
+    """out[n,m] = K(X1, X2) through ``flk_gauss_fmm``.  All tensors on one GPU, 2-D, same dtype."""
+    lib = _backend.load()
+    code = _DTYPE_CODE[X1.dtype]
+    n, d = X1.shape
+    m = X2.shape[0]
+    ws_bytes = lib.flk_gauss_fmm_workspace_bytes(n, m, d, code, int(compute_f64))
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=X1.device)
+    p1, _, r1, c1 = _mat(X1)
+    p2, _, r2, c2 = _mat(X2)
+    po, _, ro, co = _mat(out)
+    with torch.cuda.device(X1.device):
+        rc = lib.flk_gauss_fmm(p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
+                               po, ro, co, code, int(compute_f64), ws.data_ptr(), ws_bytes,
+                               _stream_handle(X1.device))
+    _backend.raise_for_status(rc, "flk_gauss_fmm")
 
 
 def fmm(kernel, opt: Optional[BaseOptions], out: Optional[torch.Tensor], diag: bool, X1: torch.Tensor,
         X2: torch.Tensor, kwargs_m1=None, kwargs_m2=None) -> torch.Tensor:
     opt = opt if opt is not None else BaseOptions()
     check_contiguity((X1, "X1"), (X2, "X2"), (out, "out"))
-    if opt.use_cpu or not torch.cuda.is_available():
-        raise RuntimeError("falkon_amd computes kernel matrices on the GPU only")
     data_devs = (X1.device, X2.device)
-    cuda_devs = [d for d in data_devs if d.type == "cuda"]
-    dev = cuda_devs[0] if cuda_devs else torch.device("cuda", torch.cuda.current_device())
-    N, M = X1.shape[0], X2.shape[0]
+    dev = _compute_device(opt, data_devs)
+    N, D = X1.shape
+    M = X2.shape[0]
     with torch.inference_mode():
         if diag:
             res = kernel.compute(X1.to(dev), X2.to(dev), None, diag=True)
             if out is None:
                 return res.to(X1.device)
             return out.copy_(res.reshape(out.shape))
+        _require_gaussian(kernel)
+        if any(t.requires_grad for t in [X1, X2] + list(kernel.diff_params.values())):
+            raise NotImplementedError("falkon_amd.fmm does not implement the autograd backward pass; "
+                                      "detach the inputs and the kernel parameters")
+        _check_dtype(X1.dtype)
         out = create_output_mat(out, data_devs, shape=(N, M), dtype=X1.dtype, other_mat=X1)
-        upcast = X1.dtype == torch.float32 and opt.no_single_kernel
-        work_dt = torch.float64 if upcast else X1.dtype
-        X2d = X2.to(device=dev, dtype=work_dt)
+        if N == 0 or M == 0:
+            return out
+        lib = _backend.load()
+        code, sz = _DTYPE_CODE[X1.dtype], sizeof_dtype(X1.dtype)
+        compute_f64 = X1.dtype == torch.float32 and bool(opt.no_single_kernel)
+        sigma_dev = kernel._sigma_on(dev, X1.dtype)
         usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack)
-        per_row = (M * 3 + X1.shape[1] * 2) * (8 if work_dt == torch.float64 else 4)
-        blk = int(max(1, min(N, usable // max(per_row, 1))))
+        x1_in, out_in = X1.device == dev, out.device == dev
+        fixed = 0 if X2.device == dev else M * D * sz
+
+        def need(rows: int) -> float:
+            stage = (0 if x1_in else rows * D * sz) + (0 if out_in else rows * M * sz)
+            return lib.flk_gauss_fmm_workspace_bytes(rows, M, D, code, int(compute_f64)) + stage + fixed
+
+        blk = _rows_that_fit(N, need, usable)
+        X2d = _on(X2, dev)
         for i in range(0, N, blk):
             li = min(blk, N - i)
-            x1 = X1[i:i + li].to(device=dev, dtype=work_dt)
-            if out.device == dev and not upcast:
-                kernel.compute(x1, X2d, out[i:i + li], diag=False)
-            else:
-                out[i:i + li].copy_(kernel.compute(x1, X2d, None, diag=False))
+            X1d = _on(X1[i:i + li], dev)
+            outd = out[i:i + li] if out_in else torch.empty((li, M), dtype=out.dtype, device=dev)
+            gauss_fmm_native(X1d, X2d, sigma_dev, outd, compute_f64)
+            if not out_in:
+                out[i:i + li].copy_(outd)
     return out

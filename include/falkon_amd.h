@@ -119,6 +119,24 @@ int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
                     void *out, int64_t out_rs, int64_t out_cs, int dtype,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- explicit kernel matrix -------------------------------------------------
+ * flk_gauss_fmm replaces falkon.mmv_ops.fmm.fmm for the dense Gaussian case
+ *   (falkon/mmv_ops/fmm.py:298-388 block loop -> distance_kernel.py:140-159):
+ *   out[n,m] = K(X1[n,d], X2[m,d]), overwritten.  out needs a unit stride in
+ *   one of its two dimensions (falkon/mmv_ops/utils.py:36-39).
+ * compute_f64 != 0 with dtype = FLK_F32 evaluates the kernel in double
+ *   precision on the single-precision data and rounds the result once, the
+ *   reference's `no_single_kernel` rule for the preconditioner's K(C,C)
+ *   (falkon/mmv_ops/fmm.py:619-622); it is ignored for dtype = FLK_F64.
+ */
+size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype, int compute_f64);
+
+int flk_gauss_fmm(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
+                  const void *X2, int64_t m, int64_t x2_rs, int64_t x2_cs, int64_t d,
+                  const void *sigma, int64_t n_sigma,
+                  void *out, int64_t out_rs, int64_t out_cs, int dtype, int compute_f64,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -208,3 +208,58 @@ def test_config1_full(dev):
     got = k.mmv(X.to(dev), C.to(dev), v.to(dev))
     exp = mmv_ref.fmmv_ref(X, C, v, sigma, max_cpu_mem=2 * 2**30)
     assert rel_err(got, exp) < 1e-11
+
+
+# --------------------------------------------------------------------------------------------------
+# explicit kernel matrix (the preconditioner's K(C, C)) through flk_gauss_fmm
+# --------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("n,m,d", [(1, 1, 1), (33, 70, 3), (200, 131, 28), (129, 257, 9), (64, 300, 110), (50, 45, 784)])
+def test_kernel_matrix_vs_oracle(dev, dtype, n, m, d):
+    """kernel(X1, X2) against rbf_core (falkon/kernels/distance_kernel.py:140-159) restated on the CPU and
+    against the fp64 difference form; per-dimension sigma; fp32 in both evaluation modes of
+    falkon/mmv_ops/fmm.py:619-622."""
+    from oracle import gaussian_ref
+    X, C, _, _ = _rand(n, d, m, 1, dtype, seed=7 * n + d, scale=0.7)
+    sigma = torch.from_numpy(np.random.default_rng(d).uniform(0.8, 1.6, d) * np.sqrt(d))
+    k = GaussianKernel(sigma)
+    exact = torch.from_numpy(brute.gaussian_brute(X, C, sigma))
+    ref = gaussian_ref.rbf_core_ref(X, C, None, sigma)
+    Xg, Cg = X.to(dev), C.to(dev)
+    if dtype == torch.float64:
+        got = k(Xg, Cg).cpu()
+        assert got.dtype == dtype and got.shape == (n, m)
+        assert float((got - ref).abs().max()) < 1e-12 and float((got - exact).abs().max()) < 1e-12
+        return
+    got64 = k(Xg, Cg, opt=FalkonOptions(no_single_kernel=True)).cpu()          # fp64 arithmetic, one rounding
+    assert got64.dtype == torch.float32
+    assert float((got64.double() - exact).abs().max()) <= 6.0e-8
+    got32 = k(Xg, Cg, opt=FalkonOptions(no_single_kernel=False)).cpu()         # fp32 arithmetic
+    err_ref = float((ref.double() - exact).abs().max())                       # what the CPU fp32 path itself loses
+    assert float((got32.double() - exact).abs().max()) <= max(2e-6, 2 * err_ref)
+    assert float((got32 - ref).norm() / ref.norm()) < 1e-5
+
+
+def test_kernel_matrix_layouts_and_out(dev):
+    """F-ordered inputs give an F-ordered result (falkon/mmv_ops/utils.py:124-155); ``out=`` is written in
+    place in either order; host inputs come back on the host; a unit diagonal for X1 == X2."""
+    from oracle import gaussian_ref
+    X, C, _, _ = _rand(150, 12, 90, 1, torch.float64, seed=5)
+    k = GaussianKernel(2.5)
+    ref = gaussian_ref.rbf_core_ref(X, C, None, k.sigma)
+    Xf = torch.empty_strided(X.shape, (1, X.shape[0]), dtype=X.dtype).copy_(X).to(dev)
+    got_f = k(Xf, C.to(dev))
+    assert got_f.stride(0) == 1 and float((got_f.cpu() - ref).abs().max()) < 1e-12
+    for strides in ((90, 1), (1, 150)):
+        out = torch.empty_strided((150, 90), strides, dtype=X.dtype, device=dev)
+        res = k(X.to(dev), C.to(dev), out=out)
+        assert res.data_ptr() == out.data_ptr() and float((out.cpu() - ref).abs().max()) < 1e-12
+    host = k(X, C)
+    assert host.device.type == "cpu" and float((host - ref).abs().max()) < 1e-12
+    # forced row blocking of X1
+    small = k(X.to(dev), C.to(dev), opt=FalkonOptions(max_gpu_mem=20_000))
+    assert float((small.cpu() - ref).abs().max()) < 1e-12
+    Kcc = k(C.to(dev), C.to(dev)).cpu()
+    assert float((Kcc.diagonal() - 1).abs().max()) < 1e-12 and float((Kcc - Kcc.T).abs().max()) < 1e-13
+    d = k(X.to(dev), X.to(dev), diag=True)
+    assert d.shape == (150,) and float((d.cpu() - 1).abs().max()) < 1e-12
