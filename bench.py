@@ -91,12 +91,103 @@ def cpu_baseline(X, C, sigma, v, w, gpu_out_fn, rows):
             "rel_err_cpu_f32_vs_f64": rel(exp, got64)}
 
 
+def make_c5(N, Nts, seed=1005, d=28):
+    """Train/test rows and +-1 labels y = sign(sin(x.a) + 0.3 eps), a ~ N(0, I/d); draw order X, Xts, a, eps, eps_ts."""
+    rng = np.random.default_rng(seed)
+    X = rng.standard_normal((N, d)).astype(np.float32)
+    Xts = rng.standard_normal((Nts, d)).astype(np.float32)
+    a = rng.standard_normal(d) / np.sqrt(d)
+    y = np.sign(np.sin(X @ a) + 0.3 * rng.standard_normal(N)).astype(np.float32)
+    yts = np.sign(np.sin(Xts @ a) + 0.3 * rng.standard_normal(Nts)).astype(np.float32)
+    return tuple(torch.from_numpy(t) for t in (X, y.reshape(-1, 1), Xts, yts.reshape(-1, 1)))
+
+
+def run_c5(args, lib):
+    """End-to-end fit + predict; returns the JSON record."""
+    from falkon_amd import Falkon, FalkonOptions, GaussianKernel
+    dev = torch.device("cuda:0")
+    N, M, d, sigma, lam, iters = args.c5_n, args.c5_m, 28, 3.8, 1e-6, 20
+    Nts = N // 10
+    X, Y, Xts, Yts = make_c5(N, Nts)
+    Xg, Yg, Xtsg = X.to(dev), Y.to(dev), Xts.to(dev)
+    n_dmmv = iters + iters // FalkonOptions().cg_full_gradient_every     # one per iteration + the full residuals
+    fit_s, pre_s, pred_s, kern_ms, launches = [], [], [], 0.0, 0
+    mse = err = None
+    for it in range(args.warmup + args.steps):
+        timed = it >= args.warmup
+        model = Falkon(GaussianKernel(sigma), lam, M=M, maxiter=iters, seed=12)
+        torch.cuda.synchronize()
+        if timed:
+            lib.flk_kernel_timing_enable(1)
+        t0 = time.perf_counter()
+        model.fit(Xg, Yg)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        if timed:
+            tot_ms, cnt = ctypes.c_double(), ctypes.c_int64()
+            lib.flk_kernel_timing_read(ctypes.byref(tot_ms), ctypes.byref(cnt))
+            lib.flk_kernel_timing_enable(0)
+            kern_ms += tot_ms.value
+            launches += cnt.value
+        pred = model.predict(Xtsg)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        if timed:
+            fit_s.append(t1 - t0)
+            pre_s.append(model.fit_times_[0])          # centres + K(C,C) + both Cholesky factorisations
+            pred_s.append(t2 - t1)
+        mse = float(((pred.cpu() - Yts) ** 2).mean())
+        err = float((torch.sign(pred.cpu()) != Yts).float().mean())
+        del model, pred
+    fit, pre, prd = float(np.mean(fit_s)), float(np.mean(pre_s)), float(np.mean(pred_s))
+    cg = fit - pre
+    flop_per_launch = N * M * (2 * d + 4 + 2)
+    kern_avg = kern_ms / max(launches, 1)
+    achieved = flop_per_launch / (kern_avg * 1e-3) / 1e12
+    res = {
+        "metric": "dfmmv kernel-entries/sec (N*M*T/s) fp32 inside Falkon.fit, 1 MI355X",
+        "value": N * M * n_dmmv / cg, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": (fit + prd) * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"C5: Falkon.fit + predict, N={N}, d={d}, M={M} uniform centres, sigma=3.8, "
+                               f"penalty=1e-6, {iters} CG iterations ({n_dmmv} dfmmv + 1 fmmv), test rows {Nts}, "
+                               f"fp32, data resident in HBM"},
+        "fit_s": fit, "preconditioner_s": pre, "cg_s": cg, "predict_s": prd, "test_mse": mse, "test_error_rate": err,
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / FP32_PEAK_TFLOPS, "traffic": None, "kernel": "mmv_small_f32_kernel",
+                     "launches_per_step": launches / max(args.steps, 1), "avg_launch_ms": kern_avg,
+                     "flop_per_launch": flop_per_launch},
+    }
+    if not args.no_cpu_baseline:
+        # the same pipeline at a size the CPU finishes in seconds, on both sides, same centres
+        from oracle import falkon_ref                  # checker only; never on the product path
+        n2, m2 = args.cpu_rows or 200_000, 5_000
+        X2, Y2, X2ts, Y2ts = make_c5(n2, n2 // 10)
+        small = Falkon(GaussianKernel(sigma), lam, M=m2, maxiter=iters, seed=12)
+        small.fit(X2.to(dev), Y2.to(dev))
+        mse_gpu = float(((small.predict(X2ts.to(dev)).cpu() - Y2ts) ** 2).mean())
+        C2 = small.ny_points_.cpu()
+        t0 = time.perf_counter()
+        alpha_ref = falkon_ref.falkon_fit_ref(X2, Y2, C2, sigma, lam, maxiter=iters)
+        dt = time.perf_counter() - t0
+        mse_cpu = float(((falkon_ref.falkon_predict_ref(X2ts, C2, alpha_ref, sigma) - Y2ts) ** 2).mean())
+        res["cpu_baseline"] = {"value": n2 * m2 * n_dmmv / dt, "unit": "kernel entries/s",
+                               "cores": torch.get_num_threads(), "kind": "port", "host_cpus": os.cpu_count(),
+                               "sample": f"whole fit (preconditioner + {iters} CG iterations) at N={n2}, M={m2}, "
+                                         f"{dt:.2f} s; the rate counts the fit's {n_dmmv} dfmmv over the whole fit time",
+                               "test_mse_cpu": mse_cpu, "test_mse_gpu_same_sample": mse_gpu,
+                               "mse_rel_diff": abs(mse_gpu - mse_cpu) / mse_cpu}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS) + ["C5"])
+    ap.add_argument("--c5-n", type=int, default=2_000_000, help="training rows of the C5 workload")
+    ap.add_argument("--c5-m", type=int, default=50_000, help="centres of the C5 workload")
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"], help="arithmetic type (the headline is f32)")
     ap.add_argument("--op", default="dmmv", choices=["dmmv", "mmv"],
                     help="dmmv = K^T(Kv+w), the headline; mmv = K v only (one launch per step)")
@@ -126,6 +217,9 @@ def main():
 
     from falkon_amd import GaussianKernel, _backend
     lib = _backend.load()                            # raises if the HIP library is missing
+    if args.workload == "C5":
+        print(json.dumps(run_c5(args, lib)), flush=True)
+        return
     dev = torch.device("cuda:0")
     seed, N, d, M, T, has_w = WORKLOADS[args.workload]
     X, C, sigma, v, w = make_inputs(args.workload)

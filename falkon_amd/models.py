@@ -74,6 +74,7 @@ class Falkon(_Base):
             Xd, Yd, Cd = X.to(dev), Y.to(dev), ny_points.to(dev)
             self.precond = FalkonPreconditioner(self.penalty, self.kernel, self.options)
             self.precond.init(Cd)
+            torch.cuda.synchronize(dev)                 # fit_times_ are wall times of finished work
             self.fit_times_.append(time.time() - t_s)
             cb = None
             if self.error_fn is not None and self.error_every is not None:

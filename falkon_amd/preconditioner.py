@@ -3,8 +3,14 @@
 Same algebra as falkon/preconditioner/flk_preconditioner.py:94-300: with K_MM the kernel matrix of
 the centres, ``T = chol(K_MM + eps*M*I)`` (upper, K = T^T T) and ``A = chol(T T^T / M + lambda*I)``
 (upper); the preconditioner is ``B = 1/sqrt(n) T^-1 A^-1``.  The reference runs this on its own
-out-of-core Cholesky/LAUUM; here the factorisations are ``torch.linalg.cholesky`` and the solves
-``torch.linalg.solve_triangular`` on the GPU (the caller side of the hot path, not accelerated).
+out-of-core Cholesky/LAUUM; here the factorisations are ``torch.linalg.cholesky`` on the GPU.
+
+The four triangular solves of every CG iteration (falkon/optim/conjgrad.py:262-285) have one to a few
+right-hand sides, where a library ``trsm`` runs far below the memory roofline (M = 50 000: about 100 ms
+per solve against 2 ms for a matrix-vector product over the same factor).  ``_BlockedTriangular`` does
+the solve by blocks instead: the diagonal blocks are inverted once when the factor is built, and a
+solve is then a chain of small matrix products with those inverses and matrix-vector products over
+the row panels of the factor, each element of which is read once.
 """
 from typing import Optional
 
@@ -14,6 +20,78 @@ from .options import FalkonOptions
 
 __all__ = ("FalkonPreconditioner",)
 
+TRSV_BLOCK = 2048        # rows per diagonal block of the blocked triangular solves
+TRSV_MIN_SIZE = 4096     # smaller factors go to torch.linalg.solve_triangular directly
+
+
+def _gram_of_lower_factor(L: torch.Tensor, block: Optional[int] = None) -> torch.Tensor:
+    """``L^T L`` for a lower-triangular ``L``, valid in the lower triangle (and the diagonal blocks); the
+    blocks above the diagonal are left zero.  Enough for a Cholesky factorisation, which reads one triangle.
+
+    Row block i of the product only involves rows i0.. of L (the rows above are zero in those columns) and
+    only its columns up to the diagonal block are needed: M^3/3 flop instead of the 2 M^3 of a full product,
+    the saving the reference gets from its LAUUM kernel (falkon/preconditioner/flk_preconditioner.py:133-138).
+    """
+    M = L.shape[0]
+    block = TRSV_BLOCK if block is None else block
+    G = torch.zeros_like(L)
+    for i0 in range(0, M, block):
+        i1 = min(i0 + block, M)
+        torch.mm(L[i0:, i0:i1].T, L[i0:, :i1], out=G[i0:i1, :i1])
+    return G
+
+
+class _BlockedTriangular:
+    """Solves with a lower-triangular factor L (M x M, row-major) and with its transpose.
+
+    Both solves apply exactly transposed operators (the same inverted diagonal blocks, the same panels),
+    which is what the preconditioned CG needs from ``invT`` / ``invTt`` and ``invA`` / ``invAt``.
+    """
+
+    def __init__(self, L: torch.Tensor, block: Optional[int] = None, min_size: Optional[int] = None):
+        self.L = L
+        M = L.shape[0]
+        block = TRSV_BLOCK if block is None else block
+        min_size = TRSV_MIN_SIZE if min_size is None else min_size
+        self.bounds = [(k, min(k + block, M)) for k in range(0, M, block)] if M >= min_size else []
+        self._build()
+
+    def _build(self):
+        L = self.L
+        self.dinv, self.panels = [], []
+        for k0, k1 in self.bounds:
+            eye = torch.eye(k1 - k0, dtype=L.dtype, device=L.device)
+            self.dinv.append(torch.linalg.solve_triangular(L[k0:k1, k0:k1], eye, upper=False))
+            self.panels.append(L[k0:k1, :k0])            # view: the rows of the block left of its diagonal block
+
+    def to(self, device):
+        self.L = self.L.to(device)
+        self._build()
+        return self
+
+    def solve(self, b: torch.Tensor) -> torch.Tensor:
+        """x with L x = b (forward substitution by blocks, row panels)."""
+        if not self.bounds:
+            return torch.linalg.solve_triangular(self.L, b, upper=False)
+        x = torch.empty_like(b, memory_format=torch.contiguous_format)
+        for (k0, k1), dinv, panel in zip(self.bounds, self.dinv, self.panels):
+            r = torch.addmm(b[k0:k1], panel, x[:k0], alpha=-1.0) if k0 > 0 else b[k0:k1]
+            torch.mm(dinv, r, out=x[k0:k1])
+        return x
+
+    def solve_t(self, b: torch.Tensor) -> torch.Tensor:
+        """x with L^T x = b (backward substitution by blocks, the same row panels transposed)."""
+        if not self.bounds:
+            return torch.linalg.solve_triangular(self.L.T, b, upper=True)
+        r = b.clone(memory_format=torch.contiguous_format)
+        x = torch.empty_like(r)
+        for (k0, k1), dinv, panel in zip(reversed(self.bounds), reversed(self.dinv), reversed(self.panels)):
+            xk = x[k0:k1]
+            torch.mm(dinv.T, r[k0:k1], out=xk)
+            if k0 > 0:
+                r[:k0].addmm_(panel.T, xk, alpha=-1.0)
+        return x
+
 
 class FalkonPreconditioner:
     def __init__(self, penalty: float, kernel, opt: Optional[FalkonOptions] = None):
@@ -22,6 +100,8 @@ class FalkonPreconditioner:
         self.kernel = kernel
         self.LT: Optional[torch.Tensor] = None   # lower factor of K_MM + eps*M*I  (T = LT^T)
         self.LA: Optional[torch.Tensor] = None   # lower factor of T T^T / M + lambda*I  (A = LA^T)
+        self._T: Optional[_BlockedTriangular] = None
+        self._A: Optional[_BlockedTriangular] = None
 
     def init(self, X: torch.Tensor, weight_vec: Optional[torch.Tensor] = None) -> None:
         if weight_vec is not None:
@@ -33,11 +113,12 @@ class FalkonPreconditioner:
             C.diagonal().add_(eps * M)
             LT = torch.linalg.cholesky(C)
             del C
-            G = LT.T @ LT                                               # T T^T
+            G = _gram_of_lower_factor(LT)                               # T T^T, lower triangle only
             G.mul_(1.0 / M)
             G.diagonal().add_(self._lambda)
             self.LA = torch.linalg.cholesky(G)
             self.LT = LT
+            self._T, self._A = _BlockedTriangular(self.LT), _BlockedTriangular(self.LA)
 
     def _check(self):
         if self.LT is None or self.LA is None:
@@ -46,24 +127,25 @@ class FalkonPreconditioner:
 
     def to(self, device):
         if self.LT is not None:
-            self.LT, self.LA = self.LT.to(device), self.LA.to(device)
+            self._T, self._A = self._T.to(device), self._A.to(device)
+            self.LT, self.LA = self._T.L, self._A.L
         return self
 
     def invA(self, v):
         self._check()
-        return torch.linalg.solve_triangular(self.LA.T, v, upper=True)
+        return self._A.solve_t(v)            # A = LA^T
 
     def invAt(self, v):
         self._check()
-        return torch.linalg.solve_triangular(self.LA, v, upper=False)
+        return self._A.solve(v)
 
     def invT(self, v):
         self._check()
-        return torch.linalg.solve_triangular(self.LT.T, v, upper=True)
+        return self._T.solve_t(v)            # T = LT^T
 
     def invTt(self, v):
         self._check()
-        return torch.linalg.solve_triangular(self.LT, v, upper=False)
+        return self._T.solve(v)
 
     def apply(self, v):
         """T^-1 A^-1 v: preconditioned solution -> kernel coefficients."""

@@ -92,6 +92,34 @@ def test_preconditioner_invariants():
     np.testing.assert_allclose(ref.A, A.numpy(), rtol=1e-8, atol=1e-10)
 
 
+def test_blocked_triangular_solves_match_lapack():
+    """The block solver behind invT / invTt / invA / invAt against scipy's triangular solve, ragged last
+    block, several right-hand sides; the two directions are exact transposes of each other."""
+    import scipy.linalg as sla
+    from falkon_amd.preconditioner import _BlockedTriangular
+    g = np.random.default_rng(3)
+    for M, blk in ((1, 4), (37, 8), (64, 16), (130, 32)):
+        B = g.standard_normal((M, M))
+        L = np.linalg.cholesky(B @ B.T + M * np.eye(M))
+        bt = _BlockedTriangular(torch.from_numpy(L), block=blk, min_size=0)
+        assert len(bt.bounds) == -(-M // blk)
+        for t in (1, 3):
+            rhs = g.standard_normal((M, t))
+            np.testing.assert_allclose(bt.solve(torch.from_numpy(rhs)).numpy(),
+                                       sla.solve_triangular(L, rhs, lower=True), rtol=1e-10, atol=1e-12)
+            np.testing.assert_allclose(bt.solve_t(torch.from_numpy(rhs)).numpy(),
+                                       sla.solve_triangular(L, rhs, lower=True, trans=1), rtol=1e-10, atol=1e-12)
+        u, v = torch.from_numpy(g.standard_normal((M, 1))), torch.from_numpy(g.standard_normal((M, 1)))
+        assert abs(float((u * bt.solve(v)).sum() - (bt.solve_t(u) * v).sum())) < 1e-12
+    from falkon_amd.preconditioner import _gram_of_lower_factor
+    for M, blk in ((5, 8), (37, 8), (64, 16)):
+        L = torch.from_numpy(np.tril(g.standard_normal((M, M))))
+        G = _gram_of_lower_factor(L, block=blk)
+        torch.testing.assert_close(torch.tril(G), torch.tril(L.T @ L), rtol=1e-12, atol=1e-12)
+    # small factors go straight to the library routine
+    assert _BlockedTriangular(torch.eye(10, dtype=torch.float64)).bounds == []
+
+
 def test_center_selection_is_seeded_uniform_without_replacement():
     X = torch.arange(200, dtype=torch.float32).reshape(100, 2)
     sel = UniformSelector(np.random.default_rng(7), num_centers=10)
@@ -151,7 +179,7 @@ def _config5(N, Nts, seed=1005, d=28):
 
 
 @pytest.mark.gpu
-def test_config5_reduced_end_to_end(dev):
+def test_config5_reduced_end_to_end(dev, monkeypatch):
     """Config 5 at N=40000, M=2000, test 8000: sigma=3.8, penalty=1e-6, 20 CG iterations, fp32.
     Test MSE of the GPU fit must be within 0.1 % (relative) of the CPU pipeline's on the same centres."""
     X, Y, Xts, Yts = _config5(40_000, 8_000)
@@ -172,6 +200,16 @@ def test_config5_reduced_end_to_end(dev):
     assert model2.alpha_.is_cuda
     mse2 = float(((model2.predict(Xts.to(dev)).cpu() - Yts) ** 2).mean())
     assert abs(mse2 - mse_gpu) / mse_gpu < 1e-3
+    # the blocked triangular solves (used from M = 4096 on) give the same model
+    import falkon_amd.preconditioner as pcm
+    monkeypatch.setattr(pcm, "TRSV_BLOCK", 256)
+    monkeypatch.setattr(pcm, "TRSV_MIN_SIZE", 512)
+    model4 = Falkon(GaussianKernel(sigma), lam, M=M, maxiter=20, center_selection=FixedSelector(C))
+    model4.fit(X.to(dev), Y.to(dev))
+    assert len(model4.precond._T.bounds) == 8
+    mse4 = float(((model4.predict(Xts.to(dev)).cpu() - Yts) ** 2).mean())
+    assert abs(mse4 - mse_ref) / mse_ref < 1e-3, (mse4, mse_ref)
+    monkeypatch.undo()
     # warm start from the preconditioned solution resumes instead of restarting
     model3 = Falkon(GaussianKernel(sigma), lam, M=M, maxiter=2, center_selection=FixedSelector(C))
     model3.fit(X.to(dev), Y.to(dev), warm_start=model2.beta_.clone())
