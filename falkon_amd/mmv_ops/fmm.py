@@ -1,7 +1,7 @@
 """Explicit kernel matrix K(X1, X2): the K(C, C) the preconditioner factorises once per fit, and
 ``kernel(X1, X2)``.
 
-Drop-in for falkon/mmv_ops/fmm.py:298-388,530-640 in the dense, non-differentiable Gaussian case:
+Drop-in for falkon/mmv_ops/fmm.py:298-388,576-640,699-708 in the dense, non-differentiable Gaussian case:
 ``flk_gauss_fmm`` packs both operands and writes the matrix in one launch (cross term on MFMA, exp2 on
 the accumulators).  With ``opt.no_single_kernel`` fp32 inputs are evaluated in fp64 and rounded once
 when stored (falkon/mmv_ops/fmm.py:619-622).  Rows of X1 are split only when the result is wanted on

@@ -121,7 +121,7 @@ int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
 
 /* ---- explicit kernel matrix -------------------------------------------------
  * flk_gauss_fmm replaces falkon.mmv_ops.fmm.fmm for the dense Gaussian case
- *   (falkon/mmv_ops/fmm.py:298-388 block loop -> distance_kernel.py:140-159):
+ *   (falkon/mmv_ops/fmm.py:699-708 -> :298-388 block loop -> distance_kernel.py:140-159):
  *   out[n,m] = K(X1[n,d], X2[m,d]), overwritten.  out needs a unit stride in
  *   one of its two dimensions (falkon/mmv_ops/utils.py:36-39).
  * compute_f64 != 0 with dtype = FLK_F32 evaluates the kernel in double
