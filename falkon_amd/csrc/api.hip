@@ -66,7 +66,7 @@ struct Plan {
     int col_chunk;         // right-hand sides per pass
 };
 
-constexpr int64_t kTargetWgsLarge = 4096;  // two 256-thread workgroups per CU: 8 rounds
+constexpr int64_t kTargetWgsLarge = 16384;  // two 256-thread workgroups per CU: 8 rounds
 
 template <typename T>
 static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t dpad, int64_t t) {

@@ -150,21 +150,36 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         commit(0);
         __syncthreads();
 
-        for (int64_t ch = 0; ch < n_chunks; ch++) {
-            const int buf = (int)(ch & 1);
-            if (ch + 1 < n_chunks) fetch(ch + 1);
-            const T *la = &ldsA[buf][(wa * WA_FR) * KC * 64 + lane];
-            const T *lb = &ldsB[buf][(wb * WB_FR) * KC * 64 + lane];
-            // Operands are read one step ahead of the MFMAs that use them.  The empty asm after each step
-            // is a compiler fence: it redefines the operands just used (so that step's MFMAs stay above it)
-            // and clobbers memory through the LDS pointer (so the reads of later steps stay below it).
-            // Left alone the compiler hoists all KC steps' reads to the top of the chunk, which costs ~40
-            // registers and pushes the global prefetch registers around.
-            T av[WA_FR], bv[WB_FR], an[WA_FR], bn[WB_FR];
+        // Operands are read from LDS one step ahead of the MFMAs that use them.  The empty asm after each
+        // step is a compiler fence: it redefines the operands just used (so that step's MFMAs stay above it)
+        // and clobbers memory through the LDS pointers (so the reads of later steps stay below it).  Left
+        // alone the compiler hoists all KC steps' reads to the top of the chunk, which costs ~40 registers
+        // and pushes the global prefetch registers around.
+        //
+        // Chunk schedule: the next chunk's global loads are issued at the top, written to the other LDS
+        // stage in the middle of the chunk (that stage has not been read since the previous barrier), and
+        // the one barrier of the chunk sits BEFORE the last step's MFMAs: by then every wave holds its last
+        // operands in registers, so right after the barrier a wave issues the reads of the next chunk's
+        // first step and covers their latency with the MFMAs it still has to issue.
+        static_assert(WA_FR == 4 && WB_FR == 2, "the step fence lists its operands explicitly");
+        constexpr int kCommitStep = KC / 2;
+        T av[WA_FR], bv[WB_FR], an[WA_FR], bn[WB_FR];
+        {
+            const T *la = &ldsA[0][(wa * WA_FR) * KC * 64 + lane];
+            const T *lb = &ldsB[0][(wb * WB_FR) * KC * 64 + lane];
 #pragma unroll
             for (int p = 0; p < WA_FR; p++) av[p] = la[(p * KC) * 64];
 #pragma unroll
             for (int q = 0; q < WB_FR; q++) bv[q] = lb[(q * KC) * 64];
+        }
+        for (int64_t ch = 0; ch < n_chunks; ch++) {
+            const int buf = (int)(ch & 1);
+            const bool more = ch + 1 < n_chunks;
+            if (more) fetch(ch + 1);
+            const T *la = &ldsA[buf][(wa * WA_FR) * KC * 64 + lane];
+            const T *lb = &ldsB[buf][(wb * WB_FR) * KC * 64 + lane];
+            const T *la2 = &ldsA[buf ^ 1][(wa * WA_FR) * KC * 64 + lane];
+            const T *lb2 = &ldsB[buf ^ 1][(wb * WB_FR) * KC * 64 + lane];
 #pragma unroll
             for (int s = 0; s < KC; s++) {
                 if (s + 1 < KC) {
@@ -172,21 +187,27 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                     for (int p = 0; p < WA_FR; p++) an[p] = la[(p * KC + s + 1) * 64];
 #pragma unroll
                     for (int q = 0; q < WB_FR; q++) bn[q] = lb[(q * KC + s + 1) * 64];
+                } else {
+                    __syncthreads();          // all waves: this chunk's LDS reads done, next stage written
+                    if (more) {
+#pragma unroll
+                        for (int p = 0; p < WA_FR; p++) an[p] = la2[(p * KC) * 64];
+#pragma unroll
+                        for (int q = 0; q < WB_FR; q++) bn[q] = lb2[(q * KC) * 64];
+                    }
                 }
 #pragma unroll
                 for (int p = 0; p < WA_FR; p++)
 #pragma unroll
                     for (int q = 0; q < WB_FR; q++) acc[p][q] = TR::mfma(av[p], bv[q], acc[p][q]);
-                static_assert(WA_FR == 4 && WB_FR == 2, "the step fence lists its operands explicitly");
                 asm volatile("" : "+v"(av[0]), "+v"(av[1]), "+v"(av[2]), "+v"(av[3]), "+v"(bv[0]), "+v"(bv[1])
                              : "v"(la), "v"(lb) : "memory");
 #pragma unroll
                 for (int p = 0; p < WA_FR; p++) av[p] = an[p];
 #pragma unroll
                 for (int q = 0; q < WB_FR; q++) bv[q] = bn[q];
+                if (s == kCommitStep && more) commit(buf ^ 1);
             }
-            if (ch + 1 < n_chunks) commit(buf ^ 1);
-            __syncthreads();
         }
 
         // epilogue: exponent = acc + hA_i + hB_j ; K = exp2 clamped ; out[q][t] += K * vec[i][t]
