@@ -132,29 +132,44 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             for (int c = 0; c < G::B_VPT; c++) *(V16 *)(&ldsB[buf][(tid + c * kLThreads) * TR::VPL]) = rb[c];
         };
 
-        // previous tile's epilogue may still be reading ldsRow and the stage buffers
-        __syncthreads();
-        // per-row values of the A tile: rows past n_a carry zero weight
-        for (int e = tid; e < (1 + (kMfmaEpi ? 16 : TT)) * G::A_ROWS; e += kLThreads) {
+        // Prologue of an A tile.  All global loads (first feature chunk, then the per-row values hA and vec)
+        // are issued before anything waits, and the barrier that protects ldsRow and the stages from the
+        // previous tile's epilogue comes after them, so one memory round trip covers the whole prologue.
+        fetch(0);
+        constexpr int kRowVals = (1 + (kMfmaEpi ? 16 : TT)) * G::A_ROWS;
+        constexpr int kRowValsPerThread = (kRowVals + kLThreads - 1) / kLThreads;
+        T rowv[kRowValsPerThread];
+#pragma unroll
+        for (int c = 0; c < kRowValsPerThread; c++) {
+            const int e = tid + c * kLThreads;
             const int which = e / G::A_ROWS, r = e % G::A_ROWS;
             const int64_t row = ablk0 * TR::BLK + r;
-            T val = T(0);
-            if (row < na_blocks * TR::BLK) {
+            T val = T(0);                      // rows past n_a carry zero weight
+            if (e < kRowVals && row < na_blocks * TR::BLK) {
                 if (which == 0) val = hA[row];
                 else if (which - 1 < tcols) val = vecp[(int64_t)(which - 1) * vec_ld + row];
             }
-            if (!kMfmaEpi || which == 0) ldsRow[e] = val;
-            else ldsRow[G::A_ROWS + r * kVecStride + (which - 1)] = val;
+            rowv[c] = val;
         }
-        fetch(0);
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < kRowValsPerThread; c++) {
+            const int e = tid + c * kLThreads;
+            const int which = e / G::A_ROWS, r = e % G::A_ROWS;
+            if (e < kRowVals) {
+                if (!kMfmaEpi || which == 0) ldsRow[e] = rowv[c];
+                else ldsRow[G::A_ROWS + r * kVecStride + (which - 1)] = rowv[c];
+            }
+        }
         commit(0);
         __syncthreads();
 
-        // Operands are read from LDS one step ahead of the MFMAs that use them.  The empty asm after each
-        // step is a compiler fence: it redefines the operands just used (so that step's MFMAs stay above it)
-        // and clobbers memory through the LDS pointers (so the reads of later steps stay below it).  Left
-        // alone the compiler hoists all KC steps' reads to the top of the chunk, which costs ~40 registers
-        // and pushes the global prefetch registers around.
+        // Operands are read from LDS one step ahead of the MFMAs that use them.  The empty asm between a
+        // step's reads (for the next step) and its MFMAs is a compiler fence: it redefines the accumulators
+        // (so the MFMAs of this step stay below it and those of the previous step above it) and clobbers
+        // memory through the LDS pointers (so reads stay on their side of it).  Left alone the compiler
+        // either hoists all KC steps' reads to the top of the chunk, which costs ~40 registers and pushes
+        // the global prefetch registers around, or issues each step's reads right before their use.
         //
         // Chunk schedule: the next chunk's global loads are issued at the top, written to the other LDS
         // stage in the middle of the chunk (that stage has not been read since the previous barrier), and
@@ -163,14 +178,15 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         // first step and covers their latency with the MFMAs it still has to issue.
         static_assert(WA_FR == 4 && WB_FR == 2, "the step fence lists its operands explicitly");
         constexpr int kCommitStep = KC / 2;
-        T av[WA_FR], bv[WB_FR], an[WA_FR], bn[WB_FR];
+        static_assert(KC % 2 == 0, "the two operand sets alternate by step and must line up across chunks");
+        T av[2][WA_FR], bv[2][WB_FR];          // operand sets: step s uses set s%2 while set (s+1)%2 is being read
         {
             const T *la = &ldsA[0][(wa * WA_FR) * KC * 64 + lane];
             const T *lb = &ldsB[0][(wb * WB_FR) * KC * 64 + lane];
 #pragma unroll
-            for (int p = 0; p < WA_FR; p++) av[p] = la[(p * KC) * 64];
+            for (int p = 0; p < WA_FR; p++) av[0][p] = la[(p * KC) * 64];
 #pragma unroll
-            for (int q = 0; q < WB_FR; q++) bv[q] = lb[(q * KC) * 64];
+            for (int q = 0; q < WB_FR; q++) bv[0][q] = lb[(q * KC) * 64];
         }
         for (int64_t ch = 0; ch < n_chunks; ch++) {
             const int buf = (int)(ch & 1);
@@ -182,30 +198,28 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             const T *lb2 = &ldsB[buf ^ 1][(wb * WB_FR) * KC * 64 + lane];
 #pragma unroll
             for (int s = 0; s < KC; s++) {
+                const int cur = s & 1, nxt = cur ^ 1;
                 if (s + 1 < KC) {
 #pragma unroll
-                    for (int p = 0; p < WA_FR; p++) an[p] = la[(p * KC + s + 1) * 64];
+                    for (int p = 0; p < WA_FR; p++) av[nxt][p] = la[(p * KC + s + 1) * 64];
 #pragma unroll
-                    for (int q = 0; q < WB_FR; q++) bn[q] = lb[(q * KC + s + 1) * 64];
+                    for (int q = 0; q < WB_FR; q++) bv[nxt][q] = lb[(q * KC + s + 1) * 64];
                 } else {
                     __syncthreads();          // all waves: this chunk's LDS reads done, next stage written
                     if (more) {
 #pragma unroll
-                        for (int p = 0; p < WA_FR; p++) an[p] = la2[(p * KC) * 64];
+                        for (int p = 0; p < WA_FR; p++) av[nxt][p] = la2[(p * KC) * 64];
 #pragma unroll
-                        for (int q = 0; q < WB_FR; q++) bn[q] = lb2[(q * KC) * 64];
+                        for (int q = 0; q < WB_FR; q++) bv[nxt][q] = lb2[(q * KC) * 64];
                     }
                 }
+                asm volatile("" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]), "+v"(acc[1][1]),
+                                  "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[3][0]), "+v"(acc[3][1])
+                             : "v"(la), "v"(lb) : "memory");
 #pragma unroll
                 for (int p = 0; p < WA_FR; p++)
 #pragma unroll
-                    for (int q = 0; q < WB_FR; q++) acc[p][q] = TR::mfma(av[p], bv[q], acc[p][q]);
-                asm volatile("" : "+v"(av[0]), "+v"(av[1]), "+v"(av[2]), "+v"(av[3]), "+v"(bv[0]), "+v"(bv[1])
-                             : "v"(la), "v"(lb) : "memory");
-#pragma unroll
-                for (int p = 0; p < WA_FR; p++) av[p] = an[p];
-#pragma unroll
-                for (int q = 0; q < WB_FR; q++) bv[q] = bn[q];
+                    for (int q = 0; q < WB_FR; q++) acc[p][q] = TR::mfma(av[cur][p], bv[cur][q], acc[p][q]);
                 if (s == kCommitStep && more) commit(buf ^ 1);
             }
         }
