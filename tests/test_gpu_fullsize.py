@@ -1,0 +1,103 @@
+"""Configurations 2, 3 and 4 at their full sizes on the GPU.
+
+The CPU oracle cannot run these sizes in test time, so parity is checked where the structure of the
+problem makes a piece of it cheap (rows of ``K v`` are independent; a few columns of ``K`` give a few
+rows of ``K^T u``) and through properties that hold at any size: the adjoint identity that ties the two
+orientations of the product kernel together, ``dmmv`` = composition of two ``mmv``, linearity in ``v``,
+invariance under a permutation of the rows of X, the closed form for sigma -> infinity, run-to-run
+determinism.  Tolerances: 1e-5 (fp32) and 1e-11 (fp64), relative, norm-wise per output column.
+"""
+import numpy as np
+import pytest
+import torch
+
+from falkon_amd import GaussianKernel
+from oracle import gaussian_ref, inputs, mmv_ref
+from conftest import check_parity, rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.float64: 1e-11}
+
+
+def _columns_of_kt_u(X, C_sub, sigma, u, block=500_000):
+    """(K(X, C_sub))^T u in fp64 on the CPU, row block by row block (rbf_core restated, fp64)."""
+    acc = torch.zeros(C_sub.shape[0], u.shape[1], dtype=torch.float64)
+    Cd = C_sub.double()
+    for i in range(0, X.shape[0], block):
+        Kb = gaussian_ref.rbf_core_ref(X[i:i + block].double(), Cd, None, sigma)
+        acc += Kb.T @ u[i:i + block].double()
+    return acc
+
+
+def _full_size_checks(dev, name, dtype, n_rows=3000, n_centres=48):
+    X, C, sigma, v, w = inputs.make_config(name, dtype=dtype)
+    N, M, T = X.shape[0], C.shape[0], v.shape[1]
+    tol = TOL[dtype]
+    g = np.random.default_rng(7)
+    k = GaussianKernel(sigma)
+    Xg, Cg, vg = X.to(dev), C.to(dev), v.to(dev)
+    wg = w.to(dev) if w is not None else None
+
+    u = k.mmv(Xg, Cg, vg)                       # N x T
+    out = k.dmmv(Xg, Cg, vg, wg)                # M x T
+    assert u.shape == (N, T) and out.shape == (M, T) and bool(torch.isfinite(out).all())
+
+    # (1) rows of K v are independent of each other: a random subset against the CPU oracle
+    rows = torch.from_numpy(np.sort(g.choice(N, n_rows, replace=False)))
+    Xs = X[rows].contiguous()
+    check_parity(u[rows.to(dev)], mmv_ref.fmmv_ref(Xs, C, v, sigma),
+                 mmv_ref.fmmv_ref(Xs.double(), C.double(), v.double(), sigma), tol)
+
+    # (2) a few rows of K^T (K v + w): needs only those columns of K, all N rows, fp64 on the CPU
+    J = torch.from_numpy(np.sort(g.choice(M, n_centres, replace=False)))
+    uw = (u if wg is None else u + wg).cpu()
+    exp_J = _columns_of_kt_u(X, C[J], sigma, uw)
+    assert rel_err(out[J.to(dev)], exp_J) < tol
+
+    # (3) adjoint identity <z, K v> = <K^T z, v> (K^T z is the other orientation of the product kernel)
+    z = torch.from_numpy(g.standard_normal((N, T))).to(dtype).to(dev)
+    ktz = k.mmv(Cg, Xg, z)
+    lhs = (z.double() * u.double()).sum(0)
+    rhs = (ktz.double() * vg.double()).sum(0)
+    scale = z.double().norm(dim=0) * u.double().norm(dim=0)
+    assert float(((lhs - rhs).abs() / scale).max()) < tol
+
+    # (4) dmmv is the composition of the two products
+    comp = k.mmv(Cg, Xg, u if wg is None else u + wg)
+    assert rel_err(out, comp) < tol / 10
+
+    # (5) linearity in v
+    v2 = torch.from_numpy(g.standard_normal((M, T))).to(dtype).to(dev)
+    lin = k.mmv(Xg, Cg, 2.0 * vg - 3.0 * v2)
+    assert rel_err(lin, 2.0 * u - 3.0 * k.mmv(Xg, Cg, v2)) < tol
+
+    # (6) a permutation of the rows of X (and w) leaves K^T (K v + w) unchanged
+    perm = torch.from_numpy(g.permutation(N)).to(dev)
+    out_p = k.dmmv(Xg[perm], Cg, vg, wg[perm] if wg is not None else None)
+    assert rel_err(out_p, out) < tol
+    del perm, out_p
+
+    # (7) sigma -> infinity: K -> 1, K v -> column sums of v
+    flat = GaussianKernel(1e7).mmv(Xg, Cg, vg)
+    sums = vg.double().sum(0, keepdim=True)
+    assert float(((flat.double() - sums).abs().max(0).values / vg.double().abs().sum(0)).max()) < tol
+
+    # (8) run-to-run determinism (fixed-order reduction, no atomics)
+    assert torch.equal(out, k.dmmv(Xg, Cg, vg, wg))
+
+
+def test_config2_full_size(dev):
+    """N=1e6, d=28, M=20000, T=1, sigma=3.8, fp32."""
+    _full_size_checks(dev, "C2", torch.float32)
+
+
+def test_config3_full_size(dev):
+    """N=1e7, d=9, M=50000, T=1, per-dimension sigma, w=None, fp32."""
+    _full_size_checks(dev, "C3", torch.float32, n_rows=2000, n_centres=24)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_config4_full_size(dev, dtype):
+    """N=5e5, d=784 (80 % zeros), M=10000, T=10, sigma=10, fp32 and fp64."""
+    _full_size_checks(dev, "C4", dtype, n_rows=2000, n_centres=32)
