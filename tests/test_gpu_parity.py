@@ -263,3 +263,48 @@ def test_kernel_matrix_layouts_and_out(dev):
     assert float((Kcc.diagonal() - 1).abs().max()) < 1e-12 and float((Kcc - Kcc.T).abs().max()) < 1e-13
     d = k(X.to(dev), X.to(dev), diag=True)
     assert d.shape == (150,) and float((d.cpu() - 1).abs().max()) < 1e-12
+
+
+# --------------------------------------------------------------------------------------------------
+# edge cases of the shapes and layouts
+# --------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_degenerate_shapes(dev, dtype):
+    """No centres (K v is an empty sum: zeros, K^T(.) has no rows), no data rows (K^T(K v + w) is an empty sum),
+    a single row on either side, a 1-D v (reshaped to one column, falkon/kernels/kernel.py:92-95)."""
+    k = GaussianKernel(1.5)
+    X, C, v, w = _rand(70, 5, 9, 2, dtype, seed=3)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    none_c, none_v = Cg[:0], vg[:0]
+    r = k.mmv(Xg, none_c, none_v)
+    assert r.shape == (70, 2) and float(r.abs().max()) == 0.0
+    r = k.dmmv(Xg, none_c, none_v, wg)
+    assert r.shape == (0, 2)
+    r = k.dmmv(Xg[:0], Cg, vg, wg[:0])
+    assert r.shape == (9, 2) and float(r.abs().max()) == 0.0
+    r = k.mmv(Xg[:0], Cg, vg)
+    assert r.shape == (0, 2)
+    for n, m in ((1, 9), (70, 1), (1, 1)):
+        got = k.dmmv(Xg[:n], Cg[:m], vg[:m], wg[:n])
+        assert rel_err(got, mmv_ref.fdmmv_ref(X[:n], C[:m], v[:m], w[:n], k.sigma)) < TOL[dtype]
+    one_d = k.mmv(Xg, Cg, vg[:, 0].contiguous())
+    assert one_d.shape == (70, 1)
+    assert rel_err(one_d, mmv_ref.fmmv_ref(X, C, v[:, :1].contiguous(), k.sigma)) < TOL[dtype]
+
+
+def test_strided_views_and_column_order(dev):
+    """Row-sliced views (row stride larger than the row length) and F-ordered v / w / out are taken as they
+    are (falkon/mmv_ops/utils.py:36-39 only asks for one unit stride); a view with no unit stride is refused."""
+    X, C, v, w = _rand(300, 12, 80, 3, torch.float64, seed=8)
+    k = GaussianKernel(2.0)
+    big = torch.zeros(300, 20, dtype=torch.float64, device=dev)
+    big[:, :12] = X.to(dev)
+    Xv = big[:, :12]                                   # strides (20, 1)
+    vf = torch.empty_strided((80, 3), (1, 80), dtype=torch.float64, device=dev).copy_(v)
+    wf = torch.empty_strided((300, 3), (1, 300), dtype=torch.float64, device=dev).copy_(w)
+    out = torch.empty_strided((80, 3), (1, 80), dtype=torch.float64, device=dev)
+    got = k.dmmv(Xv, C.to(dev), vf, wf, out=out)
+    assert got.data_ptr() == out.data_ptr()
+    assert rel_err(got, mmv_ref.fdmmv_ref(X, C, v, w, k.sigma)) < 1e-11
+    with pytest.raises(ValueError):
+        k.mmv(big[::2, ::2][:, :6], C.to(dev)[:, :6].contiguous(), v.to(dev))
