@@ -186,7 +186,7 @@ static int pack_impl(const void *X, int64_t n, int64_t d, int64_t rs, int64_t cs
     if (n > 0 && packed == nullptr) return fail(FLK_EINVAL, "packed: null pointer");
     PackedView v = packed_view<T>(packed, n, d);
     // odd-d fp32 operands of the register-resident kernel carry 1.0 in their one padding feature
-    const bool one_pad = sizeof(T) == 4 && (d & 1) && d <= mmv_small_max_d<T>();
+    const bool one_pad = sizeof(T) == 4 && f32_fold_applies(d);
     return launch_pack<T, T>((const T *)X, n, d, rs, cs, (const T *)sigma, n_sigma, (T *)v.data, (T *)v.hnorm, v.dpad,
                           v.nblk, one_pad, st);
 }

@@ -29,6 +29,13 @@ constexpr int64_t kLargeKChunk = 8;
 template <typename T> inline int64_t padded_features(int64_t d) {
     return d <= kSmallMaxD ? round_up(d, Geo<T>::KG) : round_up(d, Geo<T>::KG * kLargeKChunk);
 }
+// Odd feature counts up to kFoldMaxD (fp32 only): the one padding feature of a packed row holds 1.0 and the
+// product kernel's resident fragment puts its half norm into that slot ("fold"), so the MFMA chain adds the
+// half norm itself.  Measured: a gain for the four-blocks-per-wave kernels (d <= 32), a loss for the
+// two-blocks-per-wave ones (d = 35: 16.9 ms folded against 13.0 ms for d = 36 unfolded), which therefore
+// treat odd d like d + 1.
+constexpr int64_t kFoldMaxD = 32;
+inline bool f32_fold_applies(int64_t d) { return (d & 1) && d <= kFoldMaxD; }
 inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 
 struct PackedView {

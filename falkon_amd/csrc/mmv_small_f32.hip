@@ -23,8 +23,8 @@ int launch_mmv_small<float>(const PackedView &A, const PackedView &B, const floa
                             int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
     if (A.dpad != B.dpad || A.d != B.d)
         return fail(FLK_EINVAL, "mmv_small: operands packed with different feature counts");
-    // odd d: the padding feature holds 1.0 (see pack_kernel) and carries hB through the MFMA chain
-    if (A.d & 1) return launch_mmv_small_f32_fold(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st);
+    // odd d up to kFoldMaxD: the padding feature holds 1.0 (see pack_kernel) and carries hB through the MFMA chain
+    if (f32_fold_applies(A.d)) return launch_mmv_small_f32_fold(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st);
     return launch_mmv_small_f32_plain(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st);
 }
 
