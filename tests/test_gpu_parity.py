@@ -308,3 +308,33 @@ def test_strided_views_and_column_order(dev):
     assert rel_err(got, mmv_ref.fdmmv_ref(X, C, v, w, k.sigma)) < 1e-11
     with pytest.raises(ValueError):
         k.mmv(big[::2, ::2][:, :6], C.to(dev)[:, :6].contiguous(), v.to(dev))
+
+
+def test_dmmv_replays_from_a_hip_graph(dev):
+    """The library allocates nothing, clears memory with kernels and never synchronises, so a dmmv call can be
+    captured into a HIP graph (e.g. a whole CG iteration).  Every replay, with the program's own eager work and
+    synchronisations in between, must reproduce the eager result bit for bit."""
+    X, C, v, w = _rand(30_000, 28, 1_500, 2, torch.float32, seed=21)
+    k = GaussianKernel(3.8)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    out = torch.empty(1_500, 2, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        k.dmmv(Xg, Cg, vg, wg, out=out)               # warm-up outside the capture (sigma upload, allocator)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        k.dmmv(Xg, Cg, vg, wg, out=out)
+    g = np.random.default_rng(5)
+    for _ in range(4):
+        vg.copy_(torch.from_numpy(g.standard_normal((1_500, 2)).astype(np.float32)))
+        wg.copy_(torch.from_numpy(g.standard_normal((30_000, 2)).astype(np.float32)))
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = out.clone()
+        eager = k.dmmv(Xg, Cg, vg, wg)
+        torch.cuda.synchronize()
+        assert torch.equal(replayed, eager)
+    assert rel_err(eager, mmv_ref.fdmmv_ref(X, C, vg.cpu(), wg.cpu(), k.sigma)) < 1e-5
