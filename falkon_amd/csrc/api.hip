@@ -333,7 +333,7 @@ extern "C" {
 int flk_version(void) { return 100; }
 const char *flk_last_error(void) { return g_err; }
 int64_t flk_max_d(int dtype) { (void)dtype; return (int64_t)1 << 20; }
-int64_t flk_max_t(void) { return 65535; }
+int64_t flk_max_t(void) { return 65535 - kColPad; }   // the planar right-hand sides (t + spare planes) index grid.y
 
 int flk_kernel_timing_enable(int on) {
     std::lock_guard<std::mutex> g(g_timing_mu);
