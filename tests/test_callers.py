@@ -101,16 +101,18 @@ def test_blocked_triangular_solves_match_lapack():
     for M, blk in ((1, 4), (37, 8), (64, 16), (130, 32)):
         B = g.standard_normal((M, M))
         L = np.linalg.cholesky(B @ B.T + M * np.eye(M))
-        bt = _BlockedTriangular(torch.from_numpy(L), block=blk, min_size=0)
-        assert len(bt.bounds) == -(-M // blk)
-        for t in (1, 3):
-            rhs = g.standard_normal((M, t))
-            np.testing.assert_allclose(bt.solve(torch.from_numpy(rhs)).numpy(),
-                                       sla.solve_triangular(L, rhs, lower=True), rtol=1e-10, atol=1e-12)
-            np.testing.assert_allclose(bt.solve_t(torch.from_numpy(rhs)).numpy(),
-                                       sla.solve_triangular(L, rhs, lower=True, trans=1), rtol=1e-10, atol=1e-12)
-        u, v = torch.from_numpy(g.standard_normal((M, 1))), torch.from_numpy(g.standard_normal((M, 1)))
-        assert abs(float((u * bt.solve(v)).sum() - (bt.solve_t(u) * v).sum())) < 1e-12
+        for order in ("row-major", "column-major"):          # torch.linalg.cholesky returns column-major factors
+            Lt = torch.from_numpy(L.copy()) if order == "row-major" else torch.from_numpy(L.T.copy()).T
+            bt = _BlockedTriangular(Lt, block=blk, min_size=0)
+            assert len(bt.bounds) == -(-M // blk) and bt.row_major == (order == "row-major" or M < 2)
+            for t in (1, 3):
+                rhs = g.standard_normal((M, t))
+                np.testing.assert_allclose(bt.solve(torch.from_numpy(rhs)).numpy(),
+                                           sla.solve_triangular(L, rhs, lower=True), rtol=1e-10, atol=1e-12)
+                np.testing.assert_allclose(bt.solve_t(torch.from_numpy(rhs)).numpy(),
+                                           sla.solve_triangular(L, rhs, lower=True, trans=1), rtol=1e-10, atol=1e-12)
+            u, v = torch.from_numpy(g.standard_normal((M, 1))), torch.from_numpy(g.standard_normal((M, 1)))
+            assert abs(float((u * bt.solve(v)).sum() - (bt.solve_t(u) * v).sum())) < 1e-12
     from falkon_amd.preconditioner import _gram_of_lower_factor
     for M, blk in ((5, 8), (37, 8), (64, 16)):
         L = torch.from_numpy(np.tril(g.standard_normal((M, M))))
