@@ -118,6 +118,15 @@ def test_blocked_triangular_solves_match_lapack():
         L = torch.from_numpy(np.tril(g.standard_normal((M, M))))
         G = _gram_of_lower_factor(L, block=blk)
         torch.testing.assert_close(torch.tril(G), torch.tril(L.T @ L), rtol=1e-12, atol=1e-12)
+    from falkon_amd.preconditioner import _cholesky_lower_
+    for M, blk in ((40, 8), (37, 16), (64, 64)):
+        B = g.standard_normal((M, M))
+        A = torch.from_numpy(B @ B.T + M * np.eye(M))
+        ref = torch.linalg.cholesky(A)
+        low = torch.tril(A) + torch.triu(torch.full_like(A, float("nan")), 1)      # the upper triangle is never read
+        torch.testing.assert_close(_cholesky_lower_(low, block=blk, min_size=0), ref, rtol=1e-11, atol=1e-11)
+    with pytest.raises(torch.linalg.LinAlgError):
+        _cholesky_lower_(-torch.eye(20, dtype=torch.float64), block=8, min_size=0)
     # small factors go straight to the library routine
     assert _BlockedTriangular(torch.eye(10, dtype=torch.float64)).bounds == []
 
@@ -202,10 +211,12 @@ def test_config5_reduced_end_to_end(dev, monkeypatch):
     assert model2.alpha_.is_cuda
     mse2 = float(((model2.predict(Xts.to(dev)).cpu() - Yts) ** 2).mean())
     assert abs(mse2 - mse_gpu) / mse_gpu < 1e-3
-    # the blocked triangular solves (used from M = 4096 on) give the same model
+    # the blocked triangular solves (used from M = 4096 on) and factorisation give the same model
     import falkon_amd.preconditioner as pcm
     monkeypatch.setattr(pcm, "TRSV_BLOCK", 256)
     monkeypatch.setattr(pcm, "TRSV_MIN_SIZE", 512)
+    monkeypatch.setattr(pcm, "CHOL_BLOCK", 512)              # and the blocked Cholesky (used from M = 16384 on)
+    monkeypatch.setattr(pcm, "CHOL_MIN_SIZE", 1024)
     model4 = Falkon(GaussianKernel(sigma), lam, M=M, maxiter=20, center_selection=FixedSelector(C))
     model4.fit(X.to(dev), Y.to(dev))
     assert len(model4.precond._T.bounds) == 8
