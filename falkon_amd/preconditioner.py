@@ -3,7 +3,8 @@
 Same algebra as falkon/preconditioner/flk_preconditioner.py:94-300: with K_MM the kernel matrix of
 the centres, ``T = chol(K_MM + eps*M*I)`` (upper, K = T^T T) and ``A = chol(T T^T / M + lambda*I)``
 (upper); the preconditioner is ``B = 1/sqrt(n) T^-1 A^-1``.  The reference runs this on its own
-out-of-core Cholesky/LAUUM; here the factorisations are ``torch.linalg.cholesky`` on the GPU.
+out-of-core Cholesky/LAUUM; here everything is stock torch-ROCm linear algebra on the GPU, arranged so that
+the work lands in routines that run near their roofline (``_cholesky_lower_``, ``_gram_of_lower_factor``).
 
 The four triangular solves of every CG iteration (falkon/optim/conjgrad.py:262-285) have one to a few
 right-hand sides, where a library ``trsm`` runs far below the memory roofline (M = 50 000: about 100 ms
