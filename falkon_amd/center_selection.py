@@ -56,18 +56,19 @@ class FixedSelector(CenterSelector):
         super().__init__(0)
         self.centers, self.y_centers, self.idx_centers = centers, y_centers, idx_centers
 
-    def select(self, X, Y):
-        if Y is None:
-            return self.centers
+    def _with_targets(self, want_targets: bool, *tail):
+        """(centres[, their targets], *tail); asking for targets that were never supplied is an error."""
+        if not want_targets:
+            return (self.centers, *tail)
         if self.y_centers is None:
             raise RuntimeError("FixedSelector has no y-centers available, but `Y` is not None.")
-        return self.centers, self.y_centers
+        return (self.centers, self.y_centers, *tail)
+
+    def select(self, X, Y):
+        picked = self._with_targets(Y is not None)
+        return picked[0] if len(picked) == 1 else picked
 
     def select_indices(self, X, Y):
         if self.idx_centers is None:
             raise RuntimeError("`select_indices` method called but no indices were provided.")
-        if Y is None:
-            return self.centers, self.idx_centers
-        if self.y_centers is None:
-            raise RuntimeError("FixedSelector has no y-centers available, but `Y` is not None.")
-        return self.centers, self.y_centers, self.idx_centers
+        return self._with_targets(Y is not None, self.idx_centers)

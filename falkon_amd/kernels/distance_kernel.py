@@ -1,9 +1,9 @@
 """Gaussian kernel object (falkon/kernels/distance_kernel.py:20-38,314-432).
 
-``mmv`` / ``dmmv`` run the MI355X kernels of ``libfalkon_amd``.  ``compute`` (the
-explicit kernel block the reference's ``rbf_core`` produces) is provided with stock
-torch ops for callers that need an actual matrix (the preconditioner's K_MM); it
-is not on the kernel-vector path.
+``mmv`` / ``dmmv`` and the kernel matrix ``kernel(X1, X2)`` run the MI355X kernels of
+``libfalkon_amd``.  ``compute`` (the explicit kernel block the reference's ``rbf_core``
+produces) is kept with stock torch ops for the kernel diagonal and for callers that hand it
+their own blocks; it is not on the kernel-vector path.
 """
 from typing import Dict, Optional, Union
 
@@ -18,16 +18,18 @@ __all__ = ("GaussianKernel", "validate_sigma")
 def validate_sigma(sigma: Union[float, torch.Tensor]) -> torch.Tensor:
     """float -> 1-element fp64 tensor; 1-element tensor kept as is; vector or (d,1) matrix ->
     flat per-dimension lengthscales; anything else ValueError (distance_kernel.py:20-38)."""
-    if isinstance(sigma, torch.Tensor):
-        if sigma.numel() == 1:
-            return sigma
-        if sigma.dim() == 1 or sigma.shape[1] == 1:
-            return sigma.reshape(-1)
+    if not isinstance(sigma, torch.Tensor):
+        try:
+            value = float(sigma)
+        except TypeError:
+            raise TypeError("Sigma must be a scalar or a tensor.") from None
+        return torch.tensor([value], dtype=torch.float64)
+    if sigma.numel() == 1:
+        return sigma
+    is_vector = sigma.dim() == 1 or (sigma.dim() == 2 and sigma.shape[1] == 1)
+    if not is_vector:
         raise ValueError("sigma must be a scalar or a vector.")
-    try:
-        return torch.tensor([float(sigma)], dtype=torch.float64)
-    except TypeError:
-        raise TypeError("Sigma must be a scalar or a tensor.") from None
+    return sigma.reshape(-1)
 
 
 def _rbf_block(mat1, mat2, out: Optional[torch.Tensor], diag: bool, sigma: torch.Tensor) -> torch.Tensor:

@@ -24,76 +24,77 @@ class Kernel(torch.nn.Module, ABC):
         self.name = name
         self.params: FalkonOptions = opt if opt is not None else FalkonOptions()
 
-    # -- validation (falkon/kernels/kernel.py:44-127) ---------------------------------------
+    # -- validation: the checks, exception types and order of falkon/kernels/kernel.py:44-127 -------------
+    @staticmethod
+    def _need_matrix(name: str, t: torch.Tensor) -> None:
+        if t.dim() != 2:
+            raise ValueError(f"Matrix {name} must be 2D.")
+
+    @staticmethod
+    def _as_columns(name: str, t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        """A 1-D right-hand side becomes one column; anything but 1-D / 2-D is refused."""
+        if t is None:
+            return None
+        if t.dim() == 1:
+            t = t.reshape((-1, 1))
+        if t.dim() != 2:
+            raise ValueError(f"{name} must be a vector or a 2D matrix. Found {t.dim()}D.")
+        return t
+
+    @staticmethod
+    def _need_shape(what: str, t: Optional[torch.Tensor], rows: int, cols: int) -> None:
+        if t is not None and tuple(t.shape) != (rows, cols):
+            raise ValueError(f"{what}: Expected ({rows}, {cols}) found {tuple(t.shape)}")
+
+    @staticmethod
+    def _need_one_dtype(*tensors) -> None:
+        if not check_same_dtype(*tensors):
+            raise TypeError("Data types of input matrices must be equal.")
+
     @staticmethod
     def _check_dmmv_dimensions(X1, X2, v, w, out):
         if v is None and w is None:
             raise ValueError("One of v and w must be specified to run fdMMV.")
-        if X1.dim() != 2:
-            raise ValueError("Matrix X1 must be 2D.")
-        if X2.dim() != 2:
-            raise ValueError("Matrix X2 must be 2D.")
-        if v is not None and v.dim() == 1:
-            v = v.reshape((-1, 1))
-        if v is not None and v.dim() != 2:
-            raise ValueError(f"v must be a vector or a 2D matrix. Found {len(v.shape)}D.")
-        if w is not None and w.dim() == 1:
-            w = w.reshape((-1, 1))
-        if w is not None and w.dim() != 2:
-            raise ValueError(f"w must be a vector or a 2D matrix. Found {len(w.shape)}D.")
-        T = v.size(1) if v is not None else w.size(1)
-        M = X2.size(0)
-        if out is not None and out.shape != (M, T):
-            raise ValueError(f"Output dimension is incorrect. Expected ({M}, {T}) found {out.shape}")
-        if v is not None and v.shape != (X2.size(0), T):
-            raise ValueError(f"Dimensions of matrix v are incorrect: Expected ({M}, {T}) found {v.shape}")
-        if w is not None and w.shape != (X1.size(0), T):
-            raise ValueError(f"Dimensions of matrix w are incorrect: Expected ({X1.size(0)}, {T}) found {w.shape}")
-        if not check_same_dtype(X1, X2, v, w, out):
-            raise TypeError("Data types of input matrices must be equal.")
+        Kernel._need_matrix("X1", X1)
+        Kernel._need_matrix("X2", X2)
+        v, w = Kernel._as_columns("v", v), Kernel._as_columns("w", w)
+        n, m = X1.shape[0], X2.shape[0]
+        t = (v if v is not None else w).shape[1]
+        Kernel._need_shape("Output dimension is incorrect", out, m, t)
+        Kernel._need_shape("Dimensions of matrix v are incorrect", v, m, t)
+        Kernel._need_shape("Dimensions of matrix w are incorrect", w, n, t)
+        Kernel._need_one_dtype(X1, X2, v, w, out)
         return X1, X2, v, w, out
 
     @staticmethod
     def _check_mmv_dimensions(X1, X2, v, out):
-        if X1.dim() != 2:
-            raise ValueError("Matrix X1 must be 2D.")
-        if X2.dim() != 2:
-            raise ValueError("Matrix X2 must be 2D.")
-        if v.dim() == 1:
-            v = v.reshape((-1, 1))
-        if v.dim() != 2:
-            raise ValueError(f"v must be a vector or a 2D matrix. Found {len(v.shape)}D.")
-        if out is not None and out.shape != (X1.size(0), v.size(1)):
-            raise ValueError(f"Output dimension is incorrect. Expected ({X1.size(0)}, {v.size(1)}) found {out.shape}")
-        if v.shape != (X2.size(0), v.size(1)):
-            raise ValueError(
-                f"Dimensions of matrix v are incorrect: Expected ({X2.size(0)}, {v.size(1)}) found {v.shape}")
-        if not check_same_dtype(X1, X2, v, out):
-            raise TypeError("Data types of input matrices must be equal.")
+        Kernel._need_matrix("X1", X1)
+        Kernel._need_matrix("X2", X2)
+        v = Kernel._as_columns("v", v)
+        t = v.shape[1]
+        Kernel._need_shape("Output dimension is incorrect", out, X1.shape[0], t)
+        Kernel._need_shape("Dimensions of matrix v are incorrect", v, X2.shape[0], t)
+        Kernel._need_one_dtype(X1, X2, v, out)
         return X1, X2, v, out
 
     @staticmethod
     def _check_mm_dimensions(X1, X2, diag, out):
-        if X1.dim() != 2:
-            raise ValueError("Matrix X1 must be 2D.")
-        if X2.dim() != 2:
-            raise ValueError("Matrix X2 must be 2D.")
-        N, M = X1.size(0), X2.size(0)
-        if not diag:
-            if out is not None and out.shape != (N, M):
-                raise ValueError(f"Output dimension is incorrect. Expected ({N}, {M}) found {out.shape}.")
+        Kernel._need_matrix("X1", X1)
+        Kernel._need_matrix("X2", X2)
+        n, m = X1.shape[0], X2.shape[0]
+        if diag:
+            if n != m:
+                raise ValueError(f"Cannot compute the kernel diagonal between matrices with {n} and {m} samples.")
+            if out is not None and out.numel() != n:
+                raise ValueError(f"Output dimension is incorrect. Expected ({n}) found {tuple(out.shape)}.")
         else:
-            if N != M:
-                raise ValueError(f"Cannot compute the kernel diagonal between matrices with {N} and {M} samples.")
-            if out is not None and out.reshape(-1).shape[0] != N:
-                raise ValueError(f"Output dimension is incorrect. Expected ({N}) found {out.shape}.")
-        if not check_same_dtype(X1, X2, out):
-            raise TypeError("Data types of input matrices must be equal.")
+            Kernel._need_shape("Output dimension is incorrect", out, n, m)
+        Kernel._need_one_dtype(X1, X2, out)
         return X1, X2, out
 
     @staticmethod
-    def _check_device_properties(*args, fn_name: str, opt):
-        if not check_same_device(*args):
+    def _check_device_properties(*tensors, fn_name: str, opt):
+        if not check_same_device(*tensors):
             raise RuntimeError(f"All input arguments to {fn_name} must be on the same device")
 
     def _merged(self, opt: Optional[FalkonOptions]) -> FalkonOptions:

@@ -17,52 +17,55 @@ class StopOptimizationException(Exception):
 
 
 class ConjugateGradient:
-    """Multi right-hand-side CG on ``A X = B`` with ``A`` given as a product callback
-    (falkon/optim/conjgrad.py:53-185; differential convergence is not carried over)."""
+    """Conjugate gradient on ``A X = B`` for several right-hand sides at once (one column each, with its own
+    step lengths), ``A`` given as a product callback.  Same iteration, constants and stopping rule as
+    falkon/optim/conjgrad.py:53-185: ``eps`` guards the two divisions, the residual is recomputed from scratch
+    every ``cg_full_gradient_every`` iterations, and the solve stops once every column has
+    ``|r|^2 < cg_tolerance^2``.  Differential convergence is not carried over."""
 
     def __init__(self, opt: Optional[ConjugateGradientOptions] = None):
-        self.params = opt or ConjugateGradientOptions()
+        self.params = opt if opt is not None else ConjugateGradientOptions()
         self.num_iter = None
 
     def solve(self, X0: Optional[torch.Tensor], B: torch.Tensor, mmv: Callable[[torch.Tensor], torch.Tensor],
               max_iter: int, callback: Optional[Callable[[int, torch.Tensor, float], None]] = None) -> torch.Tensor:
-        t0 = time.time()
+        started = time.time()
         if X0 is None:
-            R = B.clone()
-            X = torch.zeros_like(B)
+            sol, resid = torch.zeros_like(B), B.clone()
         else:
-            R = B - mmv(X0)
-            X = X0
-        eps = self.params.cg_epsilon(X.dtype)
-        full_grad_every = self.params.cg_full_gradient_every or max_iter * 2
-        tol = self.params.cg_tolerance ** 2
-        P = R.clone()
-        rs_old = R.square().sum(dim=0)
-        e_train = time.time() - t0
-        for self.num_iter in range(max_iter):
-            t0 = time.time()
-            AP = mmv(P)
-            alpha = rs_old / (torch.sum(P * AP, dim=0).add_(eps))
-            X.addcmul_(P, alpha.reshape(1, -1))
-            if (self.num_iter + 1) % full_grad_every == 0:
-                if X.is_cuda:
-                    torch.cuda.synchronize()
-                R = B - mmv(X)
+            sol, resid = X0, B - mmv(X0)
+        eps = self.params.cg_epsilon(sol.dtype)
+        refresh = self.params.cg_full_gradient_every or 2 * max_iter
+        stop_below = self.params.cg_tolerance ** 2
+        direction = resid.clone()
+        rr = (resid * resid).sum(0)                       # squared residual norm of every column
+        elapsed = time.time() - started
+        for it in range(max_iter):
+            self.num_iter = it
+            started = time.time()
+            a_dir = mmv(direction)
+            step = rr / ((direction * a_dir).sum(0) + eps)
+            sol += direction * step
+            if (it + 1) % refresh:
+                resid -= a_dir * step
             else:
-                R.addcmul_(AP, alpha.reshape(1, -1), value=-1.0)
-            rs_new = R.square().sum(dim=0)
-            if torch.all(rs_new < tol):
+                if sol.is_cuda:
+                    torch.cuda.synchronize()
+                resid = B - mmv(sol)
+            rr_next = (resid * resid).sum(0)
+            if bool((rr_next < stop_below).all()):
                 break
-            P = P.mul_((rs_new / rs_old.add_(eps)).reshape(1, -1)).add_(R)
-            rs_old = rs_new
-            e_train += time.time() - t0
+            direction *= rr_next / (rr + eps)
+            direction += resid
+            rr = rr_next
+            elapsed += time.time() - started
             if callback is not None:
                 try:
-                    callback(self.num_iter + 1, X, e_train)
-                except StopOptimizationException as e:
-                    print(f"Optimization stopped from callback: {e.message}")
+                    callback(it + 1, sol, elapsed)
+                except StopOptimizationException as stop:
+                    print(f"Optimization stopped from callback: {stop.message}")
                     break
-        return X
+        return sol
 
 
 class FalkonConjugateGradient:
@@ -73,25 +76,22 @@ class FalkonConjugateGradient:
         if weight_fn is not None:
             raise NotImplementedError("weighted least squares is not part of this build")
         self.kernel, self.preconditioner, self.params = kernel, preconditioner, opt
-        self.optimizer = ConjugateGradient(ConjugateGradientOptions(
-            cg_epsilon_32=opt.cg_epsilon_32, cg_epsilon_64=opt.cg_epsilon_64, cg_tolerance=opt.cg_tolerance,
-            cg_full_gradient_every=opt.cg_full_gradient_every,
-            cg_differential_convergence=opt.cg_differential_convergence))
+        cg_fields = ("cg_epsilon_32", "cg_epsilon_64", "cg_tolerance", "cg_full_gradient_every",
+                     "cg_differential_convergence")
+        self.optimizer = ConjugateGradient(ConjugateGradientOptions(**{f: getattr(opt, f) for f in cg_fields}))
 
     def falkon_mmv(self, sol, penalty, X, M, n: int):
-        prec = self.preconditioner
-        v = prec.invA(sol)
-        v_t = prec.invT(v)
-        cc = self.kernel.dmmv(X, M, v_t, None, opt=self.params)      # K_nm^T (K_nm v_t): the hot call
-        cc_ = prec.invTt(cc.div_(n)).add_(v.mul_(penalty))
-        return prec.invAt(cc_)
+        """``A^-T (T^-T K_nm^T K_nm T^-1 / n + penalty I) A^-1 sol``: the operator of the preconditioned system
+        (falkon/optim/conjgrad.py:262-285)."""
+        pc = self.preconditioner
+        inner = pc.invA(sol)
+        gram = self.kernel.dmmv(X, M, pc.invT(inner), None, opt=self.params)      # K_nm^T K_nm (.): the hot call
+        return pc.invAt(pc.invTt(gram / n) + penalty * inner)
 
     def solve(self, X, M, Y, _lambda, initial_solution, max_iter, callback=None):
         if not torch.is_inference_mode_enabled():
             raise RuntimeError("FalkonConjugateGradient.solve must run under torch.inference_mode()")
-        n = Y.size(0)
-        y_over_n = Y / n
-        B = self.kernel.mmv(M, X, y_over_n, opt=self.params)          # K_nm^T y / n
-        B = self.preconditioner.apply_t(B)
-        mmv = functools.partial(self.falkon_mmv, penalty=_lambda, X=X, M=M, n=n)
-        return self.optimizer.solve(initial_solution, B, mmv, max_iter, callback)
+        n = Y.shape[0]
+        rhs = self.preconditioner.apply_t(self.kernel.mmv(M, X, Y / n, opt=self.params))   # B^T K_nm^T y / n
+        operator = functools.partial(self.falkon_mmv, penalty=_lambda, X=X, M=M, n=n)
+        return self.optimizer.solve(initial_solution, rhs, operator, max_iter, callback)

@@ -3,8 +3,7 @@
 Mirrors falkon/options.py:164-303 (``BaseOptions``, ``KeopsOptions``,
 ``ConjugateGradientOptions``, ``PreconditionerOptions``, ``CholeskyOptions``,
 ``FalkonOptions``) so that code written against ``falkon.FalkonOptions`` keeps
-working.  On the kernel-vector path this build reads ``use_cpu``,
-``max_gpu_mem`` and ``memory_slack``; the other fields are carried for the callers.
+working.  The comment after each field says what this build does with it.
 """
 from dataclasses import dataclass
 
@@ -15,26 +14,34 @@ __all__ = ("BaseOptions", "KeopsOptions", "ConjugateGradientOptions", "Precondit
            "CholeskyOptions", "FalkonOptions")
 
 
+def _by_precision(dtype, single, double):
+    """The fp32 or the fp64 flavour of a tolerance; other dtypes are an error."""
+    try:
+        return {torch.float32: single, torch.float64: double}[dtype]
+    except KeyError:
+        raise TypeError(f"Data-type {str(dtype)} invalid") from None
+
+
 @dataclass
 class BaseOptions:
-    debug: bool = False
-    use_cpu: bool = False
-    max_gpu_mem: float = np.inf
-    max_cpu_mem: float = np.inf
-    compute_arch_speed: bool = False
-    no_single_kernel: bool = True
-    min_cuda_pc_size_32: int = 10000
-    min_cuda_pc_size_64: int = 30000
-    min_cuda_iter_size_32: int = 10_000 * 10 * 3_000
-    min_cuda_iter_size_64: int = 30_000 * 10 * 3_000
-    never_store_kernel: bool = False
-    store_kernel_d_threshold: int = 1200
-    num_fmm_streams: int = 2
-    memory_slack: float = 0.9
+    debug: bool = False                               # carried, unused
+    use_cpu: bool = False                             # True is refused: there is no CPU compute path
+    max_gpu_mem: float = np.inf                       # cap on the device memory one call may use
+    max_cpu_mem: float = np.inf                       # carried (read by the CPU oracle in the tests only)
+    compute_arch_speed: bool = False                  # carried, unused
+    no_single_kernel: bool = True                     # kernel matrices of fp32 data are evaluated in fp64
+    min_cuda_pc_size_32: int = 10000                  # carried, unused (everything runs on the GPU)
+    min_cuda_pc_size_64: int = 30000                  # carried, unused
+    min_cuda_iter_size_32: int = 10_000 * 10 * 3_000  # carried, unused
+    min_cuda_iter_size_64: int = 30_000 * 10 * 3_000  # carried, unused
+    never_store_kernel: bool = False                  # carried: the kernel matrix is never stored anyway
+    store_kernel_d_threshold: int = 1200              # carried, unused
+    num_fmm_streams: int = 2                          # carried, unused
+    memory_slack: float = 0.9                         # fraction of the free device memory a call may plan with
 
 
 @dataclass
-class KeopsOptions:
+class KeopsOptions:                                   # KeOps is not part of this build; fields carried for compatibility
     keops_acc_dtype: str = "auto"
     keops_sum_scheme: str = "auto"
     keops_active: str = "auto"
@@ -43,36 +50,28 @@ class KeopsOptions:
 
 @dataclass
 class ConjugateGradientOptions:
-    cg_epsilon_32: float = 1e-7
-    cg_epsilon_64: float = 1e-15
-    cg_tolerance: float = 1e-7
-    cg_full_gradient_every: int = 10
-    cg_differential_convergence: bool = False
+    cg_epsilon_32: float = 1e-7                       # guards the divisions of the CG in fp32
+    cg_epsilon_64: float = 1e-15                      # ... in fp64
+    cg_tolerance: float = 1e-7                        # stop once every column has |r| below this
+    cg_full_gradient_every: int = 10                  # recompute the residual from scratch this often
+    cg_differential_convergence: bool = False         # carried, not implemented
 
     def cg_epsilon(self, dtype):
-        if dtype == torch.float32:
-            return self.cg_epsilon_32
-        if dtype == torch.float64:
-            return self.cg_epsilon_64
-        raise TypeError(f"Data-type {str(dtype)} invalid")
+        return _by_precision(dtype, self.cg_epsilon_32, self.cg_epsilon_64)
 
 
 @dataclass
 class PreconditionerOptions:
-    pc_epsilon_32: float = 1e-5
-    pc_epsilon_64: float = 1e-13
-    cpu_preconditioner: bool = False
+    pc_epsilon_32: float = 1e-5                       # jitter (times M) on the diagonal of K(C,C) in fp32
+    pc_epsilon_64: float = 1e-13                      # ... in fp64
+    cpu_preconditioner: bool = False                  # carried, unused
 
     def pc_epsilon(self, dtype):
-        if dtype == torch.float32:
-            return self.pc_epsilon_32
-        if dtype == torch.float64:
-            return self.pc_epsilon_64
-        raise TypeError(f"Data-type {str(dtype)} invalid")
+        return _by_precision(dtype, self.pc_epsilon_32, self.pc_epsilon_64)
 
 
 @dataclass
-class CholeskyOptions:
+class CholeskyOptions:                                # the reference's out-of-core Cholesky is not part of this build
     chol_force_in_core: bool = False
     chol_force_ooc: bool = False
     chol_par_blk_multiplier: int = 2
@@ -81,4 +80,3 @@ class CholeskyOptions:
 @dataclass
 class FalkonOptions(BaseOptions, ConjugateGradientOptions, PreconditionerOptions, CholeskyOptions, KeopsOptions):
     """Global options, same fields as falkon/options.py:293-303."""
-    pass
