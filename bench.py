@@ -37,9 +37,9 @@ WORKLOADS = {
 # The summaries are under profiles/.  None where it has not been measured.
 MEASURED_TRAFFIC_BYTES = {
     "C2": int((73470.7 * 2.0 + 17773.4 * 1.0) * 1024),     # 168.7 MB; algorithmic: packed X 112 MB + C + vectors
-    # 1.83 GB mean of the two passes: K v reads the packed X once (0.5 GB, the algorithmic figure), the K^T u
-    # pass reads it 6-7 times (3.1 GB): a reduction chunk of X (4.8 MB) is larger than one XCD's L2
-    "C3": int((879552.0 * 2.0 + 27737.0 * 1.0) * 1024),
+    # 0.94 GB mean of the two passes: K v reads the packed X once (0.5 GB, the algorithmic figure), the K^T u
+    # pass reads it about three times (1.3 GB): the output tiles that share a reduction chunk do not all run at once
+    "C3": int((439079.0 * 2.0 + 38190.0 * 1.0) * 1024),
     "C4": int((2.54605e7 * 2.0 + 559550.0 * 1.0) * 1024),  # 52.7 GB: tiles are re-read from L2 / MALL / HBM
 }
 

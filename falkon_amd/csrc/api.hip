@@ -56,6 +56,7 @@ constexpr int64_t kTargetWgs = 8192;  // workgroups wanted per launch: 256 CUs x
                                       // the partly filled last round costs a few percent at most
 constexpr int64_t kMinChunkBlocks = 16;
 constexpr int kMaxSplits = 4096;
+constexpr int64_t kL2ChunkBytes = 2 << 20;
 constexpr int64_t kWideChunkBlocks = 64;  // column chunks wider than 4 accumulate in one fp32 level: keep the chunks short
 
 struct Plan {
@@ -82,6 +83,13 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
         p.col_chunk = mmv_small_max_cols<T>(dpad);
         if (t > 4 && p.col_chunk > 4) {
             int64_t want = (na_blocks + kWideChunkBlocks - 1) / kWideChunkBlocks;
+            if (splits < want) splits = want;
+        }
+        // a reduction chunk is streamed by every output tile that shares it: keep it within half of one XCD's
+        // 4 MB L2 so that those re-reads hit L2 instead of HBM (only where there is more than one output tile)
+        if (b_tiles > 1) {
+            const int64_t chunk_cap = kL2ChunkBytes / (dpad * Geo<T>::BLK * (int64_t)sizeof(T));
+            const int64_t want = (na_blocks + (chunk_cap > 0 ? chunk_cap : 1) - 1) / (chunk_cap > 0 ? chunk_cap : 1);
             if (splits < want) splits = want;
         }
         if (splits > kMaxSplits) splits = kMaxSplits;
