@@ -5,10 +5,12 @@
 //
 // A wave owns FA x FB blocks (64 x 64 entries in fp32, 32 x 64 in fp64) and walks over the features; the
 // packed layout is already in MFMA operand order, so each step is one element per lane and operand
-// block straight from global memory (the tiles of neighbouring waves overlap and sit in L2), read one
-// step ahead of the MFMAs that consume it.  The epilogue adds the half norms, applies exp2 with the
+// block straight from global memory (the tiles of neighbouring waves overlap and sit in L2), read two
+// steps ahead of the MFMAs that consume it.  The epilogue adds the half norms, applies exp2 with the
 // clamp K <= 1 (the reference's clamp of the squared distance, falkon/kernels/distance_kernel.py:100)
-// and stores: consecutive lanes hold consecutive columns, so every store covers whole 128-byte runs.
+// and stores: consecutive lanes hold consecutive columns, so every store covers whole 128-byte runs.  The
+// stores are non-temporal: the result is written once and never read here, and ordinary stores evicted
+// the operand tiles from L2 (M = 50 000, d = 28: 5.9 ms with ordinary stores, 3.8 ms without).
 #include "flk_common.h"
 #include "mfma_traits.h"
 
@@ -56,26 +58,32 @@ __global__ void __launch_bounds__(64 * kFmmWavesA * kFmmWavesB)
 #pragma unroll
             for (int r = 0; r < TR::ACCN; r++) acc[p][q][r] = T(0);
 
-    T av[FA], bv[FB], an[FA], bn[FB];
+    // operands travel two steps ahead of the MFMAs that consume them (three register sets in rotation);
+    // reads past the last step repeat it
+    T av[3][FA], bv[3][FB];
+    auto read_step = [&](int set, int64_t s) {
+        const int64_t sc = s < steps ? s : steps - 1;
 #pragma unroll
-    for (int p = 0; p < FA; p++) av[p] = pa[p][0];
+        for (int p = 0; p < FA; p++) av[set][p] = pa[p][sc * TR::BLK];
 #pragma unroll
-    for (int q = 0; q < FB; q++) bv[q] = pb[q][0];
-    for (int64_t s = 0; s < steps; s++) {
-        const int64_t sn = s + 1 < steps ? s + 1 : s;            // the last step re-reads itself
-#pragma unroll
-        for (int p = 0; p < FA; p++) an[p] = pa[p][sn * TR::BLK];
-#pragma unroll
-        for (int q = 0; q < FB; q++) bn[q] = pb[q][sn * TR::BLK];
+        for (int q = 0; q < FB; q++) bv[set][q] = pb[q][sc * TR::BLK];
+    };
+    auto mfma_step = [&](int set) {
 #pragma unroll
         for (int p = 0; p < FA; p++)
 #pragma unroll
-            for (int q = 0; q < FB; q++) acc[p][q] = TR::mfma(av[p], bv[q], acc[p][q]);
-#pragma unroll
-        for (int p = 0; p < FA; p++) av[p] = an[p];
-#pragma unroll
-        for (int q = 0; q < FB; q++) bv[q] = bn[q];
+            for (int q = 0; q < FB; q++) acc[p][q] = TR::mfma(av[set][p], bv[set][q], acc[p][q]);
+    };
+    read_step(0, 0);
+    read_step(1, 1);
+    int64_t s = 0;
+    for (; s + 3 <= steps; s += 3) {
+        read_step(2, s + 2); mfma_step(0);
+        read_step(0, s + 3); mfma_step(1);
+        read_step(1, s + 4); mfma_step(2);
     }
+    if (s < steps) { read_step(2, s + 2); mfma_step(0); s++; }
+    if (s < steps) { mfma_step(1); s++; }
 
 #pragma unroll
     for (int q = 0; q < FB; q++) {
@@ -94,7 +102,7 @@ __global__ void __launch_bounds__(64 * kFmmWavesA * kFmmWavesB)
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const T k = TR::kexp(acc[p][q][4 * g + e] + (hn[e] + hb));
-                    if (row0 + e < n_a && col < n_b) out[(row0 + e) * ld + col] = (O)k;
+                    if (row0 + e < n_a && col < n_b) __builtin_nontemporal_store((O)k, &out[(row0 + e) * ld + col]);
                 }
             }
         }
