@@ -156,3 +156,24 @@ def test_product_code_never_imports_the_oracle():
                 text = open(os.path.join(base, fn)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), fn
                 assert "/root/reference" not in text, fn
+
+
+def test_bench_refuses_more_than_one_gpu_and_builds_seeded_inputs():
+    """bench.py: one GPU only (a clear message and a non-zero exit otherwise); synthetic inputs are reproducible."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
+    sys.path.insert(0, ROOT)
+    import bench
+    saved = dict(bench.WORKLOADS)
+    try:
+        bench.WORKLOADS["C2"] = (1002, 2000, 28, 50, 1, True)          # same generator, small draw
+        X, C, sigma, v, w = bench.make_inputs("C2")
+        X2, C2, _, v2, w2 = bench.make_inputs("C2")
+    finally:
+        bench.WORKLOADS.update(saved)
+    assert X.shape == (2000, 28) and C.shape == (50, 28) and v.shape == (50, 1) and w.shape == (2000, 1)
+    assert X.dtype == torch.float32 and float(sigma) == 3.8
+    assert torch.equal(X, X2) and torch.equal(C, C2) and torch.equal(v, v2) and torch.equal(w, w2)
+    assert all(bool((C[i] == X).all(1).any()) for i in range(5))        # centres are rows of X
