@@ -57,6 +57,7 @@ constexpr int64_t kTargetWgs = 8192;  // workgroups wanted per launch: 256 CUs x
 constexpr int64_t kMinChunkBlocks = 16;
 constexpr int kMaxSplits = 4096;
 constexpr int64_t kL2ChunkBytes = 2 << 20;
+constexpr int64_t kL2PartialBytes = 128 << 20;
 constexpr int64_t kWideChunkBlocks = 64;  // column chunks wider than 4 accumulate in one fp32 level: keep the chunks short
 
 struct Plan {
@@ -87,9 +88,15 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
         }
         // a reduction chunk is streamed by every output tile that shares it: keep it within half of one XCD's
         // 4 MB L2 so that those re-reads hit L2 instead of HBM (only where there is more than one output tile)
+        // ... as long as the partial results this creates stay small (kL2PartialBytes per pass)
         if (b_tiles > 1) {
-            const int64_t chunk_cap = kL2ChunkBytes / (dpad * Geo<T>::BLK * (int64_t)sizeof(T));
-            const int64_t want = (na_blocks + (chunk_cap > 0 ? chunk_cap : 1) - 1) / (chunk_cap > 0 ? chunk_cap : 1);
+            int64_t chunk_cap = kL2ChunkBytes / (dpad * Geo<T>::BLK * (int64_t)sizeof(T));
+            if (chunk_cap < 1) chunk_cap = 1;
+            int64_t want = (na_blocks + chunk_cap - 1) / chunk_cap;
+            const int64_t tc = t < p.col_chunk ? (t > 0 ? t : 1) : p.col_chunk;
+            const int64_t per_split = tc * nb_blocks * Geo<T>::BLK * (int64_t)sizeof(T);
+            const int64_t affordable = kL2PartialBytes / (per_split > 0 ? per_split : 1);
+            if (want > affordable) want = affordable;
             if (splits < want) splits = want;
         }
         if (splits > kMaxSplits) splits = kMaxSplits;
