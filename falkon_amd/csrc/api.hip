@@ -142,6 +142,15 @@ static int64_t zero_planes_needed(const Plan &p, int64_t t) {
     return instantiated_cols<T>(p, tc_last) - tc_last;
 }
 
+// Bytes of the planar copy [t + zero planes][n_a padded] of a right-hand side that multiplies the n_a rows of the
+// reduction side in a product whose output side has n_b rows.
+template <typename T>
+static size_t planar_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t) {
+    PackedView A = packed_view<T>(nullptr, n_a, d), B = packed_view<T>(nullptr, n_b, d);
+    Plan p = make_plan<T>(A.nblk, B.nblk, d, A.dpad, t);
+    return align256((size_t)(t + zero_planes_needed<T>(p, t)) * A.npad * sizeof(T));
+}
+
 template <typename T>
 static size_t partial_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t) {
     PackedView A = packed_view<T>(nullptr, n_a, d), B = packed_view<T>(nullptr, n_b, d);
@@ -217,7 +226,7 @@ static int mmv_packed_impl(const void *pa, int64_t n_a, const void *pb, int64_t 
     if (out == nullptr) return fail(FLK_EINVAL, "out: null pointer");
     if (n_a > 0 && vec == nullptr) return fail(FLK_EINVAL, "vec: null pointer");
     PackedView A = packed_view<T>(pa, n_a, d), B = packed_view<T>(pb, n_b, d);
-    size_t vec_bytes = align256((size_t)(t + kColPad) * A.npad * sizeof(T));
+    size_t vec_bytes = planar_bytes<T>(n_a, n_b, d, t);
     size_t need = vec_bytes + partial_bytes<T>(n_a, n_b, d, t);
     if (ws_bytes < need || (need > 0 && ws == nullptr))
         return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
@@ -232,17 +241,14 @@ static int mmv_packed_impl(const void *pa, int64_t n_a, const void *pb, int64_t 
 
 template <typename T>
 static size_t fmmv_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {
-    PackedView A = packed_view<T>(nullptr, m, d);
-    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + align256((size_t)(t + kColPad) * A.npad * sizeof(T)) +
-           partial_bytes<T>(m, n, d, t);
+    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + planar_bytes<T>(m, n, d, t) + partial_bytes<T>(m, n, d, t);
 }
 
 template <typename T>
 static size_t fdmmv_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {
-    PackedView X = packed_view<T>(nullptr, n, d), C = packed_view<T>(nullptr, m, d);
     size_t p1 = partial_bytes<T>(m, n, d, t), p2 = partial_bytes<T>(n, m, d, t);
-    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + align256((size_t)(t + kColPad) * C.npad * sizeof(T)) +
-           align256((size_t)(t + kColPad) * X.npad * sizeof(T)) + (p1 > p2 ? p1 : p2);
+    return packed_bytes<T>(n, d) + packed_bytes<T>(m, d) + planar_bytes<T>(m, n, d, t) + planar_bytes<T>(n, m, d, t) +
+           (p1 > p2 ? p1 : p2);
 }
 
 template <typename T>
@@ -286,8 +292,8 @@ static int fdmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, c
     char *p = (char *)ws;
     void *px = p; p += packed_bytes<T>(n, d);
     void *pc = p; p += packed_bytes<T>(m, d);
-    T *vp = (T *)p; p += align256((size_t)(t + kColPad) * C.npad * sizeof(T));
-    T *up = (T *)p; p += align256((size_t)(t + kColPad) * X.npad * sizeof(T));
+    T *vp = (T *)p; p += planar_bytes<T>(m, n, d, t);     // v multiplies the rows of C in K v
+    T *up = (T *)p; p += planar_bytes<T>(n, m, d, t);     // u multiplies the rows of X in K^T u
     T *partial = (T *)p;
     size_t partial_avail = ws_bytes - (size_t)(p - (char *)ws);
     if ((rc = pack_impl<T>(X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
@@ -390,10 +396,8 @@ int flk_gauss_pack(const void *X, int64_t n, int64_t d, int64_t x_rs, int64_t x_
 size_t flk_gauss_mmv_packed_workspace_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t, int dtype) {
     if (n_a < 0 || n_b < 0 || d < 1 || t < 0) return 0;
     if (dtype == FLK_F64)
-        return align256((size_t)(t + kColPad) * packed_view<double>(nullptr, n_a, d).npad * 8) +
-               partial_bytes<double>(n_a, n_b, d, t);
-    return align256((size_t)(t + kColPad) * packed_view<float>(nullptr, n_a, d).npad * 4) +
-           partial_bytes<float>(n_a, n_b, d, t);
+        return planar_bytes<double>(n_a, n_b, d, t) + partial_bytes<double>(n_a, n_b, d, t);
+    return planar_bytes<float>(n_a, n_b, d, t) + partial_bytes<float>(n_a, n_b, d, t);
 }
 
 int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b, int64_t n_b, int64_t d,
