@@ -1,6 +1,6 @@
-"""falkon_amd: MI355X-native Gaussian kernel-vector products behind Falkon's kernel API."""
+"""falkon_amd: MI355X-native kernel-vector products (Gaussian, Laplacian, Matern) behind Falkon's kernel API."""
 from .options import FalkonOptions  # noqa: F401
-from .kernels import GaussianKernel  # noqa: F401
+from .kernels import GaussianKernel, LaplacianKernel, MaternKernel  # noqa: F401
 from .mmv_ops import fdmmv, fmmv  # noqa: F401
 from .models import Falkon, InCoreFalkon  # noqa: F401
 

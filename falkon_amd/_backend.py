@@ -16,6 +16,7 @@ _lock = threading.Lock()
 _lib = None
 
 FLK_F32, FLK_F64 = 0, 1
+FLK_GAUSSIAN, FLK_LAPLACIAN, FLK_MATERN32, FLK_MATERN52 = 0, 1, 2, 3
 FLK_EINVAL, FLK_ENOMEM, FLK_EUNSUPPORTED, FLK_EHIP = -1, -2, -3, -4
 
 _MAT = [c_void_p, c_int64, c_int64, c_int64]        # ptr, rows, row_stride, col_stride
@@ -51,6 +52,10 @@ _SIGNATURES = {
                               c_void_p, c_int64, c_int64, c_int, c_int,
                               c_void_p, c_size_t, c_void_p]),
 }
+# the flk_kernel_* entry points: the flk_gauss_* ones with the kernel function as first argument
+for _name in ("pack", "mmv_packed", "fmmv", "fdmmv", "fmm"):
+    _res, _args = _SIGNATURES["flk_gauss_" + _name]
+    _SIGNATURES["flk_kernel_" + _name] = (_res, [c_int, *_args])
 
 
 def library_path() -> str:

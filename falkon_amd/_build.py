@@ -1,7 +1,7 @@
 """Compile the HIP sources under ``falkon_amd/csrc`` into ``falkon_amd/lib/libfalkon_amd.so``.
 
 The library is built for gfx950 only, with plain ``hipcc`` (no torch headers: the
-C ABI takes raw pointers), one object per source compiled in parallel.
+C ABI takes raw pointers), one object per source (and kernel function) compiled in parallel.
 """
 import os
 import shutil
@@ -15,7 +15,11 @@ LIB_DIR = os.path.join(_HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfalkon_amd.so")
 OBJ_DIR = os.path.join(_HERE, "build")
 
-SOURCES = ["api.hip", "pack.hip", "mmv_small_f32.hip", "mmv_small_f32_fold.hip", "mmv_small_f64.hip", "mmv_large.hip", "fmm.hip"]
+# The sources that evaluate the kernel function are compiled once per function: -DFLK_KF=0..3
+# (Gaussian, Laplacian, Matern 3/2, Matern 5/2).
+KERNEL_FNS = (0, 1, 2, 3)
+PER_KERNEL_FN = ["mmv_small_f32.hip", "mmv_small_f32_fold.hip", "mmv_small_f64.hip", "mmv_large.hip", "fmm.hip"]
+SOURCES = [("api.hip", None), ("pack.hip", None)] + [(src, kf) for kf in KERNEL_FNS for src in PER_KERNEL_FN]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -34,12 +38,15 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found; the falkon_amd native library needs ROCm's hipcc to build")
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(job) -> str:
+    src, kf = job
+    stem = os.path.splitext(src)[0] + ("" if kf is None else f"_kf{kf}")
+    obj = os.path.join(OBJ_DIR, stem + ".o")
+    defines = [] if kf is None else [f"-DFLK_KF={kf}"]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *defines, "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed on {src}:\n{res.stderr}")
+        raise RuntimeError(f"hipcc failed on {src} {' '.join(defines)}:\n{res.stderr}")
     return obj
 
 

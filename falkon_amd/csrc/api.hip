@@ -170,7 +170,7 @@ static int check_matrix(const char *name, const void *p, int64_t rows, int64_t c
 
 // out[b,t] = sum_a K(A_a,B_b) vecp[t][a] (+ addend).  vecp is planar [t][A.npad].
 template <typename T>
-static int mmv_packed_planar(const PackedView &A, const PackedView &B, const T *vecp, int64_t t, const T *addend,
+static int mmv_packed_planar(int kf, const PackedView &A, const PackedView &B, const T *vecp, int64_t t, const T *addend,
                              int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
                              T *partial, size_t partial_avail, hipStream_t st) {
     if (B.n == 0 || t == 0) return FLK_OK;
@@ -185,8 +185,8 @@ static int mmv_packed_planar(const PackedView &A, const PackedView &B, const T *
             partials = 0;  // empty reduction: finalize sums nothing and writes the addend (or zero)
         } else {
             ScopedKernelTimer timer(st);
-            int rc = p.large ? launch_mmv_large<T>(A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st)
-                             : launch_mmv_small<T>(A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st);
+            int rc = p.large ? launch_mmv_large<T>(kf, A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st)
+                             : launch_mmv_small<T>(kf, A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st);
             if (rc != FLK_OK) return rc;
         }
         int rc = launch_finalize<T>(partial, partials, tc, B.n, B.npad, addend ? addend + t0 * add_cs : nullptr,
@@ -197,7 +197,7 @@ static int mmv_packed_planar(const PackedView &A, const PackedView &B, const T *
 }
 
 template <typename T>
-static int pack_impl(const void *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const void *sigma, int64_t n_sigma,
+static int pack_impl(int kf, const void *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const void *sigma, int64_t n_sigma,
                      void *packed, size_t bytes, hipStream_t st) {
     int rc = check_matrix("X", X, n, d, rs, cs);
     if (rc) return rc;
@@ -211,12 +211,12 @@ static int pack_impl(const void *X, int64_t n, int64_t d, int64_t rs, int64_t cs
     PackedView v = packed_view<T>(packed, n, d);
     // odd-d fp32 operands of the register-resident kernel carry 1.0 in their one padding feature
     const bool one_pad = sizeof(T) == 4 && f32_fold_applies(d);
-    return launch_pack<T, T>((const T *)X, n, d, rs, cs, (const T *)sigma, n_sigma, (T *)v.data, (T *)v.hnorm, v.dpad,
-                          v.nblk, one_pad, st);
+    return launch_pack<T, T>((const T *)X, n, d, rs, cs, (const T *)sigma, n_sigma, operand_scale(kf), (T *)v.data,
+                             (T *)v.hnorm, v.dpad, v.nblk, one_pad, st);
 }
 
 template <typename T>
-static int mmv_packed_impl(const void *pa, int64_t n_a, const void *pb, int64_t n_b, int64_t d, const void *vec,
+static int mmv_packed_impl(int kf, const void *pa, int64_t n_a, const void *pb, int64_t n_b, int64_t d, const void *vec,
                            int64_t vec_rs, int64_t vec_cs, int64_t t, const void *addend, int64_t add_rs,
                            int64_t add_cs, void *out, int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes,
                            hipStream_t st) {
@@ -235,7 +235,7 @@ static int mmv_packed_impl(const void *pa, int64_t n_a, const void *pb, int64_t 
     Plan plan = make_plan<T>(A.nblk, B.nblk, A.d, A.dpad, t);
     int rc = launch_vec_planar<T>((const T *)vec, n_a, t, vec_rs, vec_cs, vecp, A.npad, zero_planes_needed<T>(plan, t), st);
     if (rc) return rc;
-    return mmv_packed_planar<T>(A, B, vecp, t, (const T *)addend, add_rs, add_cs, (T *)out, out_rs, out_cs, false,
+    return mmv_packed_planar<T>(kf, A, B, vecp, t, (const T *)addend, add_rs, add_cs, (T *)out, out_rs, out_cs, false,
                                 partial, ws_bytes - vec_bytes, st);
 }
 
@@ -252,7 +252,7 @@ static size_t fdmmv_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {
 }
 
 template <typename T>
-static int fmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
+static int fmmv_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
                      int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v, int64_t v_rs,
                      int64_t v_cs, int64_t t, void *out, int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes,
                      hipStream_t st) {
@@ -267,14 +267,14 @@ static int fmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, co
     char *p = (char *)ws;
     void *px = p; p += packed_bytes<T>(n, d);
     void *pc = p; p += packed_bytes<T>(m, d);
-    if ((rc = pack_impl<T>(X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
-    if ((rc = pack_impl<T>(X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, packed_bytes<T>(m, d), st))) return rc;
-    return mmv_packed_impl<T>(pc, m, px, n, d, v, v_rs, v_cs, t, nullptr, 0, 0, out, out_rs, out_cs, p,
+    if ((rc = pack_impl<T>(kf, X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
+    if ((rc = pack_impl<T>(kf, X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, packed_bytes<T>(m, d), st))) return rc;
+    return mmv_packed_impl<T>(kf, pc, m, px, n, d, v, v_rs, v_cs, t, nullptr, 0, 0, out, out_rs, out_cs, p,
                               ws_bytes - (size_t)(p - (char *)ws), st);
 }
 
 template <typename T>
-static int fdmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
+static int fdmmv_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
                       int64_t x2_rs, int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v,
                       int64_t v_rs, int64_t v_cs, const void *w, int64_t w_rs, int64_t w_cs, int64_t t, void *out,
                       int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes, hipStream_t st) {
@@ -296,8 +296,8 @@ static int fdmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, c
     T *up = (T *)p; p += planar_bytes<T>(n, m, d, t);     // u multiplies the rows of X in K^T u
     T *partial = (T *)p;
     size_t partial_avail = ws_bytes - (size_t)(p - (char *)ws);
-    if ((rc = pack_impl<T>(X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
-    if ((rc = pack_impl<T>(X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, packed_bytes<T>(m, d), st))) return rc;
+    if ((rc = pack_impl<T>(kf, X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
+    if ((rc = pack_impl<T>(kf, X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, packed_bytes<T>(m, d), st))) return rc;
     X = packed_view<T>(px, n, d);
     C = packed_view<T>(pc, m, d);
     Plan plan1 = make_plan<T>(C.nblk, X.nblk, d, C.dpad, t), plan2 = make_plan<T>(X.nblk, C.nblk, d, X.dpad, t);
@@ -306,17 +306,17 @@ static int fdmmv_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, c
     // u = K v + w, planar [t][X.npad] with zeroed padding (rows and the spare planes) so it can feed the
     // second product directly
     if ((rc = launch_zero_fill<T>(up + t * X.npad, zero_planes_needed<T>(plan2, t) * X.npad, st))) return rc;
-    if ((rc = mmv_packed_planar<T>(C, X, vp, t, (const T *)w, w_rs, w_cs, up, 1, X.npad, true, partial, partial_avail,
+    if ((rc = mmv_packed_planar<T>(kf, C, X, vp, t, (const T *)w, w_rs, w_cs, up, 1, X.npad, true, partial, partial_avail,
                                    st)))
         return rc;
     // out = K^T u
-    return mmv_packed_planar<T>(X, C, up, t, nullptr, 0, 0, (T *)out, out_rs, out_cs, false, partial, partial_avail,
+    return mmv_packed_planar<T>(kf, X, C, up, t, nullptr, 0, 0, (T *)out, out_rs, out_cs, false, partial, partial_avail,
                                 st);
 }
 
 // TI: element type of X1, X2, sigma and out; T: type the kernel values are computed in.
 template <typename TI, typename T>
-static int fmm_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
+static int fmm_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
                     int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, void *out, int64_t out_rs,
                     int64_t out_cs, void *ws, size_t ws_bytes, hipStream_t st) {
     if (n < 0 || m < 0 || d < 1) return fail(FLK_EINVAL, "bad shape");
@@ -333,16 +333,18 @@ static int fmm_impl(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, con
     if (ws_bytes < need || ws == nullptr)
         return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
     PackedView P1 = packed_view<T>(ws, n, d), P2 = packed_view<T>((char *)ws + packed_bytes<T>(n, d), m, d);
-    if ((rc = launch_pack<TI, T>((const TI *)X1, n, d, x1_rs, x1_cs, (const TI *)sigma, n_sigma, (T *)P1.data,
+    if ((rc = launch_pack<TI, T>((const TI *)X1, n, d, x1_rs, x1_cs, (const TI *)sigma, n_sigma, operand_scale(kf),
+                                 (T *)P1.data,
                                  (T *)P1.hnorm, P1.dpad, P1.nblk, false, st)))
         return rc;
-    if ((rc = launch_pack<TI, T>((const TI *)X2, m, d, x2_rs, x2_cs, (const TI *)sigma, n_sigma, (T *)P2.data,
+    if ((rc = launch_pack<TI, T>((const TI *)X2, m, d, x2_rs, x2_cs, (const TI *)sigma, n_sigma, operand_scale(kf),
+                                 (T *)P2.data,
                                  (T *)P2.hnorm, P2.dpad, P2.nblk, false, st)))
         return rc;
     // lanes run along the B operand: make that the dimension of out with the unit stride (a dimension of
     // extent one never has its stride applied, so it can take either role)
-    if (out_cs == 1 || m == 1) return launch_fmm<T, TI>(P1, P2, (TI *)out, out_rs, st);
-    return launch_fmm<T, TI>(P2, P1, (TI *)out, out_cs, st);
+    if (out_cs == 1 || m == 1) return launch_fmm<T, TI>(kf, P1, P2, (TI *)out, out_rs, st);
+    return launch_fmm<T, TI>(kf, P2, P1, (TI *)out, out_cs, st);
 }
 
 }  // namespace flk
@@ -385,12 +387,22 @@ size_t flk_gauss_packed_bytes(int64_t n, int64_t d, int dtype) {
     return dtype == FLK_F64 ? packed_bytes<double>(n, d) : packed_bytes<float>(n, d);
 }
 
+#define FLK_CHECK_KERNEL(kernel) \
+    if (!valid_kernel_fn(kernel)) return fail(FLK_EINVAL, "unknown kernel function %d", kernel)
+
+int flk_kernel_pack(int kernel, const void *X, int64_t n, int64_t d, int64_t x_rs, int64_t x_cs, const void *sigma,
+                    int64_t n_sigma, int dtype, void *packed, size_t packed_bytes_, void *stream) {
+    g_err[0] = 0;
+    FLK_CHECK_KERNEL(kernel);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == FLK_F32) return pack_impl<float>(kernel, X, n, d, x_rs, x_cs, sigma, n_sigma, packed, packed_bytes_, st);
+    if (dtype == FLK_F64) return pack_impl<double>(kernel, X, n, d, x_rs, x_cs, sigma, n_sigma, packed, packed_bytes_, st);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
 int flk_gauss_pack(const void *X, int64_t n, int64_t d, int64_t x_rs, int64_t x_cs, const void *sigma,
                    int64_t n_sigma, int dtype, void *packed, size_t packed_bytes_, void *stream) {
-    g_err[0] = 0;
-    if (dtype == FLK_F32) return pack_impl<float>(X, n, d, x_rs, x_cs, sigma, n_sigma, packed, packed_bytes_, (hipStream_t)stream);
-    if (dtype == FLK_F64) return pack_impl<double>(X, n, d, x_rs, x_cs, sigma, n_sigma, packed, packed_bytes_, (hipStream_t)stream);
-    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+    return flk_kernel_pack(FLK_GAUSSIAN, X, n, d, x_rs, x_cs, sigma, n_sigma, dtype, packed, packed_bytes_, stream);
 }
 
 size_t flk_gauss_mmv_packed_workspace_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t, int dtype) {
@@ -400,18 +412,27 @@ size_t flk_gauss_mmv_packed_workspace_bytes(int64_t n_a, int64_t n_b, int64_t d,
     return planar_bytes<float>(n_a, n_b, d, t) + partial_bytes<float>(n_a, n_b, d, t);
 }
 
+int flk_kernel_mmv_packed(int kernel, const void *packed_a, int64_t n_a, const void *packed_b, int64_t n_b, int64_t d,
+                          const void *vec, int64_t vec_rs, int64_t vec_cs, int64_t t, const void *addend,
+                          int64_t add_rs, int64_t add_cs, void *out, int64_t out_rs, int64_t out_cs, int dtype,
+                          void *workspace, size_t workspace_bytes, void *stream) {
+    g_err[0] = 0;
+    FLK_CHECK_KERNEL(kernel);
+    if (dtype == FLK_F32)
+        return mmv_packed_impl<float>(kernel, packed_a, n_a, packed_b, n_b, d, vec, vec_rs, vec_cs, t, addend, add_rs,
+                                      add_cs, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    if (dtype == FLK_F64)
+        return mmv_packed_impl<double>(kernel, packed_a, n_a, packed_b, n_b, d, vec, vec_rs, vec_cs, t, addend, add_rs,
+                                       add_cs, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
 int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b, int64_t n_b, int64_t d,
                          const void *vec, int64_t vec_rs, int64_t vec_cs, int64_t t, const void *addend,
                          int64_t add_rs, int64_t add_cs, void *out, int64_t out_rs, int64_t out_cs, int dtype,
                          void *workspace, size_t workspace_bytes, void *stream) {
-    g_err[0] = 0;
-    if (dtype == FLK_F32)
-        return mmv_packed_impl<float>(packed_a, n_a, packed_b, n_b, d, vec, vec_rs, vec_cs, t, addend, add_rs, add_cs,
-                                      out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    if (dtype == FLK_F64)
-        return mmv_packed_impl<double>(packed_a, n_a, packed_b, n_b, d, vec, vec_rs, vec_cs, t, addend, add_rs, add_cs,
-                                       out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+    return flk_kernel_mmv_packed(FLK_GAUSSIAN, packed_a, n_a, packed_b, n_b, d, vec, vec_rs, vec_cs, t, addend, add_rs,
+                                 add_cs, out, out_rs, out_cs, dtype, workspace, workspace_bytes, stream);
 }
 
 size_t flk_gauss_fmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
@@ -419,18 +440,27 @@ size_t flk_gauss_fmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t
     return dtype == FLK_F64 ? fmmv_ws_bytes<double>(n, m, d, t) : fmmv_ws_bytes<float>(n, m, d, t);
 }
 
+int flk_kernel_fmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
+                    int64_t x2_rs, int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v,
+                    int64_t v_rs, int64_t v_cs, int64_t t, void *out, int64_t out_rs, int64_t out_cs, int dtype,
+                    void *workspace, size_t workspace_bytes, void *stream) {
+    g_err[0] = 0;
+    FLK_CHECK_KERNEL(kernel);
+    if (dtype == FLK_F32)
+        return fmmv_impl<float>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t,
+                                out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    if (dtype == FLK_F64)
+        return fmmv_impl<double>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t,
+                                 out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
 int flk_gauss_fmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
                    int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v, int64_t v_rs,
                    int64_t v_cs, int64_t t, void *out, int64_t out_rs, int64_t out_cs, int dtype, void *workspace,
                    size_t workspace_bytes, void *stream) {
-    g_err[0] = 0;
-    if (dtype == FLK_F32)
-        return fmmv_impl<float>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t, out,
-                                out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    if (dtype == FLK_F64)
-        return fmmv_impl<double>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t, out,
-                                 out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+    return flk_kernel_fmmv(FLK_GAUSSIAN, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t,
+                           out, out_rs, out_cs, dtype, workspace, workspace_bytes, stream);
 }
 
 size_t flk_gauss_fdmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
@@ -438,18 +468,28 @@ size_t flk_gauss_fdmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t 
     return dtype == FLK_F64 ? fdmmv_ws_bytes<double>(n, m, d, t) : fdmmv_ws_bytes<float>(n, m, d, t);
 }
 
+int flk_kernel_fdmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
+                     int64_t x2_rs, int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v,
+                     int64_t v_rs, int64_t v_cs, const void *w, int64_t w_rs, int64_t w_cs, int64_t t, void *out,
+                     int64_t out_rs, int64_t out_cs, int dtype, void *workspace, size_t workspace_bytes,
+                     void *stream) {
+    g_err[0] = 0;
+    FLK_CHECK_KERNEL(kernel);
+    if (dtype == FLK_F32)
+        return fdmmv_impl<float>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
+                                 w_rs, w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    if (dtype == FLK_F64)
+        return fdmmv_impl<double>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
+                                  w_rs, w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
 int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
                     int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v, int64_t v_rs,
                     int64_t v_cs, const void *w, int64_t w_rs, int64_t w_cs, int64_t t, void *out, int64_t out_rs,
                     int64_t out_cs, int dtype, void *workspace, size_t workspace_bytes, void *stream) {
-    g_err[0] = 0;
-    if (dtype == FLK_F32)
-        return fdmmv_impl<float>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w, w_rs,
-                                 w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    if (dtype == FLK_F64)
-        return fdmmv_impl<double>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w, w_rs,
-                                  w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+    return flk_kernel_fdmmv(FLK_GAUSSIAN, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
+                            w_rs, w_cs, t, out, out_rs, out_cs, dtype, workspace, workspace_bytes, stream);
 }
 
 size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype, int compute_f64) {
@@ -458,21 +498,30 @@ size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype,
     return packed_bytes<float>(n, d) + packed_bytes<float>(m, d);
 }
 
+int flk_kernel_fmm(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
+                   int64_t x2_rs, int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, void *out,
+                   int64_t out_rs, int64_t out_cs, int dtype, int compute_f64, void *workspace, size_t workspace_bytes,
+                   void *stream) {
+    g_err[0] = 0;
+    FLK_CHECK_KERNEL(kernel);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == FLK_F64)
+        return fmm_impl<double, double>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs,
+                                        out_cs, workspace, workspace_bytes, st);
+    if (dtype == FLK_F32 && compute_f64)
+        return fmm_impl<float, double>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs,
+                                       out_cs, workspace, workspace_bytes, st);
+    if (dtype == FLK_F32)
+        return fmm_impl<float, float>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs,
+                                      out_cs, workspace, workspace_bytes, st);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
 int flk_gauss_fmm(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m, int64_t x2_rs,
                   int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, void *out, int64_t out_rs,
                   int64_t out_cs, int dtype, int compute_f64, void *workspace, size_t workspace_bytes, void *stream) {
-    g_err[0] = 0;
-    hipStream_t st = (hipStream_t)stream;
-    if (dtype == FLK_F64)
-        return fmm_impl<double, double>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs, out_cs,
-                                        workspace, workspace_bytes, st);
-    if (dtype == FLK_F32 && compute_f64)
-        return fmm_impl<float, double>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs, out_cs,
-                                       workspace, workspace_bytes, st);
-    if (dtype == FLK_F32)
-        return fmm_impl<float, float>(X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs, out_cs,
-                                      workspace, workspace_bytes, st);
-    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+    return flk_kernel_fmm(FLK_GAUSSIAN, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs, out_cs,
+                          dtype, compute_f64, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -103,12 +103,8 @@ int fail(int code, const char *fmt, ...);
 // launchers implemented in the .hip files -------------------------------------
 template <typename TI, typename T>   // TI: caller's element type, T: type of the packed operand
 int launch_pack(const TI *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const TI *sigma, int64_t n_sigma,
-                T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st);
+                double scale, T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st);
 
-// Explicit kernel matrix out[a][b] = K(A_a, B_b) from two packed operands; O is the element type of out,
-// whose rows (A side) are ld elements apart and whose columns (B side) are contiguous.
-template <typename T, typename O>
-int launch_fmm(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st);
 
 template <typename T>
 int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad,
@@ -120,10 +116,7 @@ int launch_finalize(const T *partial, int splits, int64_t t, int64_t nb, int64_t
                     int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
                     hipStream_t st);
 
-// Register-resident ("small d") product kernel.  Returns FLK_EUNSUPPORTED if dpad is out of its range.
-template <typename T>
-int launch_mmv_small(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tt,
-                     int64_t a_chunk_blocks, int splits, T *partial, hipStream_t st);
+// Register-resident ("small d") product kernel; the queries do not depend on the kernel function.
 template <typename T> int64_t mmv_small_max_d();
 template <typename T> int mmv_small_b_blocks_per_wg(int64_t dpad);
 template <typename T> int mmv_small_max_cols(int64_t dpad);   // right-hand sides per pass
@@ -134,12 +127,67 @@ constexpr int64_t kColPad = 15;
 
 // LDS-tiled ("large d") product kernel: any padded feature count, up to mmv_large_max_cols columns per pass.
 // Writes splits * mmv_large_partials_per_split partial results.
-template <typename T>
-int launch_mmv_large(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
-                     int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st);
 template <typename T> int mmv_large_a_tile_blocks();
 template <typename T> int mmv_large_b_tile_blocks();
 template <typename T> int mmv_large_partials_per_split();
 template <typename T> int mmv_large_max_cols();
+
+// The kernels that evaluate K are compiled once per kernel function (the same source with -DFLK_KF=0..3,
+// FLK_GAUSSIAN .. FLK_MATERN52): launchers carry the function in their name, and the helpers below pick one.
+//   launch_mmv_small_kf*: register-resident product kernel, FLK_EUNSUPPORTED if dpad is out of its range;
+//   launch_mmv_large_kf*: LDS-tiled product kernel, writes splits * mmv_large_partials_per_split partials;
+//   launch_fmm_kf*:       explicit kernel matrix out[a][b] = K(A_a, B_b); O is the element type of out, whose
+//                         rows (A side) are ld elements apart and whose columns (B side) are contiguous.
+#define FLK_CAT2(a, b) a##b
+#define FLK_CAT(a, b) FLK_CAT2(a, b)
+#define FLK_DECLARE_KF(KF)                                                                                        \
+    template <typename T>                                                                                         \
+    int launch_mmv_small_kf##KF(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tt,  \
+                                int64_t a_chunk_blocks, int splits, T *partial, hipStream_t st);                  \
+    template <typename T>                                                                                         \
+    int launch_mmv_large_kf##KF(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld,          \
+                                int tcols, int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st);    \
+    template <typename T, typename O>                                                                             \
+    int launch_fmm_kf##KF(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st);
+FLK_DECLARE_KF(0)
+FLK_DECLARE_KF(1)
+FLK_DECLARE_KF(2)
+FLK_DECLARE_KF(3)
+#undef FLK_DECLARE_KF
+
+constexpr int kNumKernelFns = 4;
+inline bool valid_kernel_fn(int kf) { return kf >= 0 && kf < kNumKernelFns; }
+// factor on x / sigma when packing: only the Gaussian folds the base change of its exponential into the rows
+inline double operand_scale(int kf) { return kf == FLK_GAUSSIAN ? kSqrtLog2e : 1.0; }
+
+#define FLK_SWITCH_KF(kf, CALL)                                          \
+    switch (kf) {                                                        \
+        case 0: return CALL(0);                                          \
+        case 1: return CALL(1);                                          \
+        case 2: return CALL(2);                                          \
+        case 3: return CALL(3);                                          \
+        default: return fail(FLK_EINVAL, "unknown kernel function %d", kf); \
+    }
+
+template <typename T>
+inline int launch_mmv_small(int kf, const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tt,
+                            int64_t a_chunk_blocks, int splits, T *partial, hipStream_t st) {
+#define FLK_CALL(KF) launch_mmv_small_kf##KF<T>(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st)
+    FLK_SWITCH_KF(kf, FLK_CALL)
+#undef FLK_CALL
+}
+template <typename T>
+inline int launch_mmv_large(int kf, const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
+                            int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
+#define FLK_CALL(KF) launch_mmv_large_kf##KF<T>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st)
+    FLK_SWITCH_KF(kf, FLK_CALL)
+#undef FLK_CALL
+}
+template <typename T, typename O>
+inline int launch_fmm(int kf, const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st) {
+#define FLK_CALL(KF) (launch_fmm_kf##KF<T, O>(A, B, out, ld, st))
+    FLK_SWITCH_KF(kf, FLK_CALL)
+#undef FLK_CALL
+}
 
 }  // namespace flk

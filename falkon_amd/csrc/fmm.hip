@@ -1,4 +1,4 @@
-// Explicit Gaussian kernel matrix out[a][b] = exp2(A~_a . B~_b + hA_a + hB_b) from two packed operands,
+// Explicit kernel matrix out[a][b] = f(A~_a . B~_b + hA_a + hB_b) from two packed operands (f: kernel_fn.h),
 // fp32 or fp64 arithmetic, stored as fp32 or fp64 (gfx950).  This is the K(C, C) the preconditioner
 // factorises once per fit; it is bound by the HBM writes of the result (or, computed in fp64, by the
 // software exp2), so the kernel is kept simple: no LDS, no barriers.
@@ -12,7 +12,12 @@
 // stores are non-temporal: the result is written once and never read here, and ordinary stores evicted
 // the operand tiles from L2 (M = 50 000, d = 28: 5.9 ms with ordinary stores, 3.8 ms without).
 #include "flk_common.h"
+#include "kernel_fn.h"
 #include "mfma_traits.h"
+
+#ifndef FLK_KF
+#define FLK_KF FLK_GAUSSIAN
+#endif
 
 namespace flk {
 
@@ -21,7 +26,8 @@ template <> struct FmmCfg<float>  { static constexpr int FA = 2, FB = 2; };
 template <> struct FmmCfg<double> { static constexpr int FA = 2, FB = 4; };
 constexpr int kFmmWavesA = 2, kFmmWavesB = 2;
 
-template <typename T, typename O, int FA, int FB>
+// KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
+template <typename T, typename O, int FA, int FB, int KF>
 __global__ void __launch_bounds__(64 * kFmmWavesA * kFmmWavesB)
     fmm_kernel(const T *__restrict__ PA, const T *__restrict__ hA, const T *__restrict__ PB, const T *__restrict__ hB,
                int64_t na_blocks, int64_t nb_blocks, int64_t n_a, int64_t n_b, int64_t dpad, int64_t b_tiles,
@@ -101,7 +107,7 @@ __global__ void __launch_bounds__(64 * kFmmWavesA * kFmmWavesB)
                 const vec4_t hn = *(const vec4_t *)(&hA[row0]);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const T k = TR::kexp(acc[p][q][4 * g + e] + (hn[e] + hb));
+                    const T k = kernel_value<FLK_KF>(acc[p][q][4 * g + e] + (hn[e] + hb));
                     if (row0 + e < n_a && col < n_b) __builtin_nontemporal_store((O)k, &out[(row0 + e) * ld + col]);
                 }
             }
@@ -110,21 +116,24 @@ __global__ void __launch_bounds__(64 * kFmmWavesA * kFmmWavesB)
 }
 
 template <typename T, typename O>
-int launch_fmm(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st) {
+int FLK_CAT(launch_fmm_kf, FLK_KF)(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st) {
     typedef FmmCfg<T> C;
     if (A.dpad != B.dpad || A.d != B.d) return fail(FLK_EINVAL, "fmm: operands packed with different feature counts");
     if (A.n == 0 || B.n == 0) return FLK_OK;
     const int64_t a_tiles = (A.nblk + kFmmWavesA * C::FA - 1) / (kFmmWavesA * C::FA);
     const int64_t b_tiles = (B.nblk + kFmmWavesB * C::FB - 1) / (kFmmWavesB * C::FB);
     if (a_tiles * b_tiles > (int64_t)0x7fffffff) return fail(FLK_EUNSUPPORTED, "fmm: more tiles than one launch holds");
-    hipLaunchKernelGGL((fmm_kernel<T, O, C::FA, C::FB>), dim3((unsigned)(a_tiles * b_tiles)),
+    hipLaunchKernelGGL((fmm_kernel<T, O, C::FA, C::FB, FLK_KF>), dim3((unsigned)(a_tiles * b_tiles)),
                        dim3(64 * kFmmWavesA * kFmmWavesB), 0, st, (const T *)A.data, (const T *)A.hnorm,
                        (const T *)B.data, (const T *)B.hnorm, A.nblk, B.nblk, A.n, B.n, A.dpad, b_tiles, out, ld);
     FLK_LAUNCH_CHECK("fmm_kernel");
     return FLK_OK;
 }
-template int launch_fmm<float, float>(const PackedView &, const PackedView &, float *, int64_t, hipStream_t);
-template int launch_fmm<double, double>(const PackedView &, const PackedView &, double *, int64_t, hipStream_t);
-template int launch_fmm<double, float>(const PackedView &, const PackedView &, float *, int64_t, hipStream_t);
+template int FLK_CAT(launch_fmm_kf, FLK_KF)<float, float>(const PackedView &, const PackedView &, float *, int64_t,
+                                                          hipStream_t);
+template int FLK_CAT(launch_fmm_kf, FLK_KF)<double, double>(const PackedView &, const PackedView &, double *, int64_t,
+                                                            hipStream_t);
+template int FLK_CAT(launch_fmm_kf, FLK_KF)<double, float>(const PackedView &, const PackedView &, float *, int64_t,
+                                                           hipStream_t);
 
 }  // namespace flk

@@ -24,9 +24,6 @@ template <> struct LTraits<float> {
     static __device__ __forceinline__ int out_row(int j) { return j; }
     // matrix row (within its block) of accumulator register r in lane group lg
     static __device__ __forceinline__ int acc_row(int r, int lg) { return 8 * (r >> 2) + 4 * lg + (r & 3); }
-    static __device__ __forceinline__ float kexp(float x) {
-        return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(x), 0.0f, 1.0f);
-    }
 };
 
 template <> struct LTraits<double> {
@@ -40,7 +37,6 @@ template <> struct LTraits<double> {
     static __device__ __forceinline__ int group_off(int g, int lg) { return 4 * lg; }
     static __device__ __forceinline__ int out_row(int j) { return 4 * (j & 3) + (j >> 2); }
     static __device__ __forceinline__ int acc_row(int r, int lg) { return 4 * lg + r; }
-    static __device__ __forceinline__ double kexp(double x) { return exp2(fmin(x, 0.0)); }
 };
 
 }  // namespace flk

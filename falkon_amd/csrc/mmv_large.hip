@@ -14,7 +14,12 @@
 // Waves are arranged WVA (A) x WVB (B); waves with the same wb produce partial sums for the same
 // output rows and simply write separate partials (they count as extra splits for the reduction).
 #include "flk_common.h"
+#include "kernel_fn.h"
 #include "mfma_traits.h"
+
+#ifndef FLK_KF
+#define FLK_KF FLK_GAUSSIAN
+#endif
 
 namespace flk {
 
@@ -49,7 +54,8 @@ __device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t b
     return P + (b * dpad + (int64_t)lg * DPsteps + s0 + s) * TR::BLK + jv * TR::VPL;
 }
 
-template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC, int TT>
+// KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
+template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC, int TT, int KF>
 __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   // two waves per SIMD either way
     mmv_large_kernel(const T *__restrict__ PA, const T *__restrict__ hA, const T *__restrict__ vecp, int64_t vec_ld,
                      int tcols, const T *__restrict__ PB, const T *__restrict__ hB, int64_t na_blocks,
@@ -246,7 +252,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
                 for (int q = 0; q < WB_FR; q++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) kv[q][e] = TR::kexp(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
+                    for (int e = 0; e < 4; e++) kv[q][e] = kernel_value<FLK_KF>(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
 #pragma unroll
                 for (int tg = 0; tg < NTG; tg++) {
                     const int t0 = 4 * tg;
@@ -285,7 +291,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                     for (int q = 0; q < WB_FR; q++)
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            acc[p][q][4 * g + e] = TR::kexp(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
+                            acc[p][q][4 * g + e] = kernel_value<FLK_KF>(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
                 }
             }
             // out2[q][j-rows][t] += sum_i K[i][j] vec[i][t]: accumulator register s of a lane is exactly the MFMA
@@ -353,18 +359,20 @@ template <> struct LCfg<float>  { static constexpr int WVA = 2, WVB = 2, WA_FR =
 // fp64: 8 waves (2 x 4), one workgroup per CU; tile 128 (A) x 128 (B) rows.
 template <> struct LCfg<double> { static constexpr int WVA = 2, WVB = 4, WA_FR = 4, WB_FR = 2, KC = 8; };
 
-template <typename T> int mmv_large_max_cols();
+constexpr int kLargeMaxCols = 16;
+#if FLK_KF == FLK_GAUSSIAN   // the tile geometry is the same for every kernel function: defined once
 template <typename T> int mmv_large_a_tile_blocks() { return LCfg<T>::WVA * LCfg<T>::WA_FR; }
 template <typename T> int mmv_large_b_tile_blocks() { return LCfg<T>::WVB * LCfg<T>::WB_FR; }
 template <typename T> int mmv_large_partials_per_split() { return LCfg<T>::WVA; }
-template <> int mmv_large_max_cols<float>() { return 16; }
-template <> int mmv_large_max_cols<double>() { return 16; }
+template <> int mmv_large_max_cols<float>() { return kLargeMaxCols; }
+template <> int mmv_large_max_cols<double>() { return kLargeMaxCols; }
 template int mmv_large_a_tile_blocks<float>();
 template int mmv_large_a_tile_blocks<double>();
 template int mmv_large_b_tile_blocks<float>();
 template int mmv_large_b_tile_blocks<double>();
 template int mmv_large_partials_per_split<float>();
 template int mmv_large_partials_per_split<double>();
+#endif
 
 template <typename T, int TT>
 static int launch_large_tt(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
@@ -372,7 +380,7 @@ static int launch_large_tt(const PackedView &A, const PackedView &B, const T *ve
     typedef LCfg<T> C;
     const int64_t nbb = C::WVB * C::WB_FR;
     dim3 grid((unsigned)((B.nblk + nbb - 1) / nbb), (unsigned)splits);
-    hipLaunchKernelGGL((mmv_large_kernel<T, C::WVA, C::WVB, C::WA_FR, C::WB_FR, C::KC, TT>), grid,
+    hipLaunchKernelGGL((mmv_large_kernel<T, C::WVA, C::WVB, C::WA_FR, C::WB_FR, C::KC, TT, FLK_KF>), grid,
                        dim3(64 * C::WVA * C::WVB), 0, st,
                        (const T *)A.data, (const T *)A.hnorm, vecp, vec_ld, tcols, (const T *)B.data,
                        (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, a_tiles_per_chunk, partial, B.npad, B.n > A.n);
@@ -381,19 +389,20 @@ static int launch_large_tt(const PackedView &A, const PackedView &B, const T *ve
 }
 
 template <typename T>
-int launch_mmv_large(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
-                     int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
+int FLK_CAT(launch_mmv_large_kf, FLK_KF)(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld,
+                                         int tcols, int64_t a_tiles_per_chunk, int splits, T *partial,
+                                         hipStream_t st) {
     if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_large: operands packed with different feature counts");
-    if (tcols < 1 || tcols > mmv_large_max_cols<T>())
-        return fail(FLK_EINVAL, "mmv_large: column chunk %d not in 1..%d", tcols, mmv_large_max_cols<T>());
+    if (tcols < 1 || tcols > kLargeMaxCols)
+        return fail(FLK_EINVAL, "mmv_large: column chunk %d not in 1..%d", tcols, kLargeMaxCols);
     if (tcols == 1) return launch_large_tt<T, 1>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols == 2) return launch_large_tt<T, 2>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols <= 4) return launch_large_tt<T, 4>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     return launch_large_tt<T, 16>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);   // MFMA epilogue
 }
-template int launch_mmv_large<float>(const PackedView &, const PackedView &, const float *, int64_t, int, int64_t,
-                                     int, float *, hipStream_t);
-template int launch_mmv_large<double>(const PackedView &, const PackedView &, const double *, int64_t, int, int64_t,
-                                      int, double *, hipStream_t);
+template int FLK_CAT(launch_mmv_large_kf, FLK_KF)<float>(const PackedView &, const PackedView &, const float *, int64_t,
+                                                         int, int64_t, int, float *, hipStream_t);
+template int FLK_CAT(launch_mmv_large_kf, FLK_KF)<double>(const PackedView &, const PackedView &, const double *,
+                                                          int64_t, int, int64_t, int, double *, hipStream_t);
 
 }  // namespace flk

@@ -1,14 +1,21 @@
 // Register-resident fp32 product kernel: instantiations for even feature counts, and the entry point
-// that picks between them and the folded variant.
+// that picks between them and the folded variant.  Compiled once per kernel function (-DFLK_KF=0..3).
+#ifndef FLK_KF
+#define FLK_KF 0
+#endif
 #define FLK_FOLD false
-#define FLK_LAUNCH_NAME launch_mmv_small_f32_plain
+#define FLK_PASTE2(a, b) a##b
+#define FLK_PASTE(a, b) FLK_PASTE2(a, b)
+#define FLK_LAUNCH_NAME FLK_PASTE(launch_mmv_small_f32_plain_kf, FLK_KF)
 #include "mmv_small_f32_dispatch.inc"
 
 namespace flk {
 
-int launch_mmv_small_f32_fold(const PackedView &A, const PackedView &B, const float *vecp, int64_t vec_ld, int tt,
-                              int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st);
+int FLK_CAT(launch_mmv_small_f32_fold_kf, FLK_KF)(const PackedView &A, const PackedView &B, const float *vecp,
+                                                  int64_t vec_ld, int tt, int64_t a_chunk_blocks, int splits,
+                                                  float *partial, hipStream_t st);
 
+#if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<float>() { return 2 * kMaxDpFr2; }
 template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad) {
     return kWavesPerWg * ((dpad / 2) <= kMaxDpFr4 ? 4 : 2);
@@ -17,15 +24,18 @@ template <> int mmv_small_max_cols<float>(int64_t dpad) {
     const int64_t dp = dpad / 2;   // must match the instantiations in launch_tt
     return dp <= 7 ? 16 : dp <= 12 ? 12 : dp <= 16 ? 8 : 4;
 }
+#endif
 
 template <>
-int launch_mmv_small<float>(const PackedView &A, const PackedView &B, const float *vecp, int64_t vec_ld, int tt,
-                            int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
+int FLK_CAT(launch_mmv_small_kf, FLK_KF)<float>(const PackedView &A, const PackedView &B, const float *vecp,
+                                                int64_t vec_ld, int tt, int64_t a_chunk_blocks, int splits,
+                                                float *partial, hipStream_t st) {
     if (A.dpad != B.dpad || A.d != B.d)
         return fail(FLK_EINVAL, "mmv_small: operands packed with different feature counts");
     // odd d up to kFoldMaxD: the padding feature holds 1.0 (see pack_kernel) and carries hB through the MFMA chain
-    if (f32_fold_applies(A.d)) return launch_mmv_small_f32_fold(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st);
-    return launch_mmv_small_f32_plain(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st);
+    if (f32_fold_applies(A.d))
+        return FLK_CAT(launch_mmv_small_f32_fold_kf, FLK_KF)(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st);
+    return FLK_LAUNCH_NAME(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st);
 }
 
 }  // namespace flk

@@ -1,4 +1,5 @@
-// Register-resident Gaussian kernel-vector product, fp32, gfx950.
+// Register-resident kernel-vector product for the radial kernels of kernel_fn.h, fp32, gfx950.
+// (Written for the Gaussian, K = exp2(e); the other kernel functions replace the exp2 of the epilogue.)
 //
 //   partial[split][t][b] = sum_{a in chunk(split)} exp2(A~_a . B~_b + hA_a + hB_b) * vec[a,t]
 //
@@ -16,6 +17,7 @@
 // the very end (one xor-32 shuffle to join the two lane halves).
 #pragma once
 #include "flk_common.h"
+#include "kernel_fn.h"
 
 namespace flk {
 
@@ -24,13 +26,6 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWavesPerWg = 4;
 constexpr int kFlushEvery = 16;  // A blocks between flushes of the short accumulator
-
-__device__ __forceinline__ float kexp2_clamped(float x) {
-    // min(exp2(x), 1) == exp2(min(x, 0)): the reference clamps the squared distance at
-    // 1e-20 before exp (distance_kernel.py:100,157-158), i.e. K <= 1.  The median-of-three
-    // with 0 and 1 folds into the clamp bit of v_exp_f32, so the clamp costs no instruction.
-    return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(x), 0.0f, 1.0f);
-}
 
 // Per-row quantities of an A block (half norms and right-hand side entries) reach the lanes through
 // a small wave-private LDS buffer: each lane fetches ONE dword from global memory, the wave writes the
@@ -69,7 +64,7 @@ __device__ __forceinline__ void load_a(float (&a)[DP], const float *__restrict__
     for (int s = 0; s < DP; s++) a[s] = p[s * 32];
 }
 
-template <int DP, int FR, int TT, bool FOLD>
+template <int DP, int FR, int TT, bool FOLD, int KF>
 __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds, int h, const float (&breg)[FR][DP],
                                           const float (&hb)[FR], float (&o1)[FR][TT]) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -97,7 +92,7 @@ __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds
         for (int q = 0; q < FR; q++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                float k = kexp2_clamped(acc[q][r]);
+                float k = kernel_value<KF>(acc[q][r]);
 #pragma unroll
                 for (int t = 0; t < TT; t++) o1[q][t] = __builtin_fmaf(k, vec[t][r >> 2][r & 3], o1[q][t]);
             }
@@ -112,7 +107,7 @@ __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds
 #pragma unroll
         for (int q = 0; q < FR; q++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[q][r] = kexp2_clamped(acc[q][r]);
+            for (int r = 0; r < 16; r++) acc[q][r] = kernel_value<KF>(acc[q][r]);
         // Groups of up to four columns of one row group, software pipelined by hand: the reads of the
         // next group are issued, then a compiler memory fence pins them there, then the FMAs of the
         // current group run.  Without the fences the compiler moves all 4*TT LDS reads to the front
@@ -160,7 +155,7 @@ __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds
 // FOLD (odd feature counts only): the one padding feature of the packed rows carries 1.0, and the
 // resident B fragment puts hB_j into that slot, so the MFMA chain adds hB_j by itself and the
 // accumulators start from the A block's half norms without any VALU add.
-template <int DP, int FR, int TT, bool FOLD>
+template <int DP, int FR, int TT, bool FOLD, int KF>
 __global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 registers per lane
     mmv_small_f32_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
                          int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB, int64_t na_blocks,
@@ -218,12 +213,12 @@ __global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 r
     for (int64_t ab = a0; ab < a1; ab += 2) {
         const bool has1 = ab + 1 < a1;
         if (has1) { load_a<DP>(fa1, PA, ab + 1, j, h); fetch_rowvals<TT>(rv, src, ab + 1); }
-        tile_step<DP, FR, TT, FOLD>(fa0, lds0, h, breg, hb, o1);
+        tile_step<DP, FR, TT, FOLD, KF>(fa0, lds0, h, breg, hb, o1);
         if (has1) {
             stage_rowvals<TT>(rv, lds1, lane);
             const bool has2 = ab + 2 < a1;
             if (has2) { load_a<DP>(fa0, PA, ab + 2, j, h); fetch_rowvals<TT>(rv, src, ab + 2); }
-            tile_step<DP, FR, TT, FOLD>(fa1, lds1, h, breg, hb, o1);
+            tile_step<DP, FR, TT, FOLD, KF>(fa1, lds1, h, breg, hb, o1);
             if (has2) stage_rowvals<TT>(rv, lds0, lane);
         }
         since_flush += 2;

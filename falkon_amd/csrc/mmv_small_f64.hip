@@ -1,4 +1,5 @@
-// Register-resident Gaussian kernel-vector product, fp64, gfx950.
+// Register-resident kernel-vector product for the radial kernels of kernel_fn.h, fp64, gfx950.
+// Compiled once per kernel function (-DFLK_KF=0..3).
 //
 // Same structure as the fp32 kernel with the 16x16x4 fp64 MFMA: a wave keeps FR
 // blocks of 16 output rows (B side) in registers and streams blocks of 16
@@ -9,6 +10,11 @@
 // 4*(row%4) + row/4, so a lane's four accumulator rows are the consecutive
 // matrix rows 4*q .. 4*q+3 of the A block.
 #include "flk_common.h"
+#include "kernel_fn.h"
+
+#ifndef FLK_KF
+#define FLK_KF FLK_GAUSSIAN
+#endif
 
 namespace flk {
 
@@ -16,12 +22,6 @@ typedef double doublex4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWavesPerWg64 = 4;
 constexpr int kFlushEvery64 = 16;
-
-__device__ __forceinline__ double kexp2_clamped(double x) {
-    // exp2(min(x, 0)): the reference clamps the squared distance at 1e-20 before exp
-    // (distance_kernel.py:100,157-158), i.e. K <= 1.
-    return exp2(fmin(x, 0.0));
-}
 
 template <int DP, int TT>
 struct AFrag64 {
@@ -59,13 +59,14 @@ __device__ __forceinline__ void tile_step64(const AFrag64<DP, TT> &f, const doub
     for (int c = 0; c < FR; c++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            double k = kexp2_clamped(acc[c][r]);
+            double k = kernel_value<FLK_KF>(acc[c][r]);
 #pragma unroll
             for (int t = 0; t < TT; t++) o1[c][t] = __builtin_fma(k, f.vec[t][r], o1[c][t]);
         }
 }
 
-template <int DP, int FR, int TT>
+// KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
+template <int DP, int FR, int TT, int KF>
 __global__ void __launch_bounds__(256)
     mmv_small_f64_kernel(const double *__restrict__ PA, const double *__restrict__ hA, const double *__restrict__ vecp,
                          int64_t vec_ld, const double *__restrict__ PB, const double *__restrict__ hB,
@@ -135,18 +136,20 @@ __global__ void __launch_bounds__(256)
 constexpr int kMaxDp64Fr4 = 8;   // dpad <= 32
 constexpr int kMaxDp64Fr2 = 16;  // dpad <= 64
 
+#if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<double>() { return 4 * kMaxDp64Fr2; }
 template <> int mmv_small_max_cols<double>(int64_t dpad) { (void)dpad; return 4; }
 template <> int mmv_small_b_blocks_per_wg<double>(int64_t dpad) {
     return kWavesPerWg64 * ((dpad / 4) <= kMaxDp64Fr4 ? 4 : 2);
 }
+#endif
 
 template <int DP, int FR, int TT>
 static int launch_one64(const PackedView &A, const PackedView &B, const double *vecp, int64_t vec_ld,
                         int64_t a_chunk_blocks, int splits, double *partial, hipStream_t st) {
     const int64_t per_wg = kWavesPerWg64 * FR;
     dim3 grid((unsigned)((B.nblk + per_wg - 1) / per_wg), (unsigned)splits);
-    hipLaunchKernelGGL((mmv_small_f64_kernel<DP, FR, TT>), grid, dim3(256), 0, st, (const double *)A.data,
+    hipLaunchKernelGGL((mmv_small_f64_kernel<DP, FR, TT, FLK_KF>), grid, dim3(256), 0, st, (const double *)A.data,
                        (const double *)A.hnorm, vecp, vec_ld, (const double *)B.data, (const double *)B.hnorm, A.nblk,
                        B.nblk, a_chunk_blocks, partial, B.npad, B.n > A.n);
     FLK_LAUNCH_CHECK("mmv_small_f64_kernel");
@@ -166,8 +169,9 @@ static int launch_tt64(int tt, const PackedView &A, const PackedView &B, const d
 }
 
 template <>
-int launch_mmv_small<double>(const PackedView &A, const PackedView &B, const double *vecp, int64_t vec_ld, int tt,
-                             int64_t a_chunk_blocks, int splits, double *partial, hipStream_t st) {
+int FLK_CAT(launch_mmv_small_kf, FLK_KF)<double>(const PackedView &A, const PackedView &B, const double *vecp,
+                                                 int64_t vec_ld, int tt, int64_t a_chunk_blocks, int splits,
+                                                 double *partial, hipStream_t st) {
     if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_small: operands packed with different feature counts");
     const int dp = (int)(A.dpad / 4);
 #define FLK_CASE4(DPV) \

@@ -4,7 +4,8 @@
 namespace flk {
 
 // ---------------------------------------------------------------------------
-// pack: X[n,d] (any unit-stride order) -> [nblk][dpad][BLK] scaled by sqrt(log2 e)/sigma,
+// pack: X[n,d] (any unit-stride order) -> [nblk][dpad][BLK] scaled by scale/sigma (scale = sqrt(log2 e)
+// for the Gaussian, 1 for the other kernels),
 // plus hnorm[row] = -1/2 |x~|^2.  One workgroup per block of BLK rows; a
 // BLK x 32 tile goes through LDS so that both the read (along the unit stride
 // of X) and the write (along rows of the block) are coalesced.
@@ -21,8 +22,8 @@ template <> __device__ __forceinline__ int block_pos<double>(int r) { return 4 *
 template <typename TI, typename T>
 __global__ void __launch_bounds__(256) pack_kernel(const TI *__restrict__ X, int64_t n, int64_t d, int64_t rs,
                                                    int64_t cs, const TI *__restrict__ sigma, int64_t n_sigma,
-                                                   T *__restrict__ pdata, T *__restrict__ hnorm, int64_t dpad,
-                                                   bool one_pad) {
+                                                   double scale, T *__restrict__ pdata, T *__restrict__ hnorm,
+                                                   int64_t dpad, bool one_pad) {
     constexpr int BLK = Geo<T>::BLK;
     constexpr int KT = 32;                       // features per LDS tile
     __shared__ T tile[BLK][KT + 1];
@@ -41,7 +42,7 @@ __global__ void __launch_bounds__(256) pack_kernel(const TI *__restrict__ X, int
             int64_t row = row0 + r, kk = k0 + k;
             T val = T(0);
             if (row < n && kk < d) {
-                double s = kSqrtLog2e / (double)sigma[n_sigma == 1 ? 0 : kk];
+                double s = scale / (double)sigma[n_sigma == 1 ? 0 : kk];
                 val = (T)((double)X[row * rs + kk * cs] * s);
             } else if (one_pad && kk == d) {
                 val = T(1);          // padding feature of odd-d fp32 operands: multiplies the folded half norm
@@ -67,19 +68,19 @@ __global__ void __launch_bounds__(256) pack_kernel(const TI *__restrict__ X, int
 
 template <typename TI, typename T>
 int launch_pack(const TI *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const TI *sigma, int64_t n_sigma,
-                T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st) {
+                double scale, T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st) {
     if (nblk == 0) return FLK_OK;
-    hipLaunchKernelGGL((pack_kernel<TI, T>), dim3((unsigned)nblk), dim3(256), 0, st, X, n, d, rs, cs, sigma, n_sigma, pdata,
-                       hnorm, dpad, one_pad);
+    hipLaunchKernelGGL((pack_kernel<TI, T>), dim3((unsigned)nblk), dim3(256), 0, st, X, n, d, rs, cs, sigma, n_sigma, scale,
+                       pdata, hnorm, dpad, one_pad);
     FLK_LAUNCH_CHECK("pack_kernel");
     return FLK_OK;
 }
 template int launch_pack<float, float>(const float *, int64_t, int64_t, int64_t, int64_t, const float *, int64_t,
-                                       float *, float *, int64_t, int64_t, bool, hipStream_t);
+                                       double, float *, float *, int64_t, int64_t, bool, hipStream_t);
 template int launch_pack<double, double>(const double *, int64_t, int64_t, int64_t, int64_t, const double *, int64_t,
-                                         double *, double *, int64_t, int64_t, bool, hipStream_t);
+                                         double, double *, double *, int64_t, int64_t, bool, hipStream_t);
 template int launch_pack<float, double>(const float *, int64_t, int64_t, int64_t, int64_t, const float *, int64_t,
-                                        double *, double *, int64_t, int64_t, bool, hipStream_t);
+                                        double, double *, double *, int64_t, int64_t, bool, hipStream_t);
 
 // ---------------------------------------------------------------------------
 // vec_planar: v[n,t] with element strides (rs, cs) -> vp[t + zero_planes][npad]: rows past n and the

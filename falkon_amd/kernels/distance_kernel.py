@@ -1,4 +1,4 @@
-"""Gaussian kernel object (falkon/kernels/distance_kernel.py:20-38,314-432).
+"""Distance kernels: Gaussian, Laplacian, Matern (falkon/kernels/distance_kernel.py:20-38,314-648).
 
 ``mmv`` / ``dmmv`` and the kernel matrix ``kernel(X1, X2)`` run the MI355X kernels of
 ``libfalkon_amd``.  ``compute`` (the explicit kernel block the reference's ``rbf_core``
@@ -12,7 +12,7 @@ import torch
 from ..options import FalkonOptions
 from .diff_kernel import DiffKernel
 
-__all__ = ("GaussianKernel", "validate_sigma")
+__all__ = ("GaussianKernel", "LaplacianKernel", "MaternKernel", "validate_sigma")
 
 
 def validate_sigma(sigma: Union[float, torch.Tensor]) -> torch.Tensor:
@@ -32,31 +32,36 @@ def validate_sigma(sigma: Union[float, torch.Tensor]) -> torch.Tensor:
     return sigma.reshape(-1)
 
 
-def _rbf_block(mat1, mat2, out: Optional[torch.Tensor], diag: bool, sigma: torch.Tensor) -> torch.Tensor:
-    """exp(-1/2 |mat1/sigma - mat2/sigma|^2) as a stored block, with stock torch ops."""
+_SQRT3, _SQRT5 = 3.0 ** 0.5, 5.0 ** 0.5
+
+
+def _radial_block(mat1, mat2, out: Optional[torch.Tensor], diag: bool, sigma: torch.Tensor,
+                  nu: float = float("inf")) -> torch.Tensor:
+    """A stored block of a radial kernel with stock torch ops: f(D), D = |mat1/sigma - mat2/sigma|, with
+    f = exp(-D^2/2) (nu = inf), exp(-D) (1/2), (1 + s) exp(-s) with s = sqrt(3) D (3/2),
+    (1 + s + s^2/3) exp(-s) with s = sqrt(5) D (5/2).  Off the kernel-vector path (diagonals, callers' own blocks)."""
     sigma = sigma.to(device=mat1.device, dtype=mat1.dtype)
     a, b = mat1 / sigma, mat2 / sigma
     if diag:
-        res = (a - b).square().sum(-1).mul_(-0.5).exp_()
-        return res if out is None else out.copy_(res)
-    na, nb = a.square().sum(-1, keepdim=True), b.square().sum(-1, keepdim=True)
-    if out is None:
-        out = torch.addmm(na, a, b.T, alpha=-2, beta=1)
+        d2 = (a - b).square().sum(-1)
     else:
-        out = torch.addmm(na, a, b.T, alpha=-2, beta=1, out=out)
-    out.add_(nb.T).clamp_min_(1e-20).mul_(-0.5).exp_()
-    return out
+        d2 = torch.addmm(a.square().sum(-1, keepdim=True), a, b.T, alpha=-2, beta=1)
+        d2.add_(b.square().sum(-1, keepdim=True).T).clamp_min_(1e-20)
+    if nu == float("inf"):
+        res = d2.mul_(-0.5).exp_()
+    else:
+        s = d2.sqrt_().mul_({0.5: 1.0, 1.5: _SQRT3, 2.5: _SQRT5}[nu])
+        decay = torch.exp(-s)
+        res = decay if nu == 0.5 else decay.mul_(1 + s if nu == 1.5 else 1 + s + s * s / 3)
+    return res if out is None else out.copy_(res.reshape(out.shape))
 
 
-class GaussianKernel(DiffKernel):
-    r"""k(x, x') = exp(-|x - x'|^2 / (2 sigma^2)); ``sigma`` a scalar or one lengthscale per dimension."""
+class _RadialKernel(DiffKernel):
+    """Shared part of the distance kernels: ``sigma`` (scalar or one lengthscale per dimension) as a registered
+    parameter, its cached copy on the data's device, and no per-entry scratch memory."""
 
-    kernel_name = "gaussian"
-    core_fn = _rbf_block
-
-    def __init__(self, sigma: Union[float, torch.Tensor], opt: Optional[FalkonOptions] = None):
-        sigma = validate_sigma(sigma)
-        super().__init__(self.kernel_name, opt, core_fn=GaussianKernel.core_fn, sigma=sigma)
+    def __init__(self, name: str, sigma, opt: Optional[FalkonOptions], **other_params):
+        super().__init__(name, opt, core_fn=_radial_block, sigma=validate_sigma(sigma), **other_params)
         self._sigma_cache = {}
 
     def _sigma_on(self, device: torch.device, dtype: torch.dtype) -> torch.Tensor:
@@ -74,6 +79,15 @@ class GaussianKernel(DiffKernel):
         # the fused kernels need no per-entry scratch; the packed operands are sized by the library itself
         return {}
 
+
+class GaussianKernel(_RadialKernel):
+    r"""k(x, x') = exp(-|x - x'|^2 / (2 sigma^2)); ``sigma`` a scalar or one lengthscale per dimension."""
+
+    kernel_name = "gaussian"
+
+    def __init__(self, sigma: Union[float, torch.Tensor], opt: Optional[FalkonOptions] = None):
+        super().__init__(self.kernel_name, sigma, opt)
+
     def detach(self) -> "GaussianKernel":
         return GaussianKernel(self.sigma.detach(), opt=self.params)
 
@@ -82,3 +96,62 @@ class GaussianKernel(DiffKernel):
 
     def __str__(self):
         return f"Gaussian kernel<{self.sigma}>"
+
+
+class LaplacianKernel(_RadialKernel):
+    r"""k(x, x') = exp(-|x - x'| / sigma) (falkon/kernels/distance_kernel.py:435-507)."""
+
+    kernel_name = "laplacian"
+
+    def __init__(self, sigma: Union[float, torch.Tensor], opt: Optional[FalkonOptions] = None):
+        super().__init__(self.kernel_name, sigma, opt, nu=0.5)
+
+    def detach(self) -> "LaplacianKernel":
+        return LaplacianKernel(self.sigma.detach(), opt=self.params)
+
+    def __repr__(self):
+        return f"LaplacianKernel(sigma={self.sigma})"
+
+    def __str__(self):
+        return f"Laplacian kernel<{self.sigma}>"
+
+
+class MaternKernel(_RadialKernel):
+    r"""Matern kernel for the smoothness values with a closed form, nu in {0.5, 1.5, 2.5, inf}
+    (falkon/kernels/distance_kernel.py:510-648): nu = 0.5 is the Laplacian, nu = inf the Gaussian."""
+
+    _valid_nu_values = frozenset({0.5, 1.5, 2.5, float("inf")})
+
+    def __init__(self, sigma: Union[float, torch.Tensor], nu: Union[float, torch.Tensor],
+                 opt: Optional[FalkonOptions] = None):
+        nu = self.validate_nu(nu)
+        self.kernel_name = f"{nu:.1f}-matern"
+        super().__init__(self.kernel_name, sigma, opt, nu=nu)
+
+    @staticmethod
+    def validate_nu(nu: Union[torch.Tensor, float]) -> float:
+        """A float or a tensor without gradient, rounded to two digits, one of the four closed-form values."""
+        if isinstance(nu, torch.Tensor):
+            if nu.requires_grad:
+                raise ValueError("The nu parameter of the Matern kernel is not differentiable, "
+                                 "and must not require gradients.")
+            if nu.numel() != 1:
+                raise ValueError(f"nu={nu} is not convertible to a scalar.")
+            value = float(nu.item())
+        elif isinstance(nu, float):
+            value = nu
+        else:
+            raise TypeError(f"nu must be a float or a tensor, not a {type(nu)}")
+        value = round(value, ndigits=2)
+        if value not in MaternKernel._valid_nu_values:
+            raise ValueError(f"The given value of nu = {value} can only take values {MaternKernel._valid_nu_values}.")
+        return value
+
+    def detach(self) -> "MaternKernel":
+        return MaternKernel(self.sigma.detach(), self.nondiff_params["nu"], opt=self.params)
+
+    def __repr__(self):
+        return f"MaternKernel(sigma={self.sigma}, nu={self.nondiff_params['nu']:.1f})"
+
+    def __str__(self):
+        return f"Matern kernel<{self.sigma}, {self.nondiff_params['nu']:.1f}>"

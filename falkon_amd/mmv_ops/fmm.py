@@ -1,7 +1,8 @@
 """Explicit kernel matrix K(X1, X2): the K(C, C) the preconditioner factorises once per fit, and
 ``kernel(X1, X2)``.
 
-Drop-in for falkon/mmv_ops/fmm.py:298-388,576-640,699-708 in the dense, non-differentiable Gaussian case:
+Drop-in for falkon/mmv_ops/fmm.py:298-388,576-640,699-708 in the dense, non-differentiable case of the radial
+kernels (Gaussian, Laplacian, Matern):
 ``flk_gauss_fmm`` packs both operands and writes the matrix in one launch (cross term on MFMA, exp2 on
 the accumulators).  With ``opt.no_single_kernel`` fp32 inputs are evaluated in fp64 and rounded once
 when stored (falkon/mmv_ops/fmm.py:619-622).  Rows of X1 are split only when the result is wanted on
@@ -15,15 +16,14 @@ import torch
 from .. import _backend
 from ..options import BaseOptions
 from ..utils.helpers import sizeof_dtype
-from .fmmv import _DTYPE_CODE, _check_dtype, _compute_device, _mat, _on, _require_gaussian, _rows_that_fit, \
-    _stream_handle
+from .fmmv import _DTYPE_CODE, _check_dtype, _compute_device, _kernel_fn, _mat, _on, _rows_that_fit, _stream_handle
 from .utils import check_contiguity, create_output_mat, usable_gpu_memory
 
 __all__ = ("fmm", "gauss_fmm_native")
 
 
-def gauss_fmm_native(X1, X2, sigma_dev, out, compute_f64: bool) -> None:
-    """out[n,m] = K(X1, X2) through ``flk_gauss_fmm``.  All tensors on one GPU, 2-D, same dtype."""
+def gauss_fmm_native(X1, X2, sigma_dev, out, compute_f64: bool, kernel_fn: int = _backend.FLK_GAUSSIAN) -> None:
+    """out[n,m] = K(X1, X2) through ``flk_kernel_fmm``.  All tensors on one GPU, 2-D, same dtype."""
     lib = _backend.load()
     code = _DTYPE_CODE[X1.dtype]
     n, d = X1.shape
@@ -34,10 +34,10 @@ def gauss_fmm_native(X1, X2, sigma_dev, out, compute_f64: bool) -> None:
     p2, _, r2, c2 = _mat(X2)
     po, _, ro, co = _mat(out)
     with torch.cuda.device(X1.device):
-        rc = lib.flk_gauss_fmm(p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
-                               po, ro, co, code, int(compute_f64), ws.data_ptr(), ws_bytes,
-                               _stream_handle(X1.device))
-    _backend.raise_for_status(rc, "flk_gauss_fmm")
+        rc = lib.flk_kernel_fmm(kernel_fn, p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
+                                po, ro, co, code, int(compute_f64), ws.data_ptr(), ws_bytes,
+                                _stream_handle(X1.device))
+    _backend.raise_for_status(rc, "flk_kernel_fmm")
 
 
 def fmm(kernel, opt: Optional[BaseOptions], out: Optional[torch.Tensor], diag: bool, X1: torch.Tensor,
@@ -54,7 +54,7 @@ def fmm(kernel, opt: Optional[BaseOptions], out: Optional[torch.Tensor], diag: b
             if out is None:
                 return res.to(X1.device)
             return out.copy_(res.reshape(out.shape))
-        _require_gaussian(kernel)
+        kernel_fn = _kernel_fn(kernel)
         if any(t.requires_grad for t in [X1, X2] + list(kernel.diff_params.values())):
             raise NotImplementedError("falkon_amd.fmm does not implement the autograd backward pass; "
                                       "detach the inputs and the kernel parameters")
@@ -80,7 +80,7 @@ def fmm(kernel, opt: Optional[BaseOptions], out: Optional[torch.Tensor], diag: b
             li = min(blk, N - i)
             X1d = _on(X1[i:i + li], dev)
             outd = out[i:i + li] if out_in else torch.empty((li, M), dtype=out.dtype, device=dev)
-            gauss_fmm_native(X1d, X2d, sigma_dev, outd, compute_f64)
+            gauss_fmm_native(X1d, X2d, sigma_dev, outd, compute_f64, kernel_fn)
             if not out_in:
                 out[i:i + li].copy_(outd)
     return out

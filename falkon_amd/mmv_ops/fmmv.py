@@ -1,4 +1,4 @@
-"""Gaussian kernel-vector products on the MI355X: ``fmmv`` and ``fdmmv``.
+"""Kernel-vector products of the radial kernels (Gaussian, Laplacian, Matern) on the MI355X: ``fmmv`` and ``fdmmv``.
 
 Drop-in for the two callables the reference's kernels dispatch to
 (falkon/mmv_ops/fmmv.py:960-973 ``fmmv`` and :976-1131 ``fdmmv``): same
@@ -33,8 +33,8 @@ def _stream_handle(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
-def gauss_fmmv_native(X1, X2, sigma_dev, v, out) -> None:
-    """out[n,t] = K(X1,X2) @ v through ``flk_gauss_fmmv``.  All tensors on one GPU, 2-D, same dtype."""
+def gauss_fmmv_native(X1, X2, sigma_dev, v, out, kernel_fn: int = _backend.FLK_GAUSSIAN) -> None:
+    """out[n,t] = K(X1,X2) @ v through ``flk_kernel_fmmv``.  All tensors on one GPU, 2-D, same dtype."""
     lib = _backend.load()
     code = _DTYPE_CODE[X1.dtype]
     n, d = X1.shape
@@ -46,13 +46,13 @@ def gauss_fmmv_native(X1, X2, sigma_dev, v, out) -> None:
     pv, _, rv, cv = _mat(v)
     po, _, ro, co = _mat(out)
     with torch.cuda.device(X1.device):
-        rc = lib.flk_gauss_fmmv(p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
-                                pv, rv, cv, t, po, ro, co, code, ws.data_ptr(), ws_bytes, _stream_handle(X1.device))
-    _backend.raise_for_status(rc, "flk_gauss_fmmv")
+        rc = lib.flk_kernel_fmmv(kernel_fn, p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
+                                 pv, rv, cv, t, po, ro, co, code, ws.data_ptr(), ws_bytes, _stream_handle(X1.device))
+    _backend.raise_for_status(rc, "flk_kernel_fmmv")
 
 
-def gauss_fdmmv_native(X1, X2, sigma_dev, v, w, out) -> None:
-    """out[m,t] = K^T (K v + w) through ``flk_gauss_fdmmv``.  ``w`` may be None."""
+def gauss_fdmmv_native(X1, X2, sigma_dev, v, w, out, kernel_fn: int = _backend.FLK_GAUSSIAN) -> None:
+    """out[m,t] = K^T (K v + w) through ``flk_kernel_fdmmv``.  ``w`` may be None."""
     lib = _backend.load()
     code = _DTYPE_CODE[X1.dtype]
     n, d = X1.shape
@@ -65,20 +65,29 @@ def gauss_fdmmv_native(X1, X2, sigma_dev, v, w, out) -> None:
     pw, rw, cw = (w.data_ptr(), w.stride(0), w.stride(1)) if w is not None else (None, 0, 0)
     po, _, ro, co = _mat(out)
     with torch.cuda.device(X1.device):
-        rc = lib.flk_gauss_fdmmv(p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
-                                 pv, rv, cv, pw, rw, cw, t, po, ro, co, code, ws.data_ptr(), ws_bytes,
-                                 _stream_handle(X1.device))
-    _backend.raise_for_status(rc, "flk_gauss_fdmmv")
+        rc = lib.flk_kernel_fdmmv(kernel_fn, p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
+                                  pv, rv, cv, pw, rw, cw, t, po, ro, co, code, ws.data_ptr(), ws_bytes,
+                                  _stream_handle(X1.device))
+    _backend.raise_for_status(rc, "flk_kernel_fdmmv")
 
 
 # ---------------------------------------------------------------------------
 # host-side planning
 # ---------------------------------------------------------------------------
-def _require_gaussian(kernel):
-    if getattr(kernel, "kernel_name", None) != "gaussian" or not hasattr(kernel, "sigma"):
+_KERNEL_FN = {"gaussian": _backend.FLK_GAUSSIAN, "inf-matern": _backend.FLK_GAUSSIAN,
+              "laplacian": _backend.FLK_LAPLACIAN, "0.5-matern": _backend.FLK_LAPLACIAN,
+              "1.5-matern": _backend.FLK_MATERN32, "2.5-matern": _backend.FLK_MATERN52}
+
+
+def _kernel_fn(kernel) -> int:
+    """The library's code for the kernel object's function (by ``kernel_name``, as the reference names its
+    distance kernels, falkon/kernels/distance_kernel.py:382,456,544); other kernels have no MI355X path."""
+    code = _KERNEL_FN.get(getattr(kernel, "kernel_name", None))
+    if code is None or not hasattr(kernel, "sigma"):
         raise NotImplementedError(
-            "falkon_amd accelerates the Gaussian kernel only; "
+            "falkon_amd covers the Gaussian, Laplacian and Matern kernels; "
             f"kernel '{getattr(kernel, 'name', type(kernel).__name__)}' has no MI355X kernel-vector path")
+    return code
 
 
 def _reject_block_kwargs(kwargs_m1, kwargs_m2):
@@ -135,7 +144,7 @@ def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optio
          kwargs_m2: Optional[Dict[str, torch.Tensor]] = None) -> torch.Tensor:
     """``out = K(X1, X2) @ v`` (N x T), same contract as falkon/mmv_ops/fmmv.py:960-973 / :887-932."""
     opt = opt if opt is not None else BaseOptions()
-    _require_gaussian(kernel)
+    kernel_fn = _kernel_fn(kernel)
     _reject_block_kwargs(kwargs_m1, kwargs_m2)
     check_contiguity((X1, "X1"), (X2, "X2"), (v, "v"), (out, "out"))
     if any(t.requires_grad for t in [X1, X2, v] + list(kernel.diff_params.values())):
@@ -165,7 +174,7 @@ def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optio
         if blk == N:
             X1d = _on(X1, dev)
             outd = out if out_in else torch.empty((N, T), dtype=out.dtype, device=dev)
-            gauss_fmmv_native(X1d, X2d, sigma_dev, vd, outd)
+            gauss_fmmv_native(X1d, X2d, sigma_dev, vd, outd, kernel_fn)
             if not out_in:
                 out.copy_(outd)
         else:
@@ -173,7 +182,7 @@ def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optio
                 li = min(blk, N - i)
                 X1d = _on(X1[i:i + li], dev)
                 outd = out[i:i + li] if out_in else torch.empty((li, T), dtype=out.dtype, device=dev)
-                gauss_fmmv_native(X1d, X2d, sigma_dev, vd, outd)
+                gauss_fmmv_native(X1d, X2d, sigma_dev, vd, outd, kernel_fn)
                 if not out_in:
                     out[i:i + li].copy_(outd)
     return out
@@ -191,7 +200,7 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
     if differentiable:
         raise NotImplementedError(
             "Manual D-MMV is not implemented for differentiable inputs. Try using the KeOps version instead.")
-    _require_gaussian(kernel)
+    kernel_fn = _kernel_fn(kernel)
     _reject_block_kwargs(kwargs_m1, kwargs_m2)
     check_contiguity((X1, "X1"), (X2, "X2"), (v, "v"), (out, "out"))
     if v is None:
@@ -222,13 +231,13 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
         X2d, vd = _on(X2, dev), _on(v, dev)
         outd = out if out_in else torch.empty((M, T), dtype=out.dtype, device=dev)
         if blk == N:
-            gauss_fdmmv_native(_on(X1, dev), X2d, sigma_dev, vd, _on(w, dev), outd)
+            gauss_fdmmv_native(_on(X1, dev), X2d, sigma_dev, vd, _on(w, dev), outd, kernel_fn)
         else:
             tmp = torch.empty((M, T), dtype=out.dtype, device=dev)
             for bi, i in enumerate(range(0, N, blk)):
                 li = min(blk, N - i)
                 wd = _on(w[i:i + li], dev) if w is not None else None
-                gauss_fdmmv_native(_on(X1[i:i + li], dev), X2d, sigma_dev, vd, wd, outd if bi == 0 else tmp)
+                gauss_fdmmv_native(_on(X1[i:i + li], dev), X2d, sigma_dev, vd, wd, outd if bi == 0 else tmp, kernel_fn)
                 if bi > 0:
                     outd.add_(tmp)
         if not out_in:

@@ -29,6 +29,15 @@ extern "C" {
 #define FLK_F32 0
 #define FLK_F64 1
 
+/* Radial kernels K(x, c) = f(D), D = |x/sigma - c/sigma| (falkon/kernels/distance_kernel.py):
+ * Gaussian exp(-D^2/2) (:140-159), Laplacian exp(-D) (:182-205), Matern nu = 3/2 and 5/2 (:225-269;
+ * nu = 1/2 is the Laplacian, nu = inf the Gaussian, :235-238).  The flk_gauss_* entry points are the
+ * flk_kernel_* ones with FLK_GAUSSIAN. */
+#define FLK_GAUSSIAN  0
+#define FLK_LAPLACIAN 1
+#define FLK_MATERN32  2
+#define FLK_MATERN52  3
+
 #define FLK_OK          0
 #define FLK_EINVAL     -1   /* bad argument (shape, stride, dtype, null pointer)      */
 #define FLK_ENOMEM     -2   /* workspace too small                                    */
@@ -136,6 +145,44 @@ int flk_gauss_fmm(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
                   const void *sigma, int64_t n_sigma,
                   void *out, int64_t out_rs, int64_t out_cs, int dtype, int compute_f64,
                   void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- the same entry points for any of the radial kernels ----------------------
+ * `kernel` is one of FLK_GAUSSIAN / FLK_LAPLACIAN / FLK_MATERN32 / FLK_MATERN52; everything else as in
+ * the flk_gauss_* function of the same name, whose *_workspace_bytes / flk_gauss_packed_bytes sizes
+ * apply to every kernel.  Packed operands are specific to the kernel they were packed for (the
+ * Gaussian rows carry an extra factor).  These replace fmmv / fdmmv / fmm for the reference's
+ * LaplacianKernel and MaternKernel (falkon/kernels/distance_kernel.py:434-648).
+ */
+int flk_kernel_pack(int kernel, const void *X, int64_t n, int64_t d, int64_t x_rs, int64_t x_cs,
+                    const void *sigma, int64_t n_sigma, int dtype,
+                    void *packed, size_t packed_bytes, void *stream);
+
+int flk_kernel_mmv_packed(int kernel, const void *packed_a, int64_t n_a, const void *packed_b, int64_t n_b, int64_t d,
+                          const void *vec, int64_t vec_rs, int64_t vec_cs, int64_t t,
+                          const void *addend, int64_t add_rs, int64_t add_cs,
+                          void *out, int64_t out_rs, int64_t out_cs, int dtype,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+int flk_kernel_fmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
+                    const void *X2, int64_t m, int64_t x2_rs, int64_t x2_cs, int64_t d,
+                    const void *sigma, int64_t n_sigma,
+                    const void *v, int64_t v_rs, int64_t v_cs, int64_t t,
+                    void *out, int64_t out_rs, int64_t out_cs, int dtype,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+int flk_kernel_fdmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
+                     const void *X2, int64_t m, int64_t x2_rs, int64_t x2_cs, int64_t d,
+                     const void *sigma, int64_t n_sigma,
+                     const void *v, int64_t v_rs, int64_t v_cs,
+                     const void *w, int64_t w_rs, int64_t w_cs, int64_t t,
+                     void *out, int64_t out_rs, int64_t out_cs, int dtype,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
+int flk_kernel_fmm(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
+                   const void *X2, int64_t m, int64_t x2_rs, int64_t x2_cs, int64_t d,
+                   const void *sigma, int64_t n_sigma,
+                   void *out, int64_t out_rs, int64_t out_cs, int dtype, int compute_f64,
+                   void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

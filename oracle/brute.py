@@ -31,6 +31,32 @@ def gaussian_brute(X, C, sigma) -> np.ndarray:
     return K
 
 
+def radial_brute(X, C, sigma, kernel_name: str) -> np.ndarray:
+    """K[n,m] in float64 from the distances in difference form, for the closed forms the reference documents:
+    "gaussian" exp(-D^2/2); "laplacian" exp(-D) (falkon/kernels/distance_kernel.py:449-453); "1.5-matern"
+    (1 + sqrt(3) D) exp(-sqrt(3) D) and "2.5-matern" (1 + sqrt(5) D + 5/3 D^2) exp(-sqrt(5) D) (:243-267;
+    the naive oracles of the reference's tests, falkon/tests/naive_kernels.py:28-31,48-61)."""
+    X = np.asarray(X.detach().cpu().numpy() if isinstance(X, torch.Tensor) else X, dtype=np.float64)
+    C = np.asarray(C.detach().cpu().numpy() if isinstance(C, torch.Tensor) else C, dtype=np.float64)
+    s = _sigma_vec(sigma, X.shape[1])
+    Xs, Cs = X / s, C / s
+    D2 = np.empty((X.shape[0], C.shape[0]), dtype=np.float64)
+    step = max(1, int(2**24 // max(1, C.shape[0] * X.shape[1])))
+    for i in range(0, X.shape[0], step):
+        diff = Xs[i:i + step, None, :] - Cs[None, :, :]
+        D2[i:i + step] = np.einsum("nmd,nmd->nm", diff, diff)
+    D = np.sqrt(D2)
+    if kernel_name in ("gaussian", "inf-matern"):
+        return np.exp(-0.5 * D2)
+    if kernel_name in ("laplacian", "0.5-matern"):
+        return np.exp(-D)
+    if kernel_name == "1.5-matern":
+        return (1 + np.sqrt(3) * D) * np.exp(-np.sqrt(3) * D)
+    if kernel_name == "2.5-matern":
+        return (1 + np.sqrt(5) * D + 5.0 / 3.0 * D2) * np.exp(-np.sqrt(5) * D)
+    raise ValueError(kernel_name)
+
+
 def mmv_brute(X, C, sigma, v) -> np.ndarray:
     v = np.asarray(v.detach().cpu().numpy() if isinstance(v, torch.Tensor) else v, dtype=np.float64)
     return gaussian_brute(X, C, sigma) @ v.reshape(C.shape[0], -1)

@@ -1,4 +1,4 @@
-"""Per-block Gaussian kernel arithmetic of the reference, restated in torch CPU ops.
+"""Per-block arithmetic of the reference's distance kernels (Gaussian, Laplacian, Matern), restated in torch CPU ops.
 
 Test infrastructure only (see ``oracle/__init__.py``).
 """
@@ -69,3 +69,59 @@ def rbf_core_ref(mat1: torch.Tensor, mat2: torch.Tensor, out: Optional[torch.Ten
     out.mul_(-0.5)
     out.exp_()
     return out
+
+
+def laplacian_core_ref(mat1: torch.Tensor, mat2: torch.Tensor, out: Optional[torch.Tensor], sigma: torch.Tensor) -> torch.Tensor:
+    """Follows falkon/kernels/distance_kernel.py:182-205 (``diag=False``): the clamped squared distance of the
+    scaled operands (expanded norm), then ``sqrt_``, negate, ``exp_``."""
+    sigma = sigma.to(device=mat1.device, dtype=mat1.dtype)
+    mat1_div_sig = mat1 / sigma
+    mat2_div_sig = mat2 / sigma
+    out = sq_dist_ref(mat1_div_sig, mat2_div_sig, square_norm_ref(mat1_div_sig), square_norm_ref(mat2_div_sig), out)
+    out.sqrt_()
+    out.neg_()
+    out.exp_()
+    return out
+
+
+def matern_core_ref(mat1: torch.Tensor, mat2: torch.Tensor, out: Optional[torch.Tensor], sigma: torch.Tensor,
+                    nu: float) -> torch.Tensor:
+    """Follows falkon/kernels/distance_kernel.py:225-269 (``diag=False``): nu = 0.5 and inf delegate to the
+    Laplacian and Gaussian cores; 1.5: ``D*sqrt(3)``, ``exp(-.)`` on a copy, ``(. + 1) * exp``; 2.5:
+    ``sqrt(D2)*sqrt(5)`` on a copy, ``D2 * 5/3 + . + 1``, times ``exp(-.)``."""
+    if nu == 0.5:
+        return laplacian_core_ref(mat1, mat2, out, sigma)
+    if nu == float("inf"):
+        return rbf_core_ref(mat1, mat2, out, sigma)
+    sigma = sigma.to(device=mat1.device, dtype=mat1.dtype)
+    mat1_div_sig = mat1 / sigma
+    mat2_div_sig = mat2 / sigma
+    out = sq_dist_ref(mat1_div_sig, mat2_div_sig, square_norm_ref(mat1_div_sig), square_norm_ref(mat2_div_sig), out)
+    if nu == 1.5:
+        out.sqrt_()
+        out.mul_(3.0 ** 0.5)
+        out_neg = torch.neg(out)
+        out_neg.exp_()
+        out.add_(1.0).mul_(out_neg)
+    elif nu == 2.5:
+        out_sqrt = torch.sqrt(out)
+        out_sqrt.mul_(5.0 ** 0.5)
+        out.mul_(5.0 / 3.0).add_(out_sqrt).add_(1.0)
+        out_sqrt.neg_().exp_()
+        out.mul_(out_sqrt)
+    else:
+        raise ValueError(f"nu = {nu} has no closed form")
+    return out
+
+
+def core_ref_for(kernel_name: str):
+    """The per-block function for a kernel name as the reference spells it ("gaussian", "laplacian",
+    "1.5-matern", ...), with the signature of ``rbf_core_ref``."""
+    if kernel_name == "gaussian":
+        return rbf_core_ref
+    if kernel_name == "laplacian":
+        return laplacian_core_ref
+    if kernel_name.endswith("-matern"):
+        nu = float(kernel_name.split("-")[0])
+        return lambda mat1, mat2, out, sigma: matern_core_ref(mat1, mat2, out, sigma, nu)
+    raise ValueError(kernel_name)

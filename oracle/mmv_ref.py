@@ -11,7 +11,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .gaussian_ref import rbf_core_ref, validate_sigma_ref
+from .gaussian_ref import core_ref_for, rbf_core_ref, validate_sigma_ref
 
 # falkon/mmv_ops/utils.py:44 -- head-room the reference reserves for addmm work buffers
 EXTRA_MM_RAM_BYTES = 8519680
@@ -169,7 +169,8 @@ def _check_inputs(X1, X2, v, w, out, out_rows):
     return v, w
 
 
-def fmmv_ref(X1, X2, v, sigma, out: Optional[torch.Tensor] = None, max_cpu_mem: float = float("inf")) -> torch.Tensor:
+def fmmv_ref(X1, X2, v, sigma, out: Optional[torch.Tensor] = None, max_cpu_mem: float = float("inf"),
+             kernel_name: str = "gaussian") -> torch.Tensor:
     """out[N,T] = K(X1,X2) @ v, blocked over rows of X1 and of X2.
 
     Follows falkon/mmv_ops/fmmv.py:887-932 (output creation), :117-185 (block
@@ -178,6 +179,7 @@ def fmmv_ref(X1, X2, v, sigma, out: Optional[torch.Tensor] = None, max_cpu_mem: 
     ``out_i.addmm_(K, v_j)``).
     """
     sigma = validate_sigma_ref(sigma)
+    core = core_ref_for(kernel_name)        # the kernel's per-block function (the block loop is shared)
     v, _ = _check_inputs(X1, X2, v, None, out, X1.shape[0])
     N, D = X1.shape
     M, T = v.shape
@@ -196,12 +198,13 @@ def fmmv_ref(X1, X2, v, sigma, out: Optional[torch.Tensor] = None, max_cpu_mem: 
             for j in range(0, M, blk_m):
                 lj = min(blk_m, M - j)
                 k_ij = ker_buf[:li, :lj].fill_(0.0)
-                k_ij = rbf_core_ref(x_i, X2[j:j + lj, :], k_ij, sigma)
+                k_ij = core(x_i, X2[j:j + lj, :], k_ij, sigma)
                 o_i.addmm_(k_ij, v[j:j + lj, :])
     return out
 
 
-def fdmmv_ref(X1, X2, v, w, sigma, out: Optional[torch.Tensor] = None, max_cpu_mem: float = float("inf")) -> torch.Tensor:
+def fdmmv_ref(X1, X2, v, w, sigma, out: Optional[torch.Tensor] = None, max_cpu_mem: float = float("inf"),
+              kernel_name: str = "gaussian") -> torch.Tensor:
     """out[M,T] = K(X1,X2).T @ (K(X1,X2) @ v + w), blocked over rows of X1.
 
     Follows falkon/mmv_ops/fmmv.py:1033-1061 (checks, output creation, CPU
@@ -211,6 +214,7 @@ def fdmmv_ref(X1, X2, v, w, sigma, out: Optional[torch.Tensor] = None, max_cpu_m
     reference reads ``v.shape`` unconditionally, fmmv.py:1041).
     """
     sigma = validate_sigma_ref(sigma)
+    core = core_ref_for(kernel_name)
     v, w = _check_inputs(X1, X2, v, w, out, X2.shape[0])
     N, D = X1.shape
     M, T = v.shape
@@ -231,7 +235,7 @@ def fdmmv_ref(X1, X2, v, w, sigma, out: Optional[torch.Tensor] = None, max_cpu_m
             else:
                 u_i = u_buf[:li, :].fill_(0.0)
             k_i = ker_buf[:li, :].fill_(0.0)
-            k_i = rbf_core_ref(x_i, X2, k_i, sigma)
+            k_i = core(x_i, X2, k_i, sigma)
             u_i.addmm_(k_i, v)
             out.addmm_(k_i.T, u_i)
     return out

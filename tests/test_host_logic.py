@@ -177,3 +177,41 @@ def test_bench_refuses_more_than_one_gpu_and_builds_seeded_inputs():
     assert X.dtype == torch.float32 and float(sigma) == 3.8
     assert torch.equal(X, X2) and torch.equal(C, C2) and torch.equal(v, v2) and torch.equal(w, w2)
     assert all(bool((C[i] == X).all(1).any()) for i in range(5))        # centres are rows of X
+
+
+def test_laplacian_and_matern_kernel_objects():
+    """Names, parameter handling and errors of the other distance kernels
+    (falkon/kernels/distance_kernel.py:435-507,510-648)."""
+    from falkon_amd import LaplacianKernel, MaternKernel
+    from falkon_amd.mmv_ops.fmmv import _kernel_fn
+    lap = LaplacianKernel(2.0)
+    assert lap.kernel_name == "laplacian" and lap.name == "laplacian" and _kernel_fn(lap) == _backend.FLK_LAPLACIAN
+    assert lap.sigma.dtype == torch.float64 and "sigma" in lap.diff_params and lap.nondiff_params == {"nu": 0.5}
+    names = {0.5: ("0.5-matern", _backend.FLK_LAPLACIAN), 1.5: ("1.5-matern", _backend.FLK_MATERN32),
+             2.5: ("2.5-matern", _backend.FLK_MATERN52), float("inf"): ("inf-matern", _backend.FLK_GAUSSIAN)}
+    for nu, (name, code) in names.items():
+        k = MaternKernel(torch.tensor([1.0, 2.0]), nu)
+        assert k.kernel_name == name and _kernel_fn(k) == code and k.nondiff_params["nu"] == nu
+        assert k.detach().kernel_name == name and repr(k).startswith("MaternKernel(")
+    assert MaternKernel(1.0, torch.tensor(1.5)).nondiff_params["nu"] == 1.5
+    assert MaternKernel(1.0, 2.4999).nondiff_params["nu"] == 2.5            # rounded to two digits
+    with pytest.raises(ValueError):
+        MaternKernel(1.0, 2.0)
+    with pytest.raises(TypeError):
+        MaternKernel(1.0, 2)
+    with pytest.raises(ValueError):
+        MaternKernel(1.0, torch.tensor(1.5, requires_grad=True))
+    # the stock-torch block of every kernel agrees with the oracle's restatement of the reference core
+    from oracle import gaussian_ref
+    g = np.random.default_rng(0)
+    X, C = torch.from_numpy(g.standard_normal((9, 4))), torch.from_numpy(g.standard_normal((6, 4)))
+    for k in (lap, MaternKernel(2.0, 0.5), MaternKernel(2.0, 1.5), MaternKernel(2.0, 2.5), MaternKernel(2.0, float("inf")),
+              GaussianKernel(2.0)):
+        got = k.compute(X, C, torch.empty(9, 6, dtype=torch.float64), diag=False)
+        torch.testing.assert_close(got, gaussian_ref.core_ref_for(k.kernel_name)(X, C, None, k.sigma), rtol=1e-12, atol=1e-14)
+        assert float((k.compute(X, X, None, diag=True) - 1).abs().max()) < 1e-12
+
+    class Other:
+        kernel_name = "polynomial"
+    with pytest.raises(NotImplementedError):
+        _kernel_fn(Other())

@@ -185,3 +185,88 @@ def test_config_generators_are_seeded():
     assert X.shape == (300, 784) and v.shape == (20, 10) and 0.1 < float((X != 0).float().mean()) < 0.3
     X, C, sigma, v, w = inputs.make_config("C1", N=500, M=20)
     assert X.dtype == torch.float64 and w is None
+
+
+# --------------------------------------------------------------------------------------------------
+# Laplacian and Matern cores (falkon/kernels/distance_kernel.py:182-269)
+# --------------------------------------------------------------------------------------------------
+KERNEL_NAMES = ("laplacian", "0.5-matern", "1.5-matern", "2.5-matern", "inf-matern")
+
+
+def _cdist_radial(X, C, sigma, name):
+    """The reference's naive oracles (falkon/tests/naive_kernels.py:28-31,48-61) on torch.cdist distances."""
+    s = sigma.to(X.dtype)
+    D = torch.cdist(X / s, C / s, compute_mode="donot_use_mm_for_euclid_dist")
+    if name in ("laplacian", "0.5-matern"):
+        return torch.exp(-D)
+    if name == "1.5-matern":
+        return (1.0 + D * 3 ** 0.5) * torch.exp(-D * 3 ** 0.5)
+    if name == "2.5-matern":
+        S = D * 5 ** 0.5
+        return (1.0 + S + S ** 2 / 3.0) * torch.exp(-S)
+    return torch.exp(-D ** 2 / 2.0)
+
+
+@pytest.mark.parametrize("name", KERNEL_NAMES)
+@pytest.mark.parametrize("sigma", [torch.tensor([3.0]), torch.tensor([0.7, 2.0, 5.0])])
+def test_radial_cores_reference_fixture(name, sigma):
+    """The reference's kernel-test shape (n=20 m=5 d=3 fp64, seeds 92/93, falkon/tests/test_kernels.py:32-35,75-89)
+    against the closed forms in difference form (numpy) and on torch.cdist, rtol = atol = 1e-8."""
+    A, B, _, _ = inputs.reference_test_mats(20, 5, 3, 2, np.float64, "C")
+    core = gaussian_ref.core_ref_for(name)
+    K = core(A, B, None, sigma)
+    np.testing.assert_allclose(K.numpy(), brute.radial_brute(A, B, sigma, name), rtol=1e-8, atol=1e-8)
+    torch.testing.assert_close(K, _cdist_radial(A, B, sigma, name), rtol=1e-8, atol=1e-8)
+    out = torch.empty(20, 5, dtype=torch.float64)
+    assert core(A, B, out, sigma).data_ptr() == out.data_ptr()
+    torch.testing.assert_close(out, K, rtol=0, atol=0)
+
+
+def test_radial_cores_special_cases():
+    g = np.random.default_rng(4)
+    X = torch.from_numpy(g.standard_normal((30, 6)))
+    C = torch.from_numpy(g.standard_normal((12, 6)))
+    sig = torch.tensor([1.7], dtype=torch.float64)
+    lap = gaussian_ref.laplacian_core_ref(X, C, None, sig)
+    # nu = 1/2 is the Laplacian and nu = inf the Gaussian (falkon/kernels/distance_kernel.py:235-238)
+    torch.testing.assert_close(gaussian_ref.matern_core_ref(X, C, None, sig, 0.5), lap, rtol=0, atol=0)
+    torch.testing.assert_close(gaussian_ref.matern_core_ref(X, C, None, sig, float("inf")),
+                               gaussian_ref.rbf_core_ref(X, C, None, sig), rtol=0, atol=0)
+    # textbook form of the Laplacian on a single pair
+    d01 = float(((X[0] - C[1]) / 1.7).norm())
+    assert abs(float(lap[0, 1]) - np.exp(-d01)) < 1e-12
+    for nu in (0.5, 1.5, 2.5):
+        K = gaussian_ref.matern_core_ref(X, C, None, sig, nu)
+        assert float(K.max()) <= 1.0 and float(K.min()) > 0.0
+        # coincident points: K = 1 up to the clamp of the squared distance at 1e-20 and the sqrt of rounding noise
+        Kxx = gaussian_ref.matern_core_ref(X, X, None, sig, nu)
+        assert float((Kxx.diagonal() - 1).abs().max()) < 1e-6
+        # smoother kernels decay more slowly near zero distance: at small D, 1 - K ~ D, D^2 * 3/2 ... ordering at D -> 0
+    near = X[:1] + 1e-3
+    k05, k15, k25 = (float(gaussian_ref.matern_core_ref(X[:1], near, None, sig, nu)) for nu in (0.5, 1.5, 2.5))
+    assert k05 < k15 < k25 < 1.0
+    # per-dimension lengthscales are a rescaling of the inputs
+    per_dim = torch.tensor([0.5, 1.0, 1.5, 2.0, 2.5, 3.0], dtype=torch.float64)
+    one = torch.tensor([1.0])
+    for name in KERNEL_NAMES:
+        core = gaussian_ref.core_ref_for(name)
+        torch.testing.assert_close(core(X, C, None, per_dim), core(X / per_dim, C / per_dim, None, one),
+                                   rtol=1e-12, atol=1e-14)
+    with pytest.raises(ValueError):
+        gaussian_ref.matern_core_ref(X, C, None, sig, 3.5)
+
+
+@pytest.mark.parametrize("name", KERNEL_NAMES)
+def test_radial_products_against_brute(name):
+    """fmmv / fdmmv of the block loops with another kernel's core against K from the closed form."""
+    g = np.random.default_rng(9)
+    X = torch.from_numpy(g.standard_normal((150, 7)))
+    C = torch.from_numpy(g.standard_normal((40, 7)))
+    v = torch.from_numpy(g.standard_normal((40, 3)))
+    w = torch.from_numpy(g.standard_normal((150, 3)))
+    sig = torch.tensor([2.2], dtype=torch.float64)
+    K = brute.radial_brute(X, C, sig, name)
+    np.testing.assert_allclose(mmv_ref.fmmv_ref(X, C, v, sig, kernel_name=name, max_cpu_mem=2**24).numpy(),
+                               K @ v.numpy(), rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(mmv_ref.fdmmv_ref(X, C, v, w, sig, kernel_name=name, max_cpu_mem=2**24).numpy(),
+                               K.T @ (K @ v.numpy() + w.numpy()), rtol=1e-10, atol=1e-12)
