@@ -88,11 +88,13 @@ def falkon_predict_ref(X: torch.Tensor, centers: torch.Tensor, alpha: torch.Tens
     return fmmv_ref(X, centers, alpha, validate_sigma_ref(sigma), max_cpu_mem=max_cpu_mem)
 
 
-def nystrom_krr_direct(X, Y, centers, sigma, penalty) -> np.ndarray:
+def nystrom_krr_direct(X, Y, centers, sigma, penalty, kernel_name: str = "gaussian") -> np.ndarray:
     """The linear system Falkon solves, in closed form and fp64:
     alpha = (K_nm^T K_nm + lambda n K_mm)^-1 K_nm^T y  (falkon/tests/test_conjgrad.py:100-118)."""
+    from .gaussian_ref import core_ref_for
     s = validate_sigma_ref(sigma)
-    Knm = rbf_core_ref(X.double(), centers.double(), None, s).numpy()
-    Kmm = rbf_core_ref(centers.double(), centers.double(), None, s).numpy()
+    core = core_ref_for(kernel_name)
+    Knm = core(X.double(), centers.double(), None, s).numpy()
+    Kmm = core(centers.double(), centers.double(), None, s).numpy()
     Yn = Y.double().numpy().reshape(X.shape[0], -1)
     return np.linalg.solve(Knm.T @ Knm + penalty * X.shape[0] * Kmm, Knm.T @ Yn)

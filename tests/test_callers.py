@@ -179,6 +179,25 @@ def test_falkon_cg_matches_direct_solve_on_gpu(dev):
     np.testing.assert_allclose(model.alpha_.cpu().numpy(), falkon_ref.nystrom_krr_direct(X, Y10, C, sigma, lam), rtol=1e-5)
 
 
+@pytest.mark.gpu
+def test_falkon_with_matern_and_laplacian_kernels_on_gpu(dev):
+    """The same conjugate-gradient test with the other distance kernels: preconditioner (kernel matrix), CG
+    (dfmmv) and prediction (fmmv) all run the kernel's own function."""
+    from falkon_amd import LaplacianKernel, MaternKernel
+    X, Y, C, sigma, lam = _conjgrad_problem()
+    for kernel, name in ((LaplacianKernel(sigma), "laplacian"), (MaternKernel(sigma, 1.5), "1.5-matern"),
+                         (MaternKernel(sigma, 2.5), "2.5-matern")):
+        model = Falkon(kernel, lam, M=10, center_selection=FixedSelector(C), maxiter=200,
+                       options=FalkonOptions(cg_tolerance=1e-10))
+        model.fit(X.to(dev), Y.to(dev))
+        expected = falkon_ref.nystrom_krr_direct(X, Y, C, sigma, lam, kernel_name=name)
+        np.testing.assert_allclose(model.alpha_.cpu().numpy(), expected, rtol=1e-5)
+        pred = model.predict(X[:50].to(dev)).cpu()
+        from oracle import brute
+        np.testing.assert_allclose(pred.numpy(), brute.radial_brute(X[:50], C, torch.tensor([sigma]), name) @ expected,
+                                   rtol=1e-5, atol=1e-8)
+
+
 def _config5(N, Nts, seed=1005, d=28):
     rng = np.random.default_rng(seed)
     X = rng.standard_normal((N, d)).astype(np.float32)
