@@ -69,14 +69,15 @@ def make_inputs(name):
             torch.from_numpy(w) if w is not None else None)
 
 
-def cpu_baseline(X, C, sigma, v, w, gpu_out_fn, rows):
+def cpu_baseline(X, C, sigma, v, w, gpu_out_fn, rows, kernel_name="gaussian"):
     """Reference-equivalent CPU path (the oracle restatement, torch CPU ops) on the first `rows` rows."""
     from oracle import mmv_ref                      # checker only; never on the product path
     Xs = X[:rows].contiguous()
     ws = w[:rows].contiguous() if w is not None else None
-    mmv_ref.fdmmv_ref(Xs[:2000], C, v, ws[:2000] if ws is not None else None, sigma, max_cpu_mem=4 * 2**30)  # warm-up
+    mmv_ref.fdmmv_ref(Xs[:2000], C, v, ws[:2000] if ws is not None else None, sigma, max_cpu_mem=4 * 2**30,
+                      kernel_name=kernel_name)                                                       # warm-up
     t0 = time.perf_counter()
-    exp = mmv_ref.fdmmv_ref(Xs, C, v, ws, sigma, max_cpu_mem=4 * 2**30)
+    exp = mmv_ref.fdmmv_ref(Xs, C, v, ws, sigma, max_cpu_mem=4 * 2**30, kernel_name=kernel_name)
     dt = time.perf_counter() - t0
     got, got64 = gpu_out_fn(Xs, ws)
     got, got64, exp = got.double().cpu(), got64.double().cpu(), exp.double()
@@ -194,6 +195,9 @@ def main():
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"], help="arithmetic type (the headline is f32)")
     ap.add_argument("--op", default="dmmv", choices=["dmmv", "mmv"],
                     help="dmmv = K^T(Kv+w), the headline; mmv = K v only (one launch per step)")
+    ap.add_argument("--kernel", default="gaussian", choices=["gaussian", "laplacian", "matern32", "matern52"],
+                    help="kernel function (the headline is the Gaussian; the flop count of the roofline stays the "
+                         "Gaussian's 2d+4+2T per pair, the other kernels spend a few more VALU operations per entry)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=0)
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
@@ -218,8 +222,11 @@ def main():
         print(json.dumps({"copy_calibration_bytes": src.numel() * 4, "copies": 5}))
         return
 
-    from falkon_amd import GaussianKernel, _backend
+    from falkon_amd import GaussianKernel, LaplacianKernel, MaternKernel, _backend
     lib = _backend.load()                            # raises if the HIP library is missing
+    make_kernel, kernel_name = {"gaussian": (GaussianKernel, "gaussian"), "laplacian": (LaplacianKernel, "laplacian"),
+                                "matern32": (lambda s: MaternKernel(s, 1.5), "1.5-matern"),
+                                "matern52": (lambda s: MaternKernel(s, 2.5), "2.5-matern")}[args.kernel]
     if args.workload == "C5":
         print(json.dumps(run_c5(args, lib)), flush=True)
         return
@@ -232,7 +239,7 @@ def main():
     peak = FP32_PEAK_TFLOPS if args.dtype == "f32" else FP64_PEAK_TFLOPS
     Xg, Cg, vg = X.to(dev), C.to(dev), v.to(dev)
     wg = w.to(dev) if w is not None else None
-    kernel = GaussianKernel(sigma)
+    kernel = make_kernel(sigma)
     out = torch.empty(M if args.op == "dmmv" else N, T, dtype=tdt, device=dev)
 
     def step():
@@ -266,7 +273,7 @@ def main():
         "value": value, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": f"{args.workload}: Gaussian {'dfmmv K^T(Kv+w)' if args.op == 'dmmv' else 'fmmv K v'}, N={N}, d={d}, M={M}, T={T}, "
+        "config": {"workload": f"{args.workload}: {kernel_name} {'dfmmv K^T(Kv+w)' if args.op == 'dmmv' else 'fmmv K v'}, N={N}, d={d}, M={M}, T={T}, "
                                f"{ {'C2': 'sigma=3.8', 'C3': 'per-dimension sigma', 'C4': 'sigma=10'}[args.workload] }, "
                                f"{'fp32' if args.dtype == 'f32' else 'fp64'}, "
                                f"inputs resident in HBM, packing included in every step"},
@@ -290,7 +297,7 @@ def main():
                                                                wd.double() if wd is not None else None)
             return r32, r64
 
-        res["cpu_baseline"] = cpu_baseline(X, C, sigma, v, w, gpu_on, rows)
+        res["cpu_baseline"] = cpu_baseline(X, C, sigma, v, w, gpu_on, rows, kernel_name)
     print(json.dumps(res), flush=True)
 
 
