@@ -128,6 +128,94 @@ def _rows_that_fit(n: int, bytes_for_rows, usable: float) -> int:
     return lo
 
 
+# ---------------------------------------------------------------------------
+# host-resident rows: upload overlapped with compute
+# ---------------------------------------------------------------------------
+_STREAM_MIN_BYTES = 32 << 20      # smaller host operands are uploaded in one piece
+_STREAM_PIECES = 4                # pieces a host operand that fits is cut into
+
+
+class _HostRowStream:
+    """Row chunks of host tensors on their way to the GPU, two chunks in flight.
+
+    The reference's CPU-data / GPU-compute mode copies a row block, computes on it, copies the next
+    (falkon/mmv_ops/fmmv.py:730-767).  Here the copies run on a stream of their own (default priority):
+    while the kernels of chunk k run, chunk k+1 crosses PCIe and the host stages chunk k+2 into pinned
+    memory (pageable sources only; pinned sources are copied from where they are).  Each slot's device
+    buffer is reused only after the kernels that read it have finished (event recorded by the consumer),
+    each pinned buffer only after its upload has finished.
+    """
+
+    def __init__(self, tensors, n_rows: int, dev: torch.device, chunk_rows: int):
+        self.tensors, self.n_rows, self.dev, self.chunk = list(tensors), n_rows, dev, chunk_rows
+        self.copy_stream = torch.cuda.Stream(dev)
+        on_host = [t is not None and t.device.type == "cpu" for t in self.tensors]
+        self.dev_bufs = [[self._like(t, dev, False) if h else None for t, h in zip(self.tensors, on_host)]
+                         for _ in range(2)]
+        self.pin_bufs = [[self._like(t, None, True) if h and not t.is_pinned() else None
+                          for t, h in zip(self.tensors, on_host)] for _ in range(2)]
+        self.uploaded = [None, None]
+        self.consumed = [None, None]
+
+    def _like(self, t: torch.Tensor, dev, pinned: bool) -> torch.Tensor:
+        """A chunk-sized buffer in the memory order of ``t`` (rows of an F-ordered matrix stay F-ordered)."""
+        shape = (self.chunk, t.shape[1])
+        f_order = t.shape[1] > 1 and t.stride(0) == 1
+        strides = (1, self.chunk) if f_order else (t.shape[1], 1)
+        if pinned:
+            return torch.empty_strided(shape, strides, dtype=t.dtype, pin_memory=True)
+        return torch.empty_strided(shape, strides, dtype=t.dtype, device=dev)
+
+    def _issue(self, k: int):
+        slot, i = k & 1, k * self.chunk
+        li = min(self.chunk, self.n_rows - i)
+        if self.uploaded[slot] is not None:
+            self.uploaded[slot].synchronize()                 # the pinned buffer of this slot is free again
+        chunk = []
+        with torch.cuda.stream(self.copy_stream):
+            if self.consumed[slot] is not None:
+                self.copy_stream.wait_event(self.consumed[slot])   # the device buffer of this slot is free again
+            for t, dbuf, pbuf in zip(self.tensors, self.dev_bufs[slot], self.pin_bufs[slot]):
+                if t is None or dbuf is None:                 # absent, or already on the GPU: just the rows
+                    chunk.append(None if t is None else t[i:i + li])
+                    continue
+                src = t[i:i + li]
+                if pbuf is not None:
+                    pbuf[:li].copy_(src)
+                    src = pbuf[:li]
+                dbuf[:li].copy_(src, non_blocking=True)
+                chunk.append(dbuf[:li])
+            done = torch.cuda.Event()
+            done.record(self.copy_stream)
+        self.uploaded[slot] = done
+        return i, li, chunk, done
+
+    def __iter__(self):
+        """Yields (first row, rows, [device views]); the consumer enqueues its kernels on the current stream
+        before asking for the next chunk, whose staging and upload then overlap those kernels."""
+        n_chunks = (self.n_rows + self.chunk - 1) // self.chunk
+        compute = torch.cuda.current_stream(self.dev)
+        ahead = self._issue(0) if n_chunks else None
+        for k in range(n_chunks):
+            i, li, chunk, done = ahead
+            compute.wait_event(done)
+            yield i, li, chunk
+            used = torch.cuda.Event()
+            used.record(compute)
+            self.consumed[k & 1] = used
+            ahead = self._issue(k + 1) if k + 1 < n_chunks else None
+
+
+def _streamed_chunk_rows(n: int, row_bytes: int, rows_that_fit: int) -> int:
+    """Rows per chunk for a host operand of n rows: what fits, and no more than a quarter of the operand
+    (so that upload and compute overlap) once the operand is big enough for that to matter."""
+    if n * row_bytes < _STREAM_MIN_BYTES:
+        return rows_that_fit
+    piece = -(-n // _STREAM_PIECES)
+    piece = -(-piece // 1024) * 1024
+    return max(1, min(rows_that_fit, piece))
+
+
 def _on(t: Optional[torch.Tensor], dev: torch.device) -> Optional[torch.Tensor]:
     if t is None or t.device == dev:
         return t
@@ -166,25 +254,28 @@ def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optio
         fixed = (0 if X2.device == dev else M * D * sz) + (0 if v.device == dev else M * T * sz)
 
         def need(rows: int) -> float:
-            stage = (0 if x1_in else rows * D * sz) + (0 if out_in else rows * T * sz)
-            return lib.flk_gauss_fmmv_workspace_bytes(rows, M, D, T, code) + stage + fixed
+            stage = 0 if x1_in else 2 * rows * D * sz                                    # two chunks in flight
+            result = 0 if out_in else (rows if x1_in else N) * T * sz                    # see below
+            return lib.flk_gauss_fmmv_workspace_bytes(rows, M, D, T, code) + stage + result + fixed
 
         blk = _rows_that_fit(N, need, usable) if N > 0 else 0
         X2d, vd = _on(X2, dev), _on(v, dev)
-        if blk == N:
-            X1d = _on(X1, dev)
-            outd = out if out_in else torch.empty((N, T), dtype=out.dtype, device=dev)
-            gauss_fmmv_native(X1d, X2d, sigma_dev, vd, outd, kernel_fn)
-            if not out_in:
-                out.copy_(outd)
-        else:
-            for i in range(0, N, blk):
+        if x1_in:
+            for i in range(0, N, max(blk, 1)):
                 li = min(blk, N - i)
-                X1d = _on(X1[i:i + li], dev)
                 outd = out[i:i + li] if out_in else torch.empty((li, T), dtype=out.dtype, device=dev)
-                gauss_fmmv_native(X1d, X2d, sigma_dev, vd, outd, kernel_fn)
+                gauss_fmmv_native(X1[i:i + li], X2d, sigma_dev, vd, outd, kernel_fn)
                 if not out_in:
                     out[i:i + li].copy_(outd)
+        elif N > 0:
+            # host rows stream through; their results wait on the device and leave in one copy at the end
+            # (a copy per chunk would stall the host, and with it the staging of the next chunk)
+            chunk = _streamed_chunk_rows(N, D * sz, blk)
+            full = out if out_in else torch.empty((N, T), dtype=out.dtype, device=dev)
+            for i, li, (X1d,) in _HostRowStream([X1], N, dev, chunk):
+                gauss_fmmv_native(X1d, X2d, sigma_dev, vd, full[i:i + li], kernel_fn)
+            if not out_in:
+                out.copy_(full)
     return out
 
 
@@ -223,23 +314,33 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
                  + (0 if out_in else M * T * sz))
 
         def need(rows: int) -> float:
-            stage = (0 if x1_in else rows * D * sz) + (0 if w_in else rows * T * sz)
+            stage = 2 * ((0 if x1_in else rows * D * sz) + (0 if w_in else rows * T * sz))    # two chunks in flight
             extra = M * T * sz if rows < N else 0          # per-block result that is added into out
             return lib.flk_gauss_fdmmv_workspace_bytes(rows, M, D, T, code) + stage + fixed + extra
 
         blk = _rows_that_fit(N, need, usable) if N > 0 else 0
         X2d, vd = _on(X2, dev), _on(v, dev)
         outd = out if out_in else torch.empty((M, T), dtype=out.dtype, device=dev)
-        if blk == N:
-            gauss_fdmmv_native(_on(X1, dev), X2d, sigma_dev, vd, _on(w, dev), outd, kernel_fn)
+        if x1_in and w_in:
+            chunks = ((i, min(blk, N - i), (X1[i:i + blk], None if w is None else w[i:i + blk]))
+                      for i in range(0, N, max(blk, 1)))
+        elif N > 0:
+            chunk = _streamed_chunk_rows(N, (0 if x1_in else D * sz) + (0 if w_in else T * sz), blk)
+            chunks = iter(_HostRowStream([X1, w], N, dev, chunk))
         else:
-            tmp = torch.empty((M, T), dtype=out.dtype, device=dev)
-            for bi, i in enumerate(range(0, N, blk)):
-                li = min(blk, N - i)
-                wd = _on(w[i:i + li], dev) if w is not None else None
-                gauss_fdmmv_native(_on(X1[i:i + li], dev), X2d, sigma_dev, vd, wd, outd if bi == 0 else tmp, kernel_fn)
-                if bi > 0:
-                    outd.add_(tmp)
+            chunks = iter(())
+        tmp = None
+        first = True
+        for _, _, (X1d, wd) in chunks:
+            if first:
+                gauss_fdmmv_native(X1d, X2d, sigma_dev, vd, wd, outd, kernel_fn)
+            else:
+                tmp = torch.empty((M, T), dtype=out.dtype, device=dev) if tmp is None else tmp
+                gauss_fdmmv_native(X1d, X2d, sigma_dev, vd, wd, tmp, kernel_fn)
+                outd.add_(tmp)
+            first = False
+        if first:                                           # no rows at all: K^T (K v + w) is an empty sum
+            outd.zero_()
         if not out_in:
             out.copy_(outd)
     return out

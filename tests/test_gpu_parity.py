@@ -338,3 +338,34 @@ def test_dmmv_replays_from_a_hip_graph(dev):
         torch.cuda.synchronize()
         assert torch.equal(replayed, eager)
     assert rel_err(eager, mmv_ref.fdmmv_ref(X, C, vg.cpu(), wg.cpu(), k.sigma)) < 1e-5
+
+
+@pytest.mark.parametrize("order", ["C", "F"])
+@pytest.mark.parametrize("pinned", [False, True])
+def test_host_rows_streamed_in_chunks(dev, monkeypatch, order, pinned):
+    """Host-resident X (and w) cut into chunks whose upload overlaps the kernels of the previous chunk: same
+    results as with resident data, for pageable and pinned sources, either memory order, a ragged last chunk,
+    w on either side, host and device outputs."""
+    import sys
+    drv = sys.modules["falkon_amd.mmv_ops.fmmv"]          # the package attribute of that name is the function
+    monkeypatch.setattr(drv, "_STREAM_MIN_BYTES", 0)
+    monkeypatch.setattr(drv, "_STREAM_PIECES", 5)
+    X, C, v, w = _rand(10_007, 12, 300, 3, torch.float64, seed=44)
+    if order == "F":
+        X = torch.empty_strided(X.shape, (1, X.shape[0]), dtype=X.dtype).copy_(X)
+        w = torch.empty_strided(w.shape, (1, w.shape[0]), dtype=w.dtype).copy_(w)
+    if pinned:
+        X, w = X.pin_memory(), w.pin_memory()
+    k = GaussianKernel(2.5)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    exp_m, exp_d = k.mmv(Xg, Cg, vg), k.dmmv(Xg, Cg, vg, wg)
+    got = k.mmv(X, Cg, vg)                                  # host rows, device everything else: result on the GPU
+    assert got.device.type == "cuda" and rel_err(got, exp_m) < 1e-13
+    got = k.mmv(X, C, v)                                    # everything on the host: result on the host
+    assert got.device.type == "cpu" and rel_err(got, exp_m) < 1e-13
+    out_dev = torch.empty(10_007, 3, dtype=torch.float64, device=dev)
+    assert rel_err(k.mmv(X, Cg, vg, out=out_dev), exp_m) < 1e-13
+    assert rel_err(k.dmmv(X, C, v, w), exp_d) < 1e-12       # X and w streamed together
+    assert rel_err(k.dmmv(X, Cg, vg, wg), exp_d) < 1e-12    # only X streamed
+    assert rel_err(k.dmmv(Xg, Cg, vg, w), exp_d) < 1e-12    # only w streamed
+    assert rel_err(k.dmmv(X, Cg, vg, None), k.dmmv(Xg, Cg, vg, None)) < 1e-12
