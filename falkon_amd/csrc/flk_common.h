@@ -5,12 +5,9 @@
 #include <stdint.h>
 
 #include "../../include/falkon_amd.h"
+#include "kernel_fn.h"
 
 namespace flk {
-
-// sqrt(log2(e)): rows are scaled by this over sigma so that
-// exp(-1/2 |x/s - c/s|^2) == exp2(x~.c~ - 1/2|x~|^2 - 1/2|c~|^2) with a bare v_exp_f32.
-constexpr double kSqrtLog2e = 1.2011224087864498;
 
 // Packed-operand geometry.  f32: blocks of 32 rows, features split over the two
 // lane halves of a wave (MFMA 32x32x2).  f64: blocks of 16 rows, features split
@@ -157,8 +154,6 @@ FLK_DECLARE_KF(3)
 
 constexpr int kNumKernelFns = 4;
 inline bool valid_kernel_fn(int kf) { return kf >= 0 && kf < kNumKernelFns; }
-// factor on x / sigma when packing: only the Gaussian folds the base change of its exponential into the rows
-inline double operand_scale(int kf) { return kf == FLK_GAUSSIAN ? kSqrtLog2e : 1.0; }
 
 #define FLK_SWITCH_KF(kf, CALL)                                          \
     switch (kf) {                                                        \

@@ -1,16 +1,19 @@
 // The radial kernel functions applied to the accumulator of a tile (gfx950).
 //
 // Rows are packed scaled by operand_scale(kernel)/sigma with their half norms h = -1/2 |x~|^2, so that the
-// MFMA chain plus the two half norms leaves e = x~.c~ + hA + hB = -1/2 |x~ - c~|^2 in the accumulator:
+// MFMA chain plus the two half norms leaves e = x~.c~ + hA + hB = -1/2 |x~ - c~|^2 in the accumulator.  The
+// scale is chosen per kernel so that the epilogue needs no multiplication to get at its argument
+// (D = |x/sigma - c/sigma|, L = log2 e):
 //
-//   Gaussian   (falkon/kernels/distance_kernel.py:140-159): operand_scale = sqrt(log2 e), K = exp2(e), and the
+//   Gaussian   (falkon/kernels/distance_kernel.py:140-159): scale sqrt(L), e = -L D^2/2, K = exp2(e); the
 //              reference's clamp of the squared distance at 1e-20 is K <= 1;
-//   the others (operand_scale = 1, e = -D^2/2 with D = |x/sigma - c/sigma|, D^2 clamped at 1e-20 as in
-//              distance_kernel.py:100 before the square root):
-//     Laplacian    (distance_kernel.py:182-205):  K = exp(-D)
-//     Matern nu=3/2 (distance_kernel.py:243-254): K = (1 + s) exp(-s),            s = sqrt(3) D
-//     Matern nu=5/2 (distance_kernel.py:255-267): K = (1 + s + s^2/3) exp(-s),    s = sqrt(5) D
-//   Matern nu = 1/2 is the Laplacian and nu = inf the Gaussian (distance_kernel.py:235-238).
+//   Laplacian  (distance_kernel.py:182-205): scale sqrt(2) L, -e = (L D)^2 =: q^2, K = exp(-D) = exp2(-q);
+//   Matern 3/2 (distance_kernel.py:243-254): scale sqrt(6) L, q = L s with s = sqrt(3) D,
+//              K = (1 + s) exp(-s) = (1 + q/L) exp2(-q);
+//   Matern 5/2 (distance_kernel.py:255-267): scale sqrt(10) L, q = L s with s = sqrt(5) D,
+//              K = (1 + s + s^2/3) exp(-s) = (1 + q/L + q^2/(3 L^2)) exp2(-q).
+//   The reference clamps D^2 at 1e-20 before the square root (distance_kernel.py:100): q^2 is clamped at
+//   (scale^2 / 2) * 1e-20.  Matern nu = 1/2 is the Laplacian and nu = inf the Gaussian (distance_kernel.py:235-238).
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -19,44 +22,72 @@
 namespace flk {
 
 constexpr double kLog2e = 1.4426950408889634;
+constexpr double kSqrtLog2e = 1.2011224087864498;
+constexpr double kSqrt2 = 1.4142135623730951;
+constexpr double kSqrt3 = 1.7320508075688772;
+constexpr double kSqrt5 = 2.23606797749979;
 
-template <int KF> __device__ __forceinline__ float kernel_value(float e);
-template <int KF> __device__ __forceinline__ double kernel_value(double e);
+// factor on x / sigma when a matrix is packed for the kernel
+inline double operand_scale(int kf) {
+    switch (kf) {
+        case FLK_LAPLACIAN: return kLog2e * kSqrt2;
+        case FLK_MATERN32:  return kSqrt3 * kLog2e * kSqrt2;
+        case FLK_MATERN52:  return kSqrt5 * kLog2e * kSqrt2;
+        default:            return kSqrtLog2e;
+    }
+}
+
+template <int KF> struct KernelFn;
 
 // Gaussian: the median-of-three with 0 and 1 folds into the clamp bit of v_exp_f32, so the clamp is free
-template <> __device__ __forceinline__ float kernel_value<FLK_GAUSSIAN>(float e) {
-    return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(e), 0.0f, 1.0f);
-}
-template <> __device__ __forceinline__ double kernel_value<FLK_GAUSSIAN>(double e) { return exp2(fmin(e, 0.0)); }
+template <> struct KernelFn<FLK_GAUSSIAN> {
+    static __device__ __forceinline__ float value(float e) {
+        return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(e), 0.0f, 1.0f);
+    }
+    static __device__ __forceinline__ double value(double e) { return exp2(fmin(e, 0.0)); }
+};
 
-// distance D from e = -D^2/2, with the reference's clamp
-__device__ __forceinline__ float clamped_distance(float e) { return __builtin_amdgcn_sqrtf(fmaxf(-2.0f * e, 1e-20f)); }
-__device__ __forceinline__ double clamped_distance(double e) { return sqrt(fmax(-2.0 * e, 1e-20)); }
-
-template <> __device__ __forceinline__ float kernel_value<FLK_LAPLACIAN>(float e) {
-    return __builtin_amdgcn_exp2f(clamped_distance(e) * (float)(-kLog2e));
+// q = sqrt(max(-e, clamp)): the scaled distance, with the reference's clamp carried over to q^2
+template <int KF> __device__ __forceinline__ float scaled_distance(float e) {
+    constexpr float clamp = (float)((KF == FLK_LAPLACIAN ? 1.0 : KF == FLK_MATERN32 ? 3.0 : 5.0) * kLog2e * kLog2e * 1e-20);
+    return __builtin_amdgcn_sqrtf(fmaxf(-e, clamp));
 }
-template <> __device__ __forceinline__ double kernel_value<FLK_LAPLACIAN>(double e) {
-    return exp2(clamped_distance(e) * -kLog2e);
-}
-
-template <> __device__ __forceinline__ float kernel_value<FLK_MATERN32>(float e) {
-    const float s = clamped_distance(e) * 1.7320508075688772f;
-    return (1.0f + s) * __builtin_amdgcn_exp2f(s * (float)(-kLog2e));
-}
-template <> __device__ __forceinline__ double kernel_value<FLK_MATERN32>(double e) {
-    const double s = clamped_distance(e) * 1.7320508075688772;
-    return (1.0 + s) * exp2(s * -kLog2e);
+template <int KF> __device__ __forceinline__ double scaled_distance(double e) {
+    constexpr double clamp = (KF == FLK_LAPLACIAN ? 1.0 : KF == FLK_MATERN32 ? 3.0 : 5.0) * kLog2e * kLog2e * 1e-20;
+    return sqrt(fmax(-e, clamp));
 }
 
-template <> __device__ __forceinline__ float kernel_value<FLK_MATERN52>(float e) {
-    const float s = clamped_distance(e) * 2.23606797749979f;
-    const float poly = __builtin_fmaf(s, __builtin_fmaf(s, 1.0f / 3.0f, 1.0f), 1.0f);
-    return poly * __builtin_amdgcn_exp2f(s * (float)(-kLog2e));
-}
-template <> __device__ __forceinline__ double kernel_value<FLK_MATERN52>(double e) {
-    const double s = clamped_distance(e) * 2.23606797749979;
-    return fma(s, fma(s, 1.0 / 3.0, 1.0), 1.0) * exp2(s * -kLog2e);
-}
+template <> struct KernelFn<FLK_LAPLACIAN> {
+    static __device__ __forceinline__ float value(float e) {
+        return __builtin_amdgcn_exp2f(-scaled_distance<FLK_LAPLACIAN>(e));
+    }
+    static __device__ __forceinline__ double value(double e) { return exp2(-scaled_distance<FLK_LAPLACIAN>(e)); }
+};
+
+template <> struct KernelFn<FLK_MATERN32> {
+    static __device__ __forceinline__ float value(float e) {
+        const float q = scaled_distance<FLK_MATERN32>(e);
+        return __builtin_fmaf(q, (float)(1.0 / kLog2e), 1.0f) * __builtin_amdgcn_exp2f(-q);
+    }
+    static __device__ __forceinline__ double value(double e) {
+        const double q = scaled_distance<FLK_MATERN32>(e);
+        return fma(q, 1.0 / kLog2e, 1.0) * exp2(-q);
+    }
+};
+
+template <> struct KernelFn<FLK_MATERN52> {
+    static __device__ __forceinline__ float value(float e) {
+        const float q = scaled_distance<FLK_MATERN52>(e);
+        const float poly = __builtin_fmaf(q, __builtin_fmaf(q, (float)(1.0 / (3.0 * kLog2e * kLog2e)), (float)(1.0 / kLog2e)), 1.0f);
+        return poly * __builtin_amdgcn_exp2f(-q);
+    }
+    static __device__ __forceinline__ double value(double e) {
+        const double q = scaled_distance<FLK_MATERN52>(e);
+        return fma(q, fma(q, 1.0 / (3.0 * kLog2e * kLog2e), 1.0 / kLog2e), 1.0) * exp2(-q);
+    }
+};
+
+template <int KF> __device__ __forceinline__ float kernel_value(float e) { return KernelFn<KF>::value(e); }
+template <int KF> __device__ __forceinline__ double kernel_value(double e) { return KernelFn<KF>::value(e); }
 
 }  // namespace flk
