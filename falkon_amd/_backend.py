@@ -16,7 +16,7 @@ _lock = threading.Lock()
 _lib = None
 
 FLK_F32, FLK_F64 = 0, 1
-FLK_GAUSSIAN, FLK_LAPLACIAN, FLK_MATERN32, FLK_MATERN52 = 0, 1, 2, 3
+FLK_GAUSSIAN, FLK_LAPLACIAN, FLK_MATERN32, FLK_MATERN52, FLK_LAPLACIAN_DU = 0, 1, 2, 3, 4
 FLK_EINVAL, FLK_ENOMEM, FLK_EUNSUPPORTED, FLK_EHIP = -1, -2, -3, -4
 
 _MAT = [c_void_p, c_int64, c_int64, c_int64]        # ptr, rows, row_stride, col_stride

@@ -15,9 +15,9 @@ LIB_DIR = os.path.join(_HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libfalkon_amd.so")
 OBJ_DIR = os.path.join(_HERE, "build")
 
-# The sources that evaluate the kernel function are compiled once per function: -DFLK_KF=0..3
-# (Gaussian, Laplacian, Matern 3/2, Matern 5/2).
-KERNEL_FNS = (0, 1, 2, 3)
+# The sources that evaluate the kernel function are compiled once per function: -DFLK_KF=0..4
+# (Gaussian, Laplacian, Matern 3/2, Matern 5/2, the Laplacian's derivative weight).
+KERNEL_FNS = (0, 1, 2, 3, 4)
 PER_KERNEL_FN = ["mmv_small_f32.hip", "mmv_small_f32_fold.hip", "mmv_small_f64.hip", "mmv_large.hip", "fmm.hip"]
 SOURCES = [("api.hip", None), ("pack.hip", None)] + [(src, kf) for kf in KERNEL_FNS for src in PER_KERNEL_FN]
 

@@ -129,8 +129,8 @@ template <typename T> int mmv_large_b_tile_blocks();
 template <typename T> int mmv_large_partials_per_split();
 template <typename T> int mmv_large_max_cols();
 
-// The kernels that evaluate K are compiled once per kernel function (the same source with -DFLK_KF=0..3,
-// FLK_GAUSSIAN .. FLK_MATERN52): launchers carry the function in their name, and the helpers below pick one.
+// The kernels that evaluate K are compiled once per kernel function (the same source with -DFLK_KF=0..4,
+// FLK_GAUSSIAN .. FLK_LAPLACIAN_DU): launchers carry the function in their name, and the helpers below pick one.
 //   launch_mmv_small_kf*: register-resident product kernel, FLK_EUNSUPPORTED if dpad is out of its range;
 //   launch_mmv_large_kf*: LDS-tiled product kernel, writes splits * mmv_large_partials_per_split partials;
 //   launch_fmm_kf*:       explicit kernel matrix out[a][b] = K(A_a, B_b); O is the element type of out, whose
@@ -150,9 +150,10 @@ FLK_DECLARE_KF(0)
 FLK_DECLARE_KF(1)
 FLK_DECLARE_KF(2)
 FLK_DECLARE_KF(3)
+FLK_DECLARE_KF(4)
 #undef FLK_DECLARE_KF
 
-constexpr int kNumKernelFns = 4;
+constexpr int kNumKernelFns = 5;
 inline bool valid_kernel_fn(int kf) { return kf >= 0 && kf < kNumKernelFns; }
 
 #define FLK_SWITCH_KF(kf, CALL)                                          \
@@ -161,6 +162,7 @@ inline bool valid_kernel_fn(int kf) { return kf >= 0 && kf < kNumKernelFns; }
         case 1: return CALL(1);                                          \
         case 2: return CALL(2);                                          \
         case 3: return CALL(3);                                          \
+        case 4: return CALL(4);                                          \
         default: return fail(FLK_EINVAL, "unknown kernel function %d", kf); \
     }
 

@@ -12,6 +12,8 @@
 //              K = (1 + s) exp(-s) = (1 + q/L) exp2(-q);
 //   Matern 5/2 (distance_kernel.py:255-267): scale sqrt(10) L, q = L s with s = sqrt(5) D,
 //              K = (1 + s + s^2/3) exp(-s) = (1 + q/L + q^2/(3 L^2)) exp2(-q).
+//   Laplacian derivative weight (FLK_LAPLACIAN_DU): packed like the Laplacian, K = exp(-D)/D = L exp2(-q)/q, and 0
+//              where D^2 <= 1e-20 (where the reference's clamp stops the gradient).
 //   The reference clamps D^2 at 1e-20 before the square root (distance_kernel.py:100): q^2 is clamped at
 //   (scale^2 / 2) * 1e-20.  Matern nu = 1/2 is the Laplacian and nu = inf the Gaussian (distance_kernel.py:235-238).
 #pragma once
@@ -30,7 +32,8 @@ constexpr double kSqrt5 = 2.23606797749979;
 // factor on x / sigma when a matrix is packed for the kernel
 inline double operand_scale(int kf) {
     switch (kf) {
-        case FLK_LAPLACIAN: return kLog2e * kSqrt2;
+        case FLK_LAPLACIAN:
+        case FLK_LAPLACIAN_DU: return kLog2e * kSqrt2;
         case FLK_MATERN32:  return kSqrt3 * kLog2e * kSqrt2;
         case FLK_MATERN52:  return kSqrt5 * kLog2e * kSqrt2;
         default:            return kSqrtLog2e;
@@ -48,13 +51,14 @@ template <> struct KernelFn<FLK_GAUSSIAN> {
 };
 
 // q = sqrt(max(-e, clamp)): the scaled distance, with the reference's clamp carried over to q^2
+template <int KF> constexpr double distance_clamp() {
+    return (KF == FLK_MATERN32 ? 3.0 : KF == FLK_MATERN52 ? 5.0 : 1.0) * kLog2e * kLog2e * 1e-20;
+}
 template <int KF> __device__ __forceinline__ float scaled_distance(float e) {
-    constexpr float clamp = (float)((KF == FLK_LAPLACIAN ? 1.0 : KF == FLK_MATERN32 ? 3.0 : 5.0) * kLog2e * kLog2e * 1e-20);
-    return __builtin_amdgcn_sqrtf(fmaxf(-e, clamp));
+    return __builtin_amdgcn_sqrtf(fmaxf(-e, (float)distance_clamp<KF>()));
 }
 template <int KF> __device__ __forceinline__ double scaled_distance(double e) {
-    constexpr double clamp = (KF == FLK_LAPLACIAN ? 1.0 : KF == FLK_MATERN32 ? 3.0 : 5.0) * kLog2e * kLog2e * 1e-20;
-    return sqrt(fmax(-e, clamp));
+    return sqrt(fmax(-e, distance_clamp<KF>()));
 }
 
 template <> struct KernelFn<FLK_LAPLACIAN> {
@@ -62,6 +66,18 @@ template <> struct KernelFn<FLK_LAPLACIAN> {
         return __builtin_amdgcn_exp2f(-scaled_distance<FLK_LAPLACIAN>(e));
     }
     static __device__ __forceinline__ double value(double e) { return exp2(-scaled_distance<FLK_LAPLACIAN>(e)); }
+};
+
+template <> struct KernelFn<FLK_LAPLACIAN_DU> {
+    static __device__ __forceinline__ float value(float e) {
+        const float q = scaled_distance<FLK_LAPLACIAN_DU>(e);
+        const float k = __builtin_amdgcn_exp2f(-q) * ((float)kLog2e * __builtin_amdgcn_rcpf(q));
+        return -e > (float)distance_clamp<FLK_LAPLACIAN_DU>() ? k : 0.0f;
+    }
+    static __device__ __forceinline__ double value(double e) {
+        const double q = scaled_distance<FLK_LAPLACIAN_DU>(e);
+        return -e > distance_clamp<FLK_LAPLACIAN_DU>() ? exp2(-q) * kLog2e / q : 0.0;
+    }
 };
 
 template <> struct KernelFn<FLK_MATERN32> {

@@ -1,5 +1,5 @@
 // Register-resident fp32 product kernel: instantiations for even feature counts, and the entry point
-// that picks between them and the folded variant.  Compiled once per kernel function (-DFLK_KF=0..3).
+// that picks between them and the folded variant.  Compiled once per kernel function (-DFLK_KF=0..4).
 #ifndef FLK_KF
 #define FLK_KF 0
 #endif

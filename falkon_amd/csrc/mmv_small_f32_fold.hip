@@ -1,5 +1,5 @@
 // Register-resident fp32 product kernel: instantiations for odd feature counts (half norm of the
-// output rows folded into the padding feature).  Compiled once per kernel function (-DFLK_KF=0..3).
+// output rows folded into the padding feature).  Compiled once per kernel function (-DFLK_KF=0..4).
 #ifndef FLK_KF
 #define FLK_KF 0
 #endif

@@ -1,5 +1,5 @@
 // Register-resident kernel-vector product for the radial kernels of kernel_fn.h, fp64, gfx950.
-// Compiled once per kernel function (-DFLK_KF=0..3).
+// Compiled once per kernel function (-DFLK_KF=0..4).
 //
 // Same structure as the fp32 kernel with the 16x16x4 fp64 MFMA: a wave keeps FR
 // blocks of 16 output rows (B side) in registers and streams blocks of 16

@@ -42,17 +42,20 @@ def _radial_block(mat1, mat2, out: Optional[torch.Tensor], diag: bool, sigma: to
     (1 + s + s^2/3) exp(-s) with s = sqrt(5) D (5/2).  Off the kernel-vector path (diagonals, callers' own blocks)."""
     sigma = sigma.to(device=mat1.device, dtype=mat1.dtype)
     a, b = mat1 / sigma, mat2 / sigma
+    # no in-place updates: the block may be differentiated (diagonals under autograd)
     if diag:
         d2 = (a - b).square().sum(-1)
+        if nu != float("inf") and d2.requires_grad:
+            d2 = d2.clamp_min(1e-20)                                # keeps the square root's gradient finite
     else:
         d2 = torch.addmm(a.square().sum(-1, keepdim=True), a, b.T, alpha=-2, beta=1)
-        d2.add_(b.square().sum(-1, keepdim=True).T).clamp_min_(1e-20)
+        d2 = (d2 + b.square().sum(-1, keepdim=True).T).clamp_min(1e-20)
     if nu == float("inf"):
-        res = d2.mul_(-0.5).exp_()
+        res = torch.exp(-0.5 * d2)
     else:
-        s = d2.sqrt_().mul_({0.5: 1.0, 1.5: _SQRT3, 2.5: _SQRT5}[nu])
+        s = d2.sqrt() * {0.5: 1.0, 1.5: _SQRT3, 2.5: _SQRT5}[nu]
         decay = torch.exp(-s)
-        res = decay if nu == 0.5 else decay.mul_(1 + s if nu == 1.5 else 1 + s + s * s / 3)
+        res = decay if nu == 0.5 else decay * (1 + s if nu == 1.5 else 1 + s + s * s / 3)
     return res if out is None else out.copy_(res.reshape(out.shape))
 
 
@@ -64,9 +67,13 @@ class _RadialKernel(DiffKernel):
         super().__init__(name, opt, core_fn=_radial_block, sigma=validate_sigma(sigma), **other_params)
         self._sigma_cache = {}
 
-    def _sigma_on(self, device: torch.device, dtype: torch.dtype) -> torch.Tensor:
-        """sigma on the data's device and dtype (distance_kernel.py:148), cached until sigma changes."""
+    def _sigma_on(self, device: torch.device, dtype: torch.dtype, cached: bool = True) -> torch.Tensor:
+        """sigma on the data's device and dtype (distance_kernel.py:148), cached until sigma changes.  Writes
+        through ``sigma.data`` (numerical differentiation does that) do not show in the version counter the
+        cache is keyed on: differentiable calls pass ``cached=False``."""
         sigma = self.sigma
+        if not cached:
+            return sigma.detach().reshape(-1).to(device=device, dtype=dtype).contiguous()
         key = (device, dtype)
         tag = (sigma.data_ptr(), sigma._version, sigma.numel())
         hit = self._sigma_cache.get(key)

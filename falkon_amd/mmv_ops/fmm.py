@@ -40,32 +40,69 @@ def gauss_fmm_native(X1, X2, sigma_dev, out, compute_f64: bool, kernel_fn: int =
     _backend.raise_for_status(rc, "flk_kernel_fmm")
 
 
+class _KernelMmFn(torch.autograd.Function):
+    """The kernel matrix with its backward pass (the reference's KernelMmFnFull, falkon/mmv_ops/fmm.py:441-696)."""
+
+    @staticmethod
+    def forward(ctx, kernel, opt, out, X1, X2, *kernel_params):
+        kernel_fn = _kernel_fn(kernel)
+        res = _fmm_run(kernel, kernel_fn, opt, out, X1, X2, cached_sigma=False)
+        if out is not None:
+            ctx.mark_dirty(out)
+        ctx.save_for_backward(X1, X2, *kernel_params)
+        ctx.kernel_fn, ctx.opt = kernel_fn, opt
+        return res
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_out):
+        from .fmmv_grad import fmm_backward
+        X1, X2, sigma = ctx.saved_tensors
+        grads = fmm_backward(ctx.kernel_fn, X1, X2, sigma, grad_out, ctx.needs_input_grad[3:6], ctx.opt)
+        grads = [None if g is None else g.reshape(t.shape).to(device=t.device, dtype=t.dtype)
+                 for g, t in zip(grads, (X1, X2, sigma))]
+        return (None, None, None, *grads)
+
+
 def fmm(kernel, opt: Optional[BaseOptions], out: Optional[torch.Tensor], diag: bool, X1: torch.Tensor,
         X2: torch.Tensor, kwargs_m1=None, kwargs_m2=None) -> torch.Tensor:
+    """``K(X1, X2)`` (N x M) or its diagonal (falkon/mmv_ops/fmm.py:699-717); differentiable with respect to X1, X2
+    and the kernel's lengthscale when any of them requires a gradient."""
     opt = opt if opt is not None else BaseOptions()
     check_contiguity((X1, "X1"), (X2, "X2"), (out, "out"))
-    data_devs = (X1.device, X2.device)
-    dev = _compute_device(opt, data_devs)
-    N, D = X1.shape
-    M = X2.shape[0]
-    with torch.inference_mode():
-        if diag:
+    kernel_params = list(kernel.diff_params.values())
+    differentiable = any(t.requires_grad for t in [X1, X2] + kernel_params)
+    if diag:
+        dev = _compute_device(opt, (X1.device, X2.device))
+        if differentiable:
+            # the diagonal is O(N d): stock torch ops under autograd
+            res = kernel.compute_diff(X1.to(dev), X2.to(dev), diag=True).to(X1.device)
+            return res if out is None else out.copy_(res.reshape(out.shape))
+        with torch.inference_mode():
             res = kernel.compute(X1.to(dev), X2.to(dev), None, diag=True)
             if out is None:
                 return res.to(X1.device)
             return out.copy_(res.reshape(out.shape))
-        kernel_fn = _kernel_fn(kernel)
-        if any(t.requires_grad for t in [X1, X2] + list(kernel.diff_params.values())):
-            raise NotImplementedError("falkon_amd.fmm does not implement the autograd backward pass; "
-                                      "detach the inputs and the kernel parameters")
-        _check_dtype(X1.dtype)
-        out = create_output_mat(out, data_devs, shape=(N, M), dtype=X1.dtype, other_mat=X1)
-        if N == 0 or M == 0:
-            return out
+    kernel_fn = _kernel_fn(kernel)
+    if differentiable:
+        return _KernelMmFn.apply(kernel, opt, out, X1, X2, *kernel_params)
+    return _fmm_run(kernel, kernel_fn, opt, out, X1, X2, cached_sigma=True)
+
+
+def _fmm_run(kernel, kernel_fn: int, opt: BaseOptions, out, X1, X2, cached_sigma: bool) -> torch.Tensor:
+    data_devs = (X1.device, X2.device)
+    dev = _compute_device(opt, data_devs)
+    N, D = X1.shape
+    M = X2.shape[0]
+    _check_dtype(X1.dtype)
+    out = create_output_mat(out, data_devs, shape=(N, M), dtype=X1.dtype, other_mat=X1)
+    if N == 0 or M == 0:
+        return out
+    with torch.inference_mode():
         lib = _backend.load()
         code, sz = _DTYPE_CODE[X1.dtype], sizeof_dtype(X1.dtype)
         compute_f64 = X1.dtype == torch.float32 and bool(opt.no_single_kernel)
-        sigma_dev = kernel._sigma_on(dev, X1.dtype)
+        sigma_dev = kernel._sigma_on(dev, X1.dtype, cached=cached_sigma)
         usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack)
         x1_in, out_in = X1.device == dev, out.device == dev
         fixed = 0 if X2.device == dev else M * D * sz

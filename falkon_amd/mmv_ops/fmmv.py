@@ -227,17 +227,48 @@ def _check_dtype(dtype):
         raise TypeError(f"Dtype {dtype} not valid")
 
 
+class _KernelMmvFn(torch.autograd.Function):
+    """``K(X1, X2) @ v`` with its backward pass (the reference's KernelMmvFnFull, falkon/mmv_ops/fmmv.py:771-957).
+    The forward is the plain product; the backward is closed form on the same kernels (``fmmv_grad``)."""
+
+    @staticmethod
+    def forward(ctx, kernel, opt, out, X1, X2, v, *kernel_params):
+        kernel_fn = _kernel_fn(kernel)
+        res = _fmmv_run(X1, X2, v, kernel, kernel_fn, out, opt, cached_sigma=False)
+        if out is not None:
+            ctx.mark_dirty(out)
+        ctx.save_for_backward(X1, X2, v, *kernel_params)
+        ctx.kernel_fn, ctx.opt = kernel_fn, opt
+        return res
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_out):
+        from .fmmv_grad import fmmv_backward
+        X1, X2, v, sigma = ctx.saved_tensors
+        grads = fmmv_backward(ctx.kernel_fn, X1, X2, v, sigma, grad_out, ctx.needs_input_grad[3:7], ctx.opt)
+        like = (X1, X2, v, sigma)
+        grads = [None if g is None else g.reshape(t.shape).to(device=t.device, dtype=t.dtype)
+                 for g, t in zip(grads, like)]
+        return (None, None, None, *grads)
+
+
 def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optional[torch.Tensor] = None,
          opt: Optional[BaseOptions] = None, kwargs_m1: Optional[Dict[str, torch.Tensor]] = None,
          kwargs_m2: Optional[Dict[str, torch.Tensor]] = None) -> torch.Tensor:
-    """``out = K(X1, X2) @ v`` (N x T), same contract as falkon/mmv_ops/fmmv.py:960-973 / :887-932."""
+    """``out = K(X1, X2) @ v`` (N x T), same contract as falkon/mmv_ops/fmmv.py:960-973 / :887-932; differentiable
+    with respect to X1, X2, v and the kernel's lengthscale when any of them requires a gradient."""
     opt = opt if opt is not None else BaseOptions()
     kernel_fn = _kernel_fn(kernel)
     _reject_block_kwargs(kwargs_m1, kwargs_m2)
     check_contiguity((X1, "X1"), (X2, "X2"), (v, "v"), (out, "out"))
-    if any(t.requires_grad for t in [X1, X2, v] + list(kernel.diff_params.values())):
-        raise NotImplementedError("falkon_amd.fmmv does not implement the autograd backward pass; "
-                                  "detach the inputs and the kernel parameters")
+    kernel_params = list(kernel.diff_params.values())
+    if any(t.requires_grad for t in [X1, X2, v] + kernel_params):
+        return _KernelMmvFn.apply(kernel, opt, out, X1, X2, v, *kernel_params)
+    return _fmmv_run(X1, X2, v, kernel, kernel_fn, out, opt, cached_sigma=True)
+
+
+def _fmmv_run(X1, X2, v, kernel, kernel_fn: int, out, opt: BaseOptions, cached_sigma: bool) -> torch.Tensor:
     _check_dtype(X1.dtype)
     data_devs = (X1.device, X2.device, v.device)
     dev = _compute_device(opt, data_devs)
@@ -249,7 +280,7 @@ def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optio
     x1_in, out_in = X1.device == dev, out.device == dev
 
     with torch.inference_mode():
-        sigma_dev = kernel._sigma_on(dev, X1.dtype)
+        sigma_dev = kernel._sigma_on(dev, X1.dtype, cached=cached_sigma)
         usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack)
         fixed = (0 if X2.device == dev else M * D * sz) + (0 if v.device == dev else M * T * sz)
 

@@ -32,11 +32,17 @@ extern "C" {
 /* Radial kernels K(x, c) = f(D), D = |x/sigma - c/sigma| (falkon/kernels/distance_kernel.py):
  * Gaussian exp(-D^2/2) (:140-159), Laplacian exp(-D) (:182-205), Matern nu = 3/2 and 5/2 (:225-269;
  * nu = 1/2 is the Laplacian, nu = inf the Gaussian, :235-238).  The flk_gauss_* entry points are the
- * flk_kernel_* ones with FLK_GAUSSIAN. */
+ * flk_kernel_* ones with FLK_GAUSSIAN.
+ * FLK_LAPLACIAN_DU is exp(-D)/D, and 0 where D^2 <= 1e-20: up to the factor -1/2 the derivative of the
+ * Laplacian with respect to D^2, zero where the reference's clamp of D^2 (:100) cuts the gradient.  The
+ * derivatives of the other three are multiples of kernels already in the list (Gaussian: -1/2 itself;
+ * Matern 3/2: -3/2 Laplacian with sigma/sqrt(3); Matern 5/2: -5/6 Matern 3/2 with sigma*sqrt(3/5)), so
+ * these five cover the backward pass of the kernel-vector product (falkon/mmv_ops/fmmv.py:405-485). */
 #define FLK_GAUSSIAN  0
 #define FLK_LAPLACIAN 1
 #define FLK_MATERN32  2
 #define FLK_MATERN52  3
+#define FLK_LAPLACIAN_DU 4
 
 #define FLK_OK          0
 #define FLK_EINVAL     -1   /* bad argument (shape, stride, dtype, null pointer)      */
@@ -148,7 +154,7 @@ int flk_gauss_fmm(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
                   void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- the same entry points for any of the radial kernels ----------------------
- * `kernel` is one of FLK_GAUSSIAN / FLK_LAPLACIAN / FLK_MATERN32 / FLK_MATERN52; everything else as in
+ * `kernel` is one of FLK_GAUSSIAN / FLK_LAPLACIAN / FLK_MATERN32 / FLK_MATERN52 / FLK_LAPLACIAN_DU; everything else as in
  * the flk_gauss_* function of the same name, whose *_workspace_bytes / flk_gauss_packed_bytes sizes
  * apply to every kernel.  Packed operands are specific to the kernel they were packed for (the
  * Gaussian rows carry an extra factor).  These replace fmmv / fdmmv / fmm for the reference's

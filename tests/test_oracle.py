@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import brute, brute_c, gaussian_ref, inputs, mmv_ref
+from oracle import brute, brute_c, gaussian_ref, grad_ref, inputs, mmv_ref
 
 
 def _cdist_kernel(X, C, sigma):
@@ -270,3 +270,64 @@ def test_radial_products_against_brute(name):
                                K @ v.numpy(), rtol=1e-10, atol=1e-12)
     np.testing.assert_allclose(mmv_ref.fdmmv_ref(X, C, v, w, sig, kernel_name=name, max_cpu_mem=2**24).numpy(),
                                K.T @ (K @ v.numpy() + w.numpy()), rtol=1e-10, atol=1e-12)
+
+
+# ---- gradients (oracle/grad_ref.py) -------------------------------------------------------------------
+def _grad_case(per_dim: bool, seed: int = 21, n: int = 14, m: int = 9, d: int = 4, t: int = 2):
+    g = np.random.default_rng(seed)
+    mk = lambda *s: torch.from_numpy(g.standard_normal(s))                        # noqa: E731
+    sigma = torch.from_numpy(g.uniform(1.0, 2.0, d if per_dim else 1))
+    return mk(n, d), mk(m, d), mk(m, t), sigma, mk(n, t)
+
+
+@pytest.mark.parametrize("name", KERNEL_NAMES)
+def test_autograd_restatement_is_the_core(name):
+    """The out-of-place graph evaluates to what the in-place core functions give."""
+    X, C, _, sigma, _ = _grad_case(per_dim=True)
+    torch.testing.assert_close(grad_ref.radial_kernel_autograd(X, C, sigma, name),
+                               gaussian_ref.core_ref_for(name)(X, C, None, sigma), rtol=1e-14, atol=1e-15)
+    torch.testing.assert_close(grad_ref.radial_kernel_difference_form(X, C, sigma, name),
+                               torch.from_numpy(brute.radial_brute(X, C, sigma, name)), rtol=1e-13, atol=1e-15)
+
+
+@pytest.mark.parametrize("name", KERNEL_NAMES)
+@pytest.mark.parametrize("per_dim", [False, True])
+def test_gradients_against_difference_form_and_finite_differences(name, per_dim):
+    X, C, v, sigma, G = _grad_case(per_dim)
+    got = grad_ref.fmmv_grads_ref(X, C, v, sigma, G, name)
+    exact = grad_ref.fmmv_grads_ref(X, C, v, sigma, G, name, kernel_fn=grad_ref.radial_kernel_difference_form)
+    for a, b in zip(got, exact):
+        torch.testing.assert_close(a, b, rtol=1e-9, atol=1e-11)
+
+    # central differences of L = sum(G * (K v)) built on the closed form, a few coordinates of every input
+    def loss(x, c, vv, sg):
+        return float((G.numpy() * (brute.radial_brute(x, c, sg, name) @ vv.numpy())).sum())
+
+    h = 1e-6
+    args = [X, C, v, sigma]
+    for which, grad in enumerate(got):
+        flat = grad.reshape(-1)
+        for idx in range(0, flat.numel(), max(1, flat.numel() // 5)):
+            up = [a.clone() for a in args]
+            dn = [a.clone() for a in args]
+            up[which].view(-1)[idx] += h
+            dn[which].view(-1)[idx] -= h
+            fd = (loss(*up) - loss(*dn)) / (2 * h)
+            assert abs(fd - float(flat[idx])) <= 1e-6 * max(1.0, abs(fd)), (which, idx)
+    # the kernel matrix: L = sum(G2 * K)
+    G2 = torch.from_numpy(np.random.default_rng(3).standard_normal((X.shape[0], C.shape[0])))
+    got_mm = grad_ref.fmm_grads_ref(X, C, sigma, G2, name)
+    exact_mm = grad_ref.fmm_grads_ref(X, C, sigma, G2, name, kernel_fn=grad_ref.radial_kernel_difference_form)
+    for a, b in zip(got_mm, exact_mm):
+        torch.testing.assert_close(a, b, rtol=1e-9, atol=1e-11)
+    # K @ v with v = e_j and G = e_i picks the gradient of a single kernel entry: same as the matrix form
+    E = torch.zeros_like(G2)
+    E[2, 3] = 1.0
+    vj = torch.zeros((C.shape[0], 1), dtype=torch.float64)
+    vj[3] = 1.0
+    Gi = torch.zeros((X.shape[0], 1), dtype=torch.float64)
+    Gi[2] = 1.0
+    one_mm = grad_ref.fmm_grads_ref(X, C, sigma, E, name)
+    one_mv = grad_ref.fmmv_grads_ref(X, C, vj, sigma, Gi, name)
+    for a, b in zip(one_mm, (one_mv[0], one_mv[1], one_mv[3])):
+        torch.testing.assert_close(a, b, rtol=1e-12, atol=1e-14)
