@@ -23,6 +23,23 @@ sys.path.insert(0, ROOT)
 
 FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 matrix peak = fp32 vector peak (vendor figure)
 FP64_PEAK_TFLOPS = 78.6    # MI355X fp64 matrix peak = fp64 vector peak
+BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
+
+
+def split_roofline(pairs, d, kern_ms, algorithmic_flop):
+    """Roofline of the bf16x3 product kernel: it executes 6 partial products over the features padded to whole
+    k-steps of 16 (two of them carry the half norms), on the bf16 matrix cores."""
+    ksteps = (d + 2 + 15) // 16
+    executed = pairs * 6 * 2 * 16 * ksteps
+    achieved = executed / (kern_ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": achieved / BF16_PEAK_TFLOPS, "traffic": None, "kernel": "mmv_split_kernel",
+            "avg_launch_ms": kern_ms, "flop_per_launch": executed,
+            "note": "achieved = bf16 MFMA flops the kernel executes (6 partial products, padded features); "
+                    "algorithmic fp32 flops per launch and their rate are given beside it",
+            "algorithmic_flop_per_launch": algorithmic_flop,
+            "algorithmic_tflops": algorithmic_flop / (kern_ms * 1e-3) / 1e12,
+            "algorithmic_frac_of_fp32_peak": algorithmic_flop / (kern_ms * 1e-3) / 1e12 / FP32_PEAK_TFLOPS}
 
 WORKLOADS = {
     # name: (seed, N, d, M, T, has_w)
@@ -117,9 +134,11 @@ def run_c5(args, lib):
     n_dmmv = iters + iters // FalkonOptions().cg_full_gradient_every     # one per iteration + the full residuals
     fit_s, pre_s, pred_s, kern_ms, launches = [], [], [], 0.0, 0
     mse = err = None
+    split = args.cross_term == "bf16x3"
+    opt = FalkonOptions(bf16x3_cross_term=split)
     for it in range(args.warmup + args.steps):
         timed = it >= args.warmup
-        model = Falkon(GaussianKernel(sigma), lam, M=M, maxiter=iters, seed=12)
+        model = Falkon(GaussianKernel(sigma, opt=opt), lam, M=M, maxiter=iters, seed=12, options=opt)
         torch.cuda.synchronize()
         if timed:
             lib.flk_kernel_timing_enable(1)
@@ -152,22 +171,26 @@ def run_c5(args, lib):
         "metric": "dfmmv kernel-entries/sec (N*M*T/s) fp32 inside Falkon.fit, 1 MI355X",
         "value": N * M * n_dmmv / cg, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": (fit + prd) * 1e3, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32" if not split else "f32 (cross term: bf16x3 split, fp32 accumulate)",
+        "data": "synthetic",
         "config": {"workload": f"C5: Falkon.fit + predict, N={N}, d={d}, M={M} uniform centres, sigma=3.8, "
                                f"penalty=1e-6, {iters} CG iterations ({n_dmmv} dfmmv + 1 fmmv), test rows {Nts}, "
-                               f"fp32, data resident in HBM"},
+                               f"fp32{' with the bf16x3 cross term' if split else ''}, data resident in HBM"},
         "fit_s": fit, "preconditioner_s": pre, "cg_s": cg, "predict_s": prd, "test_mse": mse, "test_error_rate": err,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_PEAK_TFLOPS, "traffic": None, "kernel": "mmv_small_f32_kernel",
                      "launches_per_step": launches / max(args.steps, 1), "avg_launch_ms": kern_avg,
                      "flop_per_launch": flop_per_launch},
     }
+    if split:
+        res["roofline"] = dict(split_roofline(N * M, d, kern_avg, flop_per_launch),
+                               launches_per_step=launches / max(args.steps, 1))
     if not args.no_cpu_baseline:
         # the same pipeline at a size the CPU finishes in seconds, on both sides, same centres
         from oracle import falkon_ref                  # checker only; never on the product path
         n2, m2 = args.cpu_rows or 200_000, 5_000
         X2, Y2, X2ts, Y2ts = make_c5(n2, n2 // 10)
-        small = Falkon(GaussianKernel(sigma), lam, M=m2, maxiter=iters, seed=12)
+        small = Falkon(GaussianKernel(sigma, opt=opt), lam, M=m2, maxiter=iters, seed=12, options=opt)
         small.fit(X2.to(dev), Y2.to(dev))
         mse_gpu = float(((small.predict(X2ts.to(dev)).cpu() - Y2ts) ** 2).mean())
         C2 = small.ny_points_.cpu()
@@ -198,6 +221,10 @@ def main():
     ap.add_argument("--kernel", default="gaussian", choices=["gaussian", "laplacian", "matern32", "matern52"],
                     help="kernel function (the headline is the Gaussian; the flop count of the roofline stays the "
                          "Gaussian's 2d+4+2T per pair, the other kernels spend a few more VALU operations per entry)")
+    ap.add_argument("--cross-term", default="f32", choices=["f32", "bf16x3"],
+                    help="f32 (the headline): fp32 MFMA.  bf16x3: the opt-in mode that forms x.c on the bf16 matrix cores "
+                         "from an exact three-way bfloat16 split of the fp32 rows (fp32 accuracy; d <= 62, fp32 data); "
+                         "its roofline is priced against the bf16 MFMA peak on the flops it executes")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=0)
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
@@ -222,16 +249,22 @@ def main():
         print(json.dumps({"copy_calibration_bytes": src.numel() * 4, "copies": 5}))
         return
 
-    from falkon_amd import GaussianKernel, LaplacianKernel, MaternKernel, _backend
+    from falkon_amd import FalkonOptions, GaussianKernel, LaplacianKernel, MaternKernel, _backend
     lib = _backend.load()                            # raises if the HIP library is missing
-    make_kernel, kernel_name = {"gaussian": (GaussianKernel, "gaussian"), "laplacian": (LaplacianKernel, "laplacian"),
-                                "matern32": (lambda s: MaternKernel(s, 1.5), "1.5-matern"),
-                                "matern52": (lambda s: MaternKernel(s, 2.5), "2.5-matern")}[args.kernel]
+    kopt = FalkonOptions(bf16x3_cross_term=args.cross_term == "bf16x3")
+    make_kernel, kernel_name = {"gaussian": (lambda s: GaussianKernel(s, opt=kopt), "gaussian"),
+                                "laplacian": (lambda s: LaplacianKernel(s, opt=kopt), "laplacian"),
+                                "matern32": (lambda s: MaternKernel(s, 1.5, opt=kopt), "1.5-matern"),
+                                "matern52": (lambda s: MaternKernel(s, 2.5, opt=kopt), "2.5-matern")}[args.kernel]
     if args.workload == "C5":
         print(json.dumps(run_c5(args, lib)), flush=True)
         return
     dev = torch.device("cuda:0")
     seed, N, d, M, T, has_w = WORKLOADS[args.workload]
+    split = args.cross_term == "bf16x3"
+    if split and (d > 62 or args.dtype != "f32"):
+        print("bench.py: --cross-term bf16x3 applies to fp32 data with d <= 62 (workloads C2, C3, C5)", file=sys.stderr)
+        sys.exit(2)
     X, C, sigma, v, w = make_inputs(args.workload)
     tdt = torch.float32 if args.dtype == "f32" else torch.float64
     X, C, v = X.to(tdt), C.to(tdt), v.to(tdt)
@@ -272,10 +305,11 @@ def main():
         "metric": f"{'dfmmv' if args.op == 'dmmv' else 'fmmv'} kernel-entries/sec (N*M*T/s) {'fp32' if args.dtype == 'f32' else 'fp64'}, 1 MI355X",
         "value": value, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.dtype, "data": "synthetic",
+        "dtype": args.dtype if not split else "f32 (cross term: bf16x3 split, fp32 accumulate)", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {kernel_name} {'dfmmv K^T(Kv+w)' if args.op == 'dmmv' else 'fmmv K v'}, N={N}, d={d}, M={M}, T={T}, "
                                f"{ {'C2': 'sigma=3.8', 'C3': 'per-dimension sigma', 'C4': 'sigma=10'}[args.workload] }, "
                                f"{'fp32' if args.dtype == 'f32' else 'fp64'}, "
+                               f"{'cross term on the bf16 matrix cores from a 3-way bfloat16 split, ' if split else ''}"
                                f"inputs resident in HBM, packing included in every step"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak,
@@ -286,6 +320,9 @@ def main():
         "whole_step_flop_frac": (N * M * ((2 if args.op == "dmmv" else 1) * (2 * d + 4 + 2 * T)))
                                 / (elapsed / args.steps) / 1e12 / peak,
     }
+    if split:
+        res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch),
+                               launches_per_step=launches.value / args.steps)
     if not args.no_cpu_baseline and args.op == "dmmv":
         rows = args.cpu_rows or {"C2": N, "C3": 400_000, "C4": 100_000}[args.workload]
 

@@ -15,7 +15,7 @@ from . import _build
 _lock = threading.Lock()
 _lib = None
 
-FLK_F32, FLK_F64 = 0, 1
+FLK_F32, FLK_F64, FLK_F32_BF16X3 = 0, 1, 2
 FLK_GAUSSIAN, FLK_LAPLACIAN, FLK_MATERN32, FLK_MATERN52, FLK_LAPLACIAN_DU = 0, 1, 2, 3, 4
 FLK_EINVAL, FLK_ENOMEM, FLK_EUNSUPPORTED, FLK_EHIP = -1, -2, -3, -4
 

@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "flk_common.h"
+#include "split_common.h"
 
 namespace flk {
 
@@ -70,42 +71,51 @@ struct Plan {
 
 constexpr int64_t kTargetWgsLarge = 16384;  // two 256-thread workgroups per CU: 8 rounds
 
+// Plan of a register-resident product kernel: per_wg output blocks per workgroup, a_block_bytes per packed
+// reduction block of blk rows, col_chunk right-hand sides per pass, results of elem_bytes per element.
+static void plan_register_resident(Plan &p, int64_t na_blocks, int64_t nb_blocks, int64_t per_wg, int64_t a_block_bytes,
+                                   int64_t blk, int col_chunk, int64_t t, int64_t elem_bytes) {
+    p.large = false;
+    const int64_t b_tiles = (nb_blocks + per_wg - 1) / per_wg;
+    int64_t splits = (kTargetWgs + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
+    int64_t max_splits = na_blocks / kMinChunkBlocks;
+    if (max_splits < 1) max_splits = 1;
+    if (splits > max_splits) splits = max_splits;
+    p.col_chunk = col_chunk;
+    if (t > 4 && p.col_chunk > 4) {
+        int64_t want = (na_blocks + kWideChunkBlocks - 1) / kWideChunkBlocks;
+        if (splits < want) splits = want;
+    }
+    // a reduction chunk is streamed by every output tile that shares it: keep it within half of one XCD's
+    // 4 MB L2 so that those re-reads hit L2 instead of HBM (only where there is more than one output tile)
+    // ... as long as the partial results this creates stay small (kL2PartialBytes per pass)
+    if (b_tiles > 1) {
+        int64_t chunk_cap = kL2ChunkBytes / a_block_bytes;
+        if (chunk_cap < 1) chunk_cap = 1;
+        int64_t want = (na_blocks + chunk_cap - 1) / chunk_cap;
+        const int64_t tc = t < p.col_chunk ? (t > 0 ? t : 1) : p.col_chunk;
+        const int64_t per_split = tc * nb_blocks * blk * elem_bytes;
+        const int64_t affordable = kL2PartialBytes / (per_split > 0 ? per_split : 1);
+        if (want > affordable) want = affordable;
+        if (splits < want) splits = want;
+    }
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    if (splits < 1) splits = 1;
+    p.chunk = (na_blocks + splits - 1) / splits;
+    if (p.chunk < 1) p.chunk = 1;
+    p.splits = (int)((na_blocks + p.chunk - 1) / p.chunk);
+    if (p.splits < 1) p.splits = 1;
+    p.partials = p.splits;
+}
+
 template <typename T>
 static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t dpad, int64_t t) {
     Plan p;
     p.large = d > mmv_small_max_d<T>();
     if (!p.large) {
-        const int64_t per_wg = mmv_small_b_blocks_per_wg<T>(dpad);
-        const int64_t b_tiles = (nb_blocks + per_wg - 1) / per_wg;
-        int64_t splits = (kTargetWgs + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
-        int64_t max_splits = na_blocks / kMinChunkBlocks;
-        if (max_splits < 1) max_splits = 1;
-        if (splits > max_splits) splits = max_splits;
-        p.col_chunk = mmv_small_max_cols<T>(dpad);
-        if (t > 4 && p.col_chunk > 4) {
-            int64_t want = (na_blocks + kWideChunkBlocks - 1) / kWideChunkBlocks;
-            if (splits < want) splits = want;
-        }
-        // a reduction chunk is streamed by every output tile that shares it: keep it within half of one XCD's
-        // 4 MB L2 so that those re-reads hit L2 instead of HBM (only where there is more than one output tile)
-        // ... as long as the partial results this creates stay small (kL2PartialBytes per pass)
-        if (b_tiles > 1) {
-            int64_t chunk_cap = kL2ChunkBytes / (dpad * Geo<T>::BLK * (int64_t)sizeof(T));
-            if (chunk_cap < 1) chunk_cap = 1;
-            int64_t want = (na_blocks + chunk_cap - 1) / chunk_cap;
-            const int64_t tc = t < p.col_chunk ? (t > 0 ? t : 1) : p.col_chunk;
-            const int64_t per_split = tc * nb_blocks * Geo<T>::BLK * (int64_t)sizeof(T);
-            const int64_t affordable = kL2PartialBytes / (per_split > 0 ? per_split : 1);
-            if (want > affordable) want = affordable;
-            if (splits < want) splits = want;
-        }
-        if (splits > kMaxSplits) splits = kMaxSplits;
-        if (splits < 1) splits = 1;
-        p.chunk = (na_blocks + splits - 1) / splits;
-        if (p.chunk < 1) p.chunk = 1;
-        p.splits = (int)((na_blocks + p.chunk - 1) / p.chunk);
-        if (p.splits < 1) p.splits = 1;
-        p.partials = p.splits;
+        plan_register_resident(p, na_blocks, nb_blocks, mmv_small_b_blocks_per_wg<T>(dpad),
+                               dpad * Geo<T>::BLK * (int64_t)sizeof(T), Geo<T>::BLK, mmv_small_max_cols<T>(dpad), t,
+                               (int64_t)sizeof(T));
     } else {
         const int64_t a_tiles = (na_blocks + mmv_large_a_tile_blocks<T>() - 1) / mmv_large_a_tile_blocks<T>();
         const int64_t b_tiles = (nb_blocks + mmv_large_b_tile_blocks<T>() - 1) / mmv_large_b_tile_blocks<T>();
@@ -347,6 +357,133 @@ static int fmm_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1
     return launch_fmm<T, TI>(kf, P2, P1, (TI *)out, out_cs, st);
 }
 
+// ---------------------------------------------------------------------------
+// bf16x3 mode of the fp32 products (split_common.h): same drivers on the split operands.  Feature counts beyond
+// kSplitMaxD have no split kernel and take the plain fp32 path (the callers below decide).
+// ---------------------------------------------------------------------------
+static Plan make_plan_split(int64_t na_blocks, int64_t nb_blocks, int64_t ks, int64_t t) {
+    Plan p;
+    plan_register_resident(p, na_blocks, nb_blocks, split_b_blocks_per_wg(ks), ks * 3 * 64 * 16, 32, kSplitMaxCols, t,
+                           (int64_t)sizeof(float));
+    return p;
+}
+static size_t split_planar_bytes(int64_t n_a, int64_t t) {
+    return align256((size_t)t * (size_t)((n_a + 31) / 32 * 32) * sizeof(float));
+}
+static size_t split_partial_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t) {
+    SplitView A = split_view(nullptr, n_a, d), B = split_view(nullptr, n_b, d);
+    Plan p = make_plan_split(A.nblk, B.nblk, A.ks, t);
+    int64_t tc = t < p.col_chunk ? t : p.col_chunk;
+    return align256((size_t)p.partials * tc * B.npad * sizeof(float));
+}
+
+// out[b,t] = sum_a K(A_a,B_b) vecp[t][a] (+ addend).  vecp is planar [t][A.npad].
+static int mmv_split_planar(int kf, const SplitView &A, const SplitView &B, const float *vecp, int64_t t,
+                            const float *addend, int64_t add_rs, int64_t add_cs, float *out, int64_t out_rs,
+                            int64_t out_cs, bool zero_pad, float *partial, size_t partial_avail, hipStream_t st) {
+    if (B.n == 0 || t == 0) return FLK_OK;
+    Plan p = make_plan_split(A.nblk, B.nblk, A.ks, t);
+    for (int64_t t0 = 0; t0 < t; t0 += p.col_chunk) {
+        int tc = (int)(t - t0 < p.col_chunk ? t - t0 : p.col_chunk);
+        if ((size_t)p.partials * tc * B.npad * sizeof(float) > partial_avail)
+            return fail(FLK_ENOMEM, "workspace too small for %d partial sums of %lld x %d", p.partials,
+                        (long long)B.npad, tc);
+        int partials = p.partials;
+        if (A.nblk == 0) {
+            partials = 0;
+        } else {
+            ScopedKernelTimer timer(st);
+            int rc = launch_mmv_split(kf, A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st);
+            if (rc != FLK_OK) return rc;
+        }
+        int rc = launch_finalize<float>(partial, partials, tc, B.n, B.npad, addend ? addend + t0 * add_cs : nullptr,
+                                        add_rs, add_cs, out + t0 * out_cs, out_rs, out_cs, zero_pad, st);
+        if (rc != FLK_OK) return rc;
+    }
+    return FLK_OK;
+}
+
+static int pack_split_impl(int kf, const char *name, const void *X, int64_t n, int64_t d, int64_t rs, int64_t cs,
+                           const void *sigma, int64_t n_sigma, void *packed, hipStream_t st) {
+    int rc = check_matrix(name, X, n, d, rs, cs);
+    if (rc) return rc;
+    if (sigma == nullptr) return fail(FLK_EINVAL, "sigma: null pointer");
+    if (n_sigma != 1 && n_sigma != d)
+        return fail(FLK_EINVAL, "The size of sigma (%lld) must match the number of features (%lld) or be 1",
+                    (long long)n_sigma, (long long)d);
+    return launch_pack_split((const float *)X, n, d, rs, cs, (const float *)sigma, n_sigma, operand_scale(kf), packed, st);
+}
+
+static size_t fmmv_split_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {
+    return split_packed_bytes(n, d) + split_packed_bytes(m, d) + split_planar_bytes(m, t) +
+           split_partial_bytes(m, n, d, t);
+}
+static size_t fdmmv_split_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {
+    size_t p1 = split_partial_bytes(m, n, d, t), p2 = split_partial_bytes(n, m, d, t);
+    return split_packed_bytes(n, d) + split_packed_bytes(m, d) + split_planar_bytes(m, t) + split_planar_bytes(n, t) +
+           (p1 > p2 ? p1 : p2);
+}
+
+static int fmmv_split_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
+                           int64_t x2_rs, int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v,
+                           int64_t v_rs, int64_t v_cs, int64_t t, void *out, int64_t out_rs, int64_t out_cs, void *ws,
+                           size_t ws_bytes, hipStream_t st) {
+    if (n < 0 || m < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
+    int rc;
+    if ((rc = check_matrix("v", v, m, t, v_rs, v_cs))) return rc;
+    if ((rc = check_matrix("out", out, n, t, out_rs, out_cs))) return rc;
+    size_t need = fmmv_split_ws_bytes(n, m, d, t);
+    if (ws_bytes < need || (need > 0 && ws == nullptr))
+        return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+    char *p = (char *)ws;
+    void *px = p; p += split_packed_bytes(n, d);
+    void *pc = p; p += split_packed_bytes(m, d);
+    float *vp = (float *)p; p += split_planar_bytes(m, t);
+    float *partial = (float *)p;
+    if ((rc = pack_split_impl(kf, "X1", X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, st))) return rc;
+    if ((rc = pack_split_impl(kf, "X2", X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, st))) return rc;
+    SplitView X = split_view(px, n, d), C = split_view(pc, m, d);
+    if (n == 0 || t == 0) return FLK_OK;
+    if ((rc = launch_vec_planar<float>((const float *)v, m, t, v_rs, v_cs, vp, C.npad, 0, st))) return rc;
+    return mmv_split_planar(kf, C, X, vp, t, nullptr, 0, 0, (float *)out, out_rs, out_cs, false, partial,
+                            ws_bytes - (size_t)(p - (char *)ws), st);
+}
+
+static int fdmmv_split_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
+                            int64_t x2_rs, int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v,
+                            int64_t v_rs, int64_t v_cs, const void *w, int64_t w_rs, int64_t w_cs, int64_t t, void *out,
+                            int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes, hipStream_t st) {
+    if (n < 0 || m < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
+    int rc;
+    if (v == nullptr && m > 0 && t > 0) return fail(FLK_EINVAL, "v: null pointer (v is required)");
+    if ((rc = check_matrix("v", v, m, t, v_rs, v_cs))) return rc;
+    if (w && (rc = check_matrix("w", w, n, t, w_rs, w_cs))) return rc;
+    if ((rc = check_matrix("out", out, m, t, out_rs, out_cs))) return rc;
+    size_t need = fdmmv_split_ws_bytes(n, m, d, t);
+    if (ws_bytes < need || (need > 0 && ws == nullptr))
+        return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+    char *p = (char *)ws;
+    void *px = p; p += split_packed_bytes(n, d);
+    void *pc = p; p += split_packed_bytes(m, d);
+    float *vp = (float *)p; p += split_planar_bytes(m, t);     // v multiplies the rows of C in K v
+    float *up = (float *)p; p += split_planar_bytes(n, t);     // u multiplies the rows of X in K^T u
+    float *partial = (float *)p;
+    size_t partial_avail = ws_bytes - (size_t)(p - (char *)ws);
+    if ((rc = pack_split_impl(kf, "X1", X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, st))) return rc;
+    if ((rc = pack_split_impl(kf, "X2", X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, st))) return rc;
+    SplitView X = split_view(px, n, d), C = split_view(pc, m, d);
+    if (m == 0 || t == 0) return FLK_OK;
+    if ((rc = launch_vec_planar<float>((const float *)v, m, t, v_rs, v_cs, vp, C.npad, 0, st))) return rc;
+    // u = K v + w, planar [t][X.npad] with zeroed padding rows so it can feed the second product directly
+    if ((rc = mmv_split_planar(kf, C, X, vp, t, (const float *)w, w_rs, w_cs, up, 1, X.npad, true, partial,
+                               partial_avail, st)))
+        return rc;
+    return mmv_split_planar(kf, X, C, up, t, nullptr, 0, 0, (float *)out, out_rs, out_cs, false, partial, partial_avail,
+                            st);
+}
+
 }  // namespace flk
 
 using namespace flk;
@@ -437,6 +574,7 @@ int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b
 
 size_t flk_gauss_fmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
+    if (dtype == FLK_F32_BF16X3 && d <= kSplitMaxD) return fmmv_split_ws_bytes(n, m, d, t);
     return dtype == FLK_F64 ? fmmv_ws_bytes<double>(n, m, d, t) : fmmv_ws_bytes<float>(n, m, d, t);
 }
 
@@ -446,7 +584,10 @@ int flk_kernel_fmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_
                     void *workspace, size_t workspace_bytes, void *stream) {
     g_err[0] = 0;
     FLK_CHECK_KERNEL(kernel);
-    if (dtype == FLK_F32)
+    if (dtype == FLK_F32_BF16X3 && d <= kSplitMaxD)
+        return fmmv_split_impl(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t, out,
+                               out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    if (dtype == FLK_F32 || dtype == FLK_F32_BF16X3)
         return fmmv_impl<float>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t,
                                 out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
     if (dtype == FLK_F64)
@@ -465,6 +606,7 @@ int flk_gauss_fmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, cons
 
 size_t flk_gauss_fdmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
+    if (dtype == FLK_F32_BF16X3 && d <= kSplitMaxD) return fdmmv_split_ws_bytes(n, m, d, t);
     return dtype == FLK_F64 ? fdmmv_ws_bytes<double>(n, m, d, t) : fdmmv_ws_bytes<float>(n, m, d, t);
 }
 
@@ -475,7 +617,10 @@ int flk_kernel_fdmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64
                      void *stream) {
     g_err[0] = 0;
     FLK_CHECK_KERNEL(kernel);
-    if (dtype == FLK_F32)
+    if (dtype == FLK_F32_BF16X3 && d <= kSplitMaxD)
+        return fdmmv_split_impl(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
+                                w_rs, w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
+    if (dtype == FLK_F32 || dtype == FLK_F32_BF16X3)
         return fdmmv_impl<float>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
                                  w_rs, w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
     if (dtype == FLK_F64)

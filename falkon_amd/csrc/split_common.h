@@ -1,0 +1,65 @@
+// "bf16x3" mode of the fp32 products, gfx950: the cross term x~.c~ runs on the bf16 matrix cores.
+//
+// Every scaled fp32 value is written as the sum of three bfloat16 numbers, x~ = hi + mid + lo (each the
+// round-to-nearest of what the previous ones leave: 3 x 8 = 24 significant bits, i.e. the fp32 value itself), and
+// the product of two such sums is accumulated from the six partial products whose weight is at least 2^-16 of
+// the leading one (hi.hi, hi.mid, mid.hi, hi.lo, lo.hi, mid.mid; the dropped ones are below 2^-24).  Products of
+// bfloat16 numbers are exact in fp32 and v_mfma_f32_32x32x16_bf16 accumulates in fp32, so the exponent has the
+// accuracy of an fp32 dot product, at 16 features per MFMA instead of 2.  bfloat16 has the exponent range of
+// fp32: no input range is lost.
+//
+// Packed operand: [block of 32 rows][k-step of 16 features][piece hi/mid/lo][lane 0..63][8 bfloat16], lane l
+// holding features 8*(l/32) .. +7 of row l%32: one global_load_dwordx4 per lane is one MFMA operand.  The last
+// two features of the padded row hold 1.0 and the row's half norm h = -1/2 |x~|^2 (split like everything else).
+// The kernel swaps that pair in the resident (B side) fragments, so that the MFMA chain adds 1*hB + hA*1 by
+// itself and the accumulator leaves the chain as the complete exponent.
+#pragma once
+#include "flk_common.h"
+
+namespace flk {
+
+constexpr int64_t kSplitMaxD = 62;          // four k-steps, two of the 64 features taken by (1, h)
+constexpr int kSplitMaxCols = 2;            // right-hand sides per pass
+
+inline int64_t split_ksteps(int64_t d) { return (d + 2 + 15) / 16; }
+
+struct SplitView {
+    const void *data;   // [nblk][ks][3][64] x 16 bytes
+    int64_t n, d, ks, nblk, npad;
+};
+inline size_t split_packed_bytes(int64_t n, int64_t d) {
+    const int64_t nblk = (n + 31) / 32;
+    return align256((size_t)nblk * split_ksteps(d) * 3 * 64 * 16);
+}
+inline SplitView split_view(const void *buf, int64_t n, int64_t d) {
+    SplitView v;
+    v.data = buf; v.n = n; v.d = d;
+    v.ks = split_ksteps(d);
+    v.nblk = (n + 31) / 32;
+    v.npad = v.nblk * 32;
+    return v;
+}
+// B blocks (of 32 output rows) per workgroup of the product kernel
+inline int split_b_blocks_per_wg(int64_t ks) { return 4 * (ks <= 2 ? 4 : 2); }
+
+int launch_pack_split(const float *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const float *sigma, int64_t n_sigma,
+                      double scale, void *packed, hipStream_t st);
+
+#define FLK_DECLARE_SPLIT_KF(KF)                                                                              \
+    int launch_mmv_split_kf##KF(const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld,    \
+                                int tcols, int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st);
+FLK_DECLARE_SPLIT_KF(0)
+FLK_DECLARE_SPLIT_KF(1)
+FLK_DECLARE_SPLIT_KF(2)
+FLK_DECLARE_SPLIT_KF(3)
+FLK_DECLARE_SPLIT_KF(4)
+#undef FLK_DECLARE_SPLIT_KF
+
+inline int launch_mmv_split(int kf, const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld, int tcols,
+                            int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
+#define FLK_CALL(KF) launch_mmv_split_kf##KF(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)
+    FLK_SWITCH_KF(kf, FLK_CALL)
+#undef FLK_CALL
+}
+
+}  // namespace flk

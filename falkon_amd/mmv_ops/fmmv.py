@@ -33,10 +33,18 @@ def _stream_handle(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
-def gauss_fmmv_native(X1, X2, sigma_dev, v, out, kernel_fn: int = _backend.FLK_GAUSSIAN) -> None:
+def _arith_code(dtype: torch.dtype, opt: Optional[BaseOptions]) -> int:
+    """The library's dtype code: the data's dtype, or the bf16x3 mode of fp32 when the options ask for it."""
+    if dtype == torch.float32 and opt is not None and getattr(opt, "bf16x3_cross_term", False):
+        return _backend.FLK_F32_BF16X3
+    return _DTYPE_CODE[dtype]
+
+
+def gauss_fmmv_native(X1, X2, sigma_dev, v, out, kernel_fn: int = _backend.FLK_GAUSSIAN,
+                      code: Optional[int] = None) -> None:
     """out[n,t] = K(X1,X2) @ v through ``flk_kernel_fmmv``.  All tensors on one GPU, 2-D, same dtype."""
     lib = _backend.load()
-    code = _DTYPE_CODE[X1.dtype]
+    code = _DTYPE_CODE[X1.dtype] if code is None else code
     n, d = X1.shape
     m, t = v.shape
     ws_bytes = lib.flk_gauss_fmmv_workspace_bytes(n, m, d, t, code)
@@ -51,10 +59,11 @@ def gauss_fmmv_native(X1, X2, sigma_dev, v, out, kernel_fn: int = _backend.FLK_G
     _backend.raise_for_status(rc, "flk_kernel_fmmv")
 
 
-def gauss_fdmmv_native(X1, X2, sigma_dev, v, w, out, kernel_fn: int = _backend.FLK_GAUSSIAN) -> None:
+def gauss_fdmmv_native(X1, X2, sigma_dev, v, w, out, kernel_fn: int = _backend.FLK_GAUSSIAN,
+                       code: Optional[int] = None) -> None:
     """out[m,t] = K^T (K v + w) through ``flk_kernel_fdmmv``.  ``w`` may be None."""
     lib = _backend.load()
-    code = _DTYPE_CODE[X1.dtype]
+    code = _DTYPE_CODE[X1.dtype] if code is None else code
     n, d = X1.shape
     m, t = v.shape
     ws_bytes = lib.flk_gauss_fdmmv_workspace_bytes(n, m, d, t, code)
@@ -276,7 +285,7 @@ def _fmmv_run(X1, X2, v, kernel, kernel_fn: int, out, opt: BaseOptions, cached_s
     M, T = v.shape
     out = create_output_mat(out, data_devs, shape=(N, T), dtype=v.dtype, other_mat=X1)
     lib = _backend.load()
-    code, sz = _DTYPE_CODE[X1.dtype], sizeof_dtype(X1.dtype)
+    code, sz = _arith_code(X1.dtype, opt), sizeof_dtype(X1.dtype)
     x1_in, out_in = X1.device == dev, out.device == dev
 
     with torch.inference_mode():
@@ -295,7 +304,7 @@ def _fmmv_run(X1, X2, v, kernel, kernel_fn: int, out, opt: BaseOptions, cached_s
             for i in range(0, N, max(blk, 1)):
                 li = min(blk, N - i)
                 outd = out[i:i + li] if out_in else torch.empty((li, T), dtype=out.dtype, device=dev)
-                gauss_fmmv_native(X1[i:i + li], X2d, sigma_dev, vd, outd, kernel_fn)
+                gauss_fmmv_native(X1[i:i + li], X2d, sigma_dev, vd, outd, kernel_fn, code)
                 if not out_in:
                     out[i:i + li].copy_(outd)
         elif N > 0:
@@ -304,7 +313,7 @@ def _fmmv_run(X1, X2, v, kernel, kernel_fn: int, out, opt: BaseOptions, cached_s
             chunk = _streamed_chunk_rows(N, D * sz, blk)
             full = out if out_in else torch.empty((N, T), dtype=out.dtype, device=dev)
             for i, li, (X1d,) in _HostRowStream([X1], N, dev, chunk):
-                gauss_fmmv_native(X1d, X2d, sigma_dev, vd, full[i:i + li], kernel_fn)
+                gauss_fmmv_native(X1d, X2d, sigma_dev, vd, full[i:i + li], kernel_fn, code)
             if not out_in:
                 out.copy_(full)
     return out
@@ -333,7 +342,7 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
     N, D = X1.shape[-2:]
     M, T = v.shape[-2:]
     lib = _backend.load()
-    code, sz = _DTYPE_CODE[X1.dtype], sizeof_dtype(X1.dtype)
+    code, sz = _arith_code(X1.dtype, opt), sizeof_dtype(X1.dtype)
 
     with torch.inference_mode():
         out = create_output_mat(out, data_devs, shape=(M, T), dtype=v.dtype, other_mat=X1)
@@ -364,10 +373,10 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
         first = True
         for _, _, (X1d, wd) in chunks:
             if first:
-                gauss_fdmmv_native(X1d, X2d, sigma_dev, vd, wd, outd, kernel_fn)
+                gauss_fdmmv_native(X1d, X2d, sigma_dev, vd, wd, outd, kernel_fn, code)
             else:
                 tmp = torch.empty((M, T), dtype=out.dtype, device=dev) if tmp is None else tmp
-                gauss_fdmmv_native(X1d, X2d, sigma_dev, vd, wd, tmp, kernel_fn)
+                gauss_fdmmv_native(X1d, X2d, sigma_dev, vd, wd, tmp, kernel_fn, code)
                 outd.add_(tmp)
             first = False
         if first:                                           # no rows at all: K^T (K v + w) is an empty sum

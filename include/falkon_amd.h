@@ -14,7 +14,13 @@
  * (falkon/mmv_ops/utils.py:36-39 requires only that some stride equals one).
  *
  * dtype: FLK_F32 (0) or FLK_F64 (1); all operands of a call share it
- * (falkon/kernels/kernel.py:78-79,102-103).
+ * (falkon/kernels/kernel.py:78-79,102-103).  FLK_F32_BF16X3 (2), accepted by the fmmv / fdmmv entry
+ * points and their workspace queries only, is fp32 data and fp32 results with the cross term x.c of the
+ * squared distance formed on the bfloat16 matrix cores: every scaled fp32 value is split exactly into
+ * three bfloat16 pieces (3 x 8 = 24 significant bits) and six partial products are accumulated in fp32,
+ * which keeps the accuracy of the fp32 dot product (measured: the same distance from the fp64 result as
+ * FLK_F32) at 16 features per matrix instruction instead of 2.  It has no counterpart in the reference;
+ * it applies to d <= 62 and is FLK_F32 otherwise.
  */
 #ifndef FALKON_AMD_H
 #define FALKON_AMD_H
@@ -28,6 +34,7 @@ extern "C" {
 
 #define FLK_F32 0
 #define FLK_F64 1
+#define FLK_F32_BF16X3 2
 
 /* Radial kernels K(x, c) = f(D), D = |x/sigma - c/sigma| (falkon/kernels/distance_kernel.py):
  * Gaussian exp(-D^2/2) (:140-159), Laplacian exp(-D) (:182-205), Matern nu = 3/2 and 5/2 (:225-269;

@@ -1,0 +1,126 @@
+"""The bf16x3 mode of the fp32 products (``FalkonOptions(bf16x3_cross_term=True)``, dtype code FLK_F32_BF16X3 of the
+C ABI): the cross term of the squared distance on the bfloat16 matrix cores from an exact three-way bfloat16 split
+of the scaled rows.  It must meet the same bar as the plain fp32 kernels (1e-5 relative, norm-wise per column,
+against the CPU oracle) and must not be less accurate than they are against the fp64 result.
+"""
+import numpy as np
+import pytest
+import torch
+
+from falkon_amd import Falkon, FalkonOptions, GaussianKernel, LaplacianKernel, MaternKernel
+from oracle import brute, inputs, mmv_ref
+from conftest import check_parity, rel_err
+
+pytestmark = pytest.mark.gpu
+
+SPLIT = FalkonOptions(bf16x3_cross_term=True)
+PLAIN = FalkonOptions(bf16x3_cross_term=False)
+
+
+def _data(n, m, d, t, seed, scale=1.0):
+    g = np.random.default_rng(seed)
+    mk = lambda *shape: torch.from_numpy(g.standard_normal(shape).astype(np.float32))     # noqa: E731
+    return mk(n, d) * scale, mk(m, d) * scale, mk(m, t), mk(n, t)
+
+
+@pytest.mark.parametrize("d", [1, 2, 9, 13, 14, 15, 28, 30, 31, 46, 47, 62])
+@pytest.mark.parametrize("t", [1, 2, 3, 5])
+def test_products_vs_oracle(dev, d, t):
+    n, m = 700 + 3 * d, 190 + d
+    X, C, v, w = _data(n, m, d, t, seed=d + 100 * t)
+    sigma = torch.tensor([0.9 * np.sqrt(d)], dtype=torch.float64)
+    k = GaussianKernel(sigma, opt=SPLIT)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+    check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)
+    check_parity(k.dmmv(Xg, Cg, vg, wg), mmv_ref.fdmmv_ref(X, C, v, w, sigma),
+                 mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), 1e-5)
+    check_parity(k.dmmv(Xg, Cg, vg, None), mmv_ref.fdmmv_ref(X, C, v, None, sigma),
+                 mmv_ref.fdmmv_ref(Xd, Cd, vd, None, sigma), 1e-5)
+
+
+def test_layouts_sigma_per_dimension_and_repeatability(dev):
+    X, C, v, w = _data(1500, 333, 11, 2, seed=7)
+    sigma = torch.from_numpy(np.random.default_rng(3).uniform(1.0, 4.0, 11))
+    k = GaussianKernel(sigma, opt=SPLIT)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    ref = k.dmmv(Xg, Cg, vg, wg)
+    check_parity(ref, mmv_ref.fdmmv_ref(X, C, v, w, sigma),
+                 mmv_ref.fdmmv_ref(X.double(), C.double(), v.double(), w.double(), sigma), 1e-5)
+    # Fortran-ordered operands, an `out` buffer, a second call: bit-identical
+    f = lambda a: a.T.contiguous().T                                                      # noqa: E731
+    out = torch.empty(333, 2, dtype=torch.float32, device=dev)
+    res = k.dmmv(f(Xg), f(Cg), f(vg), f(wg), out=out)
+    assert res.data_ptr() == out.data_ptr() and torch.equal(res, ref)
+    assert torch.equal(k.dmmv(Xg, Cg, vg, wg), ref)
+    # host data goes through the same kernels
+    assert torch.equal(k.dmmv(X, C, v, w).to(dev), ref)
+
+
+def test_feature_counts_beyond_the_split_kernels_use_plain_fp32(dev):
+    X, C, v, w = _data(400, 150, 63, 2, seed=5)
+    sigma = torch.tensor([8.0], dtype=torch.float64)
+    a = GaussianKernel(sigma, opt=SPLIT).dmmv(X.to(dev), C.to(dev), v.to(dev), w.to(dev))
+    b = GaussianKernel(sigma, opt=PLAIN).dmmv(X.to(dev), C.to(dev), v.to(dev), w.to(dev))
+    assert torch.equal(a, b)
+    X, C, v, w = _data(300, 140, 200, 3, seed=6)
+    a = GaussianKernel(15.0, opt=SPLIT).mmv(X.to(dev), C.to(dev), v.to(dev))
+    b = GaussianKernel(15.0, opt=PLAIN).mmv(X.to(dev), C.to(dev), v.to(dev))
+    assert torch.equal(a, b)
+    # fp64 data is not affected by the option
+    Xd, Cd, vd = X.double().to(dev), C.double().to(dev), v.double().to(dev)
+    assert torch.equal(GaussianKernel(15.0, opt=SPLIT).mmv(Xd, Cd, vd), GaussianKernel(15.0, opt=PLAIN).mmv(Xd, Cd, vd))
+
+
+@pytest.mark.parametrize("name,make", [("laplacian", lambda s: LaplacianKernel(s, opt=SPLIT)),
+                                       ("1.5-matern", lambda s: MaternKernel(s, 1.5, opt=SPLIT)),
+                                       ("2.5-matern", lambda s: MaternKernel(s, 2.5, opt=SPLIT))])
+def test_other_kernel_functions(dev, name, make):
+    X, C, v, w = _data(900, 260, 20, 2, seed=9)
+    sigma = torch.tensor([4.0], dtype=torch.float64)
+    k = make(sigma)
+    got = k.dmmv(X.to(dev), C.to(dev), v.to(dev), w.to(dev))
+    check_parity(got, mmv_ref.fdmmv_ref(X, C, v, w, sigma, kernel_name=name),
+                 mmv_ref.fdmmv_ref(X.double(), C.double(), v.double(), w.double(), sigma, kernel_name=name), 1e-5)
+    K = brute.radial_brute(X, C, sigma, name)
+    assert rel_err(k.mmv(X.to(dev), C.to(dev), v.to(dev)), K @ v.double().numpy()) < 5e-6
+
+
+@pytest.mark.parametrize("scale", [1e-3, 1.0, 30.0])
+def test_accuracy_is_that_of_the_fp32_kernels(dev, scale):
+    """Against the fp64 closed form the split mode may not be further away than the plain fp32 kernels (small slack):
+    data far from the origin (large norms, where the expanded squared distance cancels most) included."""
+    X, C, v, _ = _data(4000, 500, 28, 1, seed=11, scale=scale)
+    X, C = X + 2.0 * scale, C + 2.0 * scale
+    sigma = torch.tensor([3.8 * scale], dtype=torch.float64)
+    exact = brute.radial_brute(X, C, sigma, "gaussian") @ v.double().numpy()
+    Xg, Cg, vg = X.to(dev), C.to(dev), v.to(dev)
+    e_split = rel_err(GaussianKernel(sigma, opt=SPLIT).mmv(Xg, Cg, vg), exact)
+    e_plain = rel_err(GaussianKernel(sigma, opt=PLAIN).mmv(Xg, Cg, vg), exact)
+    assert e_split <= 1.5 * e_plain + 2e-7, (e_split, e_plain)
+
+
+def test_config2_and_config3_shapes_reduced(dev):
+    for name, N, M in (("C2", 100_000, 5_000), ("C3", 200_000, 5_000)):
+        X, C, sigma, v, w = inputs.make_config(name, N=N, M=M)
+        k = GaussianKernel(sigma, opt=SPLIT)
+        got = k.dmmv(X.to(dev), C.to(dev), v.to(dev), None if w is None else w.to(dev))
+        wd = None if w is None else w.double()
+        check_parity(got, mmv_ref.fdmmv_ref(X, C, v, w, sigma, max_cpu_mem=2 * 2**30),
+                     mmv_ref.fdmmv_ref(X.double(), C.double(), v.double(), wd, sigma, max_cpu_mem=4 * 2**30), 1e-5)
+
+
+def test_falkon_fit_predict_with_the_option(dev):
+    """End to end: the same model with and without the option (the preconditioner does not depend on it)."""
+    g = np.random.default_rng(21)
+    X = torch.from_numpy(g.standard_normal((20_000, 10)).astype(np.float32))
+    a = g.standard_normal(10) / np.sqrt(10)
+    y = torch.from_numpy(np.sign(np.sin(X.numpy() @ a) + 0.3 * g.standard_normal(20_000)).astype(np.float32)).reshape(-1, 1)
+    preds = []
+    for opt in (SPLIT, PLAIN):
+        model = Falkon(GaussianKernel(2.5, opt=opt), penalty=1e-6, M=1_000, maxiter=15, seed=3, options=opt)
+        model.fit(X.to(dev), y.to(dev))
+        preds.append(model.predict(X[:4000].to(dev)).cpu())
+    mse = [float(((p - y[:4000]) ** 2).mean()) for p in preds]
+    assert abs(mse[0] - mse[1]) <= 1e-3 * mse[1]
+    assert rel_err(preds[0], preds[1]) < 1e-3
