@@ -61,6 +61,12 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
+# the same for the bf16x3 product kernel (profiles/mmv_split_kernel__C2_dfmmv_bf16x3.md)
+MEASURED_TRAFFIC_BYTES_BF16X3 = {
+    "C2": int((536594.0 * 2.0 + 17773.4 * 1.0) * 1024),    # 1.12 GB: the packed centres no longer fit one L2 next to X
+}
+
+
 def make_inputs(name):
     """Synthetic inputs of the named configuration (draw order X, idx, sigma, v, w)."""
     seed, N, d, M, T, has_w = WORKLOADS[name]
