@@ -26,14 +26,15 @@ FP64_PEAK_TFLOPS = 78.6    # MI355X fp64 matrix peak = fp64 vector peak
 BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 
 
-def split_roofline(pairs, d, kern_ms, algorithmic_flop):
+def split_roofline(pairs, d, kern_ms, algorithmic_flop, traffic=None):
     """Roofline of the bf16x3 product kernel: it executes 6 partial products over the features padded to whole
     k-steps of 16 (two of them carry the half norms), on the bf16 matrix cores."""
     ksteps = (d + 2 + 15) // 16
     executed = pairs * 6 * 2 * 16 * ksteps
     achieved = executed / (kern_ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": achieved / BF16_PEAK_TFLOPS, "traffic": None, "kernel": "mmv_split_kernel",
+            "frac": achieved / BF16_PEAK_TFLOPS, "traffic": traffic,
+            "kernel": "mmv_split_kernel" if d <= 62 else "mmv_split_large_kernel",
             "avg_launch_ms": kern_ms, "flop_per_launch": executed,
             "note": "achieved = bf16 MFMA flops the kernel executes (6 partial products, padded features); "
                     "algorithmic fp32 flops per launch and their rate are given beside it",
@@ -229,7 +230,7 @@ def main():
                          "Gaussian's 2d+4+2T per pair, the other kernels spend a few more VALU operations per entry)")
     ap.add_argument("--cross-term", default="f32", choices=["f32", "bf16x3"],
                     help="f32 (the headline): fp32 MFMA.  bf16x3: the opt-in mode that forms x.c on the bf16 matrix cores "
-                         "from an exact three-way bfloat16 split of the fp32 rows (fp32 accuracy; d <= 62, fp32 data); "
+                         "from an exact three-way bfloat16 split of the fp32 rows (fp32 accuracy; fp32 data); "
                          "its roofline is priced against the bf16 MFMA peak on the flops it executes")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=0)
@@ -268,8 +269,8 @@ def main():
     dev = torch.device("cuda:0")
     seed, N, d, M, T, has_w = WORKLOADS[args.workload]
     split = args.cross_term == "bf16x3"
-    if split and (d > 62 or args.dtype != "f32"):
-        print("bench.py: --cross-term bf16x3 applies to fp32 data with d <= 62 (workloads C2, C3, C5)", file=sys.stderr)
+    if split and args.dtype != "f32":
+        print("bench.py: --cross-term bf16x3 applies to fp32 data", file=sys.stderr)
         sys.exit(2)
     X, C, sigma, v, w = make_inputs(args.workload)
     tdt = torch.float32 if args.dtype == "f32" else torch.float64
@@ -327,7 +328,8 @@ def main():
                                 / (elapsed / args.steps) / 1e12 / peak,
     }
     if split:
-        res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch),
+        res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch,
+                                              MEASURED_TRAFFIC_BYTES_BF16X3.get(args.workload)),
                                launches_per_step=launches.value / args.steps)
     if not args.no_cpu_baseline and args.op == "dmmv":
         rows = args.cpu_rows or {"C2": N, "C3": 400_000, "C4": 100_000}[args.workload]

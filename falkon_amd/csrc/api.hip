@@ -358,13 +358,31 @@ static int fmm_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1
 }
 
 // ---------------------------------------------------------------------------
-// bf16x3 mode of the fp32 products (split_common.h): same drivers on the split operands.  Feature counts beyond
-// kSplitMaxD have no split kernel and take the plain fp32 path (the callers below decide).
+// bf16x3 mode of the fp32 products (split_common.h): same drivers on the split operands; register-resident kernel
+// up to kSplitMaxD features, LDS-tiled kernel beyond.
 // ---------------------------------------------------------------------------
+constexpr int64_t kTargetWgsSplitLarge = 16384;  // two 256-thread workgroups per CU: 32 rounds
+
 static Plan make_plan_split(int64_t na_blocks, int64_t nb_blocks, int64_t ks, int64_t t) {
     Plan p;
-    plan_register_resident(p, na_blocks, nb_blocks, split_b_blocks_per_wg(ks), ks * 3 * 64 * 16, 32, kSplitMaxCols, t,
-                           (int64_t)sizeof(float));
+    if (ks * 16 <= kSplitMaxD + 2) {
+        plan_register_resident(p, na_blocks, nb_blocks, split_b_blocks_per_wg(ks), ks * 3 * 64 * 16, 32, kSplitMaxCols,
+                               t, (int64_t)sizeof(float));
+        return p;
+    }
+    p.large = true;
+    const int64_t a_tiles = (na_blocks + split_large_a_tile_blocks() - 1) / split_large_a_tile_blocks();
+    const int64_t b_tiles = (nb_blocks + split_large_b_tile_blocks() - 1) / split_large_b_tile_blocks();
+    int64_t splits = (kTargetWgsSplitLarge + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
+    if (splits > a_tiles) splits = a_tiles;
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    if (splits < 1) splits = 1;
+    p.chunk = (a_tiles + splits - 1) / splits;
+    if (p.chunk < 1) p.chunk = 1;
+    p.splits = (int)((a_tiles + p.chunk - 1) / p.chunk);
+    if (p.splits < 1) p.splits = 1;
+    p.partials = p.splits * split_large_partials_per_split();
+    p.col_chunk = split_large_max_cols();
     return p;
 }
 static size_t split_planar_bytes(int64_t n_a, int64_t t) {
@@ -393,7 +411,8 @@ static int mmv_split_planar(int kf, const SplitView &A, const SplitView &B, cons
             partials = 0;
         } else {
             ScopedKernelTimer timer(st);
-            int rc = launch_mmv_split(kf, A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st);
+            int rc = p.large ? launch_mmv_split_large(kf, A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st)
+                             : launch_mmv_split(kf, A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st);
             if (rc != FLK_OK) return rc;
         }
         int rc = launch_finalize<float>(partial, partials, tc, B.n, B.npad, addend ? addend + t0 * add_cs : nullptr,
@@ -574,7 +593,7 @@ int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b
 
 size_t flk_gauss_fmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
-    if (dtype == FLK_F32_BF16X3 && d <= kSplitMaxD) return fmmv_split_ws_bytes(n, m, d, t);
+    if (dtype == FLK_F32_BF16X3) return fmmv_split_ws_bytes(n, m, d, t);
     return dtype == FLK_F64 ? fmmv_ws_bytes<double>(n, m, d, t) : fmmv_ws_bytes<float>(n, m, d, t);
 }
 
@@ -584,10 +603,10 @@ int flk_kernel_fmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_
                     void *workspace, size_t workspace_bytes, void *stream) {
     g_err[0] = 0;
     FLK_CHECK_KERNEL(kernel);
-    if (dtype == FLK_F32_BF16X3 && d <= kSplitMaxD)
+    if (dtype == FLK_F32_BF16X3)
         return fmmv_split_impl(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t, out,
                                out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    if (dtype == FLK_F32 || dtype == FLK_F32_BF16X3)
+    if (dtype == FLK_F32)
         return fmmv_impl<float>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t,
                                 out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
     if (dtype == FLK_F64)
@@ -606,7 +625,7 @@ int flk_gauss_fmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, cons
 
 size_t flk_gauss_fdmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
-    if (dtype == FLK_F32_BF16X3 && d <= kSplitMaxD) return fdmmv_split_ws_bytes(n, m, d, t);
+    if (dtype == FLK_F32_BF16X3) return fdmmv_split_ws_bytes(n, m, d, t);
     return dtype == FLK_F64 ? fdmmv_ws_bytes<double>(n, m, d, t) : fdmmv_ws_bytes<float>(n, m, d, t);
 }
 
@@ -617,10 +636,10 @@ int flk_kernel_fdmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64
                      void *stream) {
     g_err[0] = 0;
     FLK_CHECK_KERNEL(kernel);
-    if (dtype == FLK_F32_BF16X3 && d <= kSplitMaxD)
+    if (dtype == FLK_F32_BF16X3)
         return fdmmv_split_impl(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
                                 w_rs, w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    if (dtype == FLK_F32 || dtype == FLK_F32_BF16X3)
+    if (dtype == FLK_F32)
         return fdmmv_impl<float>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
                                  w_rs, w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
     if (dtype == FLK_F64)

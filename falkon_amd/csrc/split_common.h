@@ -18,8 +18,8 @@
 
 namespace flk {
 
-constexpr int64_t kSplitMaxD = 62;          // four k-steps, two of the 64 features taken by (1, h)
-constexpr int kSplitMaxCols = 2;            // right-hand sides per pass
+constexpr int64_t kSplitMaxD = 62;          // register-resident kernel: four k-steps, two of the 64 features taken by (1, h)
+constexpr int kSplitMaxCols = 2;            // its right-hand sides per pass
 
 inline int64_t split_ksteps(int64_t d) { return (d + 2 + 15) / 16; }
 
@@ -45,9 +45,18 @@ inline int split_b_blocks_per_wg(int64_t ks) { return 4 * (ks <= 2 ? 4 : 2); }
 int launch_pack_split(const float *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const float *sigma, int64_t n_sigma,
                       double scale, void *packed, hipStream_t st);
 
+// LDS-tiled kernel for larger feature counts: tile geometry and right-hand sides per pass
+int split_large_a_tile_blocks();
+int split_large_b_tile_blocks();
+int split_large_partials_per_split();
+int split_large_max_cols();
+
 #define FLK_DECLARE_SPLIT_KF(KF)                                                                              \
     int launch_mmv_split_kf##KF(const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld,    \
-                                int tcols, int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st);
+                                int tcols, int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st); \
+    int launch_mmv_split_large_kf##KF(const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld, \
+                                      int tcols, int64_t a_tiles_per_chunk, int splits, float *partial,        \
+                                      hipStream_t st);
 FLK_DECLARE_SPLIT_KF(0)
 FLK_DECLARE_SPLIT_KF(1)
 FLK_DECLARE_SPLIT_KF(2)
@@ -58,6 +67,13 @@ FLK_DECLARE_SPLIT_KF(4)
 inline int launch_mmv_split(int kf, const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld, int tcols,
                             int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
 #define FLK_CALL(KF) launch_mmv_split_kf##KF(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)
+    FLK_SWITCH_KF(kf, FLK_CALL)
+#undef FLK_CALL
+}
+
+inline int launch_mmv_split_large(int kf, const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld,
+                                  int tcols, int64_t a_tiles_per_chunk, int splits, float *partial, hipStream_t st) {
+#define FLK_CALL(KF) launch_mmv_split_large_kf##KF(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st)
     FLK_SWITCH_KF(kf, FLK_CALL)
 #undef FLK_CALL
 }

@@ -39,7 +39,7 @@ class BaseOptions:
     num_fmm_streams: int = 2                          # carried, unused
     memory_slack: float = 0.9                         # fraction of the free device memory a call may plan with
     bf16x3_cross_term: bool = False                   # not in the reference: fp32 products form x.c on the bf16 matrix
-                                                      # cores from an exact 3-way bfloat16 split (fp32 accuracy, d <= 62)
+                                                      # cores from an exact 3-way bfloat16 split (fp32 accuracy)
 
 
 @dataclass

@@ -19,8 +19,7 @@
  * squared distance formed on the bfloat16 matrix cores: every scaled fp32 value is split exactly into
  * three bfloat16 pieces (3 x 8 = 24 significant bits) and six partial products are accumulated in fp32,
  * which keeps the accuracy of the fp32 dot product (measured: the same distance from the fp64 result as
- * FLK_F32) at 16 features per matrix instruction instead of 2.  It has no counterpart in the reference;
- * it applies to d <= 62 and is FLK_F32 otherwise.
+ * FLK_F32) at 16 features per matrix instruction instead of 2.  It has no counterpart in the reference.
  */
 #ifndef FALKON_AMD_H
 #define FALKON_AMD_H

@@ -57,19 +57,37 @@ def test_layouts_sigma_per_dimension_and_repeatability(dev):
     assert torch.equal(k.dmmv(X, C, v, w).to(dev), ref)
 
 
-def test_feature_counts_beyond_the_split_kernels_use_plain_fp32(dev):
-    X, C, v, w = _data(400, 150, 63, 2, seed=5)
-    sigma = torch.tensor([8.0], dtype=torch.float64)
-    a = GaussianKernel(sigma, opt=SPLIT).dmmv(X.to(dev), C.to(dev), v.to(dev), w.to(dev))
-    b = GaussianKernel(sigma, opt=PLAIN).dmmv(X.to(dev), C.to(dev), v.to(dev), w.to(dev))
-    assert torch.equal(a, b)
-    X, C, v, w = _data(300, 140, 200, 3, seed=6)
-    a = GaussianKernel(15.0, opt=SPLIT).mmv(X.to(dev), C.to(dev), v.to(dev))
-    b = GaussianKernel(15.0, opt=PLAIN).mmv(X.to(dev), C.to(dev), v.to(dev))
-    assert torch.equal(a, b)
-    # fp64 data is not affected by the option
+@pytest.mark.parametrize("n,m,d,t", [(400, 150, 63, 2), (300, 257, 65, 1), (129, 64, 200, 10), (64, 300, 784, 5),
+                                     (700, 129, 100, 4), (513, 260, 130, 16), (260, 513, 96, 17)])
+def test_lds_tiled_kernel_vs_oracle(dev, n, m, d, t):
+    """Feature counts beyond 62 run the LDS-tiled kernel of the mode: both epilogues, ragged tiles."""
+    X, C, v, w = _data(n, m, d, t, seed=n + d)
+    sigma = torch.tensor([0.9 * np.sqrt(d)], dtype=torch.float64)
+    k = GaussianKernel(sigma, opt=SPLIT)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+    check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)
+    check_parity(k.dmmv(Xg, Cg, vg, wg), mmv_ref.fdmmv_ref(X, C, v, w, sigma),
+                 mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), 1e-5)
+    assert torch.equal(k.dmmv(Xg, Cg, vg, wg), k.dmmv(Xg, Cg, vg, wg))
+
+
+def test_fp64_data_is_not_affected_by_the_option(dev):
+    X, C, v, _ = _data(300, 140, 40, 3, seed=6)
     Xd, Cd, vd = X.double().to(dev), C.double().to(dev), v.double().to(dev)
     assert torch.equal(GaussianKernel(15.0, opt=SPLIT).mmv(Xd, Cd, vd), GaussianKernel(15.0, opt=PLAIN).mmv(Xd, Cd, vd))
+
+
+def test_config4_shape_reduced(dev):
+    X, C, sigma, v, w = inputs.make_config("C4", N=20_000, M=2_000)
+    k = GaussianKernel(sigma, opt=SPLIT)
+    got = k.dmmv(X.to(dev), C.to(dev), v.to(dev), w.to(dev))
+    check_parity(got, mmv_ref.fdmmv_ref(X, C, v, w, sigma, max_cpu_mem=2 * 2**30),
+                 mmv_ref.fdmmv_ref(X.double(), C.double(), v.double(), w.double(), sigma, max_cpu_mem=4 * 2**30), 1e-5)
+    exact = brute.radial_brute(X[:3000], C, sigma, "gaussian") @ v.double().numpy()
+    e_split = rel_err(k.mmv(X[:3000].to(dev), C.to(dev), v.to(dev)), exact)
+    e_plain = rel_err(GaussianKernel(sigma, opt=PLAIN).mmv(X[:3000].to(dev), C.to(dev), v.to(dev)), exact)
+    assert e_split <= 1.5 * e_plain + 2e-7, (e_split, e_plain)
 
 
 @pytest.mark.parametrize("name,make", [("laplacian", lambda s: LaplacianKernel(s, opt=SPLIT)),
