@@ -361,7 +361,7 @@ static int fmm_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1
 // bf16x3 mode of the fp32 products (split_common.h): same drivers on the split operands; register-resident kernel
 // up to kSplitMaxD features, LDS-tiled kernel beyond.
 // ---------------------------------------------------------------------------
-constexpr int64_t kTargetWgsSplitLarge = 16384;  // two 256-thread workgroups per CU: 32 rounds
+constexpr int64_t kTargetWgsSplitLarge = 8192;  // one 512-thread workgroup per CU: 32 rounds
 
 static Plan make_plan_split(int64_t na_blocks, int64_t nb_blocks, int64_t ks, int64_t t) {
     Plan p;

@@ -5,8 +5,8 @@
 //
 // A workgroup owns one tile of output rows (B side) and walks over the tiles of reduction rows (A side) of its
 // chunk.  The packed operands are consumed one k-step of 16 features at a time: the three bfloat16 pieces of the
-// k-step of both tiles are staged in LDS (two stages, one barrier per k-step; the packed layout already is the
-// operand order, so a stage is a plain copy of 16-byte vectors), every wave keeps a WA_FR x WB_FR grid of MFMA
+// k-step of both tiles are staged in LDS (three stages filled two k-steps ahead by direct global-to-LDS loads, one
+// barrier per k-step; the packed layout already is the operand order), every wave keeps a WA_FR x WB_FR grid of MFMA
 // accumulators and issues the six partial products of each pair with v_mfma_f32_32x32x16_bf16.  The half norms
 // ride in the last two features (the B side swaps the pair when it reads its operands), so after the last k-step
 // the accumulators hold the exponent.  Epilogue as in the fp32 LDS-tiled kernel: per-lane FMAs for up to four
@@ -26,6 +26,15 @@ typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 
 static __device__ __forceinline__ bf16x8 bits_as_bf16x8(uintx4 v) { return __builtin_bit_cast(bf16x8, v); }
 
+// Bare workgroup barrier: the wave's own LDS traffic is drained first, and the compiler may not move memory
+// operations across it.  (__syncthreads would also wait for every vector memory operation, i.e. for the direct
+// global-to-LDS loads that are meant to stay in flight across the barrier.)
+static __device__ __forceinline__ void wg_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
 template <int WVA, int WVB, int WA_FR, int WB_FR, int TT, int KF>
 __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   // two waves per SIMD either way
@@ -33,23 +42,27 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                            const uintx4 *__restrict__ PB, int64_t na_blocks, int64_t nb_blocks, int ks_count,
                            int64_t a_tiles_per_chunk, float *__restrict__ partial, int64_t nb_pad, bool y_fastest) {
     typedef LTraits<float> TR;
-    constexpr int kThreads = 64 * WVA * WVB;
+    constexpr int kWaves = WVA * WVB, kThreads = 64 * kWaves;
     constexpr int NAB = WVA * WA_FR, NBB = WVB * WB_FR;          // blocks of 32 rows per tile
     constexpr int A_ROWS = NAB * 32;
     constexpr int kBlockVecs = 3 * 64;                            // 16-byte vectors per block and k-step
     constexpr int A_VECS = NAB * kBlockVecs, B_VECS = NBB * kBlockVecs;
-    constexpr int A_VPT = (A_VECS + kThreads - 1) / kThreads, B_VPT = (B_VECS + kThreads - 1) / kThreads;
+    // a stage is copied in units of one piece of one block (64 lanes x 16 bytes = one direct-to-LDS load of a wave)
+    constexpr int kUnits = (NAB + NBB) * 3, kUnitsPerWave = kUnits / kWaves;
+    static_assert(kUnits % kWaves == 0, "the units of a stage must split evenly over the waves");
+    constexpr int kStages = (WA_FR * WB_FR >= 8) ? 2 : 3;     // k-steps in LDS: one in use, the others in flight
     constexpr bool kMfmaEpi = TT > 4;
-    constexpr int kVecStride = 17;
+    constexpr int kVecStride = 16;
     constexpr int kRowBuf = kMfmaEpi ? A_ROWS * kVecStride : TT * A_ROWS;
-    __shared__ __attribute__((aligned(16))) uintx4 ldsA[2][A_VECS];
-    __shared__ __attribute__((aligned(16))) uintx4 ldsB[2][B_VECS];
+    __shared__ __attribute__((aligned(16))) uintx4 ldsA[kStages][A_VECS];
+    __shared__ __attribute__((aligned(16))) uintx4 ldsB[kStages][B_VECS];
     __shared__ __attribute__((aligned(32))) float ldsRow[kRowBuf];   // vec of the A tile
 
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform by construction: let the compiler know
     const int wa = wave % WVA, wb = wave / WVA;
     const int j = lane & 31, lg = lane >> 5;
     const int64_t bblk0 = (int64_t)bx * NBB;
@@ -69,29 +82,35 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
         for (int r = 0; r < 16; r++) out2[q][r] = 0.f;
 
-    // where this thread's pieces of a stage come from: vector vi of a tile is (block vi / 192, offset vi % 192);
-    // blocks past the end re-read the last block (their rows get zero weight / are not stored), and the vector
-    // indices past the tile (the tile is not a multiple of the thread count) repeat the last vector
-    const uintx4 *srcA[A_VPT], *srcB[B_VPT];
+    // The stages are filled by direct global-to-LDS loads (global_load_lds_dwordx4: lane l of the issuing wave
+    // writes its 16 bytes at the wave-uniform LDS address + 16 l, which is the packed order), three k-steps deep,
+    // without passing through registers.  The compiler does not order these loads against the LDS reads: the
+    // vmcnt waits below do (the loop issues no other vector memory instruction).  Unit u of a stage is piece u % 3
+    // of block u / 3 of the A tile, then of the B tile; blocks past the end re-read the last block (their rows get
+    // zero weight / are not stored).
+    auto issue_stage = [&](int64_t ablk0, int s, int stage) {
+#pragma unroll
+        for (int i = 0; i < kUnitsPerWave; i++) {
+            const int u = wave * kUnitsPerWave + i;
+            const bool is_a = u < NAB * 3;
+            const int blk = is_a ? u / 3 : (u - NAB * 3) / 3;
+            const int piece = u % 3;
+            int64_t b = (is_a ? ablk0 : bblk0) + blk;
+            const int64_t last = (is_a ? na_blocks : nb_blocks) - 1;
+            if (b > last) b = last;
+            const uintx4 *src = (is_a ? PA : PB) + (b * ks_count + s) * kBlockVecs + piece * 64 + lane;
+            uintx4 *dst = is_a ? &ldsA[stage][(blk * 3 + piece) * 64] : &ldsB[stage][(blk * 3 + piece) * 64];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                             (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+        }
+    };
 
+    if (at0 < at1) {
+#pragma unroll
+        for (int g = 0; g < kStages - 1; g++) issue_stage(at0 * NAB, g, g);
+    }
     for (int64_t at = at0; at < at1; at++) {
         const int64_t ablk0 = at * NAB;
-#pragma unroll
-        for (int c = 0; c < A_VPT; c++) {
-            int vi = tid + c * kThreads;
-            if (vi >= A_VECS) vi = A_VECS - 1;
-            int64_t b = ablk0 + vi / kBlockVecs;
-            if (b >= na_blocks) b = na_blocks - 1;
-            srcA[c] = PA + b * ks_count * kBlockVecs + vi % kBlockVecs;
-        }
-#pragma unroll
-        for (int c = 0; c < B_VPT; c++) {
-            int vi = tid + c * kThreads;
-            if (vi >= B_VECS) vi = B_VECS - 1;
-            int64_t b = bblk0 + vi / kBlockVecs;
-            if (b >= nb_blocks) b = nb_blocks - 1;
-            srcB[c] = PB + b * ks_count * kBlockVecs + vi % kBlockVecs;
-        }
         floatx16 acc[WA_FR][WB_FR];
 #pragma unroll
         for (int p = 0; p < WA_FR; p++)
@@ -100,29 +119,9 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[p][q][r] = 0.f;
 
-        uintx4 ra[A_VPT], rb[B_VPT];
-        auto fetch = [&](int s) {
-#pragma unroll
-            for (int c = 0; c < A_VPT; c++) ra[c] = srcA[c][(int64_t)s * kBlockVecs];
-#pragma unroll
-            for (int c = 0; c < B_VPT; c++) rb[c] = srcB[c][(int64_t)s * kBlockVecs];
-        };
-        auto commit = [&](int buf) {
-#pragma unroll
-            for (int c = 0; c < A_VPT; c++) {
-                const int vi = tid + c * kThreads;
-                if (vi < A_VECS) ldsA[buf][vi] = ra[c];
-            }
-#pragma unroll
-            for (int c = 0; c < B_VPT; c++) {
-                const int vi = tid + c * kThreads;
-                if (vi < B_VECS) ldsB[buf][vi] = rb[c];
-            }
-        };
-
-        // Prologue of an A tile: first k-step and the tile's right-hand side values are loaded before anything
-        // waits; the barrier that protects ldsRow and the stages from the previous tile's epilogue comes after.
-        fetch(0);
+        // the tile's right-hand side values: loaded, then written to ldsRow once every wave has left the previous
+        // tile's epilogue (the loads complete behind the two stages already in flight, so nothing is outstanding
+        // when the k-steps start)
         constexpr int kRowVals = (kMfmaEpi ? 16 : TT) * A_ROWS;
         constexpr int kRowValsPerThread = (kRowVals + kThreads - 1) / kThreads;
         float rowv[kRowValsPerThread];
@@ -135,7 +134,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             if (e < kRowVals && row < na_blocks * 32 && which < tcols) val = vecp[(int64_t)which * vec_ld + row];
             rowv[c] = val;
         }
-        __syncthreads();
+        wg_barrier();
 #pragma unroll
         for (int c = 0; c < kRowValsPerThread; c++) {
             const int e = tid + c * kThreads;
@@ -145,42 +144,58 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                 else ldsRow[r * kVecStride + which] = rowv[c];
             }
         }
-        commit(0);
-        __syncthreads();
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
         for (int s = 0; s < ks_count; s++) {
-            const int buf = s & 1;
-            const bool more = s + 1 < ks_count;
-            if (more) fetch(s + 1);
-            uintx4 a[WA_FR][3], b[WB_FR][3];
+            const int stage = s % kStages;
+            // this wave's loads of k-step s have landed (those of k-step s + 1 may still be in flight); after the
+            // barrier so have everybody's, and every wave has finished reading the stage that k-step s + 2 goes to
+            if (kStages == 3 && s + 1 < ks_count) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kUnitsPerWave) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            wg_barrier();
+            if (s + kStages - 1 < ks_count) issue_stage(ablk0, s + kStages - 1, (s + kStages - 1) % kStages);
+            // operands: the B fragments' three pieces stay in registers for the k-step, the A fragments come one piece
+            // at a time (lo, mid, hi: partial products roughly from the lowest order up), each LDS vector read once
+            uintx4 b[WB_FR][3];
 #pragma unroll
-            for (int c = 0; c < 3; c++) {
+            for (int c = 0; c < 3; c++)
 #pragma unroll
-                for (int p = 0; p < WA_FR; p++) a[p][c] = ldsA[buf][((wa * WA_FR + p) * 3 + c) * 64 + lane];
-#pragma unroll
-                for (int q = 0; q < WB_FR; q++) b[q][c] = ldsB[buf][((wb * WB_FR + q) * 3 + c) * 64 + lane];
-            }
+                for (int q = 0; q < WB_FR; q++) b[q][c] = ldsB[stage][((wb * WB_FR + q) * 3 + c) * 64 + lane];
             // B role, last k-step: the pair (1.0, h) in the last dword of the upper lane half becomes (h, 1.0)
-            if (!more && lg) {
+            if (s + 1 == ks_count && lg) {
 #pragma unroll
                 for (int q = 0; q < WB_FR; q++)
 #pragma unroll
                     for (int c = 0; c < 3; c++) b[q][c][3] = (b[q][c][3] >> 16) | (b[q][c][3] << 16);
             }
-            // partial products, lowest order first: (mid,mid) (hi,lo) (lo,hi) (hi,mid) (mid,hi) (hi,hi)
-            constexpr int kPieceA[6] = {1, 0, 2, 0, 1, 0}, kPieceB[6] = {1, 2, 0, 1, 0, 0};
+            // A piece -> the B pieces it meets: lo x hi | mid x (mid, hi) | hi x (lo, mid, hi)
+            constexpr int kPieceOrder[3] = {2, 1, 0};
+            constexpr int kPartners[3][3] = {{2, 1, 0}, {1, 0, -1}, {0, -1, -1}};   // indexed by A piece
 #pragma unroll
-            for (int pr = 0; pr < 6; pr++)
+            for (int o = 0; o < 3; o++) {
+                const int ca = kPieceOrder[o];
+                uintx4 a[WA_FR];
 #pragma unroll
-                for (int p = 0; p < WA_FR; p++)
+                for (int p = 0; p < WA_FR; p++) a[p] = ldsA[stage][((wa * WA_FR + p) * 3 + ca) * 64 + lane];
 #pragma unroll
-                    for (int q = 0; q < WB_FR; q++)
-                        acc[p][q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bits_as_bf16x8(a[p][kPieceA[pr]]),
-                                                                            bits_as_bf16x8(b[q][kPieceB[pr]]),
-                                                                            acc[p][q], 0, 0, 0);
-            // the other stage was last read one k-step ago, and every wave has passed the barrier since
-            if (more) commit(buf ^ 1);
-            __syncthreads();
+                for (int w = 0; w < 3; w++) {
+                    const int cb = kPartners[ca][w];
+                    if (cb < 0) continue;
+#pragma unroll
+                    for (int p = 0; p < WA_FR; p++)
+#pragma unroll
+                        for (int q = 0; q < WB_FR; q++)
+                            acc[p][q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bits_as_bf16x8(a[p]), bits_as_bf16x8(b[q][cb]),
+                                                                                acc[p][q], 0, 0, 0);
+                }
+            }
+        }
+        // every wave has read its last operands once it passes this barrier: the first two k-steps of the next
+        // tile go out before the epilogue and land while it runs
+        wg_barrier();
+        if (at + 1 < at1) {
+#pragma unroll
+            for (int g = 0; g < kStages - 1; g++) issue_stage((at + 1) * NAB, g, g);
         }
 
         // epilogue: K = kernel_value(acc) ; out[q][t] += K * vec[i][t]
@@ -264,9 +279,10 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     }
 }
 
-// 4 waves (2 x 2), two workgroups per CU so that one workgroup's barrier and LDS latencies are covered by the
-// other; tile 128 (A) x 128 (B) rows
-constexpr int kSLWavesA = 2, kSLWavesB = 2, kSLFragsA = 2, kSLFragsB = 2;
+// 8 waves (2 x 4) with 4 x 2 accumulators each, one workgroup per CU (two waves per SIMD); tile 256 (A) x 256 (B)
+// rows: every operand read from LDS feeds two or four MFMAs, and a k-step (48 MFMAs per wave) outlasts the latency
+// of the next k-step's loads
+constexpr int kSLWavesA = 2, kSLWavesB = 4, kSLFragsA = 4, kSLFragsB = 2;
 
 #if FLK_KF == FLK_GAUSSIAN   // the tile geometry is the same for every kernel function: defined once
 int split_large_a_tile_blocks() { return kSLWavesA * kSLFragsA; }
