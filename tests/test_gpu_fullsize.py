@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from falkon_amd import GaussianKernel
+from falkon_amd import FalkonOptions, GaussianKernel
 from oracle import gaussian_ref, inputs, mmv_ref
 from conftest import check_parity, rel_err
 
@@ -30,12 +30,13 @@ def _columns_of_kt_u(X, C_sub, sigma, u, block=500_000):
     return acc
 
 
-def _full_size_checks(dev, name, dtype, n_rows=3000, n_centres=48):
+def _full_size_checks(dev, name, dtype, n_rows=3000, n_centres=48, bf16x3=False):
     X, C, sigma, v, w = inputs.make_config(name, dtype=dtype)
+    opt = FalkonOptions(bf16x3_cross_term=bf16x3)
     N, M, T = X.shape[0], C.shape[0], v.shape[1]
     tol = TOL[dtype]
     g = np.random.default_rng(7)
-    k = GaussianKernel(sigma)
+    k = GaussianKernel(sigma, opt=opt)
     Xg, Cg, vg = X.to(dev), C.to(dev), v.to(dev)
     wg = w.to(dev) if w is not None else None
 
@@ -79,7 +80,7 @@ def _full_size_checks(dev, name, dtype, n_rows=3000, n_centres=48):
     del perm, out_p
 
     # (7) sigma -> infinity: K -> 1, K v -> column sums of v
-    flat = GaussianKernel(1e7).mmv(Xg, Cg, vg)
+    flat = GaussianKernel(1e7, opt=opt).mmv(Xg, Cg, vg)
     sums = vg.double().sum(0, keepdim=True)
     assert float(((flat.double() - sums).abs().max(0).values / vg.double().abs().sum(0)).max()) < tol
 
@@ -87,17 +88,20 @@ def _full_size_checks(dev, name, dtype, n_rows=3000, n_centres=48):
     assert torch.equal(out, k.dmmv(Xg, Cg, vg, wg))
 
 
-def test_config2_full_size(dev):
-    """N=1e6, d=28, M=20000, T=1, sigma=3.8, fp32."""
-    _full_size_checks(dev, "C2", torch.float32)
+@pytest.mark.parametrize("bf16x3", [False, True], ids=["fp32-mfma", "bf16x3"])
+def test_config2_full_size(dev, bf16x3):
+    """N=1e6, d=28, M=20000, T=1, sigma=3.8, fp32 (plain, and with the cross term on the bf16 matrix cores)."""
+    _full_size_checks(dev, "C2", torch.float32, bf16x3=bf16x3)
 
 
-def test_config3_full_size(dev):
+@pytest.mark.parametrize("bf16x3", [False, True], ids=["fp32-mfma", "bf16x3"])
+def test_config3_full_size(dev, bf16x3):
     """N=1e7, d=9, M=50000, T=1, per-dimension sigma, w=None, fp32."""
-    _full_size_checks(dev, "C3", torch.float32, n_rows=2000, n_centres=24)
+    _full_size_checks(dev, "C3", torch.float32, n_rows=2000, n_centres=24, bf16x3=bf16x3)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-def test_config4_full_size(dev, dtype):
-    """N=5e5, d=784 (80 % zeros), M=10000, T=10, sigma=10, fp32 and fp64."""
-    _full_size_checks(dev, "C4", dtype, n_rows=2000, n_centres=32)
+@pytest.mark.parametrize("dtype,bf16x3", [(torch.float32, False), (torch.float32, True), (torch.float64, False)],
+                         ids=["fp32-mfma", "bf16x3", "fp64"])
+def test_config4_full_size(dev, dtype, bf16x3):
+    """N=5e5, d=784 (80 % zeros), M=10000, T=10, sigma=10, fp32 (both modes) and fp64."""
+    _full_size_checks(dev, "C4", dtype, n_rows=2000, n_centres=32, bf16x3=bf16x3)
