@@ -156,9 +156,14 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             if (s + kStages - 1 < ks_count) issue_stage(ablk0, s + kStages - 1, (s + kStages - 1) % kStages);
             // operands: the B fragments' three pieces stay in registers for the k-step, the A fragments come one piece
             // at a time (lo, mid, hi: partial products roughly from the lowest order up), each LDS vector read once
-            uintx4 b[WB_FR][3];
+            // (read order: what the first partial product needs comes first, lo of A and hi of B)
+            uintx4 b[WB_FR][3], a_first[WA_FR];
 #pragma unroll
-            for (int c = 0; c < 3; c++)
+            for (int q = 0; q < WB_FR; q++) b[q][0] = ldsB[stage][((wb * WB_FR + q) * 3 + 0) * 64 + lane];
+#pragma unroll
+            for (int p = 0; p < WA_FR; p++) a_first[p] = ldsA[stage][((wa * WA_FR + p) * 3 + 2) * 64 + lane];
+#pragma unroll
+            for (int c = 1; c < 3; c++)
 #pragma unroll
                 for (int q = 0; q < WB_FR; q++) b[q][c] = ldsB[stage][((wb * WB_FR + q) * 3 + c) * 64 + lane];
             // B role, last k-step: the pair (1.0, h) in the last dword of the upper lane half becomes (h, 1.0)
@@ -176,7 +181,8 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                 const int ca = kPieceOrder[o];
                 uintx4 a[WA_FR];
 #pragma unroll
-                for (int p = 0; p < WA_FR; p++) a[p] = ldsA[stage][((wa * WA_FR + p) * 3 + ca) * 64 + lane];
+                for (int p = 0; p < WA_FR; p++)
+                    a[p] = o == 0 ? a_first[p] : ldsA[stage][((wa * WA_FR + p) * 3 + ca) * 64 + lane];
 #pragma unroll
                 for (int w = 0; w < 3; w++) {
                     const int cb = kPartners[ca][w];
