@@ -50,7 +50,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     // a stage is copied in units of one piece of one block (64 lanes x 16 bytes = one direct-to-LDS load of a wave)
     constexpr int kUnits = (NAB + NBB) * 3, kUnitsPerWave = kUnits / kWaves;
     static_assert(kUnits % kWaves == 0, "the units of a stage must split evenly over the waves");
-    constexpr int kStages = (WA_FR * WB_FR >= 8) ? 2 : 3;     // k-steps in LDS: one in use, the others in flight
+    constexpr int kStages = 3;     // k-steps in LDS: one in use, the others in flight
     constexpr bool kMfmaEpi = TT > 4;
     constexpr int kVecStride = 16;
     constexpr int kRowBuf = kMfmaEpi ? A_ROWS * kVecStride : TT * A_ROWS;
@@ -88,26 +88,37 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     // vmcnt waits below do (the loop issues no other vector memory instruction).  Unit u of a stage is piece u % 3
     // of block u / 3 of the A tile, then of the B tile; blocks past the end re-read the last block (their rows get
     // zero weight / are not stored).
-    auto issue_stage = [&](int64_t ablk0, int s, int stage) {
+    // where this wave's units of a stage come from (wave-uniform; the lane and the k-step are added at issue)
+    const uintx4 *unit_src[kUnitsPerWave];
+    auto set_tile = [&](int64_t ablk0) {
 #pragma unroll
         for (int i = 0; i < kUnitsPerWave; i++) {
             const int u = wave * kUnitsPerWave + i;
             const bool is_a = u < NAB * 3;
             const int blk = is_a ? u / 3 : (u - NAB * 3) / 3;
-            const int piece = u % 3;
             int64_t b = (is_a ? ablk0 : bblk0) + blk;
             const int64_t last = (is_a ? na_blocks : nb_blocks) - 1;
             if (b > last) b = last;
-            const uintx4 *src = (is_a ? PA : PB) + (b * ks_count + s) * kBlockVecs + piece * 64 + lane;
-            uintx4 *dst = is_a ? &ldsA[stage][(blk * 3 + piece) * 64] : &ldsB[stage][(blk * 3 + piece) * 64];
+            unit_src[i] = (is_a ? PA : PB) + b * ks_count * kBlockVecs + (u % 3) * 64;
+        }
+    };
+    auto issue_stage = [&](int s, int stage) {
+#pragma unroll
+        for (int i = 0; i < kUnitsPerWave; i++) {
+            const int u = wave * kUnitsPerWave + i;
+            const bool is_a = u < NAB * 3;
+            const int blk = is_a ? u / 3 : (u - NAB * 3) / 3;
+            const uintx4 *src = unit_src[i] + s * kBlockVecs + lane;
+            uintx4 *dst = is_a ? &ldsA[stage][(blk * 3 + u % 3) * 64] : &ldsB[stage][(blk * 3 + u % 3) * 64];
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                              (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
         }
     };
 
     if (at0 < at1) {
+        set_tile(at0 * NAB);
 #pragma unroll
-        for (int g = 0; g < kStages - 1; g++) issue_stage(at0 * NAB, g, g);
+        for (int g = 0; g < kStages - 1; g++) issue_stage(g, g);
     }
     for (int64_t at = at0; at < at1; at++) {
         const int64_t ablk0 = at * NAB;
@@ -153,7 +164,6 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             if (kStages == 3 && s + 1 < ks_count) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kUnitsPerWave) : "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             wg_barrier();
-            if (s + kStages - 1 < ks_count) issue_stage(ablk0, s + kStages - 1, (s + kStages - 1) % kStages);
             // operands: the B fragments' three pieces stay in registers for the k-step, the A fragments come one piece
             // at a time (lo, mid, hi: partial products roughly from the lowest order up), each LDS vector read once
             // (read order: what the first partial product needs comes first, lo of A and hi of B)
@@ -194,14 +204,18 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                             acc[p][q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bits_as_bf16x8(a[p]), bits_as_bf16x8(b[q][cb]),
                                                                                 acc[p][q], 0, 0, 0);
                 }
+                // the loads of a later k-step go out behind the first group of MFMAs, not in front of it: right
+                // after the barrier every wave of the CU would otherwise be issuing loads while the matrix cores idle
+                if (o == 0 && s + kStages - 1 < ks_count) issue_stage(s + kStages - 1, (s + kStages - 1) % kStages);
             }
         }
         // every wave has read its last operands once it passes this barrier: the first two k-steps of the next
         // tile go out before the epilogue and land while it runs
         wg_barrier();
         if (at + 1 < at1) {
+            set_tile((at + 1) * NAB);
 #pragma unroll
-            for (int g = 0; g < kStages - 1; g++) issue_stage((at + 1) * NAB, g, g);
+            for (int g = 0; g < kStages - 1; g++) issue_stage(g, g);
         }
 
         // epilogue: K = kernel_value(acc) ; out[q][t] += K * vec[i][t]
