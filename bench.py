@@ -65,6 +65,7 @@ MEASURED_TRAFFIC_BYTES = {
 # the same for the bf16x3 product kernel (profiles/mmv_split_kernel__C2_dfmmv_bf16x3.md)
 MEASURED_TRAFFIC_BYTES_BF16X3 = {
     "C2": int((536594.0 * 2.0 + 17773.4 * 1.0) * 1024),    # 1.12 GB: the packed centres no longer fit one L2 next to X
+    "C4": int((3.32483e7 * 2.0 + 174341.0 * 1.0) * 1024),  # 68 GB: tiles are re-read from L2 / infinity cache / HBM
 }
 
 
