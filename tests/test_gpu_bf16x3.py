@@ -142,3 +142,50 @@ def test_falkon_fit_predict_with_the_option(dev):
     mse = [float(((p - y[:4000]) ** 2).mean()) for p in preds]
     assert abs(mse[0] - mse[1]) <= 1e-3 * mse[1]
     assert rel_err(preds[0], preds[1]) < 1e-3
+
+
+@pytest.mark.parametrize("d", [9, 100])
+def test_degenerate_shapes(dev, d):
+    """No centres, no data rows, a single row on either side, in both kernels of the mode."""
+    k = GaussianKernel(1.5 * np.sqrt(d), opt=SPLIT)
+    X, C, v, w = _data(70, 9, d, 2, seed=3)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    r = k.mmv(Xg, Cg[:0], vg[:0])
+    assert r.shape == (70, 2) and float(r.abs().max()) == 0.0
+    assert k.dmmv(Xg, Cg[:0], vg[:0], wg).shape == (0, 2)
+    r = k.dmmv(Xg[:0], Cg, vg, wg[:0])
+    assert r.shape == (9, 2) and float(r.abs().max()) == 0.0
+    assert k.mmv(Xg[:0], Cg, vg).shape == (0, 2)
+    for n, m in ((1, 9), (70, 1), (1, 1)):
+        got = k.dmmv(Xg[:n], Cg[:m], vg[:m], wg[:n])
+        assert rel_err(got, mmv_ref.fdmmv_ref(X[:n], C[:m], v[:m], w[:n], k.sigma)) < 1e-5
+
+
+@pytest.mark.parametrize("d", [28, 200])
+def test_dmmv_replays_from_a_hip_graph(dev, d):
+    """As for the fp32 kernels: nothing is allocated, cleared with a memset or synchronised, so a call can be captured
+    into a HIP graph; every replay reproduces the eager result bit for bit."""
+    X, C, v, w = _data(20_000, 1_200, d, 2, seed=21)
+    k = GaussianKernel(0.7 * np.sqrt(d), opt=SPLIT)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    out = torch.empty(1_200, 2, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        k.dmmv(Xg, Cg, vg, wg, out=out)               # warm-up outside the capture (sigma upload, allocator)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        k.dmmv(Xg, Cg, vg, wg, out=out)
+    g = np.random.default_rng(5)
+    for _ in range(3):
+        vg.copy_(torch.from_numpy(g.standard_normal((1_200, 2)).astype(np.float32)))
+        wg.copy_(torch.from_numpy(g.standard_normal((20_000, 2)).astype(np.float32)))
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = out.clone()
+        eager = k.dmmv(Xg, Cg, vg, wg)
+        torch.cuda.synchronize()
+        assert torch.equal(replayed, eager)
+    assert rel_err(eager, mmv_ref.fdmmv_ref(X, C, vg.cpu(), wg.cpu(), k.sigma)) < 1e-5
