@@ -215,3 +215,35 @@ def test_laplacian_and_matern_kernel_objects():
         kernel_name = "polynomial"
     with pytest.raises(NotImplementedError):
         _kernel_fn(Other())
+
+
+def test_three_way_bfloat16_split_is_exact():
+    """The arithmetic claim behind the bf16x3 mode (falkon_amd/csrc/split_common.h), checked in numpy: an fp32 value
+    is the exact sum of three round-to-nearest bfloat16 pieces, and the six partial products the kernels keep
+    reproduce an fp32 product to about 2^-23 of |x||y|."""
+    import numpy as np
+
+    def bf16_rne(x):                                  # the conversion of pack_split.hip, bit for bit
+        u = x.astype(np.float32).view(np.uint32).astype(np.uint64)
+        r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+        return (r & 0xFFFFFFFF).astype(np.uint32).view(np.float32)
+
+    def split3(x):
+        hi = bf16_rne(x)
+        r1 = (x - hi).astype(np.float32)
+        mid = bf16_rne(r1)
+        lo = bf16_rne((r1 - mid).astype(np.float32))
+        return hi, mid, lo
+
+    g = np.random.default_rng(0)
+    x = (g.standard_normal(200_000) * np.exp(g.uniform(-30, 30, 200_000))).astype(np.float32)
+    y = (g.standard_normal(200_000) * np.exp(g.uniform(-30, 30, 200_000))).astype(np.float32)
+    xh, xm, xl = split3(x)
+    assert np.array_equal((xh.astype(np.float64) + xm + xl).astype(np.float32), x)
+    assert np.array_equal(xh.astype(np.float64) + xm.astype(np.float64) + xl.astype(np.float64), x.astype(np.float64))
+    yh, ym, yl = split3(y)
+    f = np.float64
+    kept = (xm.astype(f) * ym + xh.astype(f) * yl + xl.astype(f) * yh + xh.astype(f) * ym + xm.astype(f) * yh
+            + xh.astype(f) * yh)
+    exact = x.astype(f) * y.astype(f)
+    assert float(np.max(np.abs(kept - exact) / np.abs(exact))) < 2.0 ** -22
