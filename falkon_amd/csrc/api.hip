@@ -363,9 +363,19 @@ static int fmm_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1
 // ---------------------------------------------------------------------------
 constexpr int64_t kTargetWgsSplitLarge = 8192;  // one 512-thread workgroup per CU: 32 rounds
 
+// Where the bf16x3 kernels are the faster route to the same result.  Measured at d = 28, N = 1e6, M = 2e4, dfmmv,
+// against the fp32 MFMA kernels: 1 right-hand side 10.9 ms against 20.2, 2: 11.9 against 21.1 (register-resident
+// kernel, two columns per pass); 4: 24.3 against 22.7, 5: 34.9 against 24.5 (the fp32 kernels contract up to eight
+// columns per pass at this size); 9: 34.8 against 46.5, 16: 35.0 against 52.8 (LDS-tiled kernel, sixteen columns per
+// pass on the matrix cores).  So: every feature count beyond the register-resident kernels, and at small feature
+// counts up to two right-hand sides or more than eight; in between the fp32 MFMA kernels serve the mode.
+static bool split_applies(int64_t d, int64_t t) { return d > kSplitMaxD || t <= 2 || t > 8; }
+
 static Plan make_plan_split(int64_t na_blocks, int64_t nb_blocks, int64_t ks, int64_t t) {
     Plan p;
-    if (ks * 16 <= kSplitMaxD + 2) {
+    // up to two right-hand sides the register-resident kernel; beyond that (see split_applies) the LDS-tiled kernel,
+    // whose epilogue contracts sixteen columns per pass on the matrix cores, also for small feature counts
+    if (ks * 16 <= kSplitMaxD + 2 && t <= 2) {
         plan_register_resident(p, na_blocks, nb_blocks, split_b_blocks_per_wg(ks), ks * 3 * 64 * 16, 32, kSplitMaxCols,
                                t, (int64_t)sizeof(float));
         return p;
@@ -593,7 +603,7 @@ int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b
 
 size_t flk_gauss_fmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
-    if (dtype == FLK_F32_BF16X3) return fmmv_split_ws_bytes(n, m, d, t);
+    if (dtype == FLK_F32_BF16X3 && split_applies(d, t)) return fmmv_split_ws_bytes(n, m, d, t);
     return dtype == FLK_F64 ? fmmv_ws_bytes<double>(n, m, d, t) : fmmv_ws_bytes<float>(n, m, d, t);
 }
 
@@ -603,10 +613,10 @@ int flk_kernel_fmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_
                     void *workspace, size_t workspace_bytes, void *stream) {
     g_err[0] = 0;
     FLK_CHECK_KERNEL(kernel);
-    if (dtype == FLK_F32_BF16X3)
+    if (dtype == FLK_F32_BF16X3 && split_applies(d, t))
         return fmmv_split_impl(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t, out,
                                out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    if (dtype == FLK_F32)
+    if (dtype == FLK_F32 || dtype == FLK_F32_BF16X3)
         return fmmv_impl<float>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, t,
                                 out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
     if (dtype == FLK_F64)
@@ -625,7 +635,7 @@ int flk_gauss_fmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, cons
 
 size_t flk_gauss_fdmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
-    if (dtype == FLK_F32_BF16X3) return fdmmv_split_ws_bytes(n, m, d, t);
+    if (dtype == FLK_F32_BF16X3 && split_applies(d, t)) return fdmmv_split_ws_bytes(n, m, d, t);
     return dtype == FLK_F64 ? fdmmv_ws_bytes<double>(n, m, d, t) : fdmmv_ws_bytes<float>(n, m, d, t);
 }
 
@@ -636,10 +646,10 @@ int flk_kernel_fdmmv(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64
                      void *stream) {
     g_err[0] = 0;
     FLK_CHECK_KERNEL(kernel);
-    if (dtype == FLK_F32_BF16X3)
+    if (dtype == FLK_F32_BF16X3 && split_applies(d, t))
         return fdmmv_split_impl(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
                                 w_rs, w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
-    if (dtype == FLK_F32)
+    if (dtype == FLK_F32 || dtype == FLK_F32_BF16X3)
         return fdmmv_impl<float>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
                                  w_rs, w_cs, t, out, out_rs, out_cs, workspace, workspace_bytes, (hipStream_t)stream);
     if (dtype == FLK_F64)

@@ -1,5 +1,6 @@
-// LDS-tiled kernel-vector product of the bf16x3 mode (see split_common.h) for feature counts beyond the
-// register-resident kernel, fp32 data, gfx950.  Compiled once per kernel function (-DFLK_KF=0..4).
+// LDS-tiled kernel-vector product of the bf16x3 mode (see split_common.h), fp32 data, gfx950: feature counts beyond
+// the register-resident kernel, and more than four right-hand sides at any feature count (its epilogue contracts
+// sixteen columns per pass on the matrix cores).  Compiled once per kernel function (-DFLK_KF=0..4).
 //
 //   partial[split'][t][b] = sum_{a in chunk} K(A_a, B_b) * vec[a,t]
 //
@@ -118,7 +119,8 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     if (at0 < at1) {
         set_tile(at0 * NAB);
 #pragma unroll
-        for (int g = 0; g < kStages - 1; g++) issue_stage(g, g);
+        for (int g = 0; g < kStages - 1; g++)
+            if (g < ks_count) issue_stage(g, g);
     }
     for (int64_t at = at0; at < at1; at++) {
         const int64_t ablk0 = at * NAB;
@@ -215,7 +217,8 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         if (at + 1 < at1) {
             set_tile((at + 1) * NAB);
 #pragma unroll
-            for (int g = 0; g < kStages - 1; g++) issue_stage(g, g);
+            for (int g = 0; g < kStages - 1; g++)
+                if (g < ks_count) issue_stage(g, g);
         }
 
         // epilogue: K = kernel_value(acc) ; out[q][t] += K * vec[i][t]
