@@ -67,6 +67,7 @@ struct Plan {
     int splits;            // grid.y
     int partials;          // partial results the finalize kernel sums (= splits x partials per split)
     int col_chunk;         // right-hand sides per pass
+    int64_t dpad = 0;      // padded feature count of the operands (register-resident kernels)
 };
 
 constexpr int64_t kTargetWgsLarge = 16384;  // two 256-thread workgroups per CU: 8 rounds
@@ -111,10 +112,11 @@ static void plan_register_resident(Plan &p, int64_t na_blocks, int64_t nb_blocks
 template <typename T>
 static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t dpad, int64_t t) {
     Plan p;
+    p.dpad = dpad;
     p.large = d > mmv_small_max_d<T>();
     if (!p.large) {
-        plan_register_resident(p, na_blocks, nb_blocks, mmv_small_b_blocks_per_wg<T>(dpad),
-                               dpad * Geo<T>::BLK * (int64_t)sizeof(T), Geo<T>::BLK, mmv_small_max_cols<T>(dpad), t,
+        plan_register_resident(p, na_blocks, nb_blocks, mmv_small_b_blocks_per_wg<T>(dpad, t),
+                               dpad * Geo<T>::BLK * (int64_t)sizeof(T), Geo<T>::BLK, mmv_small_max_cols<T>(dpad, t), t,
                                (int64_t)sizeof(T));
     } else {
         const int64_t a_tiles = (na_blocks + mmv_large_a_tile_blocks<T>() - 1) / mmv_large_a_tile_blocks<T>();
@@ -137,13 +139,12 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
 // that many planes of the planar right-hand side, so the planes past the caller's columns must be zero.
 template <typename T>
 static int instantiated_cols(const Plan &p, int tc) {
-    static const int small32[] = {1, 2, 3, 4, 6, 8, 12, 16}, large[] = {1, 2, 4, 16};
+    static const int large[] = {1, 2, 4, 16};
     if (p.large) {
         for (int w : large) if (tc <= w) return w;
-    } else if (sizeof(T) == 4) {
-        for (int w : small32) if (tc <= w) return w;
+        return tc;
     }
-    return tc;
+    return mmv_small_width<T>(p.dpad, tc);
 }
 template <typename T>
 static int64_t zero_planes_needed(const Plan &p, int64_t t) {
@@ -366,10 +367,11 @@ constexpr int64_t kTargetWgsSplitLarge = 8192;  // one 512-thread workgroup per 
 // Where the bf16x3 kernels are the faster route to the same result.  Measured at d = 28, N = 1e6, M = 2e4, dfmmv,
 // against the fp32 MFMA kernels: 1 right-hand side 10.9 ms against 20.2, 2: 11.9 against 21.1 (register-resident
 // kernel, two columns per pass); 4: 24.3 against 22.7, 5: 34.9 against 24.5 (the fp32 kernels contract up to eight
-// columns per pass at this size); 9: 34.8 against 46.5, 16: 35.0 against 52.8 (LDS-tiled kernel, sixteen columns per
-// pass on the matrix cores).  So: every feature count beyond the register-resident kernels, and at small feature
-// counts up to two right-hand sides or more than eight; in between the fp32 MFMA kernels serve the mode.
-static bool split_applies(int64_t d, int64_t t) { return d > kSplitMaxD || t <= 2 || t > 8; }
+// columns per pass with per-lane FMAs at this size); 9: 34.8 against 41.9, 16: 35.0 against 42.2 (LDS-tiled kernel,
+// sixteen columns per pass on the matrix cores, against the fp32 kernel that contracts 32); 17: 50.0 against 42.2,
+// 32: 70.1 against 43.0.  So: every feature count beyond the register-resident kernels, and at small feature
+// counts 1, 2 or 9 to 16 right-hand sides; otherwise the fp32 MFMA kernels serve the mode.
+static bool split_applies(int64_t d, int64_t t) { return d > kSplitMaxD || t <= 2 || (t > 8 && t <= 16); }
 
 static Plan make_plan_split(int64_t na_blocks, int64_t nb_blocks, int64_t ks, int64_t t) {
     Plan p;

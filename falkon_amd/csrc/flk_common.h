@@ -115,12 +115,14 @@ int launch_finalize(const T *partial, int splits, int64_t t, int64_t nb, int64_t
 
 // Register-resident ("small d") product kernel; the queries do not depend on the kernel function.
 template <typename T> int64_t mmv_small_max_d();
-template <typename T> int mmv_small_b_blocks_per_wg(int64_t dpad);
-template <typename T> int mmv_small_max_cols(int64_t dpad);   // right-hand sides per pass
+// (t: right-hand sides of the call; the fp32 kernels switch to their 32-column variant beyond a few columns)
+template <typename T> int mmv_small_b_blocks_per_wg(int64_t dpad, int64_t t);
+template <typename T> int mmv_small_max_cols(int64_t dpad, int64_t t);   // right-hand sides per pass
+template <typename T> int mmv_small_width(int64_t dpad, int tc);         // planes the kernel serving tc columns reads
 
 // Planes a planar right-hand side buffer must hold for t columns: kernels compute whole column
 // chunks and read zero planes beyond the caller's columns.
-constexpr int64_t kColPad = 15;
+constexpr int64_t kColPad = 31;
 
 // LDS-tiled ("large d") product kernel: any padded feature count, up to mmv_large_max_cols columns per pass.
 // Writes splits * mmv_large_partials_per_split partial results.
@@ -141,6 +143,9 @@ template <typename T> int mmv_large_max_cols();
     template <typename T>                                                                                         \
     int launch_mmv_small_kf##KF(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tt,  \
                                 int64_t a_chunk_blocks, int splits, T *partial, hipStream_t st);                  \
+    int launch_mmv_small_f32_wide_kf##KF(const PackedView &A, const PackedView &B, const float *vecp,             \
+                                         int64_t vec_ld, int tcols, int64_t a_chunk_blocks, int splits,           \
+                                         float *partial, hipStream_t st);                                         \
     template <typename T>                                                                                         \
     int launch_mmv_large_kf##KF(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld,          \
                                 int tcols, int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st);    \

@@ -15,14 +15,30 @@ int FLK_CAT(launch_mmv_small_f32_fold_kf, FLK_KF)(const PackedView &A, const Pac
                                                   int64_t vec_ld, int tt, int64_t a_chunk_blocks, int splits,
                                                   float *partial, hipStream_t st);
 
+// Columns per pass of the per-lane FMA kernels (must match the instantiations in launch_tt); calls with more
+// right-hand sides than that go to the 32-column kernel whose contraction runs on the matrix cores
+// (mmv_small_f32_wide.hip: four resident blocks per wave up to 16 padded features, two beyond).
+static inline int fma_cols(int64_t dpad) {
+    const int64_t dp = dpad / 2;
+    return dp <= 7 ? 16 : dp <= 12 ? 12 : dp <= 16 ? 8 : 4;
+}
+constexpr int kWideColumns = 32;
+constexpr int kWideMaxDpFr4 = 8;
+
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<float>() { return 2 * kMaxDpFr2; }
-template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad) {
+template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad, int64_t t) {
+    if (t > fma_cols(dpad)) return kWavesPerWg * ((dpad / 2) <= kWideMaxDpFr4 ? 4 : 2);
     return kWavesPerWg * ((dpad / 2) <= kMaxDpFr4 ? 4 : 2);
 }
-template <> int mmv_small_max_cols<float>(int64_t dpad) {
-    const int64_t dp = dpad / 2;   // must match the instantiations in launch_tt
-    return dp <= 7 ? 16 : dp <= 12 ? 12 : dp <= 16 ? 8 : 4;
+template <> int mmv_small_max_cols<float>(int64_t dpad, int64_t t) {
+    return t > fma_cols(dpad) ? kWideColumns : fma_cols(dpad);
+}
+template <> int mmv_small_width<float>(int64_t dpad, int tc) {
+    if (tc > fma_cols(dpad)) return kWideColumns;
+    static const int widths[] = {1, 2, 3, 4, 6, 8, 12, 16};
+    for (int w : widths) if (tc <= w) return w;
+    return tc;
 }
 #endif
 
@@ -32,6 +48,8 @@ int FLK_CAT(launch_mmv_small_kf, FLK_KF)<float>(const PackedView &A, const Packe
                                                 float *partial, hipStream_t st) {
     if (A.dpad != B.dpad || A.d != B.d)
         return fail(FLK_EINVAL, "mmv_small: operands packed with different feature counts");
+    if (tt > fma_cols(A.dpad))
+        return FLK_CAT(launch_mmv_small_f32_wide_kf, FLK_KF)(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st);
     // odd d up to kFoldMaxD: the padding feature holds 1.0 (see pack_kernel) and carries hB through the MFMA chain
     if (f32_fold_applies(A.d))
         return FLK_CAT(launch_mmv_small_f32_fold_kf, FLK_KF)(A, B, vecp, vec_ld, tt, a_chunk_blocks, splits, partial, st);

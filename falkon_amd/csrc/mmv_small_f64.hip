@@ -138,8 +138,10 @@ constexpr int kMaxDp64Fr2 = 16;  // dpad <= 64
 
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<double>() { return 4 * kMaxDp64Fr2; }
-template <> int mmv_small_max_cols<double>(int64_t dpad) { (void)dpad; return 4; }
-template <> int mmv_small_b_blocks_per_wg<double>(int64_t dpad) {
+template <> int mmv_small_max_cols<double>(int64_t dpad, int64_t t) { (void)dpad; (void)t; return 4; }
+template <> int mmv_small_width<double>(int64_t dpad, int tc) { (void)dpad; return tc; }
+template <> int mmv_small_b_blocks_per_wg<double>(int64_t dpad, int64_t t) {
+    (void)t;
     return kWavesPerWg64 * ((dpad / 4) <= kMaxDp64Fr4 ? 4 : 2);
 }
 #endif

@@ -369,3 +369,23 @@ def test_host_rows_streamed_in_chunks(dev, monkeypatch, order, pinned):
     assert rel_err(k.dmmv(X, Cg, vg, wg), exp_d) < 1e-12    # only X streamed
     assert rel_err(k.dmmv(Xg, Cg, vg, w), exp_d) < 1e-12    # only w streamed
     assert rel_err(k.dmmv(X, Cg, vg, None), k.dmmv(Xg, Cg, vg, None)) < 1e-12
+
+
+@pytest.mark.parametrize("d,t", [(3, 17), (3, 40), (9, 32), (15, 13), (16, 33), (17, 9), (28, 10), (28, 32), (31, 9),
+                                 (33, 5), (40, 12), (63, 7), (64, 33)])
+def test_many_right_hand_sides_small_d(dev, d, t):
+    """More right-hand sides than the per-lane FMA kernels take in one pass: the 32-column register-resident kernel
+    (contraction on the matrix cores), folded and plain operands, four and two resident blocks per wave, a second
+    pass for the columns beyond 32."""
+    n, m = 900 + d, 260 + t
+    X, C, v, w = _rand(n, d, m, t, torch.float32, seed=d * 100 + t)
+    k = GaussianKernel(0.9 * np.sqrt(d))
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+    check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, k.sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, k.sigma), 1e-5)
+    got = k.dmmv(Xg, Cg, vg, wg)
+    check_parity(got, mmv_ref.fdmmv_ref(X, C, v, w, k.sigma), mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, k.sigma), 1e-5)
+    assert torch.equal(got, k.dmmv(Xg, Cg, vg, wg))
+    # column by column through the single-column kernels: the same numbers up to rounding
+    cols = torch.cat([k.dmmv(Xg, Cg, vg[:, i:i + 1].contiguous(), wg[:, i:i + 1].contiguous()) for i in (0, t - 1)], 1)
+    assert rel_err(got[:, [0, t - 1]], cols) < 5e-6
