@@ -289,15 +289,24 @@ def main():
         else:
             kernel.mmv(Xg, Cg, vg, out=out)
 
-    for _ in range(args.warmup):
+    first_ms = None
+    for i in range(args.warmup):
+        t0 = time.perf_counter()
         step()
+        if i == 0:                                   # the first call of the process: cold caches, lazy module load
+            torch.cuda.synchronize()
+            first_ms = (time.perf_counter() - t0) * 1e3
     torch.cuda.synchronize()
     lib.flk_kernel_timing_enable(1)                  # HIP events around each product-kernel launch, on its stream
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         step()
+        marks[i + 1].record()                        # per-step spread only; the headline uses the host clock
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
     tot_ms, launches = ctypes.c_double(), ctypes.c_int64()
     rc = lib.flk_kernel_timing_read(ctypes.byref(tot_ms), ctypes.byref(launches))
     _backend.raise_for_status(rc, "flk_kernel_timing_read")
@@ -327,7 +336,13 @@ def main():
                      "avg_launch_ms": kern_ms, "flop_per_launch": flop_per_launch},
         "whole_step_flop_frac": (N * M * ((2 if args.op == "dmmv" else 1) * (2 * d + 4 + 2 * T)))
                                 / (elapsed / args.steps) / 1e12 / peak,
+        "ms_per_step_min": per_step[0] if per_step else None,
+        "ms_per_step_median": per_step[len(per_step) // 2] if per_step else None,
+        "ms_first_call": first_ms,
     }
+    if args.op == "dmmv":
+        # the conservative count: one kernel evaluation per pair, as if K were stored between the two products
+        res["single_evaluation_flop_frac"] = (N * M * (2 * d + 4 + 4 * T)) / (elapsed / args.steps) / 1e12 / peak
     if split:
         res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch,
                                               MEASURED_TRAFFIC_BYTES_BF16X3.get(args.workload)),

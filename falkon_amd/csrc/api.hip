@@ -213,6 +213,7 @@ static int pack_impl(int kf, const void *X, int64_t n, int64_t d, int64_t rs, in
     int rc = check_matrix("X", X, n, d, rs, cs);
     if (rc) return rc;
     if (d < 1) return fail(FLK_EINVAL, "feature dimension must be positive");
+    if (d > flk_max_d(0)) return fail(FLK_EUNSUPPORTED, "more than %lld features", (long long)flk_max_d(0));
     if (sigma == nullptr) return fail(FLK_EINVAL, "sigma: null pointer");
     if (n_sigma != 1 && n_sigma != d)
         return fail(FLK_EINVAL, "The size of sigma (%lld) must match the number of features (%lld) or be 1",
@@ -232,6 +233,7 @@ static int mmv_packed_impl(int kf, const void *pa, int64_t n_a, const void *pb, 
                            int64_t add_cs, void *out, int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes,
                            hipStream_t st) {
     if (n_a < 0 || n_b < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (d > flk_max_d(0)) return fail(FLK_EUNSUPPORTED, "more than %lld features", (long long)flk_max_d(0));
     if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
     if (n_b == 0 || t == 0) return FLK_OK;
     if (out == nullptr) return fail(FLK_EINVAL, "out: null pointer");
@@ -268,6 +270,7 @@ static int fmmv_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x
                      int64_t v_cs, int64_t t, void *out, int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes,
                      hipStream_t st) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (d > flk_max_d(0)) return fail(FLK_EUNSUPPORTED, "more than %lld features", (long long)flk_max_d(0));
     if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
     int rc;
     if ((rc = check_matrix("v", v, m, t, v_rs, v_cs))) return rc;
@@ -290,6 +293,7 @@ static int fdmmv_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t 
                       int64_t v_rs, int64_t v_cs, const void *w, int64_t w_rs, int64_t w_cs, int64_t t, void *out,
                       int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes, hipStream_t st) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (d > flk_max_d(0)) return fail(FLK_EUNSUPPORTED, "more than %lld features", (long long)flk_max_d(0));
     if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
     int rc;
     if (v == nullptr && m > 0 && t > 0) return fail(FLK_EINVAL, "v: null pointer (v is required)");
@@ -331,6 +335,7 @@ static int fmm_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1
                     int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, void *out, int64_t out_rs,
                     int64_t out_cs, void *ws, size_t ws_bytes, hipStream_t st) {
     if (n < 0 || m < 0 || d < 1) return fail(FLK_EINVAL, "bad shape");
+    if (d > flk_max_d(0)) return fail(FLK_EUNSUPPORTED, "more than %lld features", (long long)flk_max_d(0));
     int rc;
     if ((rc = check_matrix("X1", X1, n, d, x1_rs, x1_cs))) return rc;
     if ((rc = check_matrix("X2", X2, m, d, x2_rs, x2_cs))) return rc;
@@ -460,6 +465,7 @@ static int fmmv_split_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int
                            int64_t v_rs, int64_t v_cs, int64_t t, void *out, int64_t out_rs, int64_t out_cs, void *ws,
                            size_t ws_bytes, hipStream_t st) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (d > flk_max_d(0)) return fail(FLK_EUNSUPPORTED, "more than %lld features", (long long)flk_max_d(0));
     if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
     int rc;
     if ((rc = check_matrix("v", v, m, t, v_rs, v_cs))) return rc;
@@ -486,6 +492,7 @@ static int fdmmv_split_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, in
                             int64_t v_rs, int64_t v_cs, const void *w, int64_t w_rs, int64_t w_cs, int64_t t, void *out,
                             int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes, hipStream_t st) {
     if (n < 0 || m < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (d > flk_max_d(0)) return fail(FLK_EUNSUPPORTED, "more than %lld features", (long long)flk_max_d(0));
     if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
     int rc;
     if (v == nullptr && m > 0 && t > 0) return fail(FLK_EINVAL, "v: null pointer (v is required)");
@@ -550,8 +557,12 @@ int flk_kernel_timing_read(double *total_ms, int64_t *launches) {
     return FLK_OK;
 }
 
+static bool known_dtype(int dtype, bool with_split) {
+    return dtype == FLK_F32 || dtype == FLK_F64 || (with_split && dtype == FLK_F32_BF16X3);
+}
+
 size_t flk_gauss_packed_bytes(int64_t n, int64_t d, int dtype) {
-    if (n < 0 || d < 1) return 0;
+    if (n < 0 || d < 1 || d > flk_max_d(dtype) || !known_dtype(dtype, false)) return 0;
     return dtype == FLK_F64 ? packed_bytes<double>(n, d) : packed_bytes<float>(n, d);
 }
 
@@ -574,7 +585,8 @@ int flk_gauss_pack(const void *X, int64_t n, int64_t d, int64_t x_rs, int64_t x_
 }
 
 size_t flk_gauss_mmv_packed_workspace_bytes(int64_t n_a, int64_t n_b, int64_t d, int64_t t, int dtype) {
-    if (n_a < 0 || n_b < 0 || d < 1 || t < 0) return 0;
+    if (n_a < 0 || n_b < 0 || d < 1 || t < 0 || d > flk_max_d(dtype) || t > flk_max_t() || !known_dtype(dtype, false))
+        return 0;
     if (dtype == FLK_F64)
         return planar_bytes<double>(n_a, n_b, d, t) + partial_bytes<double>(n_a, n_b, d, t);
     return planar_bytes<float>(n_a, n_b, d, t) + partial_bytes<float>(n_a, n_b, d, t);
@@ -604,7 +616,8 @@ int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b
 }
 
 size_t flk_gauss_fmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
-    if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
+    if (n < 0 || m < 0 || d < 1 || t < 0 || d > flk_max_d(dtype) || t > flk_max_t() || !known_dtype(dtype, true))
+        return 0;
     if (dtype == FLK_F32_BF16X3 && split_applies(d, t)) return fmmv_split_ws_bytes(n, m, d, t);
     return dtype == FLK_F64 ? fmmv_ws_bytes<double>(n, m, d, t) : fmmv_ws_bytes<float>(n, m, d, t);
 }
@@ -636,7 +649,8 @@ int flk_gauss_fmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, cons
 }
 
 size_t flk_gauss_fdmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype) {
-    if (n < 0 || m < 0 || d < 1 || t < 0) return 0;
+    if (n < 0 || m < 0 || d < 1 || t < 0 || d > flk_max_d(dtype) || t > flk_max_t() || !known_dtype(dtype, true))
+        return 0;
     if (dtype == FLK_F32_BF16X3 && split_applies(d, t)) return fdmmv_split_ws_bytes(n, m, d, t);
     return dtype == FLK_F64 ? fdmmv_ws_bytes<double>(n, m, d, t) : fdmmv_ws_bytes<float>(n, m, d, t);
 }
@@ -669,7 +683,7 @@ int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, con
 }
 
 size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype, int compute_f64) {
-    if (n < 0 || m < 0 || d < 1) return 0;
+    if (n < 0 || m < 0 || d < 1 || d > flk_max_d(dtype) || !known_dtype(dtype, false)) return 0;
     if (dtype == FLK_F64 || compute_f64) return packed_bytes<double>(n, d) + packed_bytes<double>(m, d);
     return packed_bytes<float>(n, d) + packed_bytes<float>(m, d);
 }

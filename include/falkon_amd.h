@@ -63,7 +63,8 @@ int flk_version(void);
 /* Message describing the last non-zero return on this thread ("" if none). */
 const char *flk_last_error(void);
 
-/* Largest feature dimension and number of right-hand sides the kernels cover. */
+/* Largest feature dimension and number of right-hand sides the kernels cover: calls beyond them return
+ * FLK_EUNSUPPORTED, and the size queries below return 0 for them, as for a negative shape or an unknown dtype. */
 int64_t flk_max_d(int dtype);
 int64_t flk_max_t(void);
 

@@ -43,6 +43,19 @@ def test_size_queries_need_no_gpu():
     assert 0 < small < big
     # config 2 stays far below 288 GB: nothing of size N x M is ever allocated
     assert lib.flk_gauss_fdmmv_workspace_bytes(1_000_000, 20_000, 28, 1, _backend.FLK_F32) < 512 * 2**20
+    # what no call would accept has no size: negative shapes, unknown dtypes, shapes beyond the published limits
+    too_wide, too_many = lib.flk_max_d(_backend.FLK_F32) + 1, lib.flk_max_t() + 1
+    for query in (lib.flk_gauss_fmmv_workspace_bytes, lib.flk_gauss_fdmmv_workspace_bytes,
+                  lib.flk_gauss_mmv_packed_workspace_bytes):
+        assert query(100, 10, 3, 1, _backend.FLK_F32) > 0
+        assert query(-1, 10, 3, 1, _backend.FLK_F32) == 0
+        assert query(100, 10, 3, 1, 7) == 0
+        assert query(100, 10, too_wide, 1, _backend.FLK_F32) == 0
+        assert query(100, 10, 3, too_many, _backend.FLK_F32) == 0
+    assert lib.flk_gauss_packed_bytes(10, 3, 7) == 0 and lib.flk_gauss_packed_bytes(10, too_wide, _backend.FLK_F32) == 0
+    assert lib.flk_gauss_fmmv_workspace_bytes(100, 10, 3, 1, _backend.FLK_F32_BF16X3) > 0
+    # the bf16x3 code belongs to the product entry points only
+    assert lib.flk_gauss_mmv_packed_workspace_bytes(100, 10, 3, 1, _backend.FLK_F32_BF16X3) == 0
 
 
 def test_bad_arguments_rejected_on_host_before_any_launch():
@@ -55,6 +68,10 @@ def test_bad_arguments_rejected_on_host_before_any_launch():
     assert rc == _backend.FLK_EINVAL and "stride" in _backend.last_error()
     rc = lib.flk_gauss_pack(4096, 10, 3, 3, 1, 4096, 1, 7, 4096, 1 << 20, None)
     assert rc == _backend.FLK_EINVAL
+    too_wide = lib.flk_max_d(_backend.FLK_F32) + 1
+    rc = lib.flk_gauss_fmmv(4096, 10, too_wide, 1, 4096, 5, too_wide, 1, too_wide, 4096, 1, 4096, 1, 1, 1, 4096, 1, 1,
+                            _backend.FLK_F32, 4096, 1 << 20, None)
+    assert rc == _backend.FLK_EUNSUPPORTED and "features" in _backend.last_error()
     rc = lib.flk_gauss_fmmv(4096, 10, 3, 1, 4096, 5, 3, 1, 3, 4096, 1, 4096, 1, 1, 1, 4096, 1, 1, _backend.FLK_F32,
                             4096, 16, None)
     assert rc == _backend.FLK_ENOMEM
