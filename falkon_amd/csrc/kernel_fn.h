@@ -40,6 +40,34 @@ inline double operand_scale(int kf) {
     }
 }
 
+// 2^e in double precision for e <= 0 (gfx950 has no fp64 exponential instruction; this replaces the library routine,
+// which also serves positive, huge and non-finite arguments: 8 % off the small-d fp64 products).  e = n + f with
+// n = rint(e) read from the low word of e + 1.5 * 2^52 and f = e - n in [-1/2, 1/2] exact; 2^f from the degree-11
+// interpolant at the Chebyshev nodes (relative error 3.2e-18 before rounding; 2^0 = 1 exactly); v_ldexp_f64 applies
+// 2^n and rounds results below 2^-1022 correctly.  Arguments below -1100 are raised to it (the result is 0 from
+// -1075 on), so that n always fits the low word.  (Scaling through the exponent field instead of v_ldexp_f64, with
+// results below 2^-1021 flushed to zero, measured no faster.)
+__device__ __forceinline__ double exp2_nonpositive(double e) {
+    constexpr double kRound = 6755399441055744.0;       // 1.5 * 2^52: adding it rounds to the nearest integer
+    e = fmax(e, -1100.0);
+    const double t = e + kRound;
+    const int n = (int)(unsigned)__double_as_longlong(t);  // the integer, in two's complement, is the low word
+    const double f = e - (t - kRound);
+    double p = 0x1.e9ec1fcb69a7fp-32;
+    p = fma(p, f, 0x1.e6228acd1c6e5p-28);
+    p = fma(p, f, 0x1.b524ebd13a55fp-24);
+    p = fma(p, f, 0x1.62bfc2c86d700p-20);
+    p = fma(p, f, 0x1.ffcbfc6da6ed1p-17);
+    p = fma(p, f, 0x1.430913112c61bp-13);
+    p = fma(p, f, 0x1.5d87fe78a3f9cp-10);
+    p = fma(p, f, 0x1.3b2ab6fb9f1a5p-7);
+    p = fma(p, f, 0x1.c6b08d704a0c6p-5);
+    p = fma(p, f, 0x1.ebfbdff82c5aep-3);
+    p = fma(p, f, 0x1.62e42fefa39efp-1);
+    p = fma(p, f, 1.0);
+    return __builtin_ldexp(p, n);
+}
+
 template <int KF> struct KernelFn;
 
 // Gaussian: the median-of-three with 0 and 1 folds into the clamp bit of v_exp_f32, so the clamp is free
@@ -47,7 +75,7 @@ template <> struct KernelFn<FLK_GAUSSIAN> {
     static __device__ __forceinline__ float value(float e) {
         return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(e), 0.0f, 1.0f);
     }
-    static __device__ __forceinline__ double value(double e) { return exp2(fmin(e, 0.0)); }
+    static __device__ __forceinline__ double value(double e) { return exp2_nonpositive(fmin(e, 0.0)); }
 };
 
 // q = sqrt(max(-e, clamp)): the scaled distance, with the reference's clamp carried over to q^2
@@ -65,7 +93,7 @@ template <> struct KernelFn<FLK_LAPLACIAN> {
     static __device__ __forceinline__ float value(float e) {
         return __builtin_amdgcn_exp2f(-scaled_distance<FLK_LAPLACIAN>(e));
     }
-    static __device__ __forceinline__ double value(double e) { return exp2(-scaled_distance<FLK_LAPLACIAN>(e)); }
+    static __device__ __forceinline__ double value(double e) { return exp2_nonpositive(-scaled_distance<FLK_LAPLACIAN>(e)); }
 };
 
 template <> struct KernelFn<FLK_LAPLACIAN_DU> {
@@ -76,7 +104,7 @@ template <> struct KernelFn<FLK_LAPLACIAN_DU> {
     }
     static __device__ __forceinline__ double value(double e) {
         const double q = scaled_distance<FLK_LAPLACIAN_DU>(e);
-        return -e > distance_clamp<FLK_LAPLACIAN_DU>() ? exp2(-q) * kLog2e / q : 0.0;
+        return -e > distance_clamp<FLK_LAPLACIAN_DU>() ? exp2_nonpositive(-q) * kLog2e / q : 0.0;
     }
 };
 
@@ -87,7 +115,7 @@ template <> struct KernelFn<FLK_MATERN32> {
     }
     static __device__ __forceinline__ double value(double e) {
         const double q = scaled_distance<FLK_MATERN32>(e);
-        return fma(q, 1.0 / kLog2e, 1.0) * exp2(-q);
+        return fma(q, 1.0 / kLog2e, 1.0) * exp2_nonpositive(-q);
     }
 };
 
@@ -99,7 +127,7 @@ template <> struct KernelFn<FLK_MATERN52> {
     }
     static __device__ __forceinline__ double value(double e) {
         const double q = scaled_distance<FLK_MATERN52>(e);
-        return fma(q, fma(q, 1.0 / (3.0 * kLog2e * kLog2e), 1.0 / kLog2e), 1.0) * exp2(-q);
+        return fma(q, fma(q, 1.0 / (3.0 * kLog2e * kLog2e), 1.0 / kLog2e), 1.0) * exp2_nonpositive(-q);
     }
 };
 

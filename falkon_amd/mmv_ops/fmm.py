@@ -103,7 +103,6 @@ def _fmm_run(kernel, kernel_fn: int, opt: BaseOptions, out, X1, X2, cached_sigma
         code, sz = _DTYPE_CODE[X1.dtype], sizeof_dtype(X1.dtype)
         compute_f64 = X1.dtype == torch.float32 and bool(opt.no_single_kernel)
         sigma_dev = kernel._sigma_on(dev, X1.dtype, cached=cached_sigma)
-        usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack)
         x1_in, out_in = X1.device == dev, out.device == dev
         fixed = 0 if X2.device == dev else M * D * sz
 
@@ -111,6 +110,7 @@ def _fmm_run(kernel, kernel_fn: int, opt: BaseOptions, out, X1, X2, cached_sigma
             stage = (0 if x1_in else rows * D * sz) + (0 if out_in else rows * M * sz)
             return lib.flk_gauss_fmm_workspace_bytes(rows, M, D, code, int(compute_f64)) + stage + fixed
 
+        usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack, enough=need(N))
         blk = _rows_that_fit(N, need, usable)
         X2d = _on(X2, dev)
         for i in range(0, N, blk):

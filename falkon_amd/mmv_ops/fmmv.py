@@ -290,7 +290,6 @@ def _fmmv_run(X1, X2, v, kernel, kernel_fn: int, out, opt: BaseOptions, cached_s
 
     with torch.inference_mode():
         sigma_dev = kernel._sigma_on(dev, X1.dtype, cached=cached_sigma)
-        usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack)
         fixed = (0 if X2.device == dev else M * D * sz) + (0 if v.device == dev else M * T * sz)
 
         def need(rows: int) -> float:
@@ -298,6 +297,7 @@ def _fmmv_run(X1, X2, v, kernel, kernel_fn: int, out, opt: BaseOptions, cached_s
             result = 0 if out_in else (rows if x1_in else N) * T * sz                    # see below
             return lib.flk_gauss_fmmv_workspace_bytes(rows, M, D, T, code) + stage + result + fixed
 
+        usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack, enough=need(N))
         blk = _rows_that_fit(N, need, usable) if N > 0 else 0
         X2d, vd = _on(X2, dev), _on(v, dev)
         if x1_in:
@@ -349,7 +349,6 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
         x1_in, out_in = X1.device == dev, out.device == dev
         w_in = w is None or w.device == dev
         sigma_dev = kernel._sigma_on(dev, X1.dtype)
-        usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack)
         fixed = ((0 if X2.device == dev else M * D * sz) + (0 if v.device == dev else M * T * sz)
                  + (0 if out_in else M * T * sz))
 
@@ -358,6 +357,7 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
             extra = M * T * sz if rows < N else 0          # per-block result that is added into out
             return lib.flk_gauss_fdmmv_workspace_bytes(rows, M, D, T, code) + stage + fixed + extra
 
+        usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack, enough=need(N))
         blk = _rows_that_fit(N, need, usable) if N > 0 else 0
         X2d, vd = _on(X2, dev), _on(v, dev)
         outd = out if out_in else torch.empty((M, T), dtype=out.dtype, device=dev)

@@ -38,11 +38,18 @@ def create_output_mat(out: Optional[torch.Tensor], data_devs: Sequence[torch.dev
     return create_C(shape, dtype, device=out_dev, pin_memory=pin)
 
 
-def usable_gpu_memory(dev: torch.device, max_gpu_mem: float, slack: float) -> float:
+def usable_gpu_memory(dev: torch.device, max_gpu_mem: float, slack: float, enough: float = float("inf")) -> float:
     """Bytes a call may use on ``dev``: ``slack * min(free, max_gpu_mem)``
     (falkon/mmv_ops/utils.py:47-58; free memory counts what torch's allocator holds cached,
-    falkon/utils/devices.py:84-96).  Raises MemoryError when nothing is left."""
+    falkon/utils/devices.py:84-96).  Raises MemoryError when nothing is left.
+
+    ``enough`` is what the caller needs at most: when the memory the driver reports free already covers it, the
+    allocator's statistics (by far the slowest part of a small call: two passes over a few hundred counters) are
+    not read, and the value returned is a lower bound of the usable memory that is at least ``enough``."""
     free, _total = torch.cuda.mem_get_info(dev)
+    usable = min(free * slack, max_gpu_mem * slack)
+    if usable >= enough:
+        return usable
     cached = torch.cuda.memory_reserved(dev) - torch.cuda.memory_allocated(dev)
     usable = min((free + cached) * slack, max_gpu_mem * slack)
     if usable < 0:

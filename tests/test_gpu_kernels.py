@@ -109,3 +109,29 @@ def test_config2_shape_reduced_other_kernels(dev):
         got = k.dmmv(X.to(dev), C.to(dev), v.to(dev), w.to(dev))
         check_parity(got, mmv_ref.fdmmv_ref(X, C, v, w, sigma, kernel_name=name, max_cpu_mem=2 * 2**30),
                      mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma, kernel_name=name, max_cpu_mem=4 * 2**30), 1e-5)
+
+
+@pytest.mark.parametrize("d", [1, 80])
+def test_fp64_exponential_accuracy(dev, d):
+    """The fp64 kernels evaluate 2^e with a routine of their own (the hardware has none): check it against numpy's exp
+    on a grid where the argument is exact (x = k/64 in the first feature, centre 0, sigma 1: K = exp(-k^2/8192)), from
+    K = 1 through the subnormal range down to 0, in the kernel matrix and in both product kernels (d = 1 and 80)."""
+    k = np.arange(0, 64 * 40, dtype=np.float64)         # x up to 40: argument down to -800; exp is 0 below -745.2
+    arg = -(k * k) / 8192
+    want = np.exp(arg)
+    X = torch.zeros(k.size, d, dtype=torch.float64)
+    X[:, 0] = torch.from_numpy(k / 64)
+    C = torch.zeros(1, d, dtype=torch.float64)
+    kern = GaussianKernel(1.0)
+    # the argument reaches the exponential with a relative rounding error of a few eps: allow eps * |argument| on top
+    tol = 1e-15 * (1 + np.abs(arg)) * want + 1e-323
+    for got in (kern(X.to(dev), C.to(dev))[:, 0], kern.mmv(X.to(dev), C.to(dev), torch.ones(1, 1, dtype=torch.float64, device=dev))[:, 0]):
+        got = got.cpu().numpy()
+        worst = np.max((np.abs(got - want) - tol) / np.maximum(want, 1e-300))
+        assert np.all(np.abs(got - want) <= tol), f"worst excess {worst:.3e}"
+        assert got[0] == 1.0 and np.all(got[arg < -760] == 0) and np.all(got[arg > -700] > 0)
+    # the other kernel functions share the routine: Laplacian exp(-x); at x = 0 the reference's clamp of the squared
+    # distance at 1e-20 makes it exp(-1e-10) (falkon/kernels/distance_kernel.py:100)
+    lap = LaplacianKernel(1.0)(X.to(dev), C.to(dev))[:, 0].cpu().numpy()
+    want_l = np.exp(-np.maximum(k / 64, 1e-10))
+    assert np.all(np.abs(lap - want_l) <= 1e-15 * (1 + k / 64) * want_l)
