@@ -13,6 +13,8 @@
 //
 // Waves are arranged WVA (A) x WVB (B); waves with the same wb produce partial sums for the same
 // output rows and simply write separate partials (they count as extra splits for the reduction).
+#include <type_traits>
+
 #include "flk_common.h"
 #include "kernel_fn.h"
 #include "mfma_traits.h"
@@ -38,11 +40,13 @@ template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC> struct LGe
 };
 
 // One 16-byte piece of a stage: vector index vi enumerates [block][step][lane group][row/VPL], which is
-// also the order in LDS, so the LDS side of the copy is linear.  The packed feature count is a whole
-// number of chunks (padded_features), so there is no feature tail to mask.
+// also the order in LDS, so the LDS side of the copy is linear.  MFMA step s contracts the features
+// KG s .. KG s + KG - 1 (lane group lg takes feature KG s + lg), so a step's operands are adjacent rows of the
+// packed block and the zero padding past d sits in the last steps of the last chunk, which the kernel skips.
+// The packed feature count is a whole number of chunks (padded_features), so there is no feature tail to mask.
 template <typename T, int KC>
 __device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t blk0, int64_t nblk, int64_t dpad,
-                                              int64_t DPsteps, int64_t s0, int vi) {
+                                              int64_t s0, int vi) {
     typedef LTraits<T> TR;
     constexpr int VPB = TR::BLK / TR::VPL;
     const int jv = vi % VPB;
@@ -51,7 +55,7 @@ __device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t b
     const int blk = vi / (VPB * TR::KG * KC);
     int64_t b = blk0 + blk;
     if (b >= nblk) b = nblk - 1;                 // past the end: any valid block (its rows get zero weight / are not stored)
-    return P + (b * dpad + (int64_t)lg * DPsteps + s0 + s) * TR::BLK + jv * TR::VPL;
+    return P + (b * dpad + (s0 + s) * TR::KG + lg) * TR::BLK + jv * TR::VPL;
 }
 
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
@@ -59,8 +63,8 @@ template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC, int TT, in
 __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   // two waves per SIMD either way
     mmv_large_kernel(const T *__restrict__ PA, const T *__restrict__ hA, const T *__restrict__ vecp, int64_t vec_ld,
                      int tcols, const T *__restrict__ PB, const T *__restrict__ hB, int64_t na_blocks,
-                     int64_t nb_blocks, int64_t dpad, int64_t a_tiles_per_chunk, T *__restrict__ partial,
-                     int64_t nb_pad, bool y_fastest) {
+                     int64_t nb_blocks, int64_t dpad, int last_steps, int64_t a_tiles_per_chunk,
+                     T *__restrict__ partial, int64_t nb_pad, bool y_fastest) {
     typedef LTraits<T> TR;
     typedef LGeo<T, WVA, WVB, WA_FR, WB_FR, KC> G;
     constexpr int kLWavesA = WVA, kLWavesB = WVB, kLThreads = 64 * WVA * WVB;
@@ -126,10 +130,10 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             const int64_t s0 = chunk * KC;
 #pragma unroll
             for (int c = 0; c < G::A_VPT; c++)
-                ra[c] = *(const V16 *)stage_src<T, KC>(PA, ablk0, na_blocks, dpad, DPsteps, s0, tid + c * kLThreads);
+                ra[c] = *(const V16 *)stage_src<T, KC>(PA, ablk0, na_blocks, dpad, s0, tid + c * kLThreads);
 #pragma unroll
             for (int c = 0; c < G::B_VPT; c++)
-                rb[c] = *(const V16 *)stage_src<T, KC>(PB, bblk0, nb_blocks, dpad, DPsteps, s0, tid + c * kLThreads);
+                rb[c] = *(const V16 *)stage_src<T, KC>(PB, bblk0, nb_blocks, dpad, s0, tid + c * kLThreads);
         };
         auto commit = [&](int buf) {
 #pragma unroll
@@ -194,30 +198,29 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
             for (int q = 0; q < WB_FR; q++) bv[0][q] = lb[(q * KC) * 64];
         }
-        for (int64_t ch = 0; ch < n_chunks; ch++) {
-            const int buf = (int)(ch & 1);
-            const bool more = ch + 1 < n_chunks;
-            if (more) fetch(ch + 1);
+        // The last chunk is a variant of its own (kLast): nothing to prefetch, no barrier (the next tile's prologue
+        // has one before it writes LDS), and it stops after last_steps steps: the features past d in it are padding.
+        auto run_chunk = [&](auto last_tag, const int buf) {
+            constexpr bool kLast = decltype(last_tag)::value;
             const T *la = &ldsA[buf][(wa * WA_FR) * KC * 64 + lane];
             const T *lb = &ldsB[buf][(wb * WB_FR) * KC * 64 + lane];
             const T *la2 = &ldsA[buf ^ 1][(wa * WA_FR) * KC * 64 + lane];
             const T *lb2 = &ldsB[buf ^ 1][(wb * WB_FR) * KC * 64 + lane];
 #pragma unroll
             for (int s = 0; s < KC; s++) {
+                if (kLast && s >= last_steps) break;
                 const int cur = s & 1, nxt = cur ^ 1;
                 if (s + 1 < KC) {
 #pragma unroll
                     for (int p = 0; p < WA_FR; p++) av[nxt][p] = la[(p * KC + s + 1) * 64];
 #pragma unroll
                     for (int q = 0; q < WB_FR; q++) bv[nxt][q] = lb[(q * KC + s + 1) * 64];
-                } else {
+                } else if (!kLast) {
                     __syncthreads();          // all waves: this chunk's LDS reads done, next stage written
-                    if (more) {
 #pragma unroll
-                        for (int p = 0; p < WA_FR; p++) av[nxt][p] = la2[(p * KC) * 64];
+                    for (int p = 0; p < WA_FR; p++) av[nxt][p] = la2[(p * KC) * 64];
 #pragma unroll
-                        for (int q = 0; q < WB_FR; q++) bv[nxt][q] = lb2[(q * KC) * 64];
-                    }
+                    for (int q = 0; q < WB_FR; q++) bv[nxt][q] = lb2[(q * KC) * 64];
                 }
                 asm volatile("" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]), "+v"(acc[1][1]),
                                   "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[3][0]), "+v"(acc[3][1])
@@ -226,9 +229,14 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                 for (int p = 0; p < WA_FR; p++)
 #pragma unroll
                     for (int q = 0; q < WB_FR; q++) acc[p][q] = TR::mfma(av[cur][p], bv[cur][q], acc[p][q]);
-                if (s == kCommitStep && more) commit(buf ^ 1);
+                if (!kLast && s == kCommitStep) commit(buf ^ 1);
             }
+        };
+        for (int64_t ch = 0; ch + 1 < n_chunks; ch++) {
+            fetch(ch + 1);
+            run_chunk(std::false_type{}, (int)(ch & 1));
         }
+        run_chunk(std::true_type{}, (int)((n_chunks - 1) & 1));
 
         // epilogue: exponent = acc + hA_i + hB_j ; K = exp2 clamped ; out[q][t] += K * vec[i][t]
         // Columns are contracted in groups of four whose LDS reads are issued one group ahead; the fence
@@ -380,10 +388,15 @@ static int launch_large_tt(const PackedView &A, const PackedView &B, const T *ve
     typedef LCfg<T> C;
     const int64_t nbb = C::WVB * C::WB_FR;
     dim3 grid((unsigned)((B.nblk + nbb - 1) / nbb), (unsigned)splits);
+    // MFMA steps of the last feature chunk that hold features of the data (the rest of the chunk is zero padding)
+    const int64_t chunk_features = (int64_t)C::KC * LTraits<T>::KG;
+    const int64_t tail = A.d - (A.dpad / chunk_features - 1) * chunk_features;
+    const int last_steps = (int)((tail + LTraits<T>::KG - 1) / LTraits<T>::KG);
+    if (last_steps < 1 || last_steps > C::KC) return fail(FLK_EINVAL, "mmv_large: operand padding does not match d");
     hipLaunchKernelGGL((mmv_large_kernel<T, C::WVA, C::WVB, C::WA_FR, C::WB_FR, C::KC, TT, FLK_KF>), grid,
                        dim3(64 * C::WVA * C::WVB), 0, st,
                        (const T *)A.data, (const T *)A.hnorm, vecp, vec_ld, tcols, (const T *)B.data,
-                       (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, a_tiles_per_chunk, partial, B.npad, B.n > A.n);
+                       (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, last_steps, a_tiles_per_chunk, partial, B.npad, B.n > A.n);
     FLK_LAUNCH_CHECK("mmv_large_kernel");
     return FLK_OK;
 }
