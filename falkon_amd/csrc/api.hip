@@ -201,7 +201,7 @@ static int mmv_packed_planar(int kf, const PackedView &A, const PackedView &B, c
             if (rc != FLK_OK) return rc;
         }
         int rc = launch_finalize<T>(partial, partials, tc, B.n, B.npad, addend ? addend + t0 * add_cs : nullptr,
-                                    add_rs, add_cs, out + t0 * out_cs, out_rs, out_cs, zero_pad, st);
+                                    add_rs, add_cs, out + t0 * out_cs, out_rs, out_cs, zero_pad, (const T *)B.hnorm, st);
         if (rc != FLK_OK) return rc;
     }
     return FLK_OK;
@@ -246,7 +246,8 @@ static int mmv_packed_impl(int kf, const void *pa, int64_t n_a, const void *pb, 
     T *vecp = (T *)ws;
     T *partial = (T *)((char *)ws + vec_bytes);
     Plan plan = make_plan<T>(A.nblk, B.nblk, A.d, A.dpad, t);
-    int rc = launch_vec_planar<T>((const T *)vec, n_a, t, vec_rs, vec_cs, vecp, A.npad, zero_planes_needed<T>(plan, t), st);
+    int rc = launch_vec_planar<T>((const T *)vec, n_a, t, vec_rs, vec_cs, vecp, A.npad, zero_planes_needed<T>(plan, t),
+                                  (const T *)A.hnorm, st);
     if (rc) return rc;
     return mmv_packed_planar<T>(kf, A, B, vecp, t, (const T *)addend, add_rs, add_cs, (T *)out, out_rs, out_cs, false,
                                 partial, ws_bytes - vec_bytes, st);
@@ -316,7 +317,8 @@ static int fdmmv_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t 
     X = packed_view<T>(px, n, d);
     C = packed_view<T>(pc, m, d);
     Plan plan1 = make_plan<T>(C.nblk, X.nblk, d, C.dpad, t), plan2 = make_plan<T>(X.nblk, C.nblk, d, X.dpad, t);
-    if ((rc = launch_vec_planar<T>((const T *)v, m, t, v_rs, v_cs, vp, C.npad, zero_planes_needed<T>(plan1, t), st)))
+    if ((rc = launch_vec_planar<T>((const T *)v, m, t, v_rs, v_cs, vp, C.npad, zero_planes_needed<T>(plan1, t),
+                                   (const T *)C.hnorm, st)))
         return rc;
     // u = K v + w, planar [t][X.npad] with zeroed padding (rows and the spare planes) so it can feed the
     // second product directly
@@ -433,7 +435,7 @@ static int mmv_split_planar(int kf, const SplitView &A, const SplitView &B, cons
             if (rc != FLK_OK) return rc;
         }
         int rc = launch_finalize<float>(partial, partials, tc, B.n, B.npad, addend ? addend + t0 * add_cs : nullptr,
-                                        add_rs, add_cs, out + t0 * out_cs, out_rs, out_cs, zero_pad, st);
+                                        add_rs, add_cs, out + t0 * out_cs, out_rs, out_cs, zero_pad, B.hnorm, st);
         if (rc != FLK_OK) return rc;
     }
     return FLK_OK;
@@ -482,7 +484,7 @@ static int fmmv_split_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int
     if ((rc = pack_split_impl(kf, "X2", X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, st))) return rc;
     SplitView X = split_view(px, n, d), C = split_view(pc, m, d);
     if (n == 0 || t == 0) return FLK_OK;
-    if ((rc = launch_vec_planar<float>((const float *)v, m, t, v_rs, v_cs, vp, C.npad, 0, st))) return rc;
+    if ((rc = launch_vec_planar<float>((const float *)v, m, t, v_rs, v_cs, vp, C.npad, 0, C.hnorm, st))) return rc;
     return mmv_split_planar(kf, C, X, vp, t, nullptr, 0, 0, (float *)out, out_rs, out_cs, false, partial,
                             ws_bytes - (size_t)(p - (char *)ws), st);
 }
@@ -513,7 +515,7 @@ static int fdmmv_split_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, in
     if ((rc = pack_split_impl(kf, "X2", X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, st))) return rc;
     SplitView X = split_view(px, n, d), C = split_view(pc, m, d);
     if (m == 0 || t == 0) return FLK_OK;
-    if ((rc = launch_vec_planar<float>((const float *)v, m, t, v_rs, v_cs, vp, C.npad, 0, st))) return rc;
+    if ((rc = launch_vec_planar<float>((const float *)v, m, t, v_rs, v_cs, vp, C.npad, 0, C.hnorm, st))) return rc;
     // u = K v + w, planar [t][X.npad] with zeroed padding rows so it can feed the second product directly
     if ((rc = mmv_split_planar(kf, C, X, vp, t, (const float *)w, w_rs, w_cs, up, 1, X.npad, true, partial,
                                partial_avail, st)))

@@ -103,15 +103,21 @@ int launch_pack(const TI *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const
                 double scale, T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st);
 
 
+// Non-finite data: a row holding a NaN or an infinity has a non-finite half norm.  The product kernels clamp the
+// kernel value (K <= 1, D^2 >= 1e-20), which turns such a row's NaN exponents into numbers; so that the result still
+// says NaN where the reference's does, the planar copy of a right-hand side takes NaN in the rows whose reduction-side
+// half norm (row_half_norm, may be null) is not finite, and the finalize kernel writes NaN into the output rows whose
+// half norm is not finite.
 template <typename T>
 int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad,
-                      int64_t zero_planes, hipStream_t st);   // also clears zero_planes planes after the t-th
+                      int64_t zero_planes, const T *row_half_norm,
+                      hipStream_t st);   // also clears zero_planes planes after the t-th
 template <typename T> int launch_zero_fill(T *p, int64_t count, hipStream_t st);
 
 template <typename T>
 int launch_finalize(const T *partial, int splits, int64_t t, int64_t nb, int64_t nb_pad, const T *addend,
                     int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
-                    hipStream_t st);
+                    const T *row_half_norm, hipStream_t st);
 
 // Register-resident ("small d") product kernel; the queries do not depend on the kernel function.
 template <typename T> int64_t mmv_small_max_d();

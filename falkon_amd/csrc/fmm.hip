@@ -107,7 +107,10 @@ __global__ void __launch_bounds__(64 * kFmmWavesA * kFmmWavesB)
                 const vec4_t hn = *(const vec4_t *)(&hA[row0]);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const T k = kernel_value<FLK_KF>(acc[p][q][4 * g + e] + (hn[e] + hb));
+                    // h - h is 0, or NaN where a row holds a NaN or an infinity: the kernel functions clamp their
+                    // argument, which would turn such an entry into a number
+                    const T h = hn[e] + hb;
+                    const T k = kernel_value<FLK_KF>(acc[p][q][4 * g + e] + h) + (h - h);
                     if (row0 + e < n_a && col < n_b) __builtin_nontemporal_store((O)k, &out[(row0 + e) * ld + col]);
                 }
             }

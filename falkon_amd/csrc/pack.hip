@@ -84,14 +84,24 @@ template int launch_pack<float, double>(const float *, int64_t, int64_t, int64_t
 
 // ---------------------------------------------------------------------------
 // vec_planar: v[n,t] with element strides (rs, cs) -> vp[t + zero_planes][npad]: rows past n and the
-// zero_planes planes past t are zero.
+// zero_planes planes past t are zero.  Rows whose half norm (of the operand the vector multiplies) is not
+// finite become NaN: their kernel values were clamped to numbers, and 0 * NaN brings the NaN back.
 // ---------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ bool finite_value(T x) { return x - x == T(0); }
+template <typename T> __device__ __forceinline__ T quiet_nan() { return T(0) / T(0); }
+template <> __device__ __forceinline__ float quiet_nan<float>() { return __uint_as_float(0x7fc00000u); }
+template <> __device__ __forceinline__ double quiet_nan<double>() { return __longlong_as_double(0x7ff8000000000000ll); }
+
 template <typename T>
 __global__ void __launch_bounds__(256) vec_planar_kernel(const T *__restrict__ v, int64_t n, int64_t rs, int64_t cs,
-                                                         T *__restrict__ vp, int64_t npad, int64_t tcols) {
+                                                         T *__restrict__ vp, int64_t npad, int64_t tcols,
+                                                         const T *__restrict__ row_half_norm) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     int64_t t = blockIdx.y;
-    if (i < npad) vp[t * npad + i] = (i < n && t < tcols) ? v[i * rs + t * cs] : T(0);
+    if (i >= npad) return;
+    T val = (i < n && t < tcols) ? v[i * rs + t * cs] : T(0);
+    if (row_half_norm && i < n && t < tcols && !finite_value(row_half_norm[i])) val = quiet_nan<T>();
+    vp[t * npad + i] = val;
 }
 
 template <typename T>
@@ -110,28 +120,30 @@ template int launch_zero_fill<float>(float *, int64_t, hipStream_t);
 template int launch_zero_fill<double>(double *, int64_t, hipStream_t);
 template <typename T>
 int launch_vec_planar(const T *v, int64_t n, int64_t t, int64_t rs, int64_t cs, T *vp, int64_t npad,
-                      int64_t zero_planes, hipStream_t st) {
+                      int64_t zero_planes, const T *row_half_norm, hipStream_t st) {
     if (npad == 0 || t == 0) return FLK_OK;
     hipLaunchKernelGGL(vec_planar_kernel<T>, dim3((unsigned)((npad + 255) / 256), (unsigned)(t + zero_planes)),
-                       dim3(256), 0, st, v, n, rs, cs, vp, npad, t);
+                       dim3(256), 0, st, v, n, rs, cs, vp, npad, t, row_half_norm);
     FLK_LAUNCH_CHECK("vec_planar_kernel");
     return FLK_OK;
 }
 template int launch_vec_planar<float>(const float *, int64_t, int64_t, int64_t, int64_t, float *, int64_t, int64_t,
-                                      hipStream_t);
+                                      const float *, hipStream_t);
 template int launch_vec_planar<double>(const double *, int64_t, int64_t, int64_t, int64_t, double *, int64_t, int64_t,
-                                       hipStream_t);
+                                       const double *, hipStream_t);
 
 // ---------------------------------------------------------------------------
 // finalize: out[b,t] = sum_s partial[s][t][b] (+ addend[b,t]); fixed summation
 // order, so results are reproducible run to run (no atomics anywhere).
 // With zero_pad the rows n_b..nb_pad of a planar output are cleared as well.
+// Output rows whose half norm is not finite (a NaN or an infinity in the data row) become NaN.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256) finalize_kernel(const T *__restrict__ partial, int splits, int64_t tt,
                                                        int64_t nb, int64_t nb_pad, const T *__restrict__ addend,
                                                        int64_t add_rs, int64_t add_cs, T *__restrict__ out,
-                                                       int64_t out_rs, int64_t out_cs, bool zero_pad) {
+                                                       int64_t out_rs, int64_t out_cs, bool zero_pad,
+                                                       const T *__restrict__ row_half_norm) {
     int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
     int64_t t = blockIdx.y;
     if (b >= nb_pad) return;
@@ -142,21 +154,24 @@ __global__ void __launch_bounds__(256) finalize_kernel(const T *__restrict__ par
     double s = 0.0;
     for (int sp = 0; sp < splits; sp++) s += (double)partial[((int64_t)sp * tt + t) * nb_pad + b];
     if (addend) s += (double)addend[b * add_rs + t * add_cs];
-    out[b * out_rs + t * out_cs] = (T)s;
+    T res = (T)s;
+    if (row_half_norm && !finite_value(row_half_norm[b])) res = quiet_nan<T>();
+    out[b * out_rs + t * out_cs] = res;
 }
 template <typename T>
 int launch_finalize(const T *partial, int splits, int64_t t, int64_t nb, int64_t nb_pad, const T *addend,
                     int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
-                    hipStream_t st) {
+                    const T *row_half_norm, hipStream_t st) {
     if (nb_pad == 0 || t == 0) return FLK_OK;
     hipLaunchKernelGGL(finalize_kernel<T>, dim3((unsigned)((nb_pad + 255) / 256), (unsigned)t), dim3(256), 0, st,
-                       partial, splits, t, nb, nb_pad, addend, add_rs, add_cs, out, out_rs, out_cs, zero_pad);
+                       partial, splits, t, nb, nb_pad, addend, add_rs, add_cs, out, out_rs, out_cs, zero_pad,
+                       row_half_norm);
     FLK_LAUNCH_CHECK("finalize_kernel");
     return FLK_OK;
 }
 template int launch_finalize<float>(const float *, int, int64_t, int64_t, int64_t, const float *, int64_t, int64_t,
-                                    float *, int64_t, int64_t, bool, hipStream_t);
+                                    float *, int64_t, int64_t, bool, const float *, hipStream_t);
 template int launch_finalize<double>(const double *, int, int64_t, int64_t, int64_t, const double *, int64_t, int64_t,
-                                     double *, int64_t, int64_t, bool, hipStream_t);
+                                     double *, int64_t, int64_t, bool, const double *, hipStream_t);
 
 }  // namespace flk

@@ -27,7 +27,8 @@ typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 // k-step, which carries it, is written.
 __global__ void __launch_bounds__(256) pack_split_kernel(const float *__restrict__ X, int64_t n, int64_t d, int64_t rs,
                                                          int64_t cs, const float *__restrict__ sigma, int64_t n_sigma,
-                                                         double scale, uintx4 *__restrict__ P, int ks_count) {
+                                                         double scale, uintx4 *__restrict__ P, float *__restrict__ hnorm,
+                                                         int ks_count) {
     constexpr int KT = 32;                       // features per LDS tile = two k-steps
     __shared__ float tile[32][KT + 1];
     __shared__ double nrm[32];
@@ -82,6 +83,7 @@ __global__ void __launch_bounds__(256) pack_split_kernel(const float *__restrict
             dst[128] = out[2];
         }
     }
+    if (tid < 32) hnorm[row0 + tid] = (float)(-0.5 * nrm[tid]);   // zero on the padding rows
 }
 
 int launch_pack_split(const float *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const float *sigma, int64_t n_sigma,
@@ -89,7 +91,7 @@ int launch_pack_split(const float *X, int64_t n, int64_t d, int64_t rs, int64_t 
     const int64_t nblk = (n + 31) / 32;
     if (nblk == 0) return FLK_OK;
     hipLaunchKernelGGL(pack_split_kernel, dim3((unsigned)nblk), dim3(256), 0, st, X, n, d, rs, cs, sigma, n_sigma, scale,
-                       (uintx4 *)packed, (int)split_ksteps(d));
+                       (uintx4 *)packed, (float *)((char *)packed + split_data_bytes(n, d)), (int)split_ksteps(d));
     FLK_LAUNCH_CHECK("pack_split_kernel");
     return FLK_OK;
 }

@@ -24,16 +24,22 @@ constexpr int kSplitMaxCols = 2;            // its right-hand sides per pass
 inline int64_t split_ksteps(int64_t d) { return (d + 2 + 15) / 16; }
 
 struct SplitView {
-    const void *data;   // [nblk][ks][3][64] x 16 bytes
+    const void *data;    // [nblk][ks][3][64] x 16 bytes
+    const float *hnorm;  // [npad] half norms in fp32 (the kernels use the split copy inside data; this one tells
+                         // the prologue and epilogue kernels which rows hold non-finite data)
     int64_t n, d, ks, nblk, npad;
 };
-inline size_t split_packed_bytes(int64_t n, int64_t d) {
+inline size_t split_data_bytes(int64_t n, int64_t d) {
     const int64_t nblk = (n + 31) / 32;
     return align256((size_t)nblk * split_ksteps(d) * 3 * 64 * 16);
+}
+inline size_t split_packed_bytes(int64_t n, int64_t d) {
+    return split_data_bytes(n, d) + align256((size_t)((n + 31) / 32 * 32) * sizeof(float));
 }
 inline SplitView split_view(const void *buf, int64_t n, int64_t d) {
     SplitView v;
     v.data = buf; v.n = n; v.d = d;
+    v.hnorm = buf ? (const float *)((const char *)buf + split_data_bytes(n, d)) : nullptr;
     v.ks = split_ksteps(d);
     v.nblk = (n + 31) / 32;
     v.npad = v.nblk * 32;

@@ -389,3 +389,46 @@ def test_many_right_hand_sides_small_d(dev, d, t):
     # column by column through the single-column kernels: the same numbers up to rounding
     cols = torch.cat([k.dmmv(Xg, Cg, vg[:, i:i + 1].contiguous(), wg[:, i:i + 1].contiguous()) for i in (0, t - 1)], 1)
     assert rel_err(got[:, [0, t - 1]], cols) < 5e-6
+
+
+@pytest.mark.parametrize("mode", ["f32", "f64", "bf16x3"])
+@pytest.mark.parametrize("d,t", [(8, 1), (28, 2), (28, 20), (40, 6), (100, 1), (100, 10)])
+def test_non_finite_rows_give_nan(dev, mode, d, t):
+    """A NaN or an infinity in a data row must surface as NaN where the reference's result is NaN
+    (falkon/kernels/distance_kernel.py:88-101,140-159 propagate it through the squared distance), although the
+    kernels clamp the kernel value: rows of K(X1, X2) v whose X1 row is bad, everything when an X2 row is bad (every
+    output sums over it), every entry of K^T(K v + w) either way; all other rows are what they are without the bad
+    rows.  Every kernel family is visited (d, T: register-resident, 32-column, LDS-tiled, their bf16x3 twins)."""
+    from falkon_amd import LaplacianKernel
+    dtype = torch.float64 if mode == "f64" else torch.float32
+    opt = FalkonOptions(bf16x3_cross_term=mode == "bf16x3")
+    X, C, v, w = _rand(300, d, 170, t, dtype, seed=21)
+    Xb = X.clone()
+    Xb[3, d // 2] = float("nan")
+    Xb[150, 0] = float("inf")
+    Xb[299, d - 1] = float("-inf")
+    bad = torch.zeros(300, dtype=torch.bool)
+    bad[[3, 150, 299]] = True
+    Cb = C.clone()
+    Cb[7, 0] = float("nan")
+    for K in (GaussianKernel, LaplacianKernel):
+        k = K(float(d) ** 0.5, opt=opt)
+        clean = k.mmv(X.to(dev), C.to(dev), v.to(dev)).cpu()
+        got = k.mmv(Xb.to(dev), C.to(dev), v.to(dev)).cpu()
+        assert torch.isnan(got[bad]).all()
+        assert torch.equal(got[~bad], clean[~bad])
+        assert torch.isnan(k.mmv(X.to(dev), Cb.to(dev), v.to(dev))).all()
+        assert torch.isnan(k.dmmv(Xb.to(dev), C.to(dev), v.to(dev), w.to(dev))).all()
+        assert torch.isnan(k.dmmv(X.to(dev), Cb.to(dev), v.to(dev), None)).all()
+        assert not torch.isnan(k.dmmv(X.to(dev), C.to(dev), v.to(dev), w.to(dev))).any()
+        if t == 1:
+            full_clean = k(X.to(dev), C.to(dev)).cpu()
+            full = k(Xb.to(dev), Cb.to(dev)).cpu()
+            assert torch.isnan(full[bad]).all() and torch.isnan(full[:, 7]).all()
+            keep = ~bad
+            cols = torch.arange(170) != 7
+            assert torch.equal(full[keep][:, cols], full_clean[keep][:, cols])
+    # the CPU path says NaN in the same places for a NaN entry (an infinity gives it NaN or 0, depending on signs)
+    if mode != "bf16x3" and t == 1:
+        ref = mmv_ref.fmmv_ref(Xb, C, v, float(d) ** 0.5)
+        assert torch.isnan(ref[3]).all() and not torch.isnan(ref[~bad]).any()
