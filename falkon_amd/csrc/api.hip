@@ -139,9 +139,9 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
 // that many planes of the planar right-hand side, so the planes past the caller's columns must be zero.
 template <typename T>
 static int instantiated_cols(const Plan &p, int tc) {
-    static const int large[] = {1, 2, 4, 16};
+    static const int large[] = {1, 2, 4, 8, 16};     // the 8-column instantiation exists in fp64 only
     if (p.large) {
-        for (int w : large) if (tc <= w) return w;
+        for (int w : large) if (tc <= w && (w != 8 || sizeof(T) == 8)) return w;
         return tc;
     }
     return mmv_small_width<T>(p.dpad, tc);

@@ -25,6 +25,10 @@
 
 namespace flk {
 
+// Right-hand sides up to which the epilogue contracts with per-lane FMAs (measured: the MFMA contraction is the
+// faster one from five columns on in fp32, from nine on in fp64, where it costs four 64-cycle MFMAs per 16 x 16 tile).
+template <typename T> constexpr int kLargeFmaCols = sizeof(T) == 8 ? 8 : 4;
+
 template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC> struct LGeo {
     typedef LTraits<T> TR;
     static constexpr int kLWavesA = WVA, kLWavesB = WVB, kLThreads = 64 * WVA * WVB;
@@ -74,10 +78,10 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 
     __shared__ __attribute__((aligned(16))) T ldsA[2][G::A_ELEMS];
     __shared__ __attribute__((aligned(16))) T ldsB[2][G::B_ELEMS];
-    // More than four columns: the contraction against vec runs on the MFMA as well (a second, small GEMM whose
-    // A operand are the kernel values sitting in the accumulator registers, see the epilogue), with vec staged
-    // as [row][16 columns] at a stride of 17 elements.  Up to four columns: per-lane FMAs, vec staged planar.
-    constexpr bool kMfmaEpi = TT > 4;
+    // More than four (fp32) / eight (fp64) columns: the contraction against vec runs on the MFMA as well (a second,
+    // small GEMM whose A operand are the kernel values sitting in the accumulator registers, see the epilogue), with vec staged
+    // as [row][16 columns] at a stride of 17 elements.  Fewer columns: per-lane FMAs, vec staged planar.
+    constexpr bool kMfmaEpi = TT > kLargeFmaCols<T>;
     constexpr int kVecStride = 17;
     constexpr int kRowBuf = kMfmaEpi ? G::A_ROWS * (1 + kVecStride) : (1 + TT) * G::A_ROWS;
     __shared__ __attribute__((aligned(32))) T ldsRow[kRowBuf];   // [hA | vec ...] of the A tile
@@ -411,6 +415,8 @@ int FLK_CAT(launch_mmv_large_kf, FLK_KF)(const PackedView &A, const PackedView &
     if (tcols == 1) return launch_large_tt<T, 1>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols == 2) return launch_large_tt<T, 2>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols <= 4) return launch_large_tt<T, 4>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    if constexpr (kLargeFmaCols<T> == 8)
+        if (tcols <= 8) return launch_large_tt<T, 8>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     return launch_large_tt<T, 16>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);   // MFMA epilogue
 }
 template int FLK_CAT(launch_mmv_large_kf, FLK_KF)<float>(const PackedView &, const PackedView &, const float *, int64_t,

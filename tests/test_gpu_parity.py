@@ -99,6 +99,8 @@ def test_reference_fixture_fp64(dev, order, sig):
     (700, 20, 1000, 5),
     (600, 400, 96, 16),     # a full 16-column pass (the MFMA contraction of kernel values against v)
     (333, 520, 300, 7),
+    (257, 129, 70, 8),      # eight columns (per-lane FMAs in fp64), a last feature chunk that is mostly padding
+    (130, 300, 97, 9),      # one real feature in the last chunk
 ])
 def test_large_d_vs_oracle(dev, dtype, n, m, d, t):
     """d > 64 runs the LDS-tiled kernel; same tolerances against the blocked CPU oracle."""
