@@ -260,6 +260,10 @@ def main():
     from falkon_amd import FalkonOptions, GaussianKernel, LaplacianKernel, MaternKernel, _backend
     lib = _backend.load()                            # raises if the HIP library is missing
     kopt = FalkonOptions(bf16x3_cross_term=args.cross_term == "bf16x3")
+    def make_kernel_with(o):
+        return {"gaussian": lambda s: GaussianKernel(s, opt=o), "laplacian": lambda s: LaplacianKernel(s, opt=o),
+                "matern32": lambda s: MaternKernel(s, 1.5, opt=o), "matern52": lambda s: MaternKernel(s, 2.5, opt=o)}[args.kernel]
+
     make_kernel, kernel_name = {"gaussian": (lambda s: GaussianKernel(s, opt=kopt), "gaussian"),
                                 "laplacian": (lambda s: LaplacianKernel(s, opt=kopt), "laplacian"),
                                 "matern32": (lambda s: MaternKernel(s, 1.5, opt=kopt), "1.5-matern"),
@@ -347,6 +351,24 @@ def main():
         res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch,
                                               MEASURED_TRAFFIC_BYTES_BF16X3.get(args.workload)),
                                launches_per_step=launches.value / args.steps)
+    if not split and args.dtype == "f32" and args.kernel == "gaussian":
+        # not the headline: the same step with the opt-in bf16x3 cross term (fp32 data and results, the cross term
+        # on the bf16 matrix cores from an exact three-way split), timed after the run above, and how far its
+        # result is from the fp32 kernels' result
+        ref_out = out.clone()
+        kernel = make_kernel_with(FalkonOptions(bf16x3_cross_term=True))(sigma)
+        for _ in range(max(args.warmup, 1)):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        el = time.perf_counter() - t0
+        diff = float(((out.double() - ref_out.double()).norm(dim=0) / ref_out.double().norm(dim=0)).max())
+        res["opt_in_bf16x3_cross_term"] = {"value": N * M * T / (el / args.steps), "ms_per_step": el / args.steps * 1e3,
+                                           "rel_diff_from_fp32_kernels": diff}
+        kernel = make_kernel(sigma)
     if not args.no_cpu_baseline and args.op == "dmmv":
         rows = args.cpu_rows or {"C2": N, "C3": 400_000, "C4": 100_000}[args.workload]
 

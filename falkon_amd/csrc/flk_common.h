@@ -152,6 +152,9 @@ template <typename T> int mmv_large_max_cols();
     int launch_mmv_small_f32_wide_kf##KF(const PackedView &A, const PackedView &B, const float *vecp,             \
                                          int64_t vec_ld, int tcols, int64_t a_chunk_blocks, int splits,           \
                                          float *partial, hipStream_t st);                                         \
+    int launch_mmv_small_f64_wide_kf##KF(const PackedView &A, const PackedView &B, const double *vecp,            \
+                                         int64_t vec_ld, int tcols, int64_t a_chunk_blocks, int splits,           \
+                                         double *partial, hipStream_t st);                                        \
     template <typename T>                                                                                         \
     int launch_mmv_large_kf##KF(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld,          \
                                 int tcols, int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st);    \

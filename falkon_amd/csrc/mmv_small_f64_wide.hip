@@ -1,0 +1,178 @@
+// Register-resident fp64 product kernel for many right-hand sides (up to 16 per pass), gfx950.
+// Compiled once per kernel function (-DFLK_KF=0..4).
+//
+// Same walk as mmv_small_f64_kernel (a wave keeps FR blocks of 16 output rows in registers and streams blocks of 16
+// reduction rows; K is never stored), but the contraction against vec runs on the matrix cores as well.  The fp64
+// kernel value costs about a hundred cycles per lane (software exponential), so recomputing K for every four
+// columns, as the FMA kernel does, is what many right-hand sides pay for; here 16 columns share one evaluation.
+// Once the kernel values have replaced the exponents, accumulator register r of lane l (B position j = l % 16, A row
+// 4 q + r, q = l / 16) is exactly the A operand of a 16x16x4 MFMA step whose B operand is vec[4 q + r][t = l % 16]:
+//   out2[position 4 r2 + q][t] += sum_i K[i][j] vec[i][t],
+// four more MFMAs per 16 x 16 tile whatever the number of columns, and register r2 of a lane ends up holding output
+// row 4 q + r2 of column t (positions map to rows as in the packed block), so there is no cross-lane step.
+#include "flk_common.h"
+#include "kernel_fn.h"
+
+#ifndef FLK_KF
+#define FLK_KF FLK_GAUSSIAN
+#endif
+
+namespace flk {
+
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWide64Waves = 4;
+constexpr int kWide64Cols = 16;
+constexpr int kWide64Stride = 17;                           // row stride of the staged vec values
+constexpr int kWide64Stage = 16 + 16 * kWide64Stride;       // hn(16) | vec[16 rows][17]
+constexpr int kWide64Fetch = 1 + kWide64Cols / 4;           // doubles a lane fetches per A block
+
+struct Wide64RowVals { double x[kWide64Fetch]; };
+
+template <int DP>
+__device__ __forceinline__ void wide64_load_a(double (&a)[DP], const double *__restrict__ P, int64_t blk, int j, int q) {
+    const double *p = P + (blk * (4 * DP) + (int64_t)q * DP) * 16 + j;
+#pragma unroll
+    for (int s = 0; s < DP; s++) a[s] = p[s * 16];
+}
+
+// lane l fetches hA[row l % 16] and vec[row l % 16][4c + l / 16], c = 0..3: 128-byte runs of the planes
+__device__ __forceinline__ void wide64_fetch(Wide64RowVals &rv, const double *__restrict__ hA,
+                                             const double *__restrict__ vecp, int64_t vec_ld, int64_t ab, int lane) {
+    const int r = lane & 15, hh = lane >> 4;
+    rv.x[0] = hA[ab * 16 + r];
+#pragma unroll
+    for (int c = 0; c < kWide64Cols / 4; c++) rv.x[1 + c] = vecp[(int64_t)(4 * c + hh) * vec_ld + ab * 16 + r];
+}
+__device__ __forceinline__ void wide64_stage(const Wide64RowVals &rv, double *lds, int lane) {
+    const int r = lane & 15, hh = lane >> 4;
+    if (hh == 0) lds[r] = rv.x[0];
+#pragma unroll
+    for (int c = 0; c < kWide64Cols / 4; c++) lds[16 + r * kWide64Stride + 4 * c + hh] = rv.x[1 + c];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+template <int DP, int FR, int KF>
+__device__ __forceinline__ void wide64_tile_step(const double (&a)[DP], const double *lds, int j, int q,
+                                                 const double (&breg)[FR][DP], const double (&hb)[FR],
+                                                 doublex4 (&out2)[FR]) {
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const doublex4 hn = *(const doublex4 *)(lds + 4 * q);          // rows 4q .. 4q + 3 of the A block
+    doublex4 acc[FR];
+#pragma unroll
+    for (int c = 0; c < FR; c++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[c][r] = hn[r] + hb[c];
+#pragma unroll
+    for (int s = 0; s < DP; s++)
+#pragma unroll
+        for (int c = 0; c < FR; c++) acc[c] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[s], breg[c][s], acc[c], 0, 0, 0);
+#pragma unroll
+    for (int c = 0; c < FR; c++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[c][r] = kernel_value<KF>(acc[c][r]);
+    const double *vb = lds + 16 + (4 * q) * kWide64Stride + j;     // vec[4q + r][t = j]
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const double bval = vb[r * kWide64Stride];
+#pragma unroll
+        for (int c = 0; c < FR; c++) out2[c] = __builtin_amdgcn_mfma_f64_16x16x4f64(acc[c][r], bval, out2[c], 0, 0, 0);
+    }
+}
+
+// KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
+template <int DP, int FR, int KF>
+__global__ void __launch_bounds__(256, 2)
+    mmv_small_f64_wide_kernel(const double *__restrict__ PA, const double *__restrict__ hA,
+                              const double *__restrict__ vecp, int64_t vec_ld, const double *__restrict__ PB,
+                              const double *__restrict__ hB, int64_t na_blocks, int64_t nb_blocks,
+                              int64_t a_chunk_blocks, double *__restrict__ partial, int64_t nb_pad, int tcols,
+                              bool y_fastest) {
+    // vecp must hold 16 planes (zeros beyond the caller's columns); the first tcols columns are stored
+    __shared__ __attribute__((aligned(32))) double stage[kWide64Waves][2][kWide64Stage];
+    unsigned bx, by;
+    xcd_remap(bx, by, y_fastest);
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int j = lane & 15, q = lane >> 4;
+    const int jrow = 4 * (j & 3) + (j >> 2);  // matrix row (within its block) held at position j
+    const int64_t bb0 = ((int64_t)bx * kWide64Waves + wave) * FR;
+    if (bb0 >= nb_blocks) return;             // whole wave idle; no workgroup barriers in this kernel
+    const int64_t a0 = (int64_t)by * a_chunk_blocks;
+    int64_t a1 = a0 + a_chunk_blocks;
+    if (a1 > na_blocks) a1 = na_blocks;
+
+    double breg[FR][DP];
+    double hb[FR];
+#pragma unroll
+    for (int c = 0; c < FR; c++) {
+        const int64_t bb = bb0 + c < nb_blocks ? bb0 + c : nb_blocks - 1;
+        wide64_load_a<DP>(breg[c], PB, bb, j, q);
+        hb[c] = hB[bb * 16 + jrow];
+    }
+    doublex4 out2[FR];
+#pragma unroll
+    for (int c = 0; c < FR; c++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) out2[c][r] = 0.0;
+
+    double fa0[DP], fa1[DP];
+    Wide64RowVals rv;
+    double *lds0 = stage[wave][0], *lds1 = stage[wave][1];
+    if (a0 < a1) {
+        wide64_load_a<DP>(fa0, PA, a0, j, q);
+        wide64_fetch(rv, hA, vecp, vec_ld, a0, lane);
+        wide64_stage(rv, lds0, lane);
+    }
+    for (int64_t ab = a0; ab < a1; ab += 2) {
+        const bool has1 = ab + 1 < a1;
+        if (has1) { wide64_load_a<DP>(fa1, PA, ab + 1, j, q); wide64_fetch(rv, hA, vecp, vec_ld, ab + 1, lane); }
+        wide64_tile_step<DP, FR, KF>(fa0, lds0, j, q, breg, hb, out2);
+        if (has1) {
+            wide64_stage(rv, lds1, lane);
+            const bool has2 = ab + 2 < a1;
+            if (has2) { wide64_load_a<DP>(fa0, PA, ab + 2, j, q); wide64_fetch(rv, hA, vecp, vec_ld, ab + 2, lane); }
+            wide64_tile_step<DP, FR, KF>(fa1, lds1, j, q, breg, hb, out2);
+            if (has2) wide64_stage(rv, lds0, lane);
+        }
+    }
+    // lane = column t = j, registers = output rows 4q .. 4q + 3 of each block
+    if (j < tcols) {
+#pragma unroll
+        for (int c = 0; c < FR; c++)
+            if (bb0 + c < nb_blocks)
+                *(doublex4 *)(&partial[((int64_t)by * tcols + j) * nb_pad + (bb0 + c) * 16 + 4 * q]) = out2[c];
+    }
+}
+
+template <int DP, int FR>
+static int launch_wide64_one(const PackedView &A, const PackedView &B, const double *vecp, int64_t vec_ld, int tcols,
+                             int64_t a_chunk_blocks, int splits, double *partial, hipStream_t st) {
+    const int64_t per_wg = kWide64Waves * FR;
+    dim3 grid((unsigned)((B.nblk + per_wg - 1) / per_wg), (unsigned)splits);
+    hipLaunchKernelGGL((mmv_small_f64_wide_kernel<DP, FR, FLK_KF>), grid, dim3(256), 0, st, (const double *)A.data,
+                       (const double *)A.hnorm, vecp, vec_ld, (const double *)B.data, (const double *)B.hnorm, A.nblk,
+                       B.nblk, a_chunk_blocks, partial, B.npad, tcols, B.n > A.n);
+    FLK_LAUNCH_CHECK("mmv_small_f64_wide_kernel");
+    return FLK_OK;
+}
+
+int FLK_CAT(launch_mmv_small_f64_wide_kf, FLK_KF)(const PackedView &A, const PackedView &B, const double *vecp,
+                                                  int64_t vec_ld, int tcols, int64_t a_chunk_blocks, int splits,
+                                                  double *partial, hipStream_t st) {
+    if (tcols < 1 || tcols > kWide64Cols) return fail(FLK_EINVAL, "mmv_small wide: column chunk %d not in 1..16", tcols);
+    if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_small: operands packed with different feature counts");
+    const int dp = (int)(A.dpad / 4);
+#define FLK_WIDE64(DPV, FRV) \
+    case DPV: return launch_wide64_one<DPV, FRV>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+    switch (dp) {
+        FLK_WIDE64(1, 4) FLK_WIDE64(2, 4) FLK_WIDE64(3, 4) FLK_WIDE64(4, 4) FLK_WIDE64(5, 4) FLK_WIDE64(6, 4)
+        FLK_WIDE64(7, 4) FLK_WIDE64(8, 4) FLK_WIDE64(9, 2) FLK_WIDE64(10, 2) FLK_WIDE64(11, 2) FLK_WIDE64(12, 2)
+        FLK_WIDE64(13, 2) FLK_WIDE64(14, 2) FLK_WIDE64(15, 2) FLK_WIDE64(16, 2)
+    }
+#undef FLK_WIDE64
+    return fail(FLK_EUNSUPPORTED, "mmv_small wide<f64>: padded feature count %lld not in 4..64", (long long)A.dpad);
+}
+
+}  // namespace flk

@@ -434,3 +434,27 @@ def test_non_finite_rows_give_nan(dev, mode, d, t):
     if mode != "bf16x3" and t == 1:
         ref = mmv_ref.fmmv_ref(Xb, C, v, float(d) ** 0.5)
         assert torch.isnan(ref[3]).all() and not torch.isnan(ref[~bad]).any()
+
+
+@pytest.mark.parametrize("d,t", [(1, 5), (3, 16), (9, 7), (12, 40), (28, 29), (32, 9), (33, 17), (50, 6), (64, 16), (61, 4),
+                                 (64, 20)])
+def test_many_right_hand_sides_small_d_fp64(dev, d, t):
+    """More than four right-hand sides at d <= 64 in fp64: the 16-column kernel whose contraction runs on the matrix
+    cores (one evaluation of K for 16 columns), including more columns than one pass holds and a last pass that is
+    narrow enough for the FMA kernel; 1e-11 against the CPU path, and the same numbers as column-by-column calls."""
+    n, m = 900, 333
+    X, C, v, w = _rand(n, d, m, t, torch.float64, seed=100 * d + t, scale=0.8)
+    k = GaussianKernel(0.9 * np.sqrt(d) + 0.5)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    got_mmv = k.mmv(Xg, Cg, vg)
+    got = k.dmmv(Xg, Cg, vg, wg)
+    assert rel_err(got_mmv, mmv_ref.fmmv_ref(X, C, v, k.sigma)) < 1e-11
+    assert rel_err(got, mmv_ref.fdmmv_ref(X, C, v, w, k.sigma)) < 1e-11
+    assert rel_err(got_mmv, brute.mmv_brute(X, C, k.sigma, v)) < 5e-11
+    assert torch.equal(got, k.dmmv(Xg, Cg, vg, wg))
+    cols = torch.cat([k.dmmv(Xg, Cg, vg[:, i:i + 1].contiguous(), wg[:, i:i + 1].contiguous()) for i in (0, t - 1)], 1)
+    assert rel_err(got[:, [0, t - 1]], cols) < 1e-12
+    # F-ordered right-hand sides and output
+    vf, of = vg.T.contiguous().T, torch.empty(t, n, dtype=torch.float64, device=dev).T
+    assert k.mmv(Xg, Cg, vf, out=of).data_ptr() == of.data_ptr()
+    assert torch.equal(of, got_mmv)
