@@ -69,9 +69,22 @@ MEASURED_TRAFFIC_BYTES_BF16X3 = {
 }
 
 
-def make_inputs(name):
-    """Synthetic inputs of the named configuration (draw order X, idx, sigma, v, w)."""
+def product_kernel_name(d, T, dtype):
+    """The kernel the library picks for d features and T right-hand sides (csrc/mmv_small_f32.hip, mmv_small_f64.hip)."""
+    if d > 64:
+        return "mmv_large_kernel"
+    if dtype == "f32":
+        steps = (d + 1) // 2
+        fma_cols = 16 if steps <= 7 else 12 if steps <= 12 else 8 if steps <= 16 else 4
+        return "mmv_small_f32_wide_kernel" if T > fma_cols else "mmv_small_f32_kernel"
+    return "mmv_small_f64_wide_kernel" if T > (3 if d > 56 else 4) else "mmv_small_f64_kernel"
+
+
+def make_inputs(name, rhs=0):
+    """Synthetic inputs of the named configuration (draw order X, idx, sigma, v, w); rhs > 0 replaces the
+    configuration's number of right-hand sides."""
     seed, N, d, M, T, has_w = WORKLOADS[name]
+    T = rhs or T
     rng = np.random.default_rng(seed)
     if name == "C2":
         X = rng.standard_normal((N, d), dtype=np.float32)
@@ -233,7 +246,10 @@ def main():
                     help="f32 (the headline): fp32 MFMA.  bf16x3: the opt-in mode that forms x.c on the bf16 matrix cores "
                          "from an exact three-way bfloat16 split of the fp32 rows (fp32 accuracy; fp32 data); "
                          "its roofline is priced against the bf16 MFMA peak on the flops it executes")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--rhs", type=int, default=0, metavar="T",
+                    help="right-hand sides instead of the configuration's own number (not a headline workload)")
+    ap.add_argument("--no-cpu-baseline", action="store_true",
+                    help="only the timed steps: neither the CPU baseline nor the bf16x3 side measurement (profiling runs)")
     ap.add_argument("--cpu-rows", type=int, default=0)
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run a plain device copy of BYTES bytes five times (reference point for the "
@@ -273,11 +289,12 @@ def main():
         return
     dev = torch.device("cuda:0")
     seed, N, d, M, T, has_w = WORKLOADS[args.workload]
+    T = args.rhs or T
     split = args.cross_term == "bf16x3"
     if split and args.dtype != "f32":
         print("bench.py: --cross-term bf16x3 applies to fp32 data", file=sys.stderr)
         sys.exit(2)
-    X, C, sigma, v, w = make_inputs(args.workload)
+    X, C, sigma, v, w = make_inputs(args.workload, args.rhs)
     tdt = torch.float32 if args.dtype == "f32" else torch.float64
     X, C, v = X.to(tdt), C.to(tdt), v.to(tdt)
     w = w.to(tdt) if w is not None else None
@@ -334,8 +351,8 @@ def main():
                                f"inputs resident in HBM, packing included in every step"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.dtype == "f32" else None,
-                     "kernel": ("mmv_large_kernel" if d > 64 else "mmv_small_%s_kernel" % args.dtype),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.dtype == "f32" and not args.rhs else None,
+                     "kernel": product_kernel_name(d, T, args.dtype),
                      "launches_per_step": launches.value / args.steps,
                      "avg_launch_ms": kern_ms, "flop_per_launch": flop_per_launch},
         "whole_step_flop_frac": (N * M * ((2 if args.op == "dmmv" else 1) * (2 * d + 4 + 2 * T)))
@@ -351,7 +368,7 @@ def main():
         res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch,
                                               MEASURED_TRAFFIC_BYTES_BF16X3.get(args.workload)),
                                launches_per_step=launches.value / args.steps)
-    if not split and args.dtype == "f32" and args.kernel == "gaussian":
+    if not split and args.dtype == "f32" and args.kernel == "gaussian" and not args.no_cpu_baseline:
         # not the headline: the same step with the opt-in bf16x3 cross term (fp32 data and results, the cross term
         # on the bf16 matrix cores from an exact three-way split), timed after the run above, and how far its
         # result is from the fp32 kernels' result
