@@ -458,3 +458,24 @@ def test_many_right_hand_sides_small_d_fp64(dev, d, t):
     vf, of = vg.T.contiguous().T, torch.empty(t, n, dtype=torch.float64, device=dev).T
     assert k.mmv(Xg, Cg, vf, out=of).data_ptr() == of.data_ptr()
     assert torch.equal(of, got_mmv)
+
+
+def test_torch_ops_entry_points(dev):
+    """``torch.ops.falkon.kernel_fmmv / kernel_fdmmv`` give what the kernel objects give, bit for bit, in every
+    arithmetic mode, and write ``out`` in place."""
+    import falkon_amd.torch_ops  # noqa: F401
+    from falkon_amd import LaplacianKernel
+    for dtype, bf16x3 in ((torch.float32, False), (torch.float32, True), (torch.float64, False)):
+        X, C, v, w = (a.to(dev) for a in _rand(500, 12, 130, 3, dtype, seed=5))
+        sigma = torch.tensor([1.7], dtype=dtype, device=dev)
+        opt = FalkonOptions(bf16x3_cross_term=bf16x3)
+        out = torch.empty(500, 3, dtype=dtype, device=dev)
+        assert torch.ops.falkon.kernel_fmmv(X, C, sigma, v, out, 0, bf16x3) is None
+        assert torch.equal(out, GaussianKernel(1.7, opt=opt).mmv(X, C, v))
+        out2 = torch.empty(130, 3, dtype=dtype, device=dev)
+        torch.ops.falkon.kernel_fdmmv(X, C, sigma, v, w, out2, 1, bf16x3)
+        assert torch.equal(out2, LaplacianKernel(1.7, opt=opt).dmmv(X, C, v, w))
+        torch.ops.falkon.kernel_fdmmv(X, C, sigma, v, None, out2, 0, bf16x3)
+        assert torch.equal(out2, GaussianKernel(1.7, opt=opt).dmmv(X, C, v, None))
+    with pytest.raises(TypeError):
+        torch.ops.falkon.kernel_fmmv(X, C.float(), sigma, v, out)

@@ -264,3 +264,17 @@ def test_three_way_bfloat16_split_is_exact():
             + xh.astype(f) * yh)
     exact = x.astype(f) * y.astype(f)
     assert float(np.max(np.abs(kept - exact) / np.abs(exact))) < 2.0 ** -22
+
+
+def test_torch_ops_are_registered_and_refuse_host_tensors():
+    """``torch.ops.falkon.kernel_fmmv / kernel_fdmmv`` exist once falkon_amd.torch_ops is imported (the reference
+    reaches its native code the same way, falkon/c_ext/__init__.py:13-21); there is no CPU implementation."""
+    import falkon_amd.torch_ops  # noqa: F401
+    schema = str(torch.ops.falkon.kernel_fmmv.default._schema)
+    assert "Tensor(a4!) out" in schema and "kernel_fn=0" in schema and "bf16x3=False" in schema
+    assert "Tensor? w" in str(torch.ops.falkon.kernel_fdmmv.default._schema)
+    X = torch.randn(4, 3)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        torch.ops.falkon.kernel_fmmv(X, X, torch.ones(1), torch.randn(4, 1), torch.empty(4, 1))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        torch.ops.falkon.kernel_fdmmv(X, X, torch.ones(1), torch.randn(4, 1), None, torch.empty(4, 1))
