@@ -120,4 +120,19 @@ class Falkon(_Base):
 
 
 class InCoreFalkon(Falkon):
-    """Alias: every fit is in-core on the GPU in this build (falkon/models/incore_falkon.py:178-257)."""
+    """``Falkon`` for data that already lives on the GPU (falkon/models/incore_falkon.py:21-257).  Every fit of this
+    build is in-core on the GPU, so the class adds only the reference's input checks: the tensors given to ``fit``
+    must be GPU tensors on one device, and ``predict`` wants X on the device of the fitted coefficients
+    (incore_falkon.py:139-147)."""
+
+    def fit(self, X: torch.Tensor, Y: torch.Tensor, Xts: Optional[torch.Tensor] = None,
+            Yts: Optional[torch.Tensor] = None, warm_start: Optional[torch.Tensor] = None):
+        given = [t for t in (X, Y, Xts, Yts) if t is not None]
+        if not X.is_cuda or any(t.device != X.device for t in given):
+            raise ValueError("All tensors for fitting InCoreFalkon must be CUDA tensors, located on the same GPU.")
+        return super().fit(X, Y, Xts, Yts, warm_start)
+
+    def predict(self, X: torch.Tensor) -> torch.Tensor:
+        if self.alpha_ is not None and X.device != self.alpha_.device:
+            raise ValueError(f"X must be on device {self.alpha_.device}")
+        return super().predict(X)

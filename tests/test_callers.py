@@ -247,3 +247,93 @@ def test_config5_reduced_end_to_end(dev, monkeypatch):
     model3.fit(X.to(dev), Y.to(dev), warm_start=model2.beta_.clone())
     mse3 = float(((model3.predict(Xts.to(dev)).cpu() - Yts) ** 2).mean())
     assert abs(mse3 - mse_gpu) / mse_gpu < 5e-3
+
+
+# --------------------------------------------------------------------------------------------------
+# The reference's estimator tests (tests/test_falkon.py:20-123,126-149,271-304): same sklearn data sets
+# (random_state=11), same kernels, penalties, M, seeds and accuracy thresholds, fitted through the HIP products.
+# --------------------------------------------------------------------------------------------------
+def _cls_data():
+    from sklearn import datasets
+    X, Y = datasets.make_classification(1000, 10, n_classes=2, random_state=11)
+    Y = Y.astype(np.float64).reshape(-1, 1)
+    Y[Y == 0] = -1
+    return torch.from_numpy(X.astype(np.float64)), torch.from_numpy(Y)
+
+
+def _multicls_data():
+    from sklearn import datasets
+    X, Y = datasets.make_classification(2000, 30, n_classes=20, n_informative=6, random_state=11)
+    return torch.from_numpy(X.astype(np.float64)), torch.from_numpy(np.eye(20, dtype=np.float64)[Y.astype(np.int32), :])
+
+
+def _reg_data():
+    from sklearn import datasets
+    X, Y = datasets.make_regression(1000, 30, random_state=11)
+    X, Y = X.astype(np.float64), Y.astype(np.float64).reshape(-1, 1)
+    return tuple(torch.from_numpy(a) for a in (X[:800], Y[:800], X[800:], Y[800:]))
+
+
+def _c_err(t, p):
+    return 100 * torch.sum(t * p <= 0).to(torch.float32) / t.shape[0], "c-err"
+
+
+def _rmse(t, p):
+    return torch.sqrt(torch.mean((t - p) ** 2)).item(), "RMSE"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_reference_accuracy_thresholds(dev, dtype):
+    """Binary classification error below 5 %, 20-class error below 0.23, regression test RMSE below 2.5 and above
+    the training RMSE (tests/test_falkon.py:62-123), with host tensors as there (the fit moves them to the GPU)."""
+    X, Y = (a.to(dtype) for a in _cls_data())
+    flk = Falkon(kernel=GaussianKernel(2.0), penalty=1e-6, M=500, seed=10, maxiter=10).fit(X, Y)
+    assert float(_c_err(flk.predict(X), Y)[0]) < 5
+
+    X, Y = (a.to(dtype) for a in _multicls_data())
+    flk = Falkon(kernel=GaussianKernel(10.0), penalty=1e-6, M=500, seed=10, maxiter=10).fit(X, Y)
+    preds = flk.predict(X)
+    assert preds.shape == Y.shape and preds.device == X.device
+    assert float((preds.argmax(1) != Y.argmax(1)).double().mean()) < 0.23
+
+    Xtr, Ytr, Xts, Yts = (a.to(dtype) for a in _reg_data())
+    flk = Falkon(kernel=GaussianKernel(20.0), penalty=1e-6, M=Xtr.shape[0] // 2, seed=10, maxiter=10)
+    flk.fit(Xtr, Ytr, Xts=Xts, Yts=Yts)
+    assert flk.predict(Xts).shape == (Yts.shape[0], 1)
+    ts_err, tr_err = _rmse(flk.predict(Xts), Yts)[0], _rmse(flk.predict(Xtr), Ytr)[0]
+    assert tr_err < ts_err < 2.5
+
+
+@pytest.mark.gpu
+def test_reference_gpu_predict_and_validation_callback(dev, capsys):
+    """tests/test_falkon.py:126-149: fit on host data with a validation set and an error function, move the model to
+    the GPU, predict there."""
+    Xtr, Ytr, Xts, Yts = _reg_data()
+    flk = Falkon(kernel=GaussianKernel(20.0), penalty=1e-6, M=500, seed=10, error_fn=_rmse)
+    flk.fit(Xtr, Ytr, Xts=Xts, Yts=Yts)
+    assert "validation RMSE" in capsys.readouterr().out and len(flk.val_errors_) > 0
+    flk.to("cuda:0")
+    ts_preds, tr_preds = flk.predict(Xts.to(dev)), flk.predict(Xtr.to(dev))
+    assert ts_preds.device.type == "cuda" and ts_preds.shape == (Yts.shape[0], 1)
+    ts_err, tr_err = _rmse(ts_preds.cpu(), Yts)[0], _rmse(tr_preds.cpu(), Ytr)[0]
+    assert tr_err < ts_err < 2.5
+
+
+@pytest.mark.gpu
+def test_reference_incore_falkon(dev):
+    """tests/test_falkon.py:271-304: InCoreFalkon refuses host tensors in fit and predict, and classifies the GPU
+    copy of the data with less than 5 % error."""
+    from falkon_amd import InCoreFalkon
+    X, Y = _cls_data()
+    flk = InCoreFalkon(kernel=GaussianKernel(2.0), penalty=1e-6, M=500, seed=10)
+    with pytest.raises(ValueError):
+        flk.fit(X, Y)
+    flk.fit(X.to(dev), Y.to(dev))
+    with pytest.raises(ValueError):
+        flk.predict(X)
+    flkc = InCoreFalkon(kernel=GaussianKernel(2.0), penalty=1e-6, M=500, seed=10, maxiter=20, error_fn=_c_err)
+    flkc.fit(X.to(dev), Y.to(dev))
+    preds = flkc.predict(X.to(dev))
+    assert preds.device == X.to(dev).device
+    assert float(_c_err(preds, Y.to(dev))[0]) < 5
