@@ -90,7 +90,10 @@ class FalkonConjugateGradient:
 
     def solve(self, X, M, Y, _lambda, initial_solution, max_iter, callback=None):
         if not torch.is_inference_mode_enabled():
-            raise RuntimeError("FalkonConjugateGradient.solve must run under torch.inference_mode()")
+            # the reference fails here too, with torch's own message about inference tensors (the products run under
+            # inference mode and the solver updates their results in place; falkon/tests/test_conjgrad.py:133-143)
+            raise RuntimeError("FalkonConjugateGradient.solve was called outside InferenceMode: "
+                               "wrap the call in `with torch.inference_mode():`")
         n = Y.shape[0]
         rhs = self.preconditioner.apply_t(self.kernel.mmv(M, X, Y / n, opt=self.params))   # B^T K_nm^T y / n
         operator = functools.partial(self.falkon_mmv, penalty=_lambda, X=X, M=M, n=n)

@@ -337,3 +337,33 @@ def test_reference_incore_falkon(dev):
     preds = flkc.predict(X.to(dev))
     assert preds.device == X.to(dev).device
     assert float(_c_err(preds, Y.to(dev))[0]) < 5
+
+
+def test_falkon_cg_refuses_to_run_outside_inference_mode():
+    """tests/test_conjgrad.py:133-143: RuntimeError naming InferenceMode (checked before anything touches the GPU)."""
+    from falkon_amd.optim import FalkonConjugateGradient
+    X, Y, C, sigma, lam = _conjgrad_problem()
+    solver = FalkonConjugateGradient(GaussianKernel(sigma), FalkonPreconditioner(lam, GaussianKernel(sigma), FalkonOptions()),
+                                     FalkonOptions())
+    with pytest.raises(RuntimeError, match="InferenceMode"):
+        solver.solve(X=X, M=C, Y=Y, _lambda=lam, initial_solution=None, max_iter=100)
+
+
+@pytest.mark.gpu
+def test_falkon_cg_restarts(dev):
+    """tests/test_conjgrad.py:145-166: thirty solves of six iterations each, every one started from the last
+    solution, reach the direct solution of the normal equations."""
+    from falkon_amd.optim import FalkonConjugateGradient
+    X, Y, C, sigma, lam = _conjgrad_problem()
+    kernel = GaussianKernel(sigma)
+    opt = FalkonOptions(cg_tolerance=1e-10)
+    Xd, Yd, Cd = X.to(dev), Y.to(dev), C.to(dev)
+    with torch.inference_mode():
+        prec = FalkonPreconditioner(lam, kernel, opt)
+        prec.init(Cd)
+        solver = FalkonConjugateGradient(kernel, prec, opt)
+        sol = None
+        for _ in range(30):
+            sol = solver.solve(X=Xd, M=Cd, Y=Yd, _lambda=lam, initial_solution=sol, max_iter=6)
+        alpha = prec.apply(sol)
+    np.testing.assert_allclose(alpha.cpu().numpy(), falkon_ref.nystrom_krr_direct(X, Y, C, sigma, lam), rtol=1e-5)
