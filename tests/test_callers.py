@@ -367,3 +367,35 @@ def test_falkon_cg_restarts(dev):
             sol = solver.solve(X=Xd, M=Cd, Y=Yd, _lambda=lam, initial_solution=sol, max_iter=6)
         alpha = prec.apply(sol)
     np.testing.assert_allclose(alpha.cpu().numpy(), falkon_ref.nystrom_krr_direct(X, Y, C, sigma, lam), rtol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("order", ["C", "F"])
+@pytest.mark.parametrize("dtype,la,tol", [(torch.float32, 100.0, 1e-2), (torch.float64, 100.0, 1e-10),
+                                          (torch.float64, 0.0, 1e-10)])
+def test_reference_preconditioner_invariants_on_gpu(dev, order, dtype, la, tol):
+    """The reference's preconditioner test on the GPU (tests/test_chol_prec.py:17-67,99-163): 100 uniform points,
+    GaussianKernel(10), penalty 100 and 0; with T = chol(K_MM) and A = chol(T T^T / M + la I), solving T^T x = K_MM
+    gives T, solving A^T x = A^T A gives A, invT(invTt(K_MM)) = I, and the preconditioner inverts
+    n/M K_MM^T K_MM + la n K_MM (tolerances as there).  The Gram matrix comes from the HIP kernel-matrix path."""
+    M, N = 100, 50_000
+    mat = torch.from_numpy(inputs.gen_random(M, M, "float64", F=True, seed=10)).to(dtype)
+    mat = (mat.T.contiguous().T if order == "F" else mat.contiguous()).to(dev)
+    kernel = GaussianKernel(10.0)
+    opt = FalkonOptions(no_single_kernel=True)
+    with torch.inference_mode():
+        gram = kernel(mat, mat, opt=opt)
+        prec = FalkonPreconditioner(la, kernel, opt)
+        prec.init(mat)
+        eye = torch.eye(M, dtype=dtype, device=dev)
+        T = prec.invTt(gram)
+        assert T.dtype == dtype
+        np.testing.assert_allclose((T.T @ T).cpu().numpy(), gram.cpu().numpy(), rtol=tol, atol=tol)
+        ATA = (1.0 / M) * T @ T.T + la * eye
+        A = prec.invAt(ATA)
+        np.testing.assert_allclose((A.T @ A).cpu().numpy(), ATA.cpu().numpy(), rtol=tol, atol=tol)
+        np.testing.assert_allclose(prec.invT(prec.invTt(gram)).cpu().numpy(), eye.cpu().numpy(), rtol=10 * tol, atol=10 * tol)
+        desired = (N / M) * gram.T @ gram + la * N * gram
+        out = (1 / N) * prec.invT(prec.invA(prec.invAt(prec.invTt(desired))))
+        prec_tol = 10 * tol if la else 100 * tol            # test_chol_prec.py:117,133
+        np.testing.assert_allclose(out.cpu().numpy(), eye.cpu().numpy(), rtol=prec_tol, atol=prec_tol)
