@@ -399,3 +399,30 @@ def test_reference_preconditioner_invariants_on_gpu(dev, order, dtype, la, tol):
         out = (1 / N) * prec.invT(prec.invA(prec.invAt(prec.invTt(desired))))
         prec_tol = 10 * tol if la else 100 * tol            # test_chol_prec.py:117,133
         np.testing.assert_allclose(out.cpu().numpy(), eye.cpu().numpy(), rtol=prec_tol, atol=prec_tol)
+
+
+def test_center_selection_with_targets():
+    """tests/test_nysel.py:109-125: centres and their targets come back together, orders, dtypes and devices kept."""
+    M, D, num = 10_000, 20, 100
+    X = torch.from_numpy(inputs.gen_random(M, D, "float64", F=True, seed=0))
+    Y = torch.empty(M, 1, dtype=X.dtype)
+    sel = UniformSelector(np.random.default_rng(0), num_centers=num)
+    centers, cY = sel.select(X, Y)
+    assert centers.stride() == (1, num) and centers.size() == (num, D) and cY.size() == (num, 1)
+    assert centers.dtype == X.dtype and cY.dtype == Y.dtype and centers.device == X.device
+    centers, cY, idx = sel.select_indices(X, Y)
+    assert idx.dtype == torch.long and len(idx) == centers.shape[0] == cY.shape[0]
+    assert torch.equal(centers, X[idx])
+
+
+@pytest.mark.gpu
+def test_center_selection_on_gpu_tensors(dev):
+    """tests/test_nysel.py:37-55: GPU data gives GPU centres (and indices) with the input's strides."""
+    M, D, num = 10_000, 20, 100
+    X = torch.from_numpy(inputs.gen_random(M, D, "float64", F=False, seed=0)).to(dev)
+    sel = UniformSelector(np.random.default_rng(0), num_centers=num)
+    centers = sel.select(X, None)
+    assert centers.stride() == (D, 1) and centers.size() == (num, D)
+    assert centers.dtype == X.dtype and centers.device == X.device
+    centers, idx = sel.select_indices(X, None)
+    assert centers.device == idx.device and idx.dtype == torch.long and len(idx) == num
