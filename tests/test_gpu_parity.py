@@ -479,3 +479,59 @@ def test_torch_ops_entry_points(dev):
         assert torch.equal(out2, GaussianKernel(1.7, opt=opt).dmmv(X, C, v, None))
     with pytest.raises(TypeError):
         torch.ops.falkon.kernel_fmmv(X, C.float(), sigma, v, out)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("n,m,d,t", [(1000, 300, 9, 1), (700, 130, 28, 3), (260, 200, 100, 2)])
+def test_packed_entry_points(dev, dtype, n, m, d, t):
+    """``flk_kernel_pack`` + ``flk_kernel_mmv_packed`` (pack X and C once, then K v + w and K^T u as two products on the
+    packed operands) give what ``dmmv`` gives, and the packed operand itself is the scaled data, block by block, with
+    the half squared norms behind it (the reference's ``square_norm``, falkon/c_ext/ops/cpu/cpu_square_norm.cpp:14-60,
+    pinned there against ``torch.norm``: falkon/tests/test_matrix_ops.py:72-108)."""
+    from falkon_amd import _backend
+    lib = _backend.load()
+    code = _backend.FLK_F32 if dtype == torch.float32 else _backend.FLK_F64
+    blk = 32 if dtype == torch.float32 else 16
+    X, C, v, w = (a.to(dev) for a in _rand(n, d, m, t, dtype, seed=n + d))
+    sigma = torch.linspace(1.5, 3.0, d, dtype=dtype, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    packed = {}
+    for name, A in (("X", X), ("C", C)):
+        nbytes = lib.flk_gauss_packed_bytes(A.shape[0], d, code)
+        buf = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        rc = lib.flk_gauss_pack(A.data_ptr(), A.shape[0], d, A.stride(0), A.stride(1), sigma.data_ptr(), d, code,
+                                buf.data_ptr(), nbytes, stream)
+        _backend.raise_for_status(rc, "flk_gauss_pack")
+        packed[name] = buf
+    # layout: [block][feature][row] (fp64 rows permuted inside a block), then -1/2 |x~|^2, x~ = sqrt(log2 e) x / sigma
+    if d <= 64:
+        dpad = (d + 1) // 2 * 2 if dtype == torch.float32 else (d + 3) // 4 * 4
+    else:
+        dpad = (d + 15) // 16 * 16 if dtype == torch.float32 else (d + 31) // 32 * 32
+    nblk = (n + blk - 1) // blk
+    flat = packed["X"].view(dtype)
+    data = flat[:nblk * dpad * blk].view(nblk, dpad, blk)
+    scaled = (X.double() * np.sqrt(np.log2(np.e)) / sigma.double())
+    pos = torch.arange(blk) if dtype == torch.float32 else torch.tensor([4 * (r % 4) + r // 4 for r in range(blk)])
+    rows = torch.arange(n)
+    got_rows = data[rows // blk, :d, pos[rows % blk]]
+    assert rel_err(got_rows, scaled.cpu()) < (1e-6 if dtype == torch.float32 else 1e-15)
+    off = (nblk * dpad * blk * flat.element_size() + 255) // 256 * 256 // flat.element_size()
+    half_norms = flat[off:off + n]
+    want = -0.5 * (scaled * scaled).sum(1)
+    assert rel_err(half_norms.reshape(-1, 1), want.reshape(-1, 1).cpu()) < (1e-6 if dtype == torch.float32 else 1e-15)
+    # two products on the packed operands
+    u = torch.empty(n, t, dtype=dtype, device=dev)
+    out = torch.empty(m, t, dtype=dtype, device=dev)
+    for (pa, na, pb, nb, vec, add, res) in ((packed["C"], m, packed["X"], n, v, w, u), (packed["X"], n, packed["C"], m, u, None, out)):
+        ws_bytes = lib.flk_gauss_mmv_packed_workspace_bytes(na, nb, d, t, code)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+        rc = lib.flk_gauss_mmv_packed(pa.data_ptr(), na, pb.data_ptr(), nb, d, vec.data_ptr(), vec.stride(0), vec.stride(1), t,
+                                      add.data_ptr() if add is not None else None,
+                                      add.stride(0) if add is not None else 0, add.stride(1) if add is not None else 0,
+                                      res.data_ptr(), res.stride(0), res.stride(1), code, ws.data_ptr(), ws_bytes, stream)
+        _backend.raise_for_status(rc, "flk_gauss_mmv_packed")
+    k = GaussianKernel(sigma)
+    assert torch.equal(u, k.mmv(X, C, v) + w) or rel_err(u, k.mmv(X, C, v) + w) < (1e-6 if dtype == torch.float32 else 1e-14)
+    assert torch.equal(out, k.dmmv(X, C, v, w))
+    assert rel_err(out, mmv_ref.fdmmv_ref(X.cpu(), C.cpu(), v.cpu(), w.cpu(), sigma.cpu())) < TOL[dtype]
