@@ -371,21 +371,27 @@ static int fmm_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1
 // ---------------------------------------------------------------------------
 constexpr int64_t kTargetWgsSplitLarge = 8192;  // one 512-thread workgroup per CU: 32 rounds
 
-// Where the bf16x3 kernels are the faster route to the same result.  Measured at d = 28, N = 1e6, M = 2e4, dfmmv,
-// against the fp32 MFMA kernels: 1 right-hand side 10.9 ms against 20.2, 2: 11.9 against 21.1 (register-resident
-// kernel, two columns per pass); 4: 24.3 against 22.7, 5: 34.9 against 24.5 (the fp32 kernels contract up to eight
-// columns per pass with per-lane FMAs at this size); 9: 34.8 against 41.9, 16: 35.0 against 42.2 (LDS-tiled kernel,
-// sixteen columns per pass on the matrix cores, against the fp32 kernel that contracts 32); 17: 50.0 against 42.2,
-// 32: 70.1 against 43.0.  So: every feature count beyond the register-resident kernels, and at small feature
-// counts 1, 2 or 9 to 16 right-hand sides; otherwise the fp32 MFMA kernels serve the mode.
-static bool split_applies(int64_t d, int64_t t) { return d > kSplitMaxD || t <= 2 || (t > 8 && t <= 16); }
+// Where the bf16x3 kernels are the faster route to the same result.  Measured at N = 1e6, M = 2e4, dfmmv, against the
+// fp32 MFMA kernels.  d = 28: 1 right-hand side 10.9 ms against 20.2, 2: 11.7 against 21.1, 3 or 4: 14.3 against
+// 22.4 / 22.7 (register-resident kernel, up to four columns per pass); 5: 2 x 14.3 against 24.4 (the fp32 kernels
+// contract up to eight columns per pass with per-lane FMAs up to 32 features); 9: 34.8 against 41.9, 16: 35.0 against
+// 42.2 (LDS-tiled kernel, sixteen columns per pass on the matrix cores, against the fp32 kernel that contracts 32);
+// 17: 50.0 against 42.2, 32: 70.1 against 43.0.  d = 40 / 60, where the fp32 FMA kernels take four columns per pass:
+// 4: 18.4 / 24.3 against 29.9 / 48.0, 5: 49.9 / 64.4 for the fp32 32-column kernel, i.e. two passes of the
+// register-resident bf16x3 kernel are the faster route for 5 to 8 columns.  So: every feature count beyond the
+// register-resident kernels; at small feature counts 1 to 4 and 9 to 16 right-hand sides, and 5 to 8 beyond 32
+// features; otherwise the fp32 MFMA kernels serve the mode.
+static bool split_applies(int64_t d, int64_t t) {
+    return d > kSplitMaxD || t <= kSplitMaxCols || (t <= 2 * kSplitMaxCols && d > 32) || (t > 8 && t <= 16);
+}
 
 static Plan make_plan_split(int64_t na_blocks, int64_t nb_blocks, int64_t ks, int64_t t) {
     Plan p;
-    // up to two right-hand sides the register-resident kernel; beyond that (see split_applies) the LDS-tiled kernel,
+    // up to four right-hand sides per pass the register-resident kernel (two passes for five to eight); beyond that
+    // (see split_applies) the LDS-tiled kernel,
     // whose epilogue contracts sixteen columns per pass on the matrix cores, also for small feature counts
-    if (ks * 16 <= kSplitMaxD + 2 && t <= 2) {
-        plan_register_resident(p, na_blocks, nb_blocks, split_b_blocks_per_wg(ks), ks * 3 * 64 * 16, 32, kSplitMaxCols,
+    if (ks * 16 <= kSplitMaxD + 2 && t <= 2 * kSplitMaxCols) {
+        plan_register_resident(p, na_blocks, nb_blocks, split_b_blocks_per_wg(ks, t), ks * 3 * 64 * 16, 32, kSplitMaxCols,
                                t, (int64_t)sizeof(float));
         return p;
     }

@@ -46,8 +46,9 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2)
     mmv_split_kernel(const uintx4 *__restrict__ PA, const float *__restrict__ vecp, int64_t vec_ld,
                      const uintx4 *__restrict__ PB, int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks,
                      float *__restrict__ partial, int64_t nb_pad, int tcols, bool y_fastest) {
-    static_assert(TT <= 2, "one staged dword per lane covers at most two columns of 32 rows");
-    __shared__ __attribute__((aligned(16))) float stage[kSplitWaves][2][64];
+    static_assert(TT <= 4, "two staged dwords per lane cover at most four columns of 32 rows");
+    constexpr int kStageDw = (TT + 1) / 2;      // dwords a lane stages per A block: columns lane/32 + 2c, row lane%32
+    __shared__ __attribute__((aligned(16))) float stage[kSplitWaves][2][64 * kStageDw];
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -79,15 +80,21 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2)
 #pragma unroll
         for (int t = 0; t < TT; t++) { o1[q][t] = 0.f; o2[q][t] = 0.f; }
 
-    // vec[a, t] of an A block reaches the lanes through a wave-private LDS buffer: one dword per lane from global
-    // memory (column lane/32 clamped to the last one, row lane%32), read back as broadcast 16-byte pieces
-    const float *vsrc = vecp + (int64_t)((lane >> 5) < TT ? (lane >> 5) : TT - 1) * vec_ld + (lane & 31);
+    // vec[a, t] of an A block reaches the lanes through a wave-private LDS buffer: one or two dwords per lane from
+    // global memory (column lane/32 + 2c clamped to the caller's last one, row lane%32), read back as broadcast
+    // 16-byte pieces
+    const float *vsrc[kStageDw];
+#pragma unroll
+    for (int c = 0; c < kStageDw; c++) {
+        const int col = (lane >> 5) + 2 * c;
+        vsrc[c] = vecp + (int64_t)(col < tcols ? col : tcols - 1) * vec_ld + (lane & 31);
+    }
     SplitFrag<KS> fa;
-    float rv = 0.f;
     int buf = 0;
     if (a0 < a1) {
         load_split<KS>(fa, PA, a0, lane);
-        stage[wave][0][lane] = vsrc[a0 * 32];
+#pragma unroll
+        for (int c = 0; c < kStageDw; c++) stage[wave][0][64 * c + lane] = vsrc[c][a0 * 32];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     }
@@ -143,8 +150,8 @@ __global__ void __launch_bounds__(64 * kSplitWaves, 2)
         // its own block: no branch in the loop body)
         const int64_t nxt = ab + 1 < a1 ? ab + 1 : ab;
         load_split<KS>(fa, PA, nxt, lane);
-        rv = vsrc[nxt * 32];
-        stage[wave][buf ^ 1][lane] = rv;
+#pragma unroll
+        for (int c = 0; c < kStageDw; c++) stage[wave][buf ^ 1][64 * c + lane] = vsrc[c][nxt * 32];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         buf ^= 1;
@@ -179,11 +186,13 @@ static int launch_split_one(const SplitView &A, const SplitView &B, const float 
     return FLK_OK;
 }
 
+// three and four columns: two resident fragments per wave whatever the feature count (registers)
 template <int KS, int FR>
 static int launch_split_tt(const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld, int tcols,
                            int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
     if (tcols == 1) return launch_split_one<KS, FR, 1>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
-    return launch_split_one<KS, FR, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+    if (tcols == 2) return launch_split_one<KS, FR, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+    return launch_split_one<KS, 2, 4>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
 }
 
 int FLK_CAT(launch_mmv_split_kf, FLK_KF)(const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld,
@@ -192,7 +201,7 @@ int FLK_CAT(launch_mmv_split_kf, FLK_KF)(const SplitView &A, const SplitView &B,
     if (A.ks != B.ks || A.d != B.d) return fail(FLK_EINVAL, "mmv_split: operands packed with different feature counts");
     if (tcols < 1 || tcols > kSplitMaxCols)
         return fail(FLK_EINVAL, "mmv_split: column chunk %d not in 1..%d", tcols, kSplitMaxCols);
-    if (split_b_blocks_per_wg(A.ks) != kSplitWaves * (A.ks <= 2 ? 4 : 2))
+    if (split_b_blocks_per_wg(A.ks, tcols) != kSplitWaves * (A.ks <= 2 && tcols <= 2 ? 4 : 2))
         return fail(FLK_EINVAL, "mmv_split: launch geometry out of step with the planner");
     switch (A.ks) {
         case 1: return launch_split_tt<1, 4>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);

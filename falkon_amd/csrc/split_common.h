@@ -19,7 +19,7 @@
 namespace flk {
 
 constexpr int64_t kSplitMaxD = 62;          // register-resident kernel: four k-steps, two of the 64 features taken by (1, h)
-constexpr int kSplitMaxCols = 2;            // its right-hand sides per pass
+constexpr int kSplitMaxCols = 4;            // its right-hand sides per pass
 
 inline int64_t split_ksteps(int64_t d) { return (d + 2 + 15) / 16; }
 
@@ -45,8 +45,8 @@ inline SplitView split_view(const void *buf, int64_t n, int64_t d) {
     v.npad = v.nblk * 32;
     return v;
 }
-// B blocks (of 32 output rows) per workgroup of the product kernel
-inline int split_b_blocks_per_wg(int64_t ks) { return 4 * (ks <= 2 ? 4 : 2); }
+// B blocks (of 32 output rows) per workgroup of the product kernel serving t right-hand sides per pass
+inline int split_b_blocks_per_wg(int64_t ks, int64_t t) { return 4 * (ks <= 2 && t <= 2 ? 4 : 2); }
 
 int launch_pack_split(const float *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const float *sigma, int64_t n_sigma,
                       double scale, void *packed, hipStream_t st);

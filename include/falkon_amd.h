@@ -20,7 +20,7 @@
  * three bfloat16 pieces (3 x 8 = 24 significant bits) and six partial products are accumulated in fp32,
  * which keeps the accuracy of the fp32 dot product (measured: the same distance from the fp64 result as
  * FLK_F32) at 16 features per matrix instruction instead of 2.  It has no counterpart in the reference.  Where
- * the fp32 MFMA kernels are the faster route (3 to 8 and more than 16 right-hand sides at d <= 62) they serve this code too.
+ * the fp32 MFMA kernels are the faster route (5 to 8 right-hand sides at d <= 32, more than 16 at d <= 62) they serve this code too.
  */
 #ifndef FALKON_AMD_H
 #define FALKON_AMD_H

@@ -24,7 +24,7 @@ def _data(n, m, d, t, seed, scale=1.0):
 
 
 @pytest.mark.parametrize("d", [1, 2, 9, 13, 14, 15, 28, 30, 31, 46, 47, 62])
-@pytest.mark.parametrize("t", [1, 2, 3, 5, 10])
+@pytest.mark.parametrize("t", [1, 2, 3, 4, 5, 8, 10])
 def test_products_vs_oracle(dev, d, t):
     n, m = 700 + 3 * d, 190 + d
     X, C, v, w = _data(n, m, d, t, seed=d + 100 * t)
