@@ -262,6 +262,96 @@ class _KernelMmvFn(torch.autograd.Function):
         return (None, None, None, *grads)
 
 
+# ---------------------------------------------------------------------------
+# many right-hand sides: kernel blocks stored once, contracted by library GEMMs
+# ---------------------------------------------------------------------------
+# The product kernels never store K and pay for it by evaluating K once per pass of 16 or 32 right-hand sides.
+# With many right-hand sides that is the wrong trade: a stored kernel value costs 4 (8) bytes written and a read per
+# product.  Beyond the break-even the drivers therefore do what the reference does on every call
+# (falkon/mmv_ops/fmmv.py:358-396,740-762): evaluate a block of rows of K with the kernel-matrix kernel and contract it
+# with rocBLAS (``K_b @ v``, ``K_b.T @ u``), block by block, K blocks as large as the memory budget allows, and K
+# evaluated once for both products of ``fdmmv``.  ``FalkonOptions.never_store_kernel`` switches this off.
+# Break-even in passes of the product kernels, measured on one MI355X (N = 2.5e5 .. 1e6, M = 1e4 .. 2e4):
+#   d = 784: T = 17 (2 passes) fp32 mmv 61.9 -> 45.1 ms, dmmv 122 -> 47 ms; T = 256: 989 -> 61 ms; fp64 2109 -> 120 ms;
+#   d = 100: T = 17 fp32 mmv 40.9 -> 36.3, dmmv 81 -> 45; T = 256: 741 -> 100;
+#   d = 28 fp32: T = 65 (3 passes) mmv 53.5 against 58.6 stored, T = 128 (4 passes) 86.9 -> 61.9, dmmv 172 -> 99;
+#   d = 9 fp32: T = 128 mmv 58.6 against 56.5, dmmv 116 -> 95; T = 65 dmmv 67 against 95 stored;
+#   d = 28 fp64: T = 64 (4 passes) mmv 72 against 75 stored, T = 128 143 -> 75, dmmv 286 -> 135.
+_EXPLICIT_BLOCK_BYTES = 8 * 2**30          # size of a stored block of K, memory permitting
+
+
+def _columns_per_pass(d: int, dtype: torch.dtype) -> int:
+    """Right-hand sides one evaluation of K serves in the product kernels."""
+    return 16 if d > 64 or dtype == torch.float64 else 32
+
+
+def _explicit_blocks_pay(d: int, t: int, dtype: torch.dtype, opt: BaseOptions) -> bool:
+    """Whether t right-hand sides are enough passes of the product kernels for stored blocks of K to be faster."""
+    if getattr(opt, "never_store_kernel", False):
+        return False
+    passes = -(-t // _columns_per_pass(d, dtype))
+    if d > 64:
+        return passes >= 2
+    if dtype == torch.float64:
+        return passes >= 5
+    return passes >= (4 if d <= 32 else 3)
+
+
+def _explicit_block_rows(N: int, M: int, D: int, T: int, sz: int, dev, opt: BaseOptions, upload_bytes: int) -> int:
+    """Rows of K per stored block (0: not even a sliver fits next to the operands; the caller keeps to the
+    product kernels).  Per row: the block itself, its products with v, and the packed copy of the row."""
+    usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack) - upload_bytes - 2 * M * (D + T) * sz
+    per_row = (M + 2 * T + 3 * D) * sz
+    rows = int(min(_EXPLICIT_BLOCK_BYTES, usable / 2) // per_row)
+    return min(N, rows) if rows >= 32 else 0
+
+
+def _fmmv_explicit(X1, X2, v, out, sigma_dev, kernel_fn: int, dev, opt: BaseOptions) -> bool:
+    """``out = K(X1, X2) @ v`` through stored blocks of K; False if the memory budget does not allow it."""
+    from .fmm import gauss_fmm_native
+    (N, D), (M, T), sz = X1.shape, v.shape, sizeof_dtype(X1.dtype)
+    upload = sum(t.numel() * sz for t in (X1, X2, v) if t.device != dev) + (0 if out.device == dev else N * T * sz)
+    rows = _explicit_block_rows(N, M, D, T, sz, dev, opt, upload)
+    if rows == 0:
+        return False
+    X1d, X2d, vd = _on(X1, dev), _on(X2, dev), _on(v, dev)
+    outd = out if out.device == dev else torch.empty((N, T), dtype=out.dtype, device=dev)
+    block = torch.empty((rows, M), dtype=X1.dtype, device=dev)
+    for i in range(0, N, rows):
+        li = min(rows, N - i)
+        gauss_fmm_native(X1d[i:i + li], X2d, sigma_dev, block[:li], False, kernel_fn)
+        outd[i:i + li].copy_(block[:li] @ vd)
+    if outd is not out:
+        out.copy_(outd)
+    return True
+
+
+def _fdmmv_explicit(X1, X2, v, w, out, sigma_dev, kernel_fn: int, dev, opt: BaseOptions) -> bool:
+    """``out = K^T (K v + w)`` through stored blocks of K; False if the memory budget does not allow it."""
+    from .fmm import gauss_fmm_native
+    (N, D), (M, T), sz = X1.shape, v.shape, sizeof_dtype(X1.dtype)
+    upload = (sum(t.numel() * sz for t in (X1, X2, v, w) if t is not None and t.device != dev)
+              + (0 if out.device == dev else M * T * sz))
+    rows = _explicit_block_rows(N, M, D, T, sz, dev, opt, upload)
+    if rows == 0:
+        return False
+    X1d, X2d, vd = _on(X1, dev), _on(X2, dev), _on(v, dev)
+    wd = _on(w, dev) if w is not None else None
+    outd = out if out.device == dev else torch.empty((M, T), dtype=out.dtype, device=dev)
+    outd.zero_()
+    block = torch.empty((rows, M), dtype=X1.dtype, device=dev)
+    for i in range(0, N, rows):
+        li = min(rows, N - i)
+        gauss_fmm_native(X1d[i:i + li], X2d, sigma_dev, block[:li], False, kernel_fn)
+        u = block[:li] @ vd
+        if wd is not None:
+            u += wd[i:i + li]
+        outd.addmm_(block[:li].T, u)
+    if outd is not out:
+        out.copy_(outd)
+    return True
+
+
 def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optional[torch.Tensor] = None,
          opt: Optional[BaseOptions] = None, kwargs_m1: Optional[Dict[str, torch.Tensor]] = None,
          kwargs_m2: Optional[Dict[str, torch.Tensor]] = None) -> torch.Tensor:
@@ -290,6 +380,9 @@ def _fmmv_run(X1, X2, v, kernel, kernel_fn: int, out, opt: BaseOptions, cached_s
 
     with torch.inference_mode():
         sigma_dev = kernel._sigma_on(dev, X1.dtype, cached=cached_sigma)
+        if N > 0 and M > 0 and _explicit_blocks_pay(D, T, X1.dtype, opt):
+            if _fmmv_explicit(X1, X2, v, out, sigma_dev, kernel_fn, dev, opt):
+                return out
         fixed = (0 if X2.device == dev else M * D * sz) + (0 if v.device == dev else M * T * sz)
 
         def need(rows: int) -> float:
@@ -349,6 +442,9 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
         x1_in, out_in = X1.device == dev, out.device == dev
         w_in = w is None or w.device == dev
         sigma_dev = kernel._sigma_on(dev, X1.dtype)
+        if N > 0 and M > 0 and _explicit_blocks_pay(D, T, X1.dtype, opt):
+            if _fdmmv_explicit(X1, X2, v, w, out, sigma_dev, kernel_fn, dev, opt):
+                return out
         fixed = ((0 if X2.device == dev else M * D * sz) + (0 if v.device == dev else M * T * sz)
                  + (0 if out_in else M * T * sz))
 

@@ -113,6 +113,10 @@ def test_large_d_vs_oracle(dev, dtype, n, m, d, t):
     assert rel_err(got_mmv, mmv_ref.fmmv_ref(X, C, v, sigma)) < TOL[dtype]
     assert rel_err(got_dmmv, mmv_ref.fdmmv_ref(X, C, v, w, sigma)) < TOL[dtype]
     assert rel_err(got_mmv, brute.mmv_brute(X, C, sigma, v)) < 5 * TOL[dtype]
+    if t > 16:      # enough columns for the stored-block route: the product kernels' multi-pass route as well
+        kf = GaussianKernel(sigma, opt=FalkonOptions(never_store_kernel=True))
+        assert rel_err(kf.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma)) < TOL[dtype]
+        assert rel_err(kf.dmmv(Xg, Cg, vg, wg), mmv_ref.fdmmv_ref(X, C, v, w, sigma)) < TOL[dtype]
 
 
 def test_config4_shape_reduced(dev):
@@ -535,3 +539,41 @@ def test_packed_entry_points(dev, dtype, n, m, d, t):
     assert torch.equal(u, k.mmv(X, C, v) + w) or rel_err(u, k.mmv(X, C, v) + w) < (1e-6 if dtype == torch.float32 else 1e-14)
     assert torch.equal(out, k.dmmv(X, C, v, w))
     assert rel_err(out, mmv_ref.fdmmv_ref(X.cpu(), C.cpu(), v.cpu(), w.cpu(), sigma.cpu())) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("n,m,d,t", [(700, 300, 100, 20), (300, 520, 784, 40), (2000, 333, 28, 130), (900, 257, 40, 70),
+                                     (500, 129, 9, 200)])
+def test_many_right_hand_sides_through_stored_blocks(dev, dtype, n, m, d, t, monkeypatch):
+    """Enough right-hand sides that the drivers store blocks of K and contract them with library GEMMs (the
+    reference's own scheme, falkon/mmv_ops/fmmv.py:358-396,740-762): same tolerances against the CPU path, agreement
+    with the product kernels (``never_store_kernel=True``), several blocks (block size forced down), strided
+    operands, ``out=``, host data, ``w = None``."""
+    import importlib
+    drv = importlib.import_module("falkon_amd.mmv_ops.fmmv")
+    assert drv._explicit_blocks_pay(d, t, dtype, FalkonOptions()) or dtype == torch.float64 and d <= 64 and t < 65
+    X, C, v, w = _rand(n, d, m, t, dtype, seed=n + t, scale=0.6)
+    sigma = 0.8 * np.sqrt(d)
+    k, k_free = GaussianKernel(sigma), GaussianKernel(sigma, opt=FalkonOptions(never_store_kernel=True))
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+    tol = TOL[dtype]
+    got_mmv, got_dmmv = k.mmv(Xg, Cg, vg), k.dmmv(Xg, Cg, vg, wg)
+    check_parity(got_mmv, mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), tol)
+    check_parity(got_dmmv, mmv_ref.fdmmv_ref(X, C, v, w, sigma), mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), tol)
+    assert rel_err(got_mmv, k_free.mmv(Xg, Cg, vg)) < tol and rel_err(got_dmmv, k_free.dmmv(Xg, Cg, vg, wg)) < tol
+    check_parity(k.dmmv(Xg, Cg, vg, None), mmv_ref.fdmmv_ref(X, C, v, None, sigma),
+                 mmv_ref.fdmmv_ref(Xd, Cd, vd, None, sigma), tol)
+    # several stored blocks, F-ordered operands, out=, host data
+    monkeypatch.setattr(drv, "_EXPLICIT_BLOCK_BYTES", 64 * m * X.element_size())
+    f = lambda a: a.T.contiguous().T                                                      # noqa: E731
+    out = torch.empty(t, n, dtype=dtype, device=dev).T
+    assert k.mmv(f(Xg), f(Cg), f(vg), out=out).data_ptr() == out.data_ptr()
+    # (other layouts make the library GEMMs sum in another order: compare with the CPU path again, not bit for bit)
+    ref_mmv = (mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma))
+    ref_dmmv = (mmv_ref.fdmmv_ref(X, C, v, w, sigma), mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma))
+    check_parity(out, *ref_mmv, tol)
+    check_parity(k.dmmv(f(Xg), Cg, vg, f(wg)), *ref_dmmv, tol)
+    host = k.dmmv(X, C, v, w)
+    assert host.device.type == "cpu"
+    check_parity(host, *ref_dmmv, tol)
