@@ -142,7 +142,8 @@ template <typename T> int mmv_large_max_cols();
 //   launch_mmv_small_kf*: register-resident product kernel, FLK_EUNSUPPORTED if dpad is out of its range;
 //   launch_mmv_large_kf*: LDS-tiled product kernel, writes splits * mmv_large_partials_per_split partials;
 //   launch_fmm_kf*:       explicit kernel matrix out[a][b] = K(A_a, B_b); O is the element type of out, whose
-//                         rows (A side) are ld elements apart and whose columns (B side) are contiguous.
+//                         rows (A side) are ld elements apart and whose columns (B side) are contiguous;
+//   launch_fmm_large_kf*: the same through the LDS-tiled kernel (operands packed for d > 64).
 #define FLK_CAT2(a, b) a##b
 #define FLK_CAT(a, b) FLK_CAT2(a, b)
 #define FLK_DECLARE_KF(KF)                                                                                        \
@@ -159,7 +160,9 @@ template <typename T> int mmv_large_max_cols();
     int launch_mmv_large_kf##KF(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld,          \
                                 int tcols, int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st);    \
     template <typename T, typename O>                                                                             \
-    int launch_fmm_kf##KF(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st);
+    int launch_fmm_kf##KF(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st);          \
+    template <typename T, typename O>                                                                             \
+    int launch_fmm_large_kf##KF(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st);
 FLK_DECLARE_KF(0)
 FLK_DECLARE_KF(1)
 FLK_DECLARE_KF(2)

@@ -123,6 +123,9 @@ int FLK_CAT(launch_fmm_kf, FLK_KF)(const PackedView &A, const PackedView &B, O *
     typedef FmmCfg<T> C;
     if (A.dpad != B.dpad || A.d != B.d) return fail(FLK_EINVAL, "fmm: operands packed with different feature counts");
     if (A.n == 0 || B.n == 0) return FLK_OK;
+    // beyond the register-resident feature counts the LDS-tiled kernel evaluates K faster (it stages both operand
+    // tiles in LDS instead of reading them per step)
+    if (A.d > kSmallMaxD) return FLK_CAT(launch_fmm_large_kf, FLK_KF)<T, O>(A, B, out, ld, st);
     const int64_t a_tiles = (A.nblk + kFmmWavesA * C::FA - 1) / (kFmmWavesA * C::FA);
     const int64_t b_tiles = (B.nblk + kFmmWavesB * C::FB - 1) / (kFmmWavesB * C::FB);
     if (a_tiles * b_tiles > (int64_t)0x7fffffff) return fail(FLK_EUNSUPPORTED, "fmm: more tiles than one launch holds");

@@ -63,12 +63,16 @@ __device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t b
 }
 
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
-template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC, int TT, int KF>
+// O = void: the product (partial sums of K against vec).  O = an element type: the kernel matrix itself, entry
+// (a, b) stored as O at kout[a * kout_ld + b] (then TT = 1, vecp is not read and partial not written).
+template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC, int TT, int KF, typename O = void>
 __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   // two waves per SIMD either way
     mmv_large_kernel(const T *__restrict__ PA, const T *__restrict__ hA, const T *__restrict__ vecp, int64_t vec_ld,
                      int tcols, const T *__restrict__ PB, const T *__restrict__ hB, int64_t na_blocks,
                      int64_t nb_blocks, int64_t dpad, int last_steps, int64_t a_tiles_per_chunk,
-                     T *__restrict__ partial, int64_t nb_pad, bool y_fastest) {
+                     T *__restrict__ partial, int64_t nb_pad, bool y_fastest, void *__restrict__ kout = nullptr,
+                     int64_t kout_ld = 0, int64_t n_a = 0, int64_t n_b = 0) {
+    constexpr bool kStore = !std::is_void<O>::value;
     typedef LTraits<T> TR;
     typedef LGeo<T, WVA, WVB, WA_FR, WB_FR, KC> G;
     constexpr int kLWavesA = WVA, kLWavesB = WVB, kLThreads = 64 * WVA * WVB;
@@ -247,7 +251,30 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         // after each group (the updated accumulators pass through an empty asm that also clobbers memory
         // through the LDS pointer) keeps the compiler from moving every read to the front and spilling.
         static_assert(WB_FR == 2, "the epilogue fence lists its operands explicitly");
-        if constexpr (!kMfmaEpi) {
+        if constexpr (kStore) {
+            typedef typename std::conditional<kStore, O, T>::type OT;
+            OT *dst = (OT *)kout;
+#pragma unroll
+            for (int p = 0; p < WA_FR; p++) {
+#pragma unroll
+                for (int g = 0; g < TR::NG; g++) {
+                    const int ro = (wa * WA_FR + p) * TR::BLK + TR::group_off(g, lg);     // four consecutive rows
+                    const vec4_t hn = *(const vec4_t *)(&ldsRow[ro]);
+#pragma unroll
+                    for (int q = 0; q < WB_FR; q++) {
+                        const int64_t col = (bblk0 + wb * WB_FR + q) * TR::BLK + TR::out_row(j);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            // h - h is 0, or NaN where a row holds a NaN or an infinity (the clamps would hide it)
+                            const T h = hn[e] + hb[q];
+                            const T k = kernel_value<FLK_KF>(acc[p][q][4 * g + e] + h) + (h - h);
+                            const int64_t row = ablk0 * TR::BLK + ro + e;
+                            if (row < n_a && col < n_b) __builtin_nontemporal_store((OT)k, &dst[row * kout_ld + col]);
+                        }
+                    }
+                }
+            }
+        } else if constexpr (!kMfmaEpi) {
         constexpr int NTG = (TT + 3) / 4;
 #pragma unroll
         for (int p = 0; p < WA_FR; p++) {
@@ -329,7 +356,9 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         }
     }
 
-    if constexpr (kMfmaEpi) {
+    if constexpr (kStore) {
+        // nothing left to write
+    } else if constexpr (kMfmaEpi) {
         // lane = column t (both lane groups hold different output rows): no cross-lane step
         const int tl = j & 15;
         if (j < 16 && tl < tcols) {
@@ -404,6 +433,36 @@ static int launch_large_tt(const PackedView &A, const PackedView &B, const T *ve
     FLK_LAUNCH_CHECK("mmv_large_kernel");
     return FLK_OK;
 }
+
+// The kernel matrix out[a][b] = K(A_a, B_b) through the same tiles (operands packed for d > 64): one workgroup per
+// (A tile, B tile), or a few A tiles per workgroup where the grid would not hold them all.
+template <typename T, typename O>
+int FLK_CAT(launch_fmm_large_kf, FLK_KF)(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st) {
+    typedef LCfg<T> C;
+    if (A.dpad != B.dpad || A.d != B.d) return fail(FLK_EINVAL, "fmm: operands packed with different feature counts");
+    if (A.n == 0 || B.n == 0) return FLK_OK;
+    const int64_t nab = C::WVA * C::WA_FR, nbb = C::WVB * C::WB_FR;
+    const int64_t a_tiles = (A.nblk + nab - 1) / nab;
+    const int64_t per_wg = (a_tiles + 65534) / 65535;
+    dim3 grid((unsigned)((B.nblk + nbb - 1) / nbb), (unsigned)((a_tiles + per_wg - 1) / per_wg));
+    const int64_t chunk_features = (int64_t)C::KC * LTraits<T>::KG;
+    const int64_t tail = A.d - (A.dpad / chunk_features - 1) * chunk_features;
+    const int last_steps = (int)((tail + LTraits<T>::KG - 1) / LTraits<T>::KG);
+    if (A.dpad % chunk_features != 0 || last_steps < 1 || last_steps > C::KC)
+        return fail(FLK_EINVAL, "fmm: operand padding does not match the LDS-tiled kernel");
+    hipLaunchKernelGGL((mmv_large_kernel<T, C::WVA, C::WVB, C::WA_FR, C::WB_FR, C::KC, 1, FLK_KF, O>), grid,
+                       dim3(64 * C::WVA * C::WVB), 0, st, (const T *)A.data, (const T *)A.hnorm, (const T *)nullptr,
+                       (int64_t)0, 0, (const T *)B.data, (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, last_steps, per_wg,
+                       (T *)nullptr, B.npad, B.n > A.n, (void *)out, ld, A.n, B.n);
+    FLK_LAUNCH_CHECK("mmv_large_kernel (kernel matrix)");
+    return FLK_OK;
+}
+template int FLK_CAT(launch_fmm_large_kf, FLK_KF)<float, float>(const PackedView &, const PackedView &, float *, int64_t,
+                                                                hipStream_t);
+template int FLK_CAT(launch_fmm_large_kf, FLK_KF)<double, double>(const PackedView &, const PackedView &, double *,
+                                                                  int64_t, hipStream_t);
+template int FLK_CAT(launch_fmm_large_kf, FLK_KF)<double, float>(const PackedView &, const PackedView &, float *, int64_t,
+                                                                 hipStream_t);
 
 template <typename T>
 int FLK_CAT(launch_mmv_large_kf, FLK_KF)(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld,

@@ -272,8 +272,8 @@ class _KernelMmvFn(torch.autograd.Function):
 # with rocBLAS (``K_b @ v``, ``K_b.T @ u``), block by block, K blocks as large as the memory budget allows, and K
 # evaluated once for both products of ``fdmmv``.  ``FalkonOptions.never_store_kernel`` switches this off.
 # Break-even in passes of the product kernels, measured on one MI355X (N = 2.5e5 .. 1e6, M = 1e4 .. 2e4):
-#   d = 784: T = 17 (2 passes) fp32 mmv 61.9 -> 45.1 ms, dmmv 122 -> 47 ms; T = 256: 989 -> 61 ms; fp64 2109 -> 120 ms;
-#   d = 100: T = 17 fp32 mmv 40.9 -> 36.3, dmmv 81 -> 45; T = 256: 741 -> 100;
+#   d = 784: T = 17 (2 passes) fp32 mmv 61.9 -> 32.6 ms, dmmv 122 -> 35 ms; T = 256: 986 -> 49 ms; fp64 2097 -> 114 ms;
+#   d = 100: T = 17 fp32 mmv 40.9 -> 29.1, dmmv 81 -> 36; T = 256: 741 -> 94;
 #   d = 28 fp32: T = 65 (3 passes) mmv 53.5 against 58.6 stored, T = 128 (4 passes) 86.9 -> 61.9, dmmv 172 -> 99;
 #   d = 9 fp32: T = 128 mmv 58.6 against 56.5, dmmv 116 -> 95; T = 65 dmmv 67 against 95 stored;
 #   d = 28 fp64: T = 64 (4 passes) mmv 72 against 75 stored, T = 128 143 -> 75, dmmv 286 -> 135.

@@ -220,7 +220,8 @@ def test_config1_full(dev):
 # explicit kernel matrix (the preconditioner's K(C, C)) through flk_gauss_fmm
 # --------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-@pytest.mark.parametrize("n,m,d", [(1, 1, 1), (33, 70, 3), (200, 131, 28), (129, 257, 9), (64, 300, 110), (50, 45, 784)])
+@pytest.mark.parametrize("n,m,d", [(1, 1, 1), (33, 70, 3), (200, 131, 28), (129, 257, 9), (64, 300, 110), (50, 45, 784),
+                                   (600, 700, 130), (257, 513, 65), (1, 300, 100), (300, 1, 97)])
 def test_kernel_matrix_vs_oracle(dev, dtype, n, m, d):
     """kernel(X1, X2) against rbf_core (falkon/kernels/distance_kernel.py:140-159) restated on the CPU and
     against the fp64 difference form; per-dimension sigma; fp32 in both evaluation modes of
@@ -269,6 +270,33 @@ def test_kernel_matrix_layouts_and_out(dev):
     assert float((Kcc.diagonal() - 1).abs().max()) < 1e-12 and float((Kcc - Kcc.T).abs().max()) < 1e-13
     d = k(X.to(dev), X.to(dev), diag=True)
     assert d.shape == (150,) and float((d.cpu() - 1).abs().max()) < 1e-12
+
+
+def test_kernel_matrix_layouts_large_d(dev):
+    """The same for d > 64, where the kernel matrix comes from the LDS-tiled kernel: F-ordered result (operand roles
+    swapped), ``out=`` in either order, row blocking, unit diagonal, other kernel functions, non-finite rows."""
+    from oracle import gaussian_ref
+    from falkon_amd import LaplacianKernel
+    X, C, _, _ = _rand(700, 150, 390, 1, torch.float64, seed=5, scale=0.5)
+    k = GaussianKernel(9.0)
+    ref = gaussian_ref.rbf_core_ref(X, C, None, k.sigma)
+    Xf = torch.empty_strided(X.shape, (1, X.shape[0]), dtype=X.dtype).copy_(X).to(dev)
+    got_f = k(Xf, C.to(dev))
+    assert got_f.stride(0) == 1 and float((got_f.cpu() - ref).abs().max()) < 1e-12
+    for strides in ((390, 1), (1, 700)):
+        out = torch.empty_strided((700, 390), strides, dtype=X.dtype, device=dev)
+        res = k(X.to(dev), C.to(dev), out=out)
+        assert res.data_ptr() == out.data_ptr() and float((out.cpu() - ref).abs().max()) < 1e-12
+    small = k(X.to(dev), C.to(dev), opt=FalkonOptions(max_gpu_mem=3_000_000))
+    assert float((small.cpu() - ref).abs().max()) < 1e-12
+    Kcc = k(C.to(dev), C.to(dev)).cpu()
+    assert float((Kcc.diagonal() - 1).abs().max()) < 1e-12 and float((Kcc - Kcc.T).abs().max()) < 1e-13
+    lap = LaplacianKernel(9.0)(X.to(dev), C.to(dev)).cpu()
+    assert float((lap - torch.from_numpy(brute.radial_brute(X, C, torch.tensor([9.0]), "laplacian"))).abs().max()) < 1e-9
+    Xb = X.clone()
+    Xb[5, 100] = float("nan")
+    bad, clean = k(Xb.to(dev), C.to(dev)).cpu(), k(X.to(dev), C.to(dev)).cpu()
+    assert torch.isnan(bad[5]).all() and torch.equal(bad[6:], clean[6:]) and torch.equal(bad[:5], clean[:5])
 
 
 # --------------------------------------------------------------------------------------------------
