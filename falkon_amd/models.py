@@ -31,8 +31,6 @@ class Falkon(_Base):
                  center_selection: Union[str, CenterSelector] = "uniform", maxiter: int = 20,
                  seed: Optional[int] = None, error_fn: Optional[Callable] = None, error_every: Optional[int] = 1,
                  weight_fn: Optional[Callable] = None, options: Optional[FalkonOptions] = None):
-        if weight_fn is not None:
-            raise NotImplementedError("weighted least squares is not part of this build")
         self.kernel, self.penalty, self.M, self.maxiter = kernel, penalty, M, maxiter
         self.seed, self.error_fn, self.error_every, self.weight_fn = seed, error_fn, error_every, weight_fn
         if seed is not None:
@@ -70,16 +68,21 @@ class Falkon(_Base):
         self.fit_times_, self.val_errors_ = [], []
         t_s = time.time()
         with torch.inference_mode():
-            ny_points = self.center_selection.select(X, None)
+            ny_weights = None
+            if self.weight_fn is None:
+                ny_points = self.center_selection.select(X, None)
+            else:                                       # the centres' own weights go into the preconditioner
+                ny_points, ny_indices = self.center_selection.select_indices(X, None)
+                ny_weights = self.weight_fn(Y[ny_indices], X[ny_indices], ny_indices)
             Xd, Yd, Cd = X.to(dev), Y.to(dev), ny_points.to(dev)
             self.precond = FalkonPreconditioner(self.penalty, self.kernel, self.options)
-            self.precond.init(Cd)
+            self.precond.init(Cd, weight_vec=ny_weights)
             torch.cuda.synchronize(dev)                 # fit_times_ are wall times of finished work
             self.fit_times_.append(time.time() - t_s)
             cb = None
             if self.error_fn is not None and self.error_every is not None:
                 cb = self._callback(Xd, Yd, Xts, Yts, Cd)
-            optim = FalkonConjugateGradient(self.kernel, self.precond, self.options)
+            optim = FalkonConjugateGradient(self.kernel, self.precond, self.options, weight_fn=self.weight_fn)
             ws = warm_start.to(dev) if warm_start is not None else None
             beta = optim.solve(Xd, Cd, Yd, self.penalty, initial_solution=ws, max_iter=self.maxiter, callback=cb)
             alpha = self.precond.apply(beta)

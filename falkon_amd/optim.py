@@ -70,12 +70,12 @@ class ConjugateGradient:
 
 class FalkonConjugateGradient:
     r"""Preconditioned CG on ``B^T (K_nm^T K_nm + lambda n K_mm) B beta = B^T K_nm^T y / n`` with
-    ``B = 1/sqrt(n) T^-1 A^-1`` (falkon/optim/conjgrad.py:187-306).  One ``kernel.dmmv`` per iteration."""
+    ``B = 1/sqrt(n) T^-1 A^-1`` (falkon/optim/conjgrad.py:187-306).  One ``kernel.dmmv`` per iteration; with a
+    ``weight_fn`` (weighted least squares, ``K_nm^T W K_nm`` and ``K_nm^T W y``) two ``kernel.mmv`` with the weights
+    applied in between (conjgrad.py:258-272,291-300)."""
 
     def __init__(self, kernel, preconditioner, opt: FalkonOptions, weight_fn=None):
-        if weight_fn is not None:
-            raise NotImplementedError("weighted least squares is not part of this build")
-        self.kernel, self.preconditioner, self.params = kernel, preconditioner, opt
+        self.kernel, self.preconditioner, self.params, self.weight_fn = kernel, preconditioner, opt, weight_fn
         cg_fields = ("cg_epsilon_32", "cg_epsilon_64", "cg_tolerance", "cg_full_gradient_every",
                      "cg_differential_convergence")
         self.optimizer = ConjugateGradient(ConjugateGradientOptions(**{f: getattr(opt, f) for f in cg_fields}))
@@ -88,6 +88,18 @@ class FalkonConjugateGradient:
         gram = self.kernel.dmmv(X, M, pc.invT(inner), None, opt=self.params)      # K_nm^T K_nm (.): the hot call
         return pc.invAt(pc.invTt(gram / n) + penalty * inner)
 
+    def weighted_falkon_mmv(self, sol, penalty, X, M, y_weights, n: int):
+        """The same operator with ``K_nm^T W K_nm`` in the middle (falkon/optim/conjgrad.py:258-272)."""
+        pc = self.preconditioner
+        inner = pc.invA(sol)
+        weighted = self.kernel.mmv(X, M, pc.invT(inner), None, opt=self.params).mul_(y_weights)
+        gram = self.kernel.mmv(M, X, weighted, None, opt=self.params)
+        return pc.invAt(pc.invTt(gram / n) + penalty * inner)
+
+    @property
+    def is_weighted(self) -> bool:
+        return self.weight_fn is not None
+
     def solve(self, X, M, Y, _lambda, initial_solution, max_iter, callback=None):
         if not torch.is_inference_mode_enabled():
             # the reference fails here too, with torch's own message about inference tensors (the products run under
@@ -95,6 +107,12 @@ class FalkonConjugateGradient:
             raise RuntimeError("FalkonConjugateGradient.solve was called outside InferenceMode: "
                                "wrap the call in `with torch.inference_mode():`")
         n = Y.shape[0]
-        rhs = self.preconditioner.apply_t(self.kernel.mmv(M, X, Y / n, opt=self.params))   # B^T K_nm^T y / n
-        operator = functools.partial(self.falkon_mmv, penalty=_lambda, X=X, M=M, n=n)
+        y_over_n = Y / n
+        if self.is_weighted:
+            y_weights = self.weight_fn(Y, X, torch.arange(n))
+            y_over_n.mul_(y_weights)
+            operator = functools.partial(self.weighted_falkon_mmv, penalty=_lambda, X=X, M=M, y_weights=y_weights, n=n)
+        else:
+            operator = functools.partial(self.falkon_mmv, penalty=_lambda, X=X, M=M, n=n)
+        rhs = self.preconditioner.apply_t(self.kernel.mmv(M, X, y_over_n, opt=self.params))   # B^T K_nm^T (W) y / n
         return self.optimizer.solve(initial_solution, rhs, operator, max_iter, callback)

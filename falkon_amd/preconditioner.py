@@ -163,16 +163,23 @@ class FalkonPreconditioner:
         self._A: Optional[_BlockedTriangular] = None
 
     def init(self, X: torch.Tensor, weight_vec: Optional[torch.Tensor] = None) -> None:
-        if weight_vec is not None:
-            raise NotImplementedError("weighted least squares is not part of this build")
+        """Factorise for the centres X.  ``weight_vec`` (M x 1, the weights of the centres) is for weighted least
+        squares: ``A = chol(T W T^T / M + lambda I)``, the reference's CPU algebra (flk_preconditioner.py:122-127,
+        which weighs the columns of T by sqrt(w) before the triangular product)."""
         M = X.shape[0]
+        if weight_vec is not None and weight_vec.numel() != M:
+            raise ValueError(f"weight_vec must have one entry per centre ({M}), found {weight_vec.numel()}")
         with torch.inference_mode():
             C = self.kernel(X, X, opt=self.params)                     # fp64-computed when no_single_kernel
             eps = self.params.pc_epsilon(C.dtype)
             C.diagonal().add_(eps * M)
             LT = _cholesky_lower_(C)
             del C
-            G = _gram_of_lower_factor(LT)                               # T T^T, lower triangle only
+            if weight_vec is None:
+                G = _gram_of_lower_factor(LT)                           # T T^T, lower triangle only
+            else:                                                       # T W T^T = (sqrt(W) LT)^T (sqrt(W) LT)
+                root = weight_vec.reshape(-1, 1).to(device=LT.device, dtype=LT.dtype).sqrt()
+                G = _gram_of_lower_factor(LT * root)
             G.mul_(1.0 / M)
             G.diagonal().add_(self._lambda)
             self.LA = _cholesky_lower_(G)

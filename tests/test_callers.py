@@ -426,3 +426,55 @@ def test_center_selection_on_gpu_tensors(dev):
     assert centers.dtype == X.dtype and centers.device == X.device
     centers, idx = sel.select_indices(X, None)
     assert centers.device == idx.device and idx.dtype == torch.long and len(idx) == num
+
+
+# --------------------------------------------------------------------------------------------------
+# weighted least squares (falkon/optim/conjgrad.py:258-300, flk_preconditioner.py:94-160, models/falkon.py:258-275)
+# --------------------------------------------------------------------------------------------------
+def _two_to_one(y, x, indices):
+    """The reference's test weights: class -1 counts twice (tests/test_falkon.py:212-216)."""
+    weight = torch.empty_like(y)
+    weight[y == 1] = 1
+    weight[y == -1] = 2
+    return weight
+
+
+@pytest.mark.gpu
+def test_weighted_falkon_solves_the_weighted_normal_equations(dev):
+    """alpha = (K_nm^T W K_nm + lambda n K_mm)^-1 K_nm^T W y, from the definition in fp64, for weights that depend on
+    the targets; centres are rows of the data, so that the preconditioner gets their weights."""
+    X, Y, _, sigma, lam = _conjgrad_problem()
+    Y = torch.sign(Y - 0.5)
+    idx = torch.from_numpy(np.random.default_rng(2).choice(X.shape[0], 10, replace=False))
+    C = X[idx].clone()
+    model = Falkon(GaussianKernel(sigma), lam, M=10, center_selection=FixedSelector(C, idx_centers=idx), maxiter=200,
+                   weight_fn=_two_to_one, options=FalkonOptions(cg_tolerance=1e-10))
+    model.fit(X.to(dev), Y.to(dev))
+    Knm = gaussian_ref.rbf_core_ref(X, C, None, torch.tensor([sigma])).numpy()
+    Kmm = gaussian_ref.rbf_core_ref(C, C, None, torch.tensor([sigma])).numpy()
+    W = _two_to_one(Y, X, None).numpy()
+    expected = np.linalg.solve(Knm.T @ (W * Knm) + lam * X.shape[0] * Kmm, Knm.T @ (W * Y.numpy()))
+    np.testing.assert_allclose(model.alpha_.cpu().numpy(), expected, rtol=1e-5)
+    # the preconditioner's second factor is that of T W_M T^T / M + lambda I
+    T = model.precond.LT.T.cpu().numpy()
+    Wm = _two_to_one(Y[idx], None, None).numpy().reshape(-1)
+    A = model.precond.LA.T.cpu().numpy()
+    np.testing.assert_allclose(A.T @ A, T @ (Wm[:, None] * T.T) / 10 + lam * np.eye(10), rtol=1e-9, atol=1e-12)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("where", ["incore", "mixed"])
+def test_reference_weighted_falkon_classification(dev, where):
+    """tests/test_falkon.py:191-244: weighting class -1 twice lowers its error and does not lower the other's."""
+    from falkon_amd import InCoreFalkon
+    X, Y = _cls_data()
+    cls = Falkon
+    if where == "incore":
+        X, Y, cls = X.to(dev), Y.to(dev), InCoreFalkon
+    errs = {}
+    for name, wf in (("weighted", _two_to_one), ("plain", None)):
+        flk = cls(kernel=GaussianKernel(2.0), penalty=1e-6, M=500, seed=10, weight_fn=wf).fit(X, Y)
+        preds = flk.predict(X)
+        errs[name] = (float(_c_err(preds[Y == -1], Y[Y == -1])[0]), float(_c_err(preds[Y == 1], Y[Y == 1])[0]))
+    assert errs["weighted"][0] < errs["plain"][0], "Error of weighted class is higher than without weighting"
+    assert errs["weighted"][1] >= errs["plain"][1], "Error of unweighted class is lower than in flk with no weights"
