@@ -82,12 +82,24 @@ class Falkon(_Base):
             cb = None
             if self.error_fn is not None and self.error_every is not None:
                 cb = self._callback(Xd, Yd, Xts, Yts, Cd)
-            optim = FalkonConjugateGradient(self.kernel, self.precond, self.options, weight_fn=self.weight_fn)
+            knm = self.kernel(Xd, Cd, opt=self.options) if self._can_store_knm(Xd, Cd) else None
+            optim = FalkonConjugateGradient(self.kernel, self.precond, self.options, weight_fn=self.weight_fn,
+                                            stored_knm=knm)
             ws = warm_start.to(dev) if warm_start is not None else None
             beta = optim.solve(Xd, Cd, Yd, self.penalty, initial_solution=ws, max_iter=self.maxiter, callback=cb)
             alpha = self.precond.apply(beta)
             self.alpha_, self.beta_, self.ny_points_ = alpha.to(X.device), beta.to(X.device), ny_points
         return self
+
+    def _can_store_knm(self, X, ny_points) -> bool:
+        """The reference's rule (falkon/models/model_utils.py:155-190): with more than ``store_kernel_d_threshold``
+        features a kernel evaluation costs more than the two products with a stored value, so K(X, centres) is kept
+        for the solve when it fits the memory budget (and ``never_store_kernel`` is not set)."""
+        if self.options.never_store_kernel or X.shape[1] <= self.options.store_kernel_d_threshold:
+            return False
+        from .mmv_ops.utils import usable_gpu_memory
+        need = 1.1 * X.shape[0] * ny_points.shape[0] * X.element_size()
+        return usable_gpu_memory(X.device, self.options.max_gpu_mem, self.options.memory_slack) > need
 
     def _callback(self, X, Y, Xts, Yts, ny_points):
         def val_cback(it, beta, train_time):

@@ -74,8 +74,12 @@ class FalkonConjugateGradient:
     ``weight_fn`` (weighted least squares, ``K_nm^T W K_nm`` and ``K_nm^T W y``) two ``kernel.mmv`` with the weights
     applied in between (conjgrad.py:258-272,291-300)."""
 
-    def __init__(self, kernel, preconditioner, opt: FalkonOptions, weight_fn=None):
+    def __init__(self, kernel, preconditioner, opt: FalkonOptions, weight_fn=None, stored_knm=None):
+        """``stored_knm``: K(X, M) kept in memory for the solve (what the reference's ``PrecomputedKernel`` is for,
+        falkon/kernels/precomputed_kernel.py, falkon/models/model_utils.py:155-190): the products of every iteration
+        are then library GEMMs on it instead of kernel evaluations."""
         self.kernel, self.preconditioner, self.params, self.weight_fn = kernel, preconditioner, opt, weight_fn
+        self.stored_knm = stored_knm
         cg_fields = ("cg_epsilon_32", "cg_epsilon_64", "cg_tolerance", "cg_full_gradient_every",
                      "cg_differential_convergence")
         self.optimizer = ConjugateGradient(ConjugateGradientOptions(**{f: getattr(opt, f) for f in cg_fields}))
@@ -85,15 +89,21 @@ class FalkonConjugateGradient:
         (falkon/optim/conjgrad.py:262-285)."""
         pc = self.preconditioner
         inner = pc.invA(sol)
-        gram = self.kernel.dmmv(X, M, pc.invT(inner), None, opt=self.params)      # K_nm^T K_nm (.): the hot call
+        if self.stored_knm is not None:
+            gram = self.stored_knm.T @ (self.stored_knm @ pc.invT(inner))
+        else:
+            gram = self.kernel.dmmv(X, M, pc.invT(inner), None, opt=self.params)  # K_nm^T K_nm (.): the hot call
         return pc.invAt(pc.invTt(gram / n) + penalty * inner)
 
     def weighted_falkon_mmv(self, sol, penalty, X, M, y_weights, n: int):
         """The same operator with ``K_nm^T W K_nm`` in the middle (falkon/optim/conjgrad.py:258-272)."""
         pc = self.preconditioner
         inner = pc.invA(sol)
-        weighted = self.kernel.mmv(X, M, pc.invT(inner), None, opt=self.params).mul_(y_weights)
-        gram = self.kernel.mmv(M, X, weighted, None, opt=self.params)
+        if self.stored_knm is not None:
+            gram = self.stored_knm.T @ (self.stored_knm @ pc.invT(inner)).mul_(y_weights)
+        else:
+            weighted = self.kernel.mmv(X, M, pc.invT(inner), None, opt=self.params).mul_(y_weights)
+            gram = self.kernel.mmv(M, X, weighted, None, opt=self.params)
         return pc.invAt(pc.invTt(gram / n) + penalty * inner)
 
     @property
@@ -114,5 +124,6 @@ class FalkonConjugateGradient:
             operator = functools.partial(self.weighted_falkon_mmv, penalty=_lambda, X=X, M=M, y_weights=y_weights, n=n)
         else:
             operator = functools.partial(self.falkon_mmv, penalty=_lambda, X=X, M=M, n=n)
-        rhs = self.preconditioner.apply_t(self.kernel.mmv(M, X, y_over_n, opt=self.params))   # B^T K_nm^T (W) y / n
+        kty = self.stored_knm.T @ y_over_n if self.stored_knm is not None else self.kernel.mmv(M, X, y_over_n, opt=self.params)
+        rhs = self.preconditioner.apply_t(kty)                                                # B^T K_nm^T (W) y / n
         return self.optimizer.solve(initial_solution, rhs, operator, max_iter, callback)

@@ -35,7 +35,7 @@ class BaseOptions:
     min_cuda_iter_size_32: int = 10_000 * 10 * 3_000  # carried, unused
     min_cuda_iter_size_64: int = 30_000 * 10 * 3_000  # carried, unused
     never_store_kernel: bool = False                  # True: never store blocks of K, however many right-hand sides
-    store_kernel_d_threshold: int = 1200              # carried, unused
+    store_kernel_d_threshold: int = 1200              # beyond this many features a fit keeps K(X, centres) if it fits
     num_fmm_streams: int = 2                          # carried, unused
     memory_slack: float = 0.9                         # fraction of the free device memory a call may plan with
     bf16x3_cross_term: bool = False                   # not in the reference: fp32 products form x.c on the bf16 matrix

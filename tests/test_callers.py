@@ -478,3 +478,30 @@ def test_reference_weighted_falkon_classification(dev, where):
         errs[name] = (float(_c_err(preds[Y == -1], Y[Y == -1])[0]), float(_c_err(preds[Y == 1], Y[Y == 1])[0]))
     assert errs["weighted"][0] < errs["plain"][0], "Error of weighted class is higher than without weighting"
     assert errs["weighted"][1] >= errs["plain"][1], "Error of unweighted class is lower than in flk with no weights"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("incore", [False, True])
+def test_reference_precomputed_kernel_fit(dev, incore):
+    """tests/test_falkon.py:167-189,306-340: with ``store_kernel_d_threshold`` below the feature count the fit keeps
+    K(X, centres) in memory and runs its products on it; same accuracy bounds, and the same coefficients as the fit
+    that evaluates the kernel in every iteration."""
+    from falkon_amd import InCoreFalkon
+    Xtr, Ytr, Xts, Yts = _reg_data()
+    if incore:
+        Xtr, Ytr, Xts, Yts = (a.to(dev) for a in (Xtr, Ytr, Xts, Yts))
+    cls = InCoreFalkon if incore else Falkon
+    opt = FalkonOptions(never_store_kernel=False, store_kernel_d_threshold=Xtr.shape[1] - 1)
+    flk = cls(kernel=GaussianKernel(20.0), penalty=1e-6, M=Xtr.shape[0] // 2, seed=10, options=opt, maxiter=10)
+    assert flk._can_store_knm(Xtr.to(dev), Xtr[:400].to(dev))
+    flk.fit(Xtr, Ytr, Xts=Xts, Yts=Yts)
+    assert flk.predict(Xts).shape == (Yts.shape[0], 1)
+    ts_err, tr_err = _rmse(flk.predict(Xts), Yts)[0], _rmse(flk.predict(Xtr), Ytr)[0]
+    assert tr_err < ts_err < 2.5
+    plain = cls(kernel=GaussianKernel(20.0), penalty=1e-6, M=Xtr.shape[0] // 2, seed=10, maxiter=10,
+                options=FalkonOptions(never_store_kernel=True, store_kernel_d_threshold=Xtr.shape[1] - 1))
+    assert not plain._can_store_knm(Xtr.to(dev), Xtr[:400].to(dev))
+    plain.fit(Xtr, Ytr)
+    # (penalty 1e-6, ten iterations: the coefficients feel the different summation order of the two routes)
+    a, b = flk.alpha_.cpu().numpy(), plain.alpha_.cpu().numpy()
+    np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-6 * np.abs(b).max())
