@@ -13,12 +13,12 @@ import numpy as np
 import torch
 
 from .center_selection import CenterSelector, UniformSelector
-from .optim import FalkonConjugateGradient
+from .optim import ConjugateGradient, FalkonConjugateGradient
 from .options import FalkonOptions
-from .preconditioner import FalkonPreconditioner
+from .preconditioner import FalkonPreconditioner, LogisticPreconditioner
 from .utils.helpers import check_same_dtype
 
-__all__ = ("Falkon", "InCoreFalkon")
+__all__ = ("Falkon", "InCoreFalkon", "LogisticFalkon")
 
 try:                                    # keep sklearn's get_params / set_params / clone when it is there
     from sklearn.base import BaseEstimator as _Base
@@ -151,3 +151,75 @@ class InCoreFalkon(Falkon):
         if self.alpha_ is not None and X.device != self.alpha_.device:
             raise ValueError(f"X must be on device {self.alpha_.device}")
         return super().predict(X)
+
+
+class LogisticFalkon(Falkon):
+    """Kernel classification with a generalised self-concordant loss by Newton's method, every step a preconditioned CG
+    whose operator is two ``kernel.mmv`` (falkon/models/logistic_falkon.py:17-271): ``penalty_list[i]`` and
+    ``iter_list[i]`` are the regularisation and the CG iterations of Newton step i."""
+
+    def __init__(self, kernel, penalty_list, iter_list, loss, M: int,
+                 center_selection: Union[str, CenterSelector] = "uniform", seed: Optional[int] = None,
+                 error_fn: Optional[Callable] = None, error_every: Optional[int] = 1,
+                 options: Optional[FalkonOptions] = None):
+        super().__init__(kernel, penalty_list, M, center_selection=center_selection, maxiter=iter_list, seed=seed,
+                         error_fn=error_fn, error_every=error_every, options=options)
+        if len(iter_list) != len(penalty_list):
+            raise ValueError(f"Iteration list must be of same length as penalty list "
+                             f"(found {len(iter_list)} and {len(penalty_list)})")
+        self.penalty_list, self.iter_list, self.loss = penalty_list, iter_list, loss
+
+    def fit(self, X: torch.Tensor, Y: torch.Tensor, Xts: Optional[torch.Tensor] = None,
+            Yts: Optional[torch.Tensor] = None):
+        if X.shape[0] != Y.shape[0]:
+            raise ValueError(f"X and Y must have the same number of samples (found {X.shape[0]} and {Y.shape[0]})")
+        if Y.dim() == 1:
+            Y = Y.unsqueeze(1)
+        if not check_same_dtype(X, Y):
+            raise TypeError("X and Y must have the same data-type.")
+        dev = X.device if X.is_cuda else self._device()
+        self.alpha_ = self.ny_points_ = None
+        self.fit_times_, self.val_errors_ = [0.0], []
+        t_s, elapsed = time.time(), 0.0
+        with torch.inference_mode():
+            ny_X, ny_Y = self.center_selection.select(X, Y)
+            Xd, Yd, Cd, Yc = X.to(dev), Y.to(dev), ny_X.to(dev), ny_Y.to(dev)
+            beta = torch.zeros(Cd.shape[0], 1, dtype=X.dtype, device=dev)
+            optim = ConjugateGradient(self.options)
+            precond = LogisticPreconditioner(self.kernel, self.loss, self.options)
+            self.precond = precond
+            for step, penalty in enumerate(self.penalty_list):
+                precond.init(Cd, Yc, beta, penalty, X.shape[0])
+                grad, f_vals = self.loss.knmp_grad(Xd, Cd, Yd, precond.invT(beta), opt=self.options)
+                grad_p = precond.invAt(precond.invTt(grad).add_(penalty * beta))
+
+                def newton_operator(sol, f_vals=f_vals, penalty=penalty):
+                    inner = precond.invA(sol)
+                    hess = self.loss.knmp_hess(Xd, Cd, Yd, f_vals, precond.invT(inner), opt=self.options)
+                    return precond.invAt(precond.invTt(hess).add_(inner.mul_(penalty)))
+
+                direction = optim.solve(None, grad_p, newton_operator, self.iter_list[step])
+                beta -= precond.invA(direction)
+                torch.cuda.synchronize(dev)
+                elapsed += time.time() - t_s
+                if self.error_fn is not None and self.error_every is not None:
+                    self._logistic_callback(step, beta, elapsed, Xd, Yd, Xts, Yts, Cd)
+                t_s = time.time()
+            self.alpha_, self.ny_points_ = precond.invT(beta).to(X.device), ny_X
+        return self
+
+    def _logistic_callback(self, it, beta, train_time, X, Y, Xts, Yts, ny_points):
+        self.fit_times_.append(self.fit_times_[0] + train_time)
+        if it % self.error_every != 0:
+            print(f"Iteration {it:3d} - Elapsed {self.fit_times_[-1]:.2f}s", flush=True)
+            return
+        on_val = Xts is not None and Yts is not None
+        pred = self._predict(Xts if on_val else X, ny_points, self.precond.invT(beta))
+        true = (Yts if on_val else Y).to(pred.device)
+        err, name = self.error_fn(true, pred), "error"
+        if isinstance(err, tuple) and len(err) == 2:
+            err, name = err
+        kind = "validation" if on_val else "training"
+        print(f"Iteration {it:3d} - Elapsed {self.fit_times_[-1]:.2f}s - {kind} loss "
+              f"{torch.mean(self.loss(true, pred)).item():.4f} - {kind} {name} {float(err):.4f} ", flush=True)
+        self.val_errors_.append(err)

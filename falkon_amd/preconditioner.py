@@ -19,7 +19,7 @@ import torch
 
 from .options import FalkonOptions
 
-__all__ = ("FalkonPreconditioner",)
+__all__ = ("FalkonPreconditioner", "LogisticPreconditioner")
 
 TRSV_BLOCK = 2048        # rows per diagonal block of the blocked triangular solves
 TRSV_MIN_SIZE = 4096     # smaller factors go to torch.linalg.solve_triangular directly
@@ -220,3 +220,33 @@ class FalkonPreconditioner:
     def apply_t(self, v):
         """A^-T T^-T v."""
         return self.invAt(self.invTt(v))
+
+
+class LogisticPreconditioner(FalkonPreconditioner):
+    """The preconditioner of one Newton step of Logistic Falkon (falkon/preconditioner/logistic_preconditioner.py:17-350):
+    ``T = chol(K_MM + eps*M*I)`` once, then for every step ``A = chol(T W T^T / N + penalty*I)`` with
+    ``W = diag(l''(Y_M, T^T beta))``, the loss' curvature at the centres for the current iterate (``T^T beta`` are
+    the function values at the centres, since the coefficients are ``T^-1 beta``)."""
+
+    def __init__(self, kernel, loss, opt: Optional[FalkonOptions] = None):
+        super().__init__(0.0, kernel, opt)
+        self.loss = loss
+
+    def init(self, X: torch.Tensor, Y: torch.Tensor, alpha: torch.Tensor, penalty: float, N: int) -> None:
+        if Y.shape[1] != 1:
+            raise ValueError("Logistic preconditioner can only deal with 1D outputs.")
+        M = X.shape[0]
+        with torch.inference_mode():
+            if self.LT is None:                                         # first step only
+                C = self.kernel(X, X, opt=self.params)
+                C.diagonal().add_(self.params.pc_epsilon(C.dtype) * M)
+                self.LT = _cholesky_lower_(C)
+                self._T = _BlockedTriangular(self.LT)
+            at_centres = self.LT @ alpha.to(self.LT.dtype)              # T^T beta
+            root = self.loss.ddf(Y.to(self.LT.dtype), at_centres).reshape(-1, 1).sqrt()
+            G = _gram_of_lower_factor(self.LT * root)                   # T W T^T, lower triangle
+            G.mul_(1.0 / N)                                             # 1/N here, not 1/M (logistic_preconditioner.py:146)
+            G.diagonal().add_(penalty)
+            self.LA = _cholesky_lower_(G)
+            self._A = _BlockedTriangular(self.LA)
+            self._lambda = penalty
