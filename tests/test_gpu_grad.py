@@ -169,3 +169,73 @@ def test_gradients_with_centres_from_the_data(dev, name):
         shape = (g_64.shape[0], -1)
         assert torch.isfinite(g_gpu).all()
         assert rel_err(g_gpu.reshape(shape), g_64.reshape(shape)) <= max(1e-5, rel_err(g_cpu.reshape(shape), g_64.reshape(shape)))
+
+
+def _hopt_data(dtype, n=1000, d=10):
+    """The synthetic regression set of the reference's hyperparameter-optimisation tests
+    (falkon/tests/test_hopt.py:31-50): linear targets with noise, standardised, 80 % for training."""
+    g = torch.Generator().manual_seed(12)
+    X = torch.randn((n, d), dtype=dtype, generator=g)
+    Y = X @ torch.arange(d, dtype=dtype).reshape(-1, 1) + torch.randn((n, 1), dtype=dtype, generator=g) * 0.3
+    ntr = int(n * 0.8)
+    xm, xs, ym, ys = X[:ntr].mean(0, keepdim=True), X[:ntr].std(0, keepdim=True), Y[:ntr].mean(), Y[:ntr].std()
+    X, Y = (X - xm) / xs, (Y - ym) / ys
+    return X[:ntr], Y[:ntr], X[ntr:], Y[ntr:]
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_gradient_descent_on_a_holdout_objective(dev, dtype):
+    """What the backward pass is for (the reference's ``falkon.hopt`` objectives, e.g.
+    falkon/hopt/objectives/exact_objectives/holdout.py:37-83): lengthscales (one per feature), centres and penalty
+    are optimised by Adam on the hold-out error of the Nystroem estimator, every kernel matrix and its gradient
+    coming from the MI355X kernels.  The hold-out error must drop, and so must the error on unseen data."""
+    Xtr, Ytr, Xts, Yts = (a.to(dev) for a in _hopt_data(dtype))
+    fit_idx, val_idx = torch.arange(0, 600, device=dev), torch.arange(600, 800, device=dev)
+    kernel = GaussianKernel(torch.full((10,), 5.0, dtype=torch.float32).requires_grad_())
+    centres = Xtr[:100].clone().requires_grad_()
+    log_penalty = torch.tensor(np.log(1e-3), dtype=dtype, device=dev, requires_grad=True)
+
+    def coefficients(Xf, Yf):
+        kmn, kmm = kernel(centres, Xf), kernel(centres, centres)
+        reg = torch.exp(log_penalty) * Xf.shape[0]
+        lhs = kmn @ kmn.T + reg * kmm + 1e-6 * reg * torch.eye(100, dtype=dtype, device=dev)
+        return torch.linalg.solve(lhs, kmn @ Yf)
+
+    def holdout():
+        alpha = coefficients(Xtr[fit_idx], Ytr[fit_idx])
+        return torch.mean((Ytr[val_idx] - kernel(Xtr[val_idx], centres) @ alpha) ** 2)
+
+    def test_error():
+        with torch.no_grad():
+            return float(torch.mean((Yts - kernel(Xts, centres) @ coefficients(Xtr, Ytr)) ** 2))
+
+    optimiser = torch.optim.Adam([kernel.sigma, centres, log_penalty], lr=0.1)
+    first, before = None, test_error()
+    for _ in range(40):
+        optimiser.zero_grad()
+        loss = holdout()
+        loss.backward()
+        assert all(torch.isfinite(p.grad).all() for p in (kernel.sigma, centres, log_penalty))
+        optimiser.step()
+        first = float(loss) if first is None else first
+    assert float(holdout()) < 0.5 * first
+    assert test_error() < 0.7 * before
+
+
+def test_gradient_descent_through_the_kernel_vector_product(dev):
+    """The same through ``kernel.mmv`` (K is never stored, forward or backward): lengthscale, centres and
+    coefficients of ``f(x) = K(x, C) v`` are fitted to the training targets by Adam; the squared error must fall by
+    an order of magnitude."""
+    Xtr, Ytr, _, _ = (a.to(dev) for a in _hopt_data(torch.float32))
+    kernel = GaussianKernel(torch.tensor([4.0]).requires_grad_())
+    centres = Xtr[:64].clone().requires_grad_()
+    v = torch.zeros(64, 1, device=dev, requires_grad=True)
+    optimiser = torch.optim.Adam([kernel.sigma, centres, v], lr=0.05)
+    losses = []
+    for _ in range(150):
+        optimiser.zero_grad()
+        loss = torch.mean((kernel.mmv(Xtr, centres, v) - Ytr) ** 2)
+        loss.backward()
+        optimiser.step()
+        losses.append(float(loss))
+    assert losses[-1] < 0.1 * losses[0] and np.isfinite(losses).all()
