@@ -338,7 +338,7 @@ def main():
     # one launch of the product kernel evaluates all N*M pairs once: (2d+4) flop per kernel value + 2T to contract
     flop_per_launch = N * M * (2 * d + 4 + 2 * T)
     kern_ms = tot_ms.value / max(launches.value, 1)
-    achieved = flop_per_launch / (kern_ms * 1e-3) / 1e12
+    achieved = flop_per_launch / (kern_ms * 1e-3) / 1e12 if kern_ms > 0 else 0.0
     res = {
         "metric": f"{'dfmmv' if args.op == 'dmmv' else 'fmmv'} kernel-entries/sec (N*M*T/s) {'fp32' if args.dtype == 'f32' else 'fp64'}, 1 MI355X",
         "value": value, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -364,7 +364,15 @@ def main():
     if args.op == "dmmv":
         # the conservative count: one kernel evaluation per pair, as if K were stored between the two products
         res["single_evaluation_flop_frac"] = (N * M * (2 * d + 4 + 4 * T)) / (elapsed / args.steps) / 1e12 / peak
-    if split:
+    if launches.value == 0:
+        # many right-hand sides: the drivers stored blocks of K (kernel-matrix kernel + rocBLAS GEMMs), no product
+        # kernel ran and K was evaluated once per step: the rate is that flop count (E(d) + 2T or 4T per pair) over
+        # the step time
+        once = res.get("single_evaluation_flop_frac", res["whole_step_flop_frac"])
+        res["roofline"] = {"bound": "mfma", "achieved": once * peak, "peak": peak, "unit": "TFLOP/s", "frac": once,
+                           "traffic": None, "kernel": "kernel-matrix kernel + rocBLAS GEMMs on stored blocks of K",
+                           "launches_per_step": 0.0, "avg_launch_ms": None, "flop_per_launch": None}
+    if split and launches.value > 0:
         res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch,
                                               MEASURED_TRAFFIC_BYTES_BF16X3.get(args.workload)),
                                launches_per_step=launches.value / args.steps)
