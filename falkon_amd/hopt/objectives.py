@@ -13,8 +13,8 @@ the hat matrix of the Nystroem estimator is H = C^T C, its coefficients are alph
     tr(H) = |C|_F^2,   diag(H) = column sums of C^2,   H Y = C^T (C Y),   Y^T (I - H) Y = |Y|^2 - |C Y|^2,
     1/2 log det(B) = sum(log(diag(L_B))),   tr(K_nn - Q_nn) = tr(K_nn) - v * tr(A A^T)   (Q_nn the Nystroem kernel).
 
-The stochastic objective of the reference (trace estimators on top of ``kernel.mmv``,
-falkon/hopt/objectives/stoch_objectives/stoch_new_compreg.py) is not part of this module.
+``StochasticNystromCompReg`` (at the end) is the matrix-free counterpart of ``NystromCompReg``: trace estimators and
+the Falkon solver on top of ``kernel.mmv`` and its backward pass.
 """
 from typing import Dict, Optional
 
@@ -23,7 +23,8 @@ import torch.nn.functional as F
 
 from ..kernels.diff_kernel import DiffKernel
 
-__all__ = ("PositiveTransform", "HyperoptObjective", "HoldOut", "GCV", "LOOCV", "SGPR", "CompReg", "NystromCompReg")
+__all__ = ("PositiveTransform", "HyperoptObjective", "HoldOut", "GCV", "LOOCV", "SGPR", "CompReg", "NystromCompReg",
+           "StochasticNystromCompReg")
 
 
 class PositiveTransform:
@@ -218,3 +219,66 @@ class NystromCompReg(HyperoptObjective):
         trace = gap * data_fit / (f.variance * X.shape[0])
         self._remember(X, Y, **{"d_eff": deff, "data_fit": data_fit, "trace": trace})
         return deff + data_fit + trace
+
+
+class StochasticNystromCompReg(HyperoptObjective):
+    r"""``NystromCompReg`` without any n x m matrix: traces by Hutchinson's estimator, linear systems by the Falkon solver,
+    every kernel product a ``kernel.mmv`` (the reference's objective of the same name,
+    falkon/hopt/objectives/stoch_objectives/stoch_new_compreg.py:21-505, which hand-writes the backward pass).
+
+    With S = (K_mn K_nm + v K_mm)^-1, random vectors Z (n x t, standard normal) and ZY = [Z, Y]:
+
+        tr(H) ~ 1/t sum_j z_j^T K_nm S K_mn z_j,      Y^T (I - H) Y = |Y|^2 - Y^T K_nm S K_mn Y,
+        tr(Q_nn) ~ 1/t sum_j |L^-1 K_mn z_j|^2         (K_mm = L L^T).
+
+    The quadratic forms ``b^T S b`` (b = K_mn z, depending on the hyperparameters through K_mn and S) are differentiated
+    without differentiating the solver: with u = S b from the Falkon solver held fixed,
+    ``2 u^T b - u^T (K_mn K_nm + v K_mm) u`` has the value and the gradient of ``b^T S b`` at the current
+    hyperparameters, and its pieces are kernel-vector products whose backward pass is the MI355X one
+    (falkon_amd/mmv_ops/fmmv_grad.py).  The solver runs ``flk_maxiter`` iterations to ``flk_opt.cg_tolerance``."""
+
+    def __init__(self, kernel, centers_init, penalty_init, opt_centers: bool, opt_penalty: bool, flk_opt=None,
+                 flk_maxiter: int = 10, num_trace_est: int = 20, centers_transform=None, pen_transform=None):
+        super().__init__(kernel, centers_init, penalty_init, opt_centers, opt_penalty, centers_transform, pen_transform)
+        from ..options import FalkonOptions
+        self.flk_opt = flk_opt or FalkonOptions()
+        self.flk_maxiter, self.num_trace_est = flk_maxiter, num_trace_est
+        self.trace_vectors: Optional[torch.Tensor] = None    # fixed Z (n x t) instead of a fresh draw per call
+
+    def _solve(self, X, centres, rhs, penalty: float) -> torch.Tensor:
+        """(K_mn K_nm + penalty n K_mm)^-1 K_mn rhs with the preconditioned CG of the estimator."""
+        from ..optim import FalkonConjugateGradient
+        from ..preconditioner import FalkonPreconditioner
+        kernel = self.kernel.detach()                          # the solver is not differentiated
+        with torch.inference_mode():
+            precond = FalkonPreconditioner(penalty, kernel, self.flk_opt)
+            precond.init(centres)
+            solver = FalkonConjugateGradient(kernel, precond, self.flk_opt)
+            coeff = precond.apply(solver.solve(X, centres, rhs, penalty, None, self.flk_maxiter))
+        return coeff.clone()                                   # an ordinary tensor, usable in the graph below
+
+    def forward(self, X, Y):
+        n, t = X.shape[0], self.num_trace_est
+        Z = self.trace_vectors if self.trace_vectors is not None else torch.randn(n, t, dtype=X.dtype, device=X.device)
+        t = Z.shape[1]
+        ZY = torch.cat([Z, Y], dim=1)
+        centres, variance = self.centers, self.penalty * n
+        U = self._solve(X.detach(), centres.detach(), ZY, float(self.penalty.detach()))
+        B = self.kernel.mmv(centres, X, ZY)                    # K_mn [Z, Y], differentiable
+        KU = self.kernel.mmv(X, centres, U)                    # K_nm U
+        kmm = self.kernel(centres, centres)
+        quad = 2 * (U * B).sum(0) - KU.square().sum(0) - variance * (U * (kmm @ U)).sum(0)
+        deff = quad[:t].sum() / t
+        data_fit = Y.square().sum() - quad[t:].sum()
+        half = torch.linalg.solve_triangular(_jittered_cholesky(kmm), B[:, :t], upper=False)
+        gap = self.kernel(X, X, diag=True).sum() - half.square().sum() / t
+        trace = gap * data_fit / (variance * n)
+        self._remember(X, Y, **{"d_eff": deff, "data_fit": data_fit, "trace": trace})
+        return deff + data_fit + trace
+
+    def predict(self, X):
+        if self.x_train is None or self.y_train is None:
+            raise RuntimeError("Call forward at least once before calling predict.")
+        with torch.no_grad():
+            alpha = self._solve(self.x_train, self.centers.detach(), self.y_train, float(self.penalty.detach()))
+            return self.kernel.detach().mmv(X, self.centers.detach(), alpha)

@@ -118,3 +118,53 @@ def test_reference_exact_objectives_optimise(dev, cls):
         optimiser.step()
     after = float(torch.mean((model.predict(Xts) - Yts) ** 2))
     assert np.isfinite(after) and after < max(before, 0.05)
+
+
+def test_stochastic_objective_equals_the_exact_one_for_exact_traces(dev):
+    """With the Hutchinson vectors replaced by sqrt(n) e_1 .. sqrt(n) e_n the trace estimates are exact, and with the
+    solver run to convergence the matrix-free objective and its gradient (lengthscales, centres, penalty) must equal
+    those of ``NystromCompReg``, whose gradient is plain autograd through the factorised formula."""
+    from falkon_amd import FalkonOptions
+    from falkon_amd.hopt import StochasticNystromCompReg
+    X, Y, C, sigma, penalty = _small_problem(dev, n=80, m=10)
+    Xg, Yg = X.to(dev), Y.to(dev)
+    exact = _build(NystromCompReg, C, sigma, penalty, dev)
+    stoch = _build(StochasticNystromCompReg, C, sigma, penalty, dev, flk_maxiter=300,
+                   flk_opt=FalkonOptions(cg_tolerance=1e-13, pc_epsilon_64=1e-8, cg_full_gradient_every=5))
+    stoch.trace_vectors = (np.sqrt(80.0) * torch.eye(80, dtype=torch.float64)).to(dev)
+    values, grads = [], []
+    for model in (exact, stoch):
+        loss = model(Xg, Yg)
+        loss.backward()
+        values.append(loss.item())
+        grads.append([model.kernel.sigma.grad.cpu(), model.centers_.grad.cpu(), model.penalty_.grad.cpu()])
+    assert abs(values[0] - values[1]) < 1e-6 * abs(values[0])
+    for a, b in zip(*grads):
+        np.testing.assert_allclose(b.double().numpy(), a.double().numpy(), rtol=2e-4, atol=1e-6 * float(a.abs().max()))
+
+
+def test_reference_stochastic_objective_optimises(dev):
+    """falkon/tests/test_hopt.py:73-115: fp32, 100 centres, 10 trace vectors, 100 solver iterations to 1e-4; 60 Adam
+    steps; the test error must end far below the reference's bound of 60 (targets are standardised)."""
+    from falkon_amd import FalkonOptions
+    from falkon_amd.hopt import StochasticNystromCompReg
+    torch.manual_seed(12)
+    n, d, dtype = 1000, 10, torch.float32
+    X = torch.randn((n, d), dtype=dtype)
+    Y = X @ torch.arange(d, dtype=dtype).reshape(-1, 1) + torch.randn((n, 1), dtype=dtype) * 0.1
+    ntr = int(n * 0.8)
+    xm, xs, ym, ys = X[:ntr].mean(0, keepdim=True), X[:ntr].std(0, keepdim=True), Y[:ntr].mean(), Y[:ntr].std()
+    X, Y = ((X - xm) / xs).to(dev), ((Y - ym) / ys).to(dev)
+    kernel = GaussianKernel(sigma=torch.tensor([5.0] * d, dtype=torch.float32, requires_grad=True))
+    model = StochasticNystromCompReg(kernel, X[:100].clone(), torch.tensor(1e-1, dtype=dtype, device=dev), True, True,
+                                     flk_opt=FalkonOptions(pc_epsilon_32=1e-4, cg_tolerance=1e-4), flk_maxiter=100,
+                                     num_trace_est=10)
+    optimiser = torch.optim.Adam(model.parameters(), lr=0.1)
+    for _ in range(60):
+        optimiser.zero_grad()
+        loss = model(X[:ntr], Y[:ntr])
+        assert torch.isfinite(loss)
+        loss.backward()
+        optimiser.step()
+    ts_err = float(torch.mean((model.predict(X[ntr:]) - Y[ntr:]) ** 2))
+    assert ts_err < 0.5
