@@ -246,6 +246,9 @@ def main():
                     help="f32 (the headline): fp32 MFMA.  bf16x3: the opt-in mode that forms x.c on the bf16 matrix cores "
                          "from an exact three-way bfloat16 split of the fp32 rows (fp32 accuracy; fp32 data); "
                          "its roofline is priced against the bf16 MFMA peak on the flops it executes")
+    ap.add_argument("--stored-blocks", action="store_true",
+                    help="FalkonOptions(dmmv_stored_blocks=True): dfmmv beyond 64 features through stored blocks of K "
+                         "(not the headline path, which never materialises K)")
     ap.add_argument("--rhs", type=int, default=0, metavar="T",
                     help="right-hand sides instead of the configuration's own number (not a headline workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true",
@@ -275,7 +278,7 @@ def main():
 
     from falkon_amd import FalkonOptions, GaussianKernel, LaplacianKernel, MaternKernel, _backend
     lib = _backend.load()                            # raises if the HIP library is missing
-    kopt = FalkonOptions(bf16x3_cross_term=args.cross_term == "bf16x3")
+    kopt = FalkonOptions(bf16x3_cross_term=args.cross_term == "bf16x3", dmmv_stored_blocks=args.stored_blocks)
     def make_kernel_with(o):
         return {"gaussian": lambda s: GaussianKernel(s, opt=o), "laplacian": lambda s: LaplacianKernel(s, opt=o),
                 "matern32": lambda s: MaternKernel(s, 1.5, opt=o), "matern52": lambda s: MaternKernel(s, 2.5, opt=o)}[args.kernel]

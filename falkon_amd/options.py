@@ -40,6 +40,8 @@ class BaseOptions:
     memory_slack: float = 0.9                         # fraction of the free device memory a call may plan with
     bf16x3_cross_term: bool = False                   # not in the reference: fp32 products form x.c on the bf16 matrix
                                                       # cores from an exact 3-way bfloat16 split (fp32 accuracy)
+    dmmv_stored_blocks: bool = False                  # not in the reference's options: K^T(K v + w) beyond 64 features
+                                                      # evaluates K once, into stored blocks, whatever T (see fmmv.py)
 
 
 @dataclass

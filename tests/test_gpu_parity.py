@@ -605,3 +605,20 @@ def test_many_right_hand_sides_through_stored_blocks(dev, dtype, n, m, d, t, mon
     host = k.dmmv(X, C, v, w)
     assert host.device.type == "cpu"
     check_parity(host, *ref_dmmv, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_dmmv_stored_blocks_option(dev, dtype):
+    """``FalkonOptions(dmmv_stored_blocks=True)``: K^T(K v + w) beyond 64 features through stored blocks of K for any
+    number of right-hand sides; same tolerances; at 64 features or fewer the option changes nothing."""
+    opt = FalkonOptions(dmmv_stored_blocks=True)
+    for (n, m, d, t) in ((600, 257, 100, 1), (513, 300, 784, 10)):
+        X, C, v, w = _rand(n, d, m, t, dtype, seed=n + d, scale=0.5)
+        sigma = 0.6 * np.sqrt(d)
+        Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+        got = GaussianKernel(sigma, opt=opt).dmmv(Xg, Cg, vg, wg)
+        Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+        check_parity(got, mmv_ref.fdmmv_ref(X, C, v, w, sigma), mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), TOL[dtype])
+        assert rel_err(got, GaussianKernel(sigma).dmmv(Xg, Cg, vg, wg)) < TOL[dtype]
+    X, C, v, w = (a.to(dev) for a in _rand(500, 28, 200, 2, dtype, seed=1))
+    assert torch.equal(GaussianKernel(3.0, opt=opt).dmmv(X, C, v, w), GaussianKernel(3.0).dmmv(X, C, v, w))
