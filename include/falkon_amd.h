@@ -123,6 +123,9 @@ int flk_gauss_mmv_packed(const void *packed_a, int64_t n_a, const void *packed_b
  * Both pack X1 and X2 into the workspace, never materialise K, and leave the
  * inputs untouched.  The workspace must hold at least the number of bytes the
  * matching *_workspace_bytes call returns.
+ * A NaN or an infinity in a row of X1 or X2 gives NaN in every result that row
+ * enters, as in the reference (falkon/kernels/distance_kernel.py:88-101), although
+ * the kernels clamp the kernel value: the rows' half norms carry the information.
  */
 size_t flk_gauss_fmmv_workspace_bytes(int64_t n, int64_t m, int64_t d, int64_t t, int dtype);
 
