@@ -278,3 +278,26 @@ def test_torch_ops_are_registered_and_refuse_host_tensors():
         torch.ops.falkon.kernel_fmmv(X, X, torch.ones(1), torch.randn(4, 1), torch.empty(4, 1))
     with pytest.raises(RuntimeError, match="GPU only"):
         torch.ops.falkon.kernel_fdmmv(X, X, torch.ones(1), torch.randn(4, 1), None, torch.empty(4, 1))
+
+
+def test_stored_block_route_rules(monkeypatch):
+    """When the drivers store blocks of K instead of re-evaluating it per pass (many right-hand sides), how large
+    the blocks are, and the options that switch the route off or on."""
+    import importlib
+    drv = importlib.import_module("falkon_amd.mmv_ops.fmmv")
+    opt = FalkonOptions()
+    f32, f64 = torch.float32, torch.float64
+    # one pass of the product kernels: never; two passes beyond 64 features; four (fp32) / five (fp64) at small d
+    assert not drv._explicit_blocks_pay(784, 16, f32, opt) and drv._explicit_blocks_pay(784, 17, f32, opt)
+    assert not drv._explicit_blocks_pay(28, 96, f32, opt) and drv._explicit_blocks_pay(28, 97, f32, opt)
+    assert not drv._explicit_blocks_pay(40, 64, f32, opt) and drv._explicit_blocks_pay(40, 65, f32, opt)
+    assert not drv._explicit_blocks_pay(28, 64, f64, opt) and drv._explicit_blocks_pay(28, 65, f64, opt)
+    assert drv._explicit_blocks_pay(100, 17, f64, opt)
+    assert not drv._explicit_blocks_pay(784, 1000, f32, FalkonOptions(never_store_kernel=True))
+    # block rows: within the block size, within half of what the budget leaves, nothing below 32 rows
+    monkeypatch.setattr(drv, "usable_gpu_memory", lambda dev, cap, slack, enough=float("inf"): 64 * 2**30)
+    rows = drv._explicit_block_rows(10**6, 10_000, 784, 256, 4, None, opt, upload_bytes=0)
+    assert 32 <= rows <= 10**6 and rows * (10_000 + 512 + 3 * 784) * 4 <= drv._EXPLICIT_BLOCK_BYTES
+    assert drv._explicit_block_rows(500, 10_000, 784, 256, 4, None, opt, upload_bytes=0) == 500
+    monkeypatch.setattr(drv, "usable_gpu_memory", lambda dev, cap, slack, enough=float("inf"): 2**20)
+    assert drv._explicit_block_rows(10**6, 10_000, 784, 256, 4, None, opt, upload_bytes=0) == 0
