@@ -38,14 +38,17 @@ def main():
     ap.add_argument("--d", type=int, default=256)
     ap.add_argument("--reps", type=int, default=5)
     ap.add_argument("--resident", action="store_true", help="also time the call with A (and the result) on the GPU")
+    ap.add_argument("--bf16x3", action="store_true",
+                    help="FalkonOptions(bf16x3_cross_term=True): serves the fp32 evaluation beyond 64 features")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("mm_timings: no GPU visible")
     A = torch.randn(args.n, args.d, dtype=torch.float32, generator=torch.Generator().manual_seed(0)).pin_memory()
     for no_single_kernel in (True, False):
-        kernel = GaussianKernel(5.0, opt=FalkonOptions(no_single_kernel=no_single_kernel))
+        kernel = GaussianKernel(5.0, opt=FalkonOptions(no_single_kernel=no_single_kernel,
+                                                       bf16x3_cross_term=args.bf16x3))
         kernel(A[:1000], A[:1000])                           # first call: library load
-        rec = {"exp": "kernel matrix", "N": args.n, "D": args.d, "no_single_kernel": no_single_kernel,
+        rec = {"exp": "kernel matrix" + (" (bf16x3 cross term)" if args.bf16x3 else ""), "N": args.n, "D": args.d, "no_single_kernel": no_single_kernel,
                "seconds": _best_of(lambda: kernel(A, A), args.reps)}
         if args.resident:
             Ag = A.cuda()

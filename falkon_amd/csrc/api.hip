@@ -530,6 +530,32 @@ static int fdmmv_split_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, in
                             st);
 }
 
+// bf16x3 mode of the kernel matrix: beyond the register-resident feature counts, fp32 arithmetic only (the fp64
+// evaluation of fp32 data, compute_f64, keeps its own kernels).
+static bool fmm_split_applies(int64_t d, int dtype, int compute_f64) {
+    return dtype == FLK_F32_BF16X3 && !compute_f64 && d > kSmallMaxD;
+}
+
+static int fmm_split_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
+                          int64_t x2_rs, int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, void *out,
+                          int64_t out_rs, int64_t out_cs, void *ws, size_t ws_bytes, hipStream_t st) {
+    if (n < 0 || m < 0 || d < 1) return fail(FLK_EINVAL, "bad shape");
+    if (d > flk_max_d(0)) return fail(FLK_EUNSUPPORTED, "more than %lld features", (long long)flk_max_d(0));
+    int rc;
+    if ((rc = check_matrix("out", out, n, m, out_rs, out_cs))) return rc;
+    if (n == 0 || m == 0) return FLK_OK;
+    const size_t need = split_packed_bytes(n, d) + split_packed_bytes(m, d);
+    if (ws_bytes < need || ws == nullptr)
+        return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+    void *p1 = ws, *p2 = (char *)ws + split_packed_bytes(n, d);
+    if ((rc = pack_split_impl(kf, "X1", X1, n, d, x1_rs, x1_cs, sigma, n_sigma, p1, st))) return rc;
+    if ((rc = pack_split_impl(kf, "X2", X2, m, d, x2_rs, x2_cs, sigma, n_sigma, p2, st))) return rc;
+    SplitView P1 = split_view(p1, n, d), P2 = split_view(p2, m, d);
+    // lanes run along the B operand: make that the dimension of out with the unit stride
+    if (out_cs == 1 || m == 1) return launch_fmm_split_large(kf, P1, P2, (float *)out, out_rs, st);
+    return launch_fmm_split_large(kf, P2, P1, (float *)out, out_cs, st);
+}
+
 }  // namespace flk
 
 using namespace flk;
@@ -691,7 +717,8 @@ int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, con
 }
 
 size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype, int compute_f64) {
-    if (n < 0 || m < 0 || d < 1 || d > flk_max_d(dtype) || !known_dtype(dtype, false)) return 0;
+    if (n < 0 || m < 0 || d < 1 || d > flk_max_d(dtype) || !known_dtype(dtype, true)) return 0;
+    if (fmm_split_applies(d, dtype, compute_f64)) return split_packed_bytes(n, d) + split_packed_bytes(m, d);
     if (dtype == FLK_F64 || compute_f64) return packed_bytes<double>(n, d) + packed_bytes<double>(m, d);
     return packed_bytes<float>(n, d) + packed_bytes<float>(m, d);
 }
@@ -703,6 +730,10 @@ int flk_kernel_fmm(int kernel, const void *X1, int64_t n, int64_t x1_rs, int64_t
     g_err[0] = 0;
     FLK_CHECK_KERNEL(kernel);
     hipStream_t st = (hipStream_t)stream;
+    if (fmm_split_applies(d, dtype, compute_f64))
+        return fmm_split_impl(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs, out_cs,
+                              workspace, workspace_bytes, st);
+    if (dtype == FLK_F32_BF16X3) dtype = FLK_F32;      // where the mode has no kernel of its own: the fp32 kernels
     if (dtype == FLK_F64)
         return fmm_impl<double, double>(kernel, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, out, out_rs,
                                         out_cs, workspace, workspace_bytes, st);

@@ -37,11 +37,16 @@ static __device__ __forceinline__ void wg_barrier() {
 }
 
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
-template <int WVA, int WVB, int WA_FR, int WB_FR, int TT, int KF>
+// STORE: the kernel matrix instead of the product: entry (a, b) goes to kout[a * kout_ld + b] (then TT = 1, tcols = 0,
+// vecp is not read and partial not written); hnA / hnB are the operands' fp32 half norms, read only to give the rows
+// that hold a NaN or an infinity their NaN back (the clamps of the kernel functions would hide it).
+template <int WVA, int WVB, int WA_FR, int WB_FR, int TT, int KF, bool STORE = false>
 __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   // two waves per SIMD either way
     mmv_split_large_kernel(const uintx4 *__restrict__ PA, const float *__restrict__ vecp, int64_t vec_ld, int tcols,
                            const uintx4 *__restrict__ PB, int64_t na_blocks, int64_t nb_blocks, int ks_count,
-                           int64_t a_tiles_per_chunk, float *__restrict__ partial, int64_t nb_pad, bool y_fastest) {
+                           int64_t a_tiles_per_chunk, float *__restrict__ partial, int64_t nb_pad, bool y_fastest,
+                           float *__restrict__ kout = nullptr, int64_t kout_ld = 0, int64_t n_a = 0, int64_t n_b = 0,
+                           const float *__restrict__ hnA = nullptr, const float *__restrict__ hnB = nullptr) {
     typedef LTraits<float> TR;
     constexpr int kWaves = WVA * WVB, kThreads = 64 * kWaves;
     constexpr int NAB = WVA * WA_FR, NBB = WVB * WB_FR;          // blocks of 32 rows per tile
@@ -222,7 +227,34 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         }
 
         // epilogue: K = kernel_value(acc) ; out[q][t] += K * vec[i][t]
-        if constexpr (!kMfmaEpi) {
+        if constexpr (STORE) {
+#pragma unroll
+            for (int p = 0; p < WA_FR; p++) {
+                const int64_t ablk = ablk0 + wa * WA_FR + p;
+                if (ablk < na_blocks) {
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const int64_t row0 = ablk * 32 + TR::group_off(g, lg);       // four consecutive rows
+                        const floatx4 ha = *(const floatx4 *)(hnA + row0);
+#pragma unroll
+                        for (int q = 0; q < WB_FR; q++) {
+                            const int64_t bb = bblk0 + wb * WB_FR + q;
+                            if (bb < nb_blocks) {
+                                const int64_t col = bb * 32 + j;
+                                const float hb = hnB[col];
+#pragma unroll
+                                for (int e = 0; e < 4; e++) {
+                                    const float h = ha[e] + hb;                       // h - h: 0, or NaN for a bad row
+                                    const float k = kernel_value<KF>(acc[p][q][4 * g + e]) + (h - h);
+                                    if (row0 + e < n_a && col < n_b)
+                                        __builtin_nontemporal_store(k, &kout[(row0 + e) * kout_ld + col]);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        } else if constexpr (!kMfmaEpi) {
 #pragma unroll
             for (int p = 0; p < WA_FR; p++) {
                 const int rbase = (wa * WA_FR + p) * 32;
@@ -273,7 +305,9 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         }
     }
 
-    if constexpr (kMfmaEpi) {
+    if constexpr (STORE) {
+        // nothing left to write
+    } else if constexpr (kMfmaEpi) {
         const int tl = j & 15;
         if (j < 16 && tl < tcols) {
 #pragma unroll
@@ -324,6 +358,26 @@ static int launch_split_large_tt(const SplitView &A, const SplitView &B, const f
                        (const uintx4 *)B.data, A.nblk, B.nblk, (int)A.ks, a_tiles_per_chunk, partial, B.npad,
                        B.n > A.n);
     FLK_LAUNCH_CHECK("mmv_split_large_kernel");
+    return FLK_OK;
+}
+
+// The kernel matrix out[a][b] = K(A_a, B_b) in the bf16x3 mode: one workgroup per (A tile, B tile), or a few A tiles
+// per workgroup where the grid would not hold them all.
+int FLK_CAT(launch_fmm_split_large_kf, FLK_KF)(const SplitView &A, const SplitView &B, float *out, int64_t ld,
+                                               hipStream_t st) {
+    if (A.ks != B.ks || A.d != B.d)
+        return fail(FLK_EINVAL, "fmm (bf16x3): operands packed with different feature counts");
+    if (A.n == 0 || B.n == 0) return FLK_OK;
+    if (A.hnorm == nullptr || B.hnorm == nullptr) return fail(FLK_EINVAL, "fmm (bf16x3): operands without half norms");
+    const int64_t nab = kSLWavesA * kSLFragsA, nbb = kSLWavesB * kSLFragsB;
+    const int64_t a_tiles = (A.nblk + nab - 1) / nab;
+    const int64_t per_wg = (a_tiles + 65534) / 65535;
+    dim3 grid((unsigned)((B.nblk + nbb - 1) / nbb), (unsigned)((a_tiles + per_wg - 1) / per_wg));
+    hipLaunchKernelGGL((mmv_split_large_kernel<kSLWavesA, kSLWavesB, kSLFragsA, kSLFragsB, 1, FLK_KF, true>), grid,
+                       dim3(64 * kSLWavesA * kSLWavesB), 0, st, (const uintx4 *)A.data, (const float *)nullptr,
+                       (int64_t)0, 0, (const uintx4 *)B.data, A.nblk, B.nblk, (int)A.ks, per_wg, (float *)nullptr,
+                       B.npad, B.n > A.n, out, ld, A.n, B.n, A.hnorm, B.hnorm);
+    FLK_LAUNCH_CHECK("mmv_split_large_kernel (kernel matrix)");
     return FLK_OK;
 }
 

@@ -62,7 +62,8 @@ int split_large_max_cols();
                                 int tcols, int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st); \
     int launch_mmv_split_large_kf##KF(const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld, \
                                       int tcols, int64_t a_tiles_per_chunk, int splits, float *partial,        \
-                                      hipStream_t st);
+                                      hipStream_t st);                                                         \
+    int launch_fmm_split_large_kf##KF(const SplitView &A, const SplitView &B, float *out, int64_t ld, hipStream_t st);
 FLK_DECLARE_SPLIT_KF(0)
 FLK_DECLARE_SPLIT_KF(1)
 FLK_DECLARE_SPLIT_KF(2)
@@ -80,6 +81,14 @@ inline int launch_mmv_split(int kf, const SplitView &A, const SplitView &B, cons
 inline int launch_mmv_split_large(int kf, const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld,
                                   int tcols, int64_t a_tiles_per_chunk, int splits, float *partial, hipStream_t st) {
 #define FLK_CALL(KF) launch_mmv_split_large_kf##KF(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st)
+    FLK_SWITCH_KF(kf, FLK_CALL)
+#undef FLK_CALL
+}
+
+// explicit kernel matrix out[a][b] = K(A_a, B_b) (rows ld elements apart, columns contiguous) in the bf16x3 mode
+inline int launch_fmm_split_large(int kf, const SplitView &A, const SplitView &B, float *out, int64_t ld,
+                                  hipStream_t st) {
+#define FLK_CALL(KF) launch_fmm_split_large_kf##KF(A, B, out, ld, st)
     FLK_SWITCH_KF(kf, FLK_CALL)
 #undef FLK_CALL
 }

@@ -16,16 +16,19 @@ import torch
 from .. import _backend
 from ..options import BaseOptions
 from ..utils.helpers import sizeof_dtype
-from .fmmv import _DTYPE_CODE, _check_dtype, _compute_device, _kernel_fn, _mat, _on, _rows_that_fit, _stream_handle
+from .fmmv import (_DTYPE_CODE, _arith_code, _check_dtype, _compute_device, _kernel_fn, _mat, _on, _rows_that_fit,
+                   _stream_handle)
 from .utils import check_contiguity, create_output_mat, usable_gpu_memory
 
 __all__ = ("fmm", "gauss_fmm_native")
 
 
-def gauss_fmm_native(X1, X2, sigma_dev, out, compute_f64: bool, kernel_fn: int = _backend.FLK_GAUSSIAN) -> None:
-    """out[n,m] = K(X1, X2) through ``flk_kernel_fmm``.  All tensors on one GPU, 2-D, same dtype."""
+def gauss_fmm_native(X1, X2, sigma_dev, out, compute_f64: bool, kernel_fn: int = _backend.FLK_GAUSSIAN,
+                     code: Optional[int] = None) -> None:
+    """out[n,m] = K(X1, X2) through ``flk_kernel_fmm``.  All tensors on one GPU, 2-D, same dtype; ``code`` is the
+    library's dtype code (the data's dtype, or the bf16x3 mode of fp32)."""
     lib = _backend.load()
-    code = _DTYPE_CODE[X1.dtype]
+    code = _DTYPE_CODE[X1.dtype] if code is None else code
     n, d = X1.shape
     m = X2.shape[0]
     ws_bytes = lib.flk_gauss_fmm_workspace_bytes(n, m, d, code, int(compute_f64))
@@ -100,7 +103,7 @@ def _fmm_run(kernel, kernel_fn: int, opt: BaseOptions, out, X1, X2, cached_sigma
         return out
     with torch.inference_mode():
         lib = _backend.load()
-        code, sz = _DTYPE_CODE[X1.dtype], sizeof_dtype(X1.dtype)
+        code, sz = _arith_code(X1.dtype, opt), sizeof_dtype(X1.dtype)      # (the bf16x3 mode of fp32 where it applies)
         compute_f64 = X1.dtype == torch.float32 and bool(opt.no_single_kernel)
         sigma_dev = kernel._sigma_on(dev, X1.dtype, cached=cached_sigma)
         x1_in, out_in = X1.device == dev, out.device == dev
@@ -117,7 +120,7 @@ def _fmm_run(kernel, kernel_fn: int, opt: BaseOptions, out, X1, X2, cached_sigma
             li = min(blk, N - i)
             X1d = _on(X1[i:i + li], dev)
             outd = out[i:i + li] if out_in else torch.empty((li, M), dtype=out.dtype, device=dev)
-            gauss_fmm_native(X1d, X2d, sigma_dev, outd, compute_f64, kernel_fn)
+            gauss_fmm_native(X1d, X2d, sigma_dev, outd, compute_f64, kernel_fn, code)
             if not out_in:
                 out[i:i + li].copy_(outd)
     return out

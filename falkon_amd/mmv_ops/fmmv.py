@@ -319,7 +319,7 @@ def _fmmv_explicit(X1, X2, v, out, sigma_dev, kernel_fn: int, dev, opt: BaseOpti
     block = torch.empty((rows, M), dtype=X1.dtype, device=dev)
     for i in range(0, N, rows):
         li = min(rows, N - i)
-        gauss_fmm_native(X1d[i:i + li], X2d, sigma_dev, block[:li], False, kernel_fn)
+        gauss_fmm_native(X1d[i:i + li], X2d, sigma_dev, block[:li], False, kernel_fn, _arith_code(X1.dtype, opt))
         outd[i:i + li].copy_(block[:li] @ vd)
     if outd is not out:
         out.copy_(outd)
@@ -342,7 +342,7 @@ def _fdmmv_explicit(X1, X2, v, w, out, sigma_dev, kernel_fn: int, dev, opt: Base
     block = torch.empty((rows, M), dtype=X1.dtype, device=dev)
     for i in range(0, N, rows):
         li = min(rows, N - i)
-        gauss_fmm_native(X1d[i:i + li], X2d, sigma_dev, block[:li], False, kernel_fn)
+        gauss_fmm_native(X1d[i:i + li], X2d, sigma_dev, block[:li], False, kernel_fn, _arith_code(X1.dtype, opt))
         u = block[:li] @ vd
         if wd is not None:
             u += wd[i:i + li]

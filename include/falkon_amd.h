@@ -14,8 +14,8 @@
  * (falkon/mmv_ops/utils.py:36-39 requires only that some stride equals one).
  *
  * dtype: FLK_F32 (0) or FLK_F64 (1); all operands of a call share it
- * (falkon/kernels/kernel.py:78-79,102-103).  FLK_F32_BF16X3 (2), accepted by the fmmv / fdmmv entry
- * points and their workspace queries only, is fp32 data and fp32 results with the cross term x.c of the
+ * (falkon/kernels/kernel.py:78-79,102-103).  FLK_F32_BF16X3 (2), accepted by the fmmv / fdmmv / fmm entry
+ * points and their workspace queries only (fmm: beyond 64 features and without compute_f64; otherwise as FLK_F32), is fp32 data and fp32 results with the cross term x.c of the
  * squared distance formed on the bfloat16 matrix cores: every scaled fp32 value is split exactly into
  * three bfloat16 pieces (3 x 8 = 24 significant bits) and six partial products are accumulated in fp32,
  * which keeps the accuracy of the fp32 dot product (measured: the same distance from the fp64 result as

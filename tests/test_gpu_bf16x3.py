@@ -189,3 +189,49 @@ def test_dmmv_replays_from_a_hip_graph(dev, d):
         torch.cuda.synchronize()
         assert torch.equal(replayed, eager)
     assert rel_err(eager, mmv_ref.fdmmv_ref(X, C, vg.cpu(), wg.cpu(), k.sigma)) < 1e-5
+
+
+@pytest.mark.parametrize("n,m,d", [(600, 700, 130), (257, 513, 65), (64, 300, 110), (50, 45, 784), (1, 300, 100), (300, 1, 97)])
+def test_kernel_matrix_in_the_mode(dev, n, m, d):
+    """Beyond 64 features the option also serves the kernel matrix evaluated in fp32 (``no_single_kernel=False``): as
+    close to the fp64 closed form as the fp32 kernels, both memory orders, a NaN row stays a NaN row, other kernel
+    functions; with ``no_single_kernel=True`` (fp64 evaluation) the option changes nothing."""
+    from oracle import brute
+    g = np.random.default_rng(n + d)
+    X = torch.from_numpy(g.standard_normal((n, d)).astype(np.float32) * 0.6)
+    C = torch.from_numpy(g.standard_normal((m, d)).astype(np.float32) * 0.6)
+    sigma = torch.from_numpy(g.uniform(0.8, 1.6, d) * np.sqrt(d))
+    exact = torch.from_numpy(brute.gaussian_brute(X, C, sigma))
+    split_opt = FalkonOptions(bf16x3_cross_term=True, no_single_kernel=False)
+    k = GaussianKernel(sigma, opt=split_opt)
+    Xg, Cg = X.to(dev), C.to(dev)
+    got = k(Xg, Cg).cpu()
+    plain = GaussianKernel(sigma, opt=FalkonOptions(no_single_kernel=False))(Xg, Cg).cpu()
+    err, err_plain = float((got.double() - exact).abs().max()), float((plain.double() - exact).abs().max())
+    assert got.dtype == torch.float32 and err <= 1.5 * err_plain + 2e-7
+    out = torch.empty(m, n, dtype=torch.float32, device=dev).T                       # F-ordered result
+    assert k(Xg, Cg, out=out).data_ptr() == out.data_ptr()      # operands change roles: same terms, another order
+    assert float((out.cpu().double() - exact).abs().max()) <= 1.5 * err_plain + 2e-7
+    Xb = X.clone()
+    Xb[n // 2, 3] = float("nan")
+    bad = k(Xb.to(dev), Cg).cpu()
+    keep = torch.arange(n) != n // 2
+    assert torch.isnan(bad[n // 2]).all() and torch.equal(bad[keep], got[keep])
+    lap = LaplacianKernel(float(np.sqrt(d)), opt=split_opt)(Xg, Cg).cpu()
+    want = torch.from_numpy(brute.radial_brute(X, C, torch.tensor([np.sqrt(d)]), "laplacian"))
+    assert float((lap.double() - want).abs().max()) < 5e-6
+    both = GaussianKernel(sigma, opt=FalkonOptions(bf16x3_cross_term=True, no_single_kernel=True))(Xg, Cg)
+    assert torch.equal(both, GaussianKernel(sigma, opt=FalkonOptions(no_single_kernel=True))(Xg, Cg))
+
+
+def test_stored_block_route_in_the_mode(dev):
+    """Many right-hand sides beyond 64 features with the option: the stored blocks of K come from the bf16x3 kernel."""
+    n, m, d, t = 700, 300, 100, 40
+    X, C, v, w = _data(n, m, d, t, seed=11)
+    sigma = torch.tensor([0.9 * np.sqrt(d)], dtype=torch.float64)
+    k = GaussianKernel(sigma, opt=SPLIT)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+    check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)
+    check_parity(k.dmmv(Xg, Cg, vg, wg), mmv_ref.fdmmv_ref(X, C, v, w, sigma),
+                 mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), 1e-5)
