@@ -375,6 +375,13 @@ def main():
         res["roofline"] = {"bound": "mfma", "achieved": once * peak, "peak": peak, "unit": "TFLOP/s", "frac": once,
                            "traffic": None, "kernel": "kernel-matrix kernel + rocBLAS GEMMs on stored blocks of K",
                            "launches_per_step": 0.0, "avg_launch_ms": None, "flop_per_launch": None}
+        if split and d > 64:
+            # the stored blocks come from the bf16x3 kernel-matrix kernel: priced, like the bf16x3 product kernels,
+            # on the bf16 matrix flops executed (one evaluation of K per step), the fp32 count kept beside it
+            executed = N * M * 6 * 2 * 16 * ((d + 2 + 15) // 16)
+            res["roofline"].update(achieved=executed / (elapsed / args.steps) / 1e12, peak=BF16_PEAK_TFLOPS,
+                                   frac=executed / (elapsed / args.steps) / 1e12 / BF16_PEAK_TFLOPS,
+                                   algorithmic_frac_of_fp32_peak=once)
     if split and launches.value > 0:
         res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch,
                                               MEASURED_TRAFFIC_BYTES_BF16X3.get(args.workload)),
