@@ -105,3 +105,25 @@ def test_config3_full_size(dev, bf16x3):
 def test_config4_full_size(dev, dtype, bf16x3):
     """N=5e5, d=784 (80 % zeros), M=10000, T=10, sigma=10, fp32 (both modes) and fp64."""
     _full_size_checks(dev, "C4", dtype, n_rows=2000, n_centres=32, bf16x3=bf16x3)
+
+
+@pytest.mark.parametrize("bf16x3", [False, True], ids=["fp32-mfma", "bf16x3"])
+def test_kernel_matrix_large_square(dev, bf16x3):
+    """K(A, A) for 30 000 rows of 256 features, evaluated in fp32 (3.6 GB): properties no sample can miss — a unit
+    diagonal and symmetry (each to rounding of the expanded norm), the F-ordered result equal to the transpose —
+    and 40 rows against the fp64 closed form."""
+    from oracle import brute
+    n, d, sigma = 30_000, 256, 16.0
+    g = torch.Generator().manual_seed(77)
+    A = torch.randn(n, d, generator=g, dtype=torch.float32)
+    Ag = A.to(dev)
+    k = GaussianKernel(sigma, opt=FalkonOptions(no_single_kernel=False, bf16x3_cross_term=bf16x3))
+    K = k(Ag, Ag)
+    assert float((K.diagonal() - 1).abs().max()) < 2e-5
+    assert float((K - K.T).abs().max()) < 2e-6
+    Kf = k(Ag, Ag, out=torch.empty(n, n, dtype=torch.float32, device=dev).T)
+    assert float((Kf - K).abs().max()) < 2e-6
+    rows = torch.randint(0, n, (40,), generator=g)
+    exact = torch.from_numpy(brute.gaussian_brute(A[rows], A, torch.tensor([sigma], dtype=torch.float64)))
+    assert float((K[rows.to(dev)].cpu().double() - exact).abs().max()) < 2e-6
+    assert torch.isfinite(K).all()
