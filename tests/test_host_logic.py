@@ -54,8 +54,17 @@ def test_size_queries_need_no_gpu():
         assert query(100, 10, 3, too_many, _backend.FLK_F32) == 0
     assert lib.flk_gauss_packed_bytes(10, 3, 7) == 0 and lib.flk_gauss_packed_bytes(10, too_wide, _backend.FLK_F32) == 0
     assert lib.flk_gauss_fmmv_workspace_bytes(100, 10, 3, 1, _backend.FLK_F32_BF16X3) > 0
-    # the bf16x3 code belongs to the product entry points only
+    # the bf16x3 code belongs to the product entry points and the kernel matrix, not to the packed entry points
     assert lib.flk_gauss_mmv_packed_workspace_bytes(100, 10, 3, 1, _backend.FLK_F32_BF16X3) == 0
+    # kernel matrix: the code has operands of its own beyond 64 features in fp32 arithmetic (three bfloat16 planes per
+    # 16-feature step, 32-row blocks, fp32 half norms), and asks for what FLK_F32 asks otherwise
+    fmm = lib.flk_gauss_fmm_workspace_bytes
+    a256 = lambda b: (b + 255) // 256 * 256
+    split_operand = lambda n, d: a256((n + 31) // 32 * ((d + 2 + 15) // 16) * 3 * 64 * 16) + a256((n + 31) // 32 * 32 * 4)
+    assert fmm(1000, 300, 100, _backend.FLK_F32_BF16X3, 0) == split_operand(1000, 100) + split_operand(300, 100)
+    assert fmm(1000, 300, 100, _backend.FLK_F32_BF16X3, 1) == fmm(1000, 300, 100, _backend.FLK_F32, 1)
+    assert fmm(1000, 300, 64, _backend.FLK_F32_BF16X3, 0) == fmm(1000, 300, 64, _backend.FLK_F32, 0)
+    assert fmm(1000, 300, 100, 7, 0) == 0 and fmm(-1, 300, 100, _backend.FLK_F32, 0) == 0
 
 
 def test_bad_arguments_rejected_on_host_before_any_launch():
