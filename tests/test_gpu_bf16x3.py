@@ -235,3 +235,29 @@ def test_stored_block_route_in_the_mode(dev):
     check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)
     check_parity(k.dmmv(Xg, Cg, vg, wg), mmv_ref.fdmmv_ref(X, C, v, w, sigma),
                  mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), 1e-5)
+
+
+def test_kernel_matrix_in_the_mode_blocking_and_inputs(dev):
+    """The drivers' row blocking of X1 under a small memory budget, F-ordered inputs (F-ordered result) and host inputs
+    (result on the host) reach the same bf16x3 kernel: the blocked result equals the one-piece result bitwise, the
+    others agree with the fp64 closed form like it."""
+    from oracle import brute
+    n, m, d = 900, 410, 150
+    g = np.random.default_rng(3)
+    X = torch.from_numpy(g.standard_normal((n, d)).astype(np.float32) * 0.5)
+    C = torch.from_numpy(g.standard_normal((m, d)).astype(np.float32) * 0.5)
+    exact = torch.from_numpy(brute.gaussian_brute(X, C, torch.tensor([9.0], dtype=torch.float64)))
+    opt = FalkonOptions(bf16x3_cross_term=True, no_single_kernel=False)
+    k = GaussianKernel(9.0, opt=opt)
+    Xg, Cg = X.to(dev), C.to(dev)
+    whole = k(Xg, Cg).cpu()
+    err = float((whole.double() - exact).abs().max())
+    assert err < 4e-7
+    blocked = k(Xg, Cg, opt=FalkonOptions(bf16x3_cross_term=True, no_single_kernel=False, max_gpu_mem=2_500_000))
+    assert torch.equal(blocked.cpu(), whole)
+    Xf = torch.empty_strided(X.shape, (1, n), dtype=X.dtype).copy_(X).to(dev)
+    Cf = torch.empty_strided(C.shape, (1, m), dtype=C.dtype).copy_(C).to(dev)
+    got_f = k(Xf, Cf)
+    assert got_f.stride(0) == 1 and float((got_f.cpu().double() - exact).abs().max()) < 4e-7
+    host = k(X, C)
+    assert host.device.type == "cpu" and float((host.double() - exact).abs().max()) < 4e-7
