@@ -80,6 +80,21 @@ __device__ __forceinline__ void xcd_remap(unsigned &bx, unsigned &by, bool y_fas
         by = logical / gx;
     }
 }
+// The same XCD-contiguous numbering for kernels whose workgroups each own one (x, y) tile and share nothing through
+// a loop (the kernel-matrix store mode): consecutive workgroups of an XCD walk bands of kBandY tiles in y, y fastest,
+// so the 32 workgroups resident on an XCD cover 8 x 4 tiles and fetch 12 operand tiles through its L2 instead of 33.
+constexpr unsigned kBandY = 8;
+__device__ __forceinline__ void xcd_remap_banded(unsigned &bx, unsigned &by) {
+    const unsigned gx = gridDim.x, gy = gridDim.y, total = gx * gy;
+    const unsigned id = blockIdx.y * gx + blockIdx.x;
+    const unsigned q = total / 8, r = total % 8, xcd = id % 8, local = id / 8;
+    const unsigned logical = xcd * q + (xcd < r ? xcd : r) + local;
+    const unsigned band = logical / (kBandY * gx), first = band * kBandY;
+    const unsigned height = gy - first < kBandY ? gy - first : kBandY;
+    const unsigned within = logical - band * kBandY * gx;
+    by = first + within % height;
+    bx = within / height;
+}
 #endif
 
 // error plumbing -------------------------------------------------------------

@@ -91,7 +91,8 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     __shared__ __attribute__((aligned(32))) T ldsRow[kRowBuf];   // [hA | vec ...] of the A tile
 
     unsigned bx, by;
-    xcd_remap(bx, by, y_fastest);
+    if constexpr (kStore) xcd_remap_banded(bx, by);
+    else xcd_remap(bx, by, y_fastest);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wa = wave % kLWavesA, wb = wave / kLWavesA;

@@ -65,7 +65,8 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     __shared__ __attribute__((aligned(32))) float ldsRow[kRowBuf];   // vec of the A tile
 
     unsigned bx, by;
-    xcd_remap(bx, by, y_fastest);
+    if constexpr (STORE) xcd_remap_banded(bx, by);
+    else xcd_remap(bx, by, y_fastest);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform by construction: let the compiler know
