@@ -297,11 +297,18 @@ def _explicit_blocks_pay(d: int, t: int, dtype: torch.dtype, opt: BaseOptions) -
     return passes >= (4 if d <= 32 else 3)
 
 
+def _block_leading_dim(M: int, sz: int) -> int:
+    """Leading dimension of a stored block: rows start on multiples of 128 bytes, so that the kernel-matrix kernel's
+    128-byte store segments never straddle two lines."""
+    per_line = 128 // sz
+    return -(-M // per_line) * per_line
+
+
 def _explicit_block_rows(N: int, M: int, D: int, T: int, sz: int, dev, opt: BaseOptions, upload_bytes: int) -> int:
     """Rows of K per stored block (0: not even a sliver fits next to the operands; the caller keeps to the
     product kernels).  Per row: the block itself, its products with v, and the packed copy of the row."""
     usable = usable_gpu_memory(dev, opt.max_gpu_mem, opt.memory_slack) - upload_bytes - 2 * M * (D + T) * sz
-    per_row = (M + 2 * T + 3 * D) * sz
+    per_row = (_block_leading_dim(M, sz) + 2 * T + 3 * D) * sz
     rows = int(min(_EXPLICIT_BLOCK_BYTES, usable / 2) // per_row)
     return min(N, rows) if rows >= 32 else 0
 
@@ -316,7 +323,7 @@ def _fmmv_explicit(X1, X2, v, out, sigma_dev, kernel_fn: int, dev, opt: BaseOpti
         return False
     X1d, X2d, vd = _on(X1, dev), _on(X2, dev), _on(v, dev)
     outd = out if out.device == dev else torch.empty((N, T), dtype=out.dtype, device=dev)
-    block = torch.empty((rows, M), dtype=X1.dtype, device=dev)
+    block = torch.empty((rows, _block_leading_dim(M, sz)), dtype=X1.dtype, device=dev)[:, :M]
     for i in range(0, N, rows):
         li = min(rows, N - i)
         gauss_fmm_native(X1d[i:i + li], X2d, sigma_dev, block[:li], False, kernel_fn, _arith_code(X1.dtype, opt))
@@ -339,7 +346,7 @@ def _fdmmv_explicit(X1, X2, v, w, out, sigma_dev, kernel_fn: int, dev, opt: Base
     wd = _on(w, dev) if w is not None else None
     outd = out if out.device == dev else torch.empty((M, T), dtype=out.dtype, device=dev)
     outd.zero_()
-    block = torch.empty((rows, M), dtype=X1.dtype, device=dev)
+    block = torch.empty((rows, _block_leading_dim(M, sz)), dtype=X1.dtype, device=dev)[:, :M]
     for i in range(0, N, rows):
         li = min(rows, N - i)
         gauss_fmm_native(X1d[i:i + li], X2d, sigma_dev, block[:li], False, kernel_fn, _arith_code(X1.dtype, opt))
