@@ -39,10 +39,19 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found; the falkon_amd native library needs ROCm's hipcc to build")
 
 
+def _headers_mtime() -> float:
+    hdrs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".inc"))]
+    hdrs.append(os.path.join(_HERE, "..", "include", "falkon_amd.h"))
+    return max(os.path.getmtime(h) for h in hdrs)
+
+
 def _compile(job) -> str:
-    src, kf = job
+    src, kf, only_changed = job
     stem = os.path.splitext(src)[0] + ("" if kf is None else f"_kf{kf}")
     obj = os.path.join(OBJ_DIR, stem + ".o")
+    if only_changed and os.path.exists(obj):
+        if os.path.getmtime(obj) > max(os.path.getmtime(os.path.join(CSRC, src)), _headers_mtime()):
+            return obj
     defines = [] if kf is None else [f"-DFLK_KF={kf}"]
     cmd = [_hipcc(), *HIPCC_FLAGS, *defines, "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -51,13 +60,14 @@ def _compile(job) -> str:
     return obj
 
 
-def build(verbose: bool = True, jobs: int = 0) -> str:
-    """Compile every source (always, also when a library is already there) and link."""
+def build(verbose: bool = True, jobs: int = 0, only_changed: bool = False) -> str:
+    """Compile every source (always, also when a library is already there) and link.  With ``only_changed`` an
+    object newer than its source and every header is kept (a developer's shortcut; the default rebuilds all)."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(_compile, SOURCES))
+        objs = list(ex.map(_compile, [(src, kf, only_changed) for src, kf in SOURCES]))
     tmp = LIB_PATH + ".tmp"
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", tmp]
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -70,4 +80,4 @@ def build(verbose: bool = True, jobs: int = 0) -> str:
 
 
 if __name__ == "__main__":
-    build()
+    build(only_changed="--changed" in sys.argv)
