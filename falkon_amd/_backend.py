@@ -52,10 +52,17 @@ _SIGNATURES = {
                               c_void_p, c_int64, c_int64, c_int, c_int,
                               c_void_p, c_size_t, c_void_p]),
 }
+# (added below the loop that derives the flk_kernel_* signatures: this one has no flk_kernel_* twin)
+_NOALLOC = {"flk_gauss_fdmmv_noalloc": (c_int, [*_MAT, *_MAT, c_int64, c_void_p, c_int64,
+                                               c_void_p, c_int64, c_int64,
+                                               c_void_p, c_int64, c_int64, c_int64,
+                                               c_void_p, c_int64, c_int64, c_int, c_void_p])}
 # the flk_kernel_* entry points: the flk_gauss_* ones with the kernel function as first argument
 for _name in ("pack", "mmv_packed", "fmmv", "fdmmv", "fmm"):
     _res, _args = _SIGNATURES["flk_gauss_" + _name]
     _SIGNATURES["flk_kernel_" + _name] = (_res, [c_int, *_args])
+_SIGNATURES.update(_NOALLOC)
+NOALLOC_SCRATCH_BYTES = 64 << 20
 
 
 def library_path() -> str:

@@ -556,6 +556,33 @@ static int fmm_split_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int6
     return launch_fmm_split_large(kf, P2, P1, (float *)out, out_cs, st);
 }
 
+// ---------------------------------------------------------------------------
+// Scratch memory of the entry point that allocates nothing (flk_gauss_fdmmv_noalloc): one array per GPU, part of the
+// loaded code object, held until the process ends.  `scratch` is only a host-side handle of the symbol: the device
+// address comes from hipGetSymbolAddress, once per device, and only that address is ever handed to kernels.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[FLK_NOALLOC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of the current device's copy of `scratch` (looked up on the first call on that device).
+static int scratch_address(void **ptr) {
+    int dev = -1;
+    FLK_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(FLK_EUNSUPPORTED, "device ordinal %d beyond %d", dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> g(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        FLK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr) return fail(FLK_EHIP, "hipGetSymbolAddress returned a null address for the scratch array");
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return FLK_OK;
+}
+
 }  // namespace flk
 
 using namespace flk;
@@ -714,6 +741,30 @@ int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, con
                     int64_t out_cs, int dtype, void *workspace, size_t workspace_bytes, void *stream) {
     return flk_kernel_fdmmv(FLK_GAUSSIAN, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
                             w_rs, w_cs, t, out, out_rs, out_cs, dtype, workspace, workspace_bytes, stream);
+}
+
+int flk_gauss_fdmmv_noalloc(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, const void *X2, int64_t m,
+                            int64_t x2_rs, int64_t x2_cs, int64_t d, const void *sigma, int64_t n_sigma, const void *v,
+                            int64_t v_rs, int64_t v_cs, const void *w, int64_t w_rs, int64_t w_cs, int64_t t, void *out,
+                            int64_t out_rs, int64_t out_cs, int dtype, void *stream) {
+    g_err[0] = 0;
+    if (n < 0 || m < 0 || d < 1 || t < 0) return fail(FLK_EINVAL, "bad shape");
+    if (!known_dtype(dtype, true)) return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+    if (d > flk_max_d(dtype)) return fail(FLK_EUNSUPPORTED, "more than %lld features", (long long)flk_max_d(dtype));
+    if (t > flk_max_t()) return fail(FLK_EUNSUPPORTED, "more than %lld right-hand sides", (long long)flk_max_t());
+    const size_t need = flk_gauss_fdmmv_workspace_bytes(n, m, d, t, dtype);
+    if (need > (size_t)FLK_NOALLOC_SCRATCH_BYTES)
+        return fail(FLK_ENOMEM,
+                    "flk_gauss_fdmmv_noalloc: this problem (n=%lld, m=%lld, d=%lld, t=%lld) needs %zu bytes of scratch "
+                    "memory, the built-in array holds %zu; use flk_gauss_fdmmv with a workspace of the caller's",
+                    (long long)n, (long long)m, (long long)d, (long long)t, need, (size_t)FLK_NOALLOC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    int rc = scratch_address(&ws);
+    if (rc != FLK_OK) return rc;
+    // every byte of the workspace a product reads it has written before in the same call (packed operands, planar
+    // vectors including their zero planes, partial sums), so what the previous call left behind needs no clearing
+    return flk_kernel_fdmmv(FLK_GAUSSIAN, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
+                            w_rs, w_cs, t, out, out_rs, out_cs, dtype, ws, (size_t)FLK_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype, int compute_f64) {

@@ -146,6 +146,26 @@ int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
                     void *out, int64_t out_rs, int64_t out_cs, int dtype,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- fdmmv for callers that cannot allocate ---------------------------------
+ * flk_gauss_fdmmv_noalloc has no counterpart in the reference.  It is flk_gauss_fdmmv without the workspace
+ * argument, for callers that cannot obtain device memory at the call: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  The workspace is an array of FLK_NOALLOC_SCRATCH_BYTES
+ * bytes that is part of the library's device code: every GPU the library runs on holds its own copy from the
+ * first call on it until the process ends.  The call allocates and frees nothing and enqueues the same kernels
+ * as flk_gauss_fdmmv, so the results are bit-identical to it.  A problem whose
+ * flk_gauss_fdmmv_workspace_bytes(n, m, d, t, dtype) exceeds FLK_NOALLOC_SCRATCH_BYTES is refused with
+ * FLK_ENOMEM and a message naming both sizes.  All calls on one GPU share that GPU's array: two calls whose
+ * kernels overlap in time (different streams, different threads) race on it, so keep them on one stream or
+ * order them yourself.  The array keeps the previous call's contents; every call writes what it reads. */
+#define FLK_NOALLOC_SCRATCH_BYTES (64u << 20)
+
+int flk_gauss_fdmmv_noalloc(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
+                            const void *X2, int64_t m, int64_t x2_rs, int64_t x2_cs, int64_t d,
+                            const void *sigma, int64_t n_sigma,
+                            const void *v, int64_t v_rs, int64_t v_cs,
+                            const void *w, int64_t w_rs, int64_t w_cs, int64_t t,
+                            void *out, int64_t out_rs, int64_t out_cs, int dtype, void *stream);
+
 /* ---- explicit kernel matrix -------------------------------------------------
  * flk_gauss_fmm replaces falkon.mmv_ops.fmm.fmm for the dense Gaussian case
  *   (falkon/mmv_ops/fmm.py:699-708 -> :298-388 block loop -> distance_kernel.py:140-159):
