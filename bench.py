@@ -49,24 +49,26 @@ WORKLOADS = {
     "C4": (1004, 500_000, 784, 10_000, 10, True),
 }
 
-# HBM bytes per launch of the product kernel, keyed by workload: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (KiB per dispatch, mean over the launches of the kernel) scaled by what the same counters read for a plain
-# 1 GiB device copy (FETCH_SIZE reads half the true bytes on this box: factor 2.0; WRITE_SIZE factor 1.0).
-# The summaries are under profiles/.  None where it has not been measured.
-MEASURED_TRAFFIC_BYTES = {
-    "C2": int((73470.7 * 2.0 + 17773.4 * 1.0) * 1024),     # 168.7 MB; algorithmic: packed X 112 MB + C + vectors
-    # 0.94 GB mean of the two passes: K v reads the packed X once (0.5 GB, the algorithmic figure), the K^T u
-    # pass reads it about three times (1.3 GB): the output tiles that share a reduction chunk do not all run at once
-    "C3": int((439079.0 * 2.0 + 38190.0 * 1.0) * 1024),
-    "C4": int((2.54605e7 * 2.0 + 559550.0 * 1.0) * 1024),  # 52.7 GB: tiles are re-read from L2 / MALL / HBM
-}
+# HBM bytes per launch of the product kernel come from profiles/hbm_traffic.json, written together with the
+# rocprofv3 counter summaries under profiles/ (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, mean over the launches of
+# the kernel, each scaled by what the same counter reads for a plain 1 GiB device copy; the file names the commit
+# the counters were taken on and the commands).  None where a workload has no entry.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 
 
-# the same for the bf16x3 product kernel (profiles/mmv_split_kernel__C2_dfmmv_bf16x3.md)
-MEASURED_TRAFFIC_BYTES_BF16X3 = {
-    "C2": int((536594.0 * 2.0 + 17773.4 * 1.0) * 1024),    # 1.12 GB: the packed centres no longer fit one L2 next to X
-    "C4": int((3.32483e7 * 2.0 + 174341.0 * 1.0) * 1024),  # 68 GB: tiles are re-read from L2 / infinity cache / HBM
-}
+def measured_traffic(workload, dtype, cross_term="f32"):
+    """(bytes per launch, provenance) of the product kernel on `workload`, or (None, None)."""
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            table = json.load(fh)
+    except (OSError, ValueError):
+        return None, None
+    entry = table.get("kernels", {}).get(f"{workload}/{dtype}/{cross_term}")
+    if not entry:
+        return None, None
+    cal = table.get("copy_calibration", {})
+    nbytes = int((entry["fetch_kib"] * cal.get("fetch_factor", 1.0) + entry["write_kib"] * cal.get("write_factor", 1.0)) * 1024)
+    return nbytes, {"file": "profiles/hbm_traffic.json", "commit": table.get("commit"), "kernel": entry.get("kernel")}
 
 
 def product_kernel_name(d, T, dtype):
@@ -107,30 +109,75 @@ def make_inputs(name, rhs=0):
             torch.from_numpy(w) if w is not None else None)
 
 
-def cpu_baseline(X, C, sigma, v, w, gpu_out_fn, rows, kernel_name="gaussian"):
-    """Reference-equivalent CPU path (the oracle restatement, torch CPU ops) on the first `rows` rows."""
+CPU_MEM = 16 * 2**30           # max_cpu_mem of the CPU path (the reference's default of inf would allocate N x M)
+
+
+def _rel(a, b):
+    """Norm-wise relative error per output column, worst column."""
+    a, b = a.double().cpu(), b.double().cpu()
+    return float(((a - b).norm(dim=0) / b.norm(dim=0)).max())
+
+
+def cpu_baseline(X, C, sigma, v, w, gpu_out_fn, rows, time_rows, reps, kernel_name="gaussian"):
+    """Reference-equivalent CPU path (the oracle restatement, torch CPU ops).
+
+    Timing: dfmmv on the first `time_rows` rows with the full M, two warm-ups and `reps` timed repetitions (min and
+    median).  Parity: on the first `rows` rows (all of them for config 2) the CPU path in the data's dtype at
+    max_cpu_mem = 16 GiB and at 4 GiB (the fp32 accumulation order follows the row blocks), and the same path in
+    fp64 on the same inputs as the anchor -- every distance is to a CPU-computed result; the GPU's own fp64 result
+    is only reported beside them."""
     from oracle import mmv_ref                      # checker only; never on the product path
+    M, T = v.shape
+    Xt = X[:time_rows].contiguous()
+    wt = w[:time_rows].contiguous() if w is not None else None
+    times = []
+    for i in range(2 + reps):
+        t0 = time.perf_counter()
+        mmv_ref.fdmmv_ref(Xt, C, v, wt, sigma, max_cpu_mem=CPU_MEM, kernel_name=kernel_name)
+        if i >= 2:
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
     Xs = X[:rows].contiguous()
     ws = w[:rows].contiguous() if w is not None else None
-    mmv_ref.fdmmv_ref(Xs[:2000], C, v, ws[:2000] if ws is not None else None, sigma, max_cpu_mem=4 * 2**30,
-                      kernel_name=kernel_name)                                                       # warm-up
-    t0 = time.perf_counter()
-    exp = mmv_ref.fdmmv_ref(Xs, C, v, ws, sigma, max_cpu_mem=4 * 2**30, kernel_name=kernel_name)
-    dt = time.perf_counter() - t0
-    got, got64 = gpu_out_fn(Xs, ws)
-    got, got64, exp = got.double().cpu(), got64.double().cpu(), exp.double()
-
-    def rel(a, b):
-        return float(((a - b).norm(dim=0) / b.norm(dim=0)).max())
-
-    M, T = v.shape
-    return {"value": rows * M * T / dt, "unit": "kernel entries/s", "cores": torch.get_num_threads(),
+    base = {"value": time_rows * M * T / med, "unit": "kernel entries/s", "cores": torch.get_num_threads(),
             "kind": "port", "host_cpus": os.cpu_count(),
-            "sample": f"first {rows} rows of X with the full M={M} (dfmmv is linear in N), "
-                      f"max_cpu_mem=4GiB, {dt:.2f} s",
-            # fp64 anchor = the same product in fp64 on the same fp32-valued inputs (GPU fp64 kernel)
-            "rel_err_gpu_f32_vs_cpu_f32": rel(got, exp), "rel_err_gpu_f32_vs_f64": rel(got, got64),
-            "rel_err_cpu_f32_vs_f64": rel(exp, got64)}
+            "sample": f"dfmmv on the first {time_rows} rows of X with the full M={M} (linear in N), "
+                      f"max_cpu_mem=16GiB, 2 warm-ups + {reps} repetitions: median {med:.2f} s, min {times[0]:.2f} s",
+            "value_at_min_time": time_rows * M * T / times[0], "parity_rows": rows}
+    t0 = time.perf_counter()
+    cpu64 = mmv_ref.fdmmv_ref(Xs.double(), C.double(), v.double(), ws.double() if ws is not None else None, sigma,
+                              max_cpu_mem=CPU_MEM, kernel_name=kernel_name)
+    f64_s = time.perf_counter() - t0
+    got, got64 = gpu_out_fn(Xs, ws)
+    tol32, tol64 = 1e-5, 1e-11
+    e_gpu64 = _rel(got64, cpu64)
+    base.update({"rel_err_gpu_f64_vs_cpu_f64": e_gpu64, "fp64_within_1e-11": e_gpu64 <= tol64})
+    if X.dtype == torch.float64:
+        base["parity_run_s"] = {"cpu_f64_16GiB": f64_s}
+        base["parity_statement"] = f"GPU fp64 result {e_gpu64:.2e} from the fp64 CPU path (bar {tol64:g})"
+        return base
+    t0 = time.perf_counter()
+    cpu32 = mmv_ref.fdmmv_ref(Xs, C, v, ws, sigma, max_cpu_mem=CPU_MEM, kernel_name=kernel_name)
+    full_s = time.perf_counter() - t0
+    cpu32_4g = mmv_ref.fdmmv_ref(Xs, C, v, ws, sigma, max_cpu_mem=4 * 2**30, kernel_name=kernel_name)
+    e_gpu32, e_cpu32, e_cpu32_4g = _rel(got, cpu64), _rel(cpu32, cpu64), _rel(cpu32_4g, cpu64)
+    e_pair, e_pair_4g = _rel(got, cpu32), _rel(got, cpu32_4g)
+    if e_pair <= tol32:
+        statement = f"GPU fp32 result within {tol32:g} of the fp32 CPU path ({e_pair:.2e})"
+    else:
+        statement = (f"fp32 CPU path is {e_cpu32:.2e} from its fp64 twin (CPU), the GPU fp32 result {e_gpu32:.2e}: "
+                     f"the two fp32 results differ by {e_pair:.2e} > {tol32:g} because of the CPU path's own fp32 "
+                     f"accumulation; the 1e-5 bar is read as 'no further from the fp64 CPU result than the fp32 CPU path'")
+    base.update({"parity_run_s": {"cpu_f32_16GiB": full_s, "cpu_f64_16GiB": f64_s},
+                 "value_parity_run": rows * M * T / full_s,
+                 # every anchor below is computed on the CPU
+                 "rel_err_gpu_f32_vs_cpu_f64": e_gpu32, "rel_err_cpu_f32_vs_cpu_f64": e_cpu32,
+                 "rel_err_cpu_f32_4GiB_vs_cpu_f64": e_cpu32_4g,
+                 "rel_err_gpu_f32_vs_cpu_f32": e_pair, "rel_err_gpu_f32_vs_cpu_f32_4GiB": e_pair_4g,
+                 "rel_err_gpu_f32_vs_gpu_f64": _rel(got, got64),          # extra: GPU against GPU, not an anchor
+                 "parity_statement": statement})
+    return base
 
 
 def make_c5(N, Nts, seed=1005, d=28):
@@ -231,7 +278,7 @@ def run_c5(args, lib):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS) + ["C5"])
     ap.add_argument("--c5-n", type=int, default=2_000_000, help="training rows of the C5 workload")
@@ -342,6 +389,8 @@ def main():
     flop_per_launch = N * M * (2 * d + 4 + 2 * T)
     kern_ms = tot_ms.value / max(launches.value, 1)
     achieved = flop_per_launch / (kern_ms * 1e-3) / 1e12 if kern_ms > 0 else 0.0
+    traffic, traffic_src = (None, None) if args.rhs or args.op != "dmmv" or args.kernel != "gaussian" else \
+        measured_traffic(args.workload, args.dtype, args.cross_term)
     res = {
         "metric": f"{'dfmmv' if args.op == 'dmmv' else 'fmmv'} kernel-entries/sec (N*M*T/s) {'fp32' if args.dtype == 'f32' else 'fp64'}, 1 MI355X",
         "value": value, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -354,7 +403,7 @@ def main():
                                f"inputs resident in HBM, packing included in every step"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.dtype == "f32" and not args.rhs else None,
+                     "traffic": traffic, "traffic_source": traffic_src,
                      "kernel": product_kernel_name(d, T, args.dtype),
                      "launches_per_step": launches.value / args.steps,
                      "avg_launch_ms": kern_ms, "flop_per_launch": flop_per_launch},
@@ -383,9 +432,8 @@ def main():
                                    frac=executed / (elapsed / args.steps) / 1e12 / BF16_PEAK_TFLOPS,
                                    algorithmic_frac_of_fp32_peak=once)
     if split and launches.value > 0:
-        res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch,
-                                              MEASURED_TRAFFIC_BYTES_BF16X3.get(args.workload)),
-                               launches_per_step=launches.value / args.steps)
+        res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch, traffic),
+                               launches_per_step=launches.value / args.steps, traffic_source=traffic_src)
     if not split and args.dtype == "f32" and args.kernel == "gaussian" and not args.no_cpu_baseline:
         # not the headline: the same step with the opt-in bf16x3 cross term (fp32 data and results, the cross term
         # on the bf16 matrix cores from an exact three-way split), timed after the run above, and how far its
@@ -404,10 +452,46 @@ def main():
         res["opt_in_bf16x3_cross_term"] = {"value": N * M * T / (el / args.steps), "ms_per_step": el / args.steps * 1e3,
                                            "rel_diff_from_fp32_kernels": diff}
         kernel = make_kernel(sigma)
+    side64 = None
+    if not split and args.dtype == "f32" and args.kernel == "gaussian" and args.op == "dmmv" and not args.no_cpu_baseline:
+        # the fp64 half of the metric: the same step on the same inputs widened to fp64 (fewer steps: it is not
+        # the headline), product-kernel time from the library's HIP events as above
+        X64, C64, v64 = Xg.double(), Cg.double(), vg.double()
+        w64 = wg.double() if wg is not None else None
+        out64 = torch.empty(M, T, dtype=torch.float64, device=dev)
+        steps64 = max(5, args.steps // 5)
+        for _ in range(2):
+            kernel.dmmv(X64, C64, v64, w64, out=out64)
+        torch.cuda.synchronize()
+        lib.flk_kernel_timing_enable(1)
+        t0 = time.perf_counter()
+        for _ in range(steps64):
+            kernel.dmmv(X64, C64, v64, w64, out=out64)
+        torch.cuda.synchronize()
+        el64 = (time.perf_counter() - t0) / steps64
+        tot64, n64 = ctypes.c_double(), ctypes.c_int64()
+        _backend.raise_for_status(lib.flk_kernel_timing_read(ctypes.byref(tot64), ctypes.byref(n64)), "flk_kernel_timing_read")
+        lib.flk_kernel_timing_enable(0)
+        k64 = tot64.value / max(n64.value, 1)
+        a64 = flop_per_launch / (k64 * 1e-3) / 1e12 if k64 > 0 else 0.0
+        tr64, tr64_src = measured_traffic(args.workload, "f64")
+        side64 = {"metric": "dfmmv kernel-entries/sec (N*M*T/s) fp64, 1 MI355X", "value": N * M * T / el64,
+                  "unit": "kernel entries/s", "dtype": "f64", "steps": steps64, "warmup": 2, "ms_per_step": el64 * 1e3,
+                  "roofline": {"bound": "mfma", "achieved": a64, "peak": FP64_PEAK_TFLOPS, "unit": "TFLOP/s",
+                               "frac": a64 / FP64_PEAK_TFLOPS, "traffic": tr64, "traffic_source": tr64_src,
+                               "kernel": product_kernel_name(d, T, "f64"), "launches_per_step": n64.value / steps64,
+                               "avg_launch_ms": k64, "flop_per_launch": flop_per_launch}}
+        res["fp64"] = side64
+        del X64, C64, v64, w64
     if not args.no_cpu_baseline and args.op == "dmmv":
-        rows = args.cpu_rows or {"C2": N, "C3": 400_000, "C4": 100_000}[args.workload]
+        full = args.workload == "C2" and not args.cpu_rows
+        rows = args.cpu_rows or {"C2": N, "C3": 200_000, "C4": 100_000}[args.workload]
+        time_rows = min(rows, {"C2": 200_000, "C3": 100_000, "C4": 50_000}[args.workload])
 
         def gpu_on(Xs, ws):
+            if full and tdt == torch.float32 and side64 is not None:
+                step()
+                return out.clone(), out64                       # the timed steps' own results, all N rows
             Xd = Xs.to(dev)
             wd = ws.to(dev) if ws is not None else None
             r32 = kernel.dmmv(Xd, Cg, vg, wd)
@@ -415,7 +499,10 @@ def main():
                                                                wd.double() if wd is not None else None)
             return r32, r64
 
-        res["cpu_baseline"] = cpu_baseline(X, C, sigma, v, w, gpu_on, rows, kernel_name)
+        res["cpu_baseline"] = cpu_baseline(X, C, sigma, v, w, gpu_on, rows, time_rows, 5 if full else 3, kernel_name)
+        if side64 is not None:
+            side64["rel_err_vs_cpu_f64"] = res["cpu_baseline"]["rel_err_gpu_f64_vs_cpu_f64"]
+            side64["parity_rows"] = rows
     print(json.dumps(res), flush=True)
 
 
