@@ -193,7 +193,7 @@ def make_c5(N, Nts, seed=1005, d=28):
 
 def run_c5(args, lib):
     """End-to-end fit + predict; returns the JSON record."""
-    from falkon_amd import Falkon, FalkonOptions, GaussianKernel
+    from falkon_amd import Falkon, FalkonOptions, GaussianKernel, _backend
     dev = torch.device("cuda:0")
     N, M, d, sigma, lam, iters = args.c5_n, args.c5_m, 28, 3.8, 1e-6, 20
     Nts = N // 10
@@ -203,7 +203,7 @@ def run_c5(args, lib):
     fit_s, pre_s, pred_s, kern_ms, launches = [], [], [], 0.0, 0
     mse = err = None
     split = args.cross_term == "bf16x3"
-    opt = FalkonOptions(bf16x3_cross_term=split)
+    opt = FalkonOptions(bf16x3_cross_term=split, cg_capture_graph=args.cg_graph)
     for it in range(args.warmup + args.steps):
         timed = it >= args.warmup
         model = Falkon(GaussianKernel(sigma, opt=opt), lam, M=M, maxiter=iters, seed=12, options=opt)
@@ -216,7 +216,8 @@ def run_c5(args, lib):
         t1 = time.perf_counter()
         if timed:
             tot_ms, cnt = ctypes.c_double(), ctypes.c_int64()
-            lib.flk_kernel_timing_read(ctypes.byref(tot_ms), ctypes.byref(cnt))
+            _backend.raise_for_status(lib.flk_kernel_timing_read(ctypes.byref(tot_ms), ctypes.byref(cnt)),
+                                      "flk_kernel_timing_read")
             lib.flk_kernel_timing_enable(0)
             kern_ms += tot_ms.value
             launches += cnt.value
@@ -245,6 +246,8 @@ def run_c5(args, lib):
                                f"penalty=1e-6, {iters} CG iterations ({n_dmmv} dfmmv + 1 fmmv), test rows {Nts}, "
                                f"fp32{' with the bf16x3 cross term' if split else ''}, data resident in HBM"},
         "fit_s": fit, "preconditioner_s": pre, "cg_s": cg, "predict_s": prd, "test_mse": mse, "test_error_rate": err,
+        "cg_graph": bool(args.cg_graph), "product_kernel_s_per_fit": kern_ms * 1e-3 / max(args.steps, 1),
+        "cg_s_over_product_kernel_s": cg / (kern_ms * 1e-3 / max(args.steps, 1)) if kern_ms > 0 else None,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_PEAK_TFLOPS, "traffic": None, "kernel": "mmv_small_f32_kernel",
                      "launches_per_step": launches / max(args.steps, 1), "avg_launch_ms": kern_avg,
@@ -296,6 +299,8 @@ def main():
     ap.add_argument("--stored-blocks", action="store_true",
                     help="FalkonOptions(dmmv_stored_blocks=True): dfmmv beyond 64 features through stored blocks of K "
                          "(not the headline path, which never materialises K)")
+    ap.add_argument("--cg-graph", action="store_true",
+                    help="C5 only: FalkonOptions(cg_capture_graph=True), the CG iterations replayed from HIP graphs")
     ap.add_argument("--rhs", type=int, default=0, metavar="T",
                     help="right-hand sides instead of the configuration's own number (not a headline workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true",

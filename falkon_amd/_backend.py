@@ -62,6 +62,10 @@ for _name in ("pack", "mmv_packed", "fmmv", "fdmmv", "fmm"):
     _res, _args = _SIGNATURES["flk_gauss_" + _name]
     _SIGNATURES["flk_kernel_" + _name] = (_res, [c_int, *_args])
 _SIGNATURES.update(_NOALLOC)
+_SIGNATURES["flk_cg_state_ints"] = (c_int64, [c_int64])
+_SIGNATURES["flk_cg_update"] = (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                        c_int64, c_int64, c_void_p, c_void_p, c_int64, ctypes.c_double, ctypes.c_double,
+                                        c_int, c_int, c_void_p])
 NOALLOC_SCRATCH_BYTES = 64 << 20
 
 

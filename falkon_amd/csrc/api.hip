@@ -42,6 +42,13 @@ struct ScopedKernelTimer {
     explicit ScopedKernelTimer(hipStream_t s) : st(s) {
         std::lock_guard<std::mutex> g(g_timing_mu);
         if (!g_timing_on) return;
+        // a launch that is being captured into a graph is not timed: events recorded during capture become graph
+        // nodes, and asking them for a time afterwards is an error
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return;
+        }
         if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { e0 = e1 = nullptr; return; }
         (void)hipEventRecord(e0, st);
     }
@@ -607,9 +614,14 @@ int flk_kernel_timing_read(double *total_ms, int64_t *launches) {
     std::lock_guard<std::mutex> g(g_timing_mu);
     double tot = 0.0;
     for (auto &e : g_timing_events) {
-        FLK_HIP(hipEventSynchronize(e.second));
         float ms = 0.f;
-        FLK_HIP(hipEventElapsedTime(&ms, e.first, e.second));
+        hipError_t err = hipEventSynchronize(e.second);
+        if (err == hipSuccess) err = hipEventElapsedTime(&ms, e.first, e.second);
+        if (err != hipSuccess) {
+            (void)hipGetLastError();       // do not leave the error for the next launch check to find
+            timing_clear_locked();
+            return fail(FLK_EHIP, "reading a kernel timing event failed: %s", hipGetErrorString(err));
+        }
         tot += ms;
     }
     *total_ms = tot;
@@ -765,6 +777,30 @@ int flk_gauss_fdmmv_noalloc(const void *X1, int64_t n, int64_t x1_rs, int64_t x1
     // vectors including their zero planes, partial sums), so what the previous call left behind needs no clearing
     return flk_kernel_fdmmv(FLK_GAUSSIAN, X1, n, x1_rs, x1_cs, X2, m, x2_rs, x2_cs, d, sigma, n_sigma, v, v_rs, v_cs, w,
                             w_rs, w_cs, t, out, out_rs, out_cs, dtype, ws, (size_t)FLK_NOALLOC_SCRATCH_BYTES, stream);
+}
+
+int64_t flk_cg_state_ints(int64_t t) { return t < 0 ? 0 : 2 + 3 * t; }
+
+int flk_cg_update(int mode, void *X, void *R, void *P, const void *Q, const void *B, int64_t m, int64_t t, int64_t rs,
+                  int64_t cs, void *rsold, int32_t *state, int64_t iteration, double eps, double tol2, int differential,
+                  int dtype, void *stream) {
+    g_err[0] = 0;
+    if (mode < 0 || mode > 2) return fail(FLK_EINVAL, "flk_cg_update: mode %d (0: whole iteration, 1 / 2: its halves)", mode);
+    if (m < 0 || t < 0 || iteration < 0) return fail(FLK_EINVAL, "flk_cg_update: negative size or iteration");
+    if (t > 65535) return fail(FLK_EUNSUPPORTED, "flk_cg_update: more than 65535 right-hand sides");
+    if (m == 0 || t == 0) return FLK_OK;
+    if (!X || !P || !Q || !rsold || !state || (mode != 1 && !R) || (mode == 2 && !B))
+        return fail(FLK_EINVAL, "flk_cg_update: null pointer");
+    if (m > 1 && t > 1 && rs != 1 && cs != 1) return fail(FLK_EINVAL, "flk_cg_update: neither stride is one");
+    const int parity = (int)(iteration & 1);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == FLK_F32)
+        return launch_cg_update<float>(mode, (float *)X, (float *)R, (float *)P, (const float *)Q, (const float *)B, m, t, rs,
+                                       cs, (float *)rsold, state, parity, eps, tol2, differential, st);
+    if (dtype == FLK_F64)
+        return launch_cg_update<double>(mode, (double *)X, (double *)R, (double *)P, (const double *)Q, (const double *)B,
+                                        m, t, rs, cs, (double *)rsold, state, parity, eps, tol2, differential, st);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
 }
 
 size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype, int compute_f64) {

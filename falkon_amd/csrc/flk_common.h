@@ -134,6 +134,11 @@ int launch_finalize(const T *partial, int splits, int64_t t, int64_t nb, int64_t
                     int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
                     const T *row_half_norm, hipStream_t st);
 
+// One conjugate-gradient iteration's vector updates for t right-hand sides (cg.hip).
+template <typename T>
+int launch_cg_update(int mode, T *X, T *R, T *P, const T *Q, const T *B, int64_t m, int64_t t, int64_t rs, int64_t cs,
+                     T *rsold, int *state, int parity, double eps, double tol2, int differential, hipStream_t st);
+
 // Register-resident ("small d") product kernel; the queries do not depend on the kernel function.
 template <typename T> int64_t mmv_small_max_d();
 // (t: right-hand sides of the call; the fp32 kernels switch to their 32-column variant beyond a few columns)

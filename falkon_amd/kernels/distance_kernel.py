@@ -68,17 +68,17 @@ class _RadialKernel(DiffKernel):
         self._sigma_cache = {}
 
     def _sigma_on(self, device: torch.device, dtype: torch.dtype, cached: bool = True) -> torch.Tensor:
-        """sigma on the data's device and dtype (distance_kernel.py:148), cached until sigma changes.  Writes
-        through ``sigma.data`` (numerical differentiation does that) do not show in the version counter the
-        cache is keyed on: differentiable calls pass ``cached=False``."""
-        sigma = self.sigma
-        if not cached:
-            return sigma.detach().reshape(-1).to(device=device, dtype=dtype).contiguous()
+        """sigma on the data's device and dtype (distance_kernel.py:148).  A host-resident sigma (the usual case) is
+        uploaded once per (device, dtype) and again whenever its VALUES differ from the snapshot taken at the upload:
+        the comparison is of 1 or d host numbers, and unlike the tensor's version counter it also sees writes through
+        ``sigma.data``.  A sigma that already lives on the GPU is used (or converted) as it is on every call."""
+        sigma = self.sigma.detach().reshape(-1)
+        if not cached or sigma.device.type != "cpu":
+            return sigma.to(device=device, dtype=dtype).contiguous()
         key = (device, dtype)
-        tag = (sigma.data_ptr(), sigma._version, sigma.numel())
         hit = self._sigma_cache.get(key)
-        if hit is None or hit[0] != tag:
-            hit = (tag, sigma.detach().reshape(-1).to(device=device, dtype=dtype).contiguous())
+        if hit is None or hit[0].shape != sigma.shape or not torch.equal(hit[0], sigma):
+            hit = (sigma.clone(), sigma.to(device=device, dtype=dtype).contiguous())
             self._sigma_cache[key] = hit
         return hit[1]
 

@@ -265,12 +265,13 @@ class _KernelMmvFn(torch.autograd.Function):
 # ---------------------------------------------------------------------------
 # many right-hand sides: kernel blocks stored once, contracted by library GEMMs
 # ---------------------------------------------------------------------------
-# The product kernels never store K and pay for it by evaluating K once per pass of 16 or 32 right-hand sides.
-# With many right-hand sides that is the wrong trade: a stored kernel value costs 4 (8) bytes written and a read per
-# product.  Beyond the break-even the drivers therefore do what the reference does on every call
+# The product kernels never store K and pay for it by evaluating K once per pass of 16 to 64 right-hand sides.  That
+# is the default for any number of right-hand sides.  ``FalkonOptions(many_rhs_stored_blocks=True)`` opts into the
+# other trade where it is the faster one: a stored kernel value costs 4 (8) bytes written and a read per product, so
+# beyond a break-even the drivers then do what the reference does on every call
 # (falkon/mmv_ops/fmmv.py:358-396,740-762): evaluate a block of rows of K with the kernel-matrix kernel and contract it
 # with rocBLAS (``K_b @ v``, ``K_b.T @ u``), block by block, K blocks as large as the memory budget allows, and K
-# evaluated once for both products of ``fdmmv``.  ``FalkonOptions.never_store_kernel`` switches this off.
+# evaluated once for both products of ``fdmmv``.  ``FalkonOptions.never_store_kernel`` overrides the option.
 # Break-even in passes of the product kernels, measured on one MI355X (N = 2.5e5 .. 1e6, M = 1e4 .. 2e4):
 #   d = 784: T = 17 (2 passes) fp32 mmv 61.9 -> 32.6 ms, dmmv 122 -> 35 ms; T = 256: 986 -> 49 ms; fp64 2097 -> 114 ms;
 #   d = 100: T = 17 fp32 mmv 40.9 -> 29.1, dmmv 81 -> 36; T = 256: 741 -> 94;
@@ -286,8 +287,9 @@ def _columns_per_pass(d: int, dtype: torch.dtype) -> int:
 
 
 def _explicit_blocks_pay(d: int, t: int, dtype: torch.dtype, opt: BaseOptions) -> bool:
-    """Whether t right-hand sides are enough passes of the product kernels for stored blocks of K to be faster."""
-    if getattr(opt, "never_store_kernel", False):
+    """Whether the caller opted into stored blocks of K (``many_rhs_stored_blocks``) and t right-hand sides are
+    enough passes of the product kernels for them to be the faster route."""
+    if getattr(opt, "never_store_kernel", False) or not getattr(opt, "many_rhs_stored_blocks", False):
         return False
     passes = -(-t // _columns_per_pass(d, dtype))
     if d > 64:
@@ -452,7 +454,8 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
         # (opt-in beyond 64 features whatever T: a stored block costs about one pass of the product kernel there,
         # and K^T(K v + w) then needs K once instead of twice; C4: 122 -> 69 ms.  Off by default: the path is
         # specified as one that never materialises K.)
-        stored = _explicit_blocks_pay(D, T, X1.dtype, opt) or (getattr(opt, "dmmv_stored_blocks", False) and D > 64)
+        stored = _explicit_blocks_pay(D, T, X1.dtype, opt) or (
+            getattr(opt, "dmmv_stored_blocks", False) and D > 64 and not getattr(opt, "never_store_kernel", False))
         if N > 0 and M > 0 and stored:
             if _fdmmv_explicit(X1, X2, v, w, out, sigma_dev, kernel_fn, dev, opt):
                 return out

@@ -20,8 +20,19 @@ class ConjugateGradient:
     """Conjugate gradient on ``A X = B`` for several right-hand sides at once (one column each, with its own
     step lengths), ``A`` given as a product callback.  Same iteration, constants and stopping rule as
     falkon/optim/conjgrad.py:53-185: ``eps`` guards the two divisions, the residual is recomputed from scratch
-    every ``cg_full_gradient_every`` iterations, and the solve stops once every column has
-    ``|r|^2 < cg_tolerance^2``.  Differential convergence is not carried over."""
+    every ``cg_full_gradient_every`` iterations, the solve stops once every column has
+    ``|r|^2 < cg_tolerance^2``, and with ``cg_differential_convergence`` a column that has converged is frozen at
+    its value while the others go on (:113-161).
+
+    GPU tensors take the device-resident iteration (``flk_cg_update``): one launch does the vector work of an
+    iteration, step lengths and convergence flags stay on the device, and the host looks at the flags only every
+    ``CHECK_EVERY`` iterations (every iteration when a callback wants the solution), so iterations are enqueued
+    without waiting for each other.  Once every column has converged the remaining launches of that window leave the
+    solution untouched: the result is the one the reference's ``break`` gives.  With ``cg_capture_graph`` every kind
+    of iteration is captured once into a HIP graph (operator and update together) and replayed.  Host tensors run
+    the same iteration in torch ops."""
+
+    CHECK_EVERY = 5
 
     def __init__(self, opt: Optional[ConjugateGradientOptions] = None):
         self.params = opt if opt is not None else ConjugateGradientOptions()
@@ -29,6 +40,97 @@ class ConjugateGradient:
 
     def solve(self, X0: Optional[torch.Tensor], B: torch.Tensor, mmv: Callable[[torch.Tensor], torch.Tensor],
               max_iter: int, callback: Optional[Callable[[int, torch.Tensor, float], None]] = None) -> torch.Tensor:
+        if B.is_cuda and B.dim() == 2 and B.dtype in (torch.float32, torch.float64) and B.numel() > 0:
+            return self._solve_on_device(X0, B, mmv, max_iter, callback)
+        return self._solve_in_torch_ops(X0, B, mmv, max_iter, callback)
+
+    # ------------------------------------------------------------------ GPU tensors
+    def _solve_on_device(self, X0, B, mmv, max_iter, callback) -> torch.Tensor:
+        from . import _backend
+        lib = _backend.load()
+        started = time.time()
+        dev, (m, t) = B.device, B.shape
+        if 1 not in B.stride() and m > 1 and t > 1:
+            B = B.contiguous()
+        strides = B.stride()
+
+        def like_b(src=None):
+            buf = torch.empty_strided((m, t), strides, dtype=B.dtype, device=dev)
+            return buf if src is None else buf.copy_(src)
+
+        def same_layout(x):
+            return x if (x.stride() == strides and x.dtype == B.dtype) else like_b(x)
+
+        if X0 is None:
+            sol, resid = like_b().zero_(), like_b(B)
+        else:
+            sol, resid = same_layout(X0), like_b(B - mmv(X0))
+        direction = like_b(resid)
+        rsold = (resid * resid).sum(0).contiguous()
+        state = torch.zeros(int(lib.flk_cg_state_ints(t)), dtype=torch.int32, device=dev)
+        code = _backend.FLK_F32 if B.dtype == torch.float32 else _backend.FLK_F64
+        eps = float(self.params.cg_epsilon(B.dtype))
+        tol2 = float(self.params.cg_tolerance) ** 2
+        refresh = self.params.cg_full_gradient_every or 2 * max_iter
+        differential = int(bool(self.params.cg_differential_convergence) and t > 1)
+        rs, cs = strides
+
+        def update(mode, q, it):
+            q = same_layout(q)
+            with torch.cuda.device(dev):
+                rc = lib.flk_cg_update(mode, sol.data_ptr(), resid.data_ptr(), direction.data_ptr(), q.data_ptr(),
+                                       B.data_ptr(), m, t, rs, cs, rsold.data_ptr(), state.data_ptr(), it, eps, tol2,
+                                       differential, code, torch.cuda.current_stream(dev).cuda_stream)
+            _backend.raise_for_status(rc, "flk_cg_update")
+
+        def iteration(it):
+            if (it + 1) % refresh:
+                update(0, mmv(direction), it)
+            else:                                   # step, then the residual from scratch: R = B - A X
+                update(1, mmv(direction), it)
+                update(2, mmv(sol), it)
+
+        graphs, pool = {}, None
+        use_graph = bool(getattr(self.params, "cg_capture_graph", False))
+        every = 1 if callback is not None else self.CHECK_EVERY
+        elapsed = time.time() - started
+        applied = 0
+        for it in range(max_iter):
+            started = time.time()
+            if use_graph and it > 0:                # the first iteration runs eagerly (library set-up, lazy loads)
+                key = (bool((it + 1) % refresh), it & 1)
+                if key not in graphs:
+                    g = torch.cuda.CUDAGraph()
+                    pool = torch.cuda.graph_pool_handle() if pool is None else pool
+                    with torch.cuda.graph(g, pool=pool):
+                        iteration(it)
+                    graphs[key] = g
+                graphs[key].replay()
+            else:
+                iteration(it)
+            applied = it + 1
+            stop = False
+            if (it + 1) % every == 0 or it + 1 == max_iter:
+                flags = state.cpu()                 # waits for the iterations enqueued so far
+                applied = int(flags[1])
+                stop = bool(flags[2 + (it & 1) * t: 2 + (it & 1) * t + t].all())
+            if stop:
+                break
+            elapsed += time.time() - started
+            if callback is not None:
+                try:
+                    callback(it + 1, sol, elapsed)
+                except StopOptimizationException as stop_exc:
+                    print(f"Optimization stopped from callback: {stop_exc.message}")
+                    break
+        self.num_iter = max(applied - 1, 0) if max_iter > 0 else None
+        if X0 is not None and sol is not X0:
+            X0.copy_(sol)
+            return X0
+        return sol
+
+    # ------------------------------------------------------------------ host tensors
+    def _solve_in_torch_ops(self, X0, B, mmv, max_iter, callback) -> torch.Tensor:
         started = time.time()
         if X0 is None:
             sol, resid = torch.zeros_like(B), B.clone()
@@ -37,6 +139,8 @@ class ConjugateGradient:
         eps = self.params.cg_epsilon(sol.dtype)
         refresh = self.params.cg_full_gradient_every or 2 * max_iter
         stop_below = self.params.cg_tolerance ** 2
+        differential = bool(self.params.cg_differential_convergence) and sol.dim() == 2 and sol.shape[1] > 1
+        frozen = torch.zeros(sol.shape[1], dtype=torch.bool, device=sol.device) if differential else None
         direction = resid.clone()
         rr = (resid * resid).sum(0)                       # squared residual norm of every column
         elapsed = time.time() - started
@@ -45,15 +149,22 @@ class ConjugateGradient:
             started = time.time()
             a_dir = mmv(direction)
             step = rr / ((direction * a_dir).sum(0) + eps)
+            if differential:
+                step = torch.where(frozen, torch.zeros_like(step), step)      # frozen columns no longer move
             sol += direction * step
             if (it + 1) % refresh:
                 resid -= a_dir * step
             else:
                 if sol.is_cuda:
                     torch.cuda.synchronize()
-                resid = B - mmv(sol)
+                fresh = B - mmv(sol)
+                resid = torch.where(frozen, resid, fresh) if differential else fresh
             rr_next = (resid * resid).sum(0)
-            if bool((rr_next < stop_below).all()):
+            converged = rr_next < stop_below
+            if differential:
+                frozen |= converged
+                converged = frozen
+            if bool(converged.all()):
                 break
             direction *= rr_next / (rr + eps)
             direction += resid
@@ -81,7 +192,7 @@ class FalkonConjugateGradient:
         self.kernel, self.preconditioner, self.params, self.weight_fn = kernel, preconditioner, opt, weight_fn
         self.stored_knm = stored_knm
         cg_fields = ("cg_epsilon_32", "cg_epsilon_64", "cg_tolerance", "cg_full_gradient_every",
-                     "cg_differential_convergence")
+                     "cg_differential_convergence", "cg_capture_graph")
         self.optimizer = ConjugateGradient(ConjugateGradientOptions(**{f: getattr(opt, f) for f in cg_fields}))
 
     def falkon_mmv(self, sol, penalty, X, M, n: int):

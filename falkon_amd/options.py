@@ -34,12 +34,16 @@ class BaseOptions:
     min_cuda_pc_size_64: int = 30000                  # carried, unused
     min_cuda_iter_size_32: int = 10_000 * 10 * 3_000  # carried, unused
     min_cuda_iter_size_64: int = 30_000 * 10 * 3_000  # carried, unused
-    never_store_kernel: bool = False                  # True: never store blocks of K, however many right-hand sides
+    never_store_kernel: bool = False                  # True: never store K (overrides the two *_stored_blocks options
+                                                      # and the stored K(X, centres) of a fit)
     store_kernel_d_threshold: int = 1200              # beyond this many features a fit keeps K(X, centres) if it fits
     num_fmm_streams: int = 2                          # carried, unused
     memory_slack: float = 0.9                         # fraction of the free device memory a call may plan with
     bf16x3_cross_term: bool = False                   # not in the reference: fp32 products form x.c on the bf16 matrix
                                                       # cores from an exact 3-way bfloat16 split (fp32 accuracy)
+    many_rhs_stored_blocks: bool = False              # not in the reference's options: with many right-hand sides
+                                                      # (several passes of the product kernels) store blocks of K and
+                                                      # contract them with rocBLAS; off: every product is matrix-free
     dmmv_stored_blocks: bool = False                  # not in the reference's options: K^T(K v + w) beyond 64 features
                                                       # evaluates K once, into stored blocks, whatever T (see fmmv.py)
 
@@ -58,7 +62,9 @@ class ConjugateGradientOptions:
     cg_epsilon_64: float = 1e-15                      # ... in fp64
     cg_tolerance: float = 1e-7                        # stop once every column has |r| below this
     cg_full_gradient_every: int = 10                  # recompute the residual from scratch this often
-    cg_differential_convergence: bool = False         # carried, not implemented
+    cg_differential_convergence: bool = False         # a converged column is frozen while the others go on
+    cg_capture_graph: bool = False                    # not in the reference: GPU solves capture each kind of iteration
+                                                      # (operator + update) into a HIP graph once and replay it
 
     def cg_epsilon(self, dtype):
         return _by_precision(dtype, self.cg_epsilon_32, self.cg_epsilon_64)

@@ -166,6 +166,30 @@ int flk_gauss_fdmmv_noalloc(const void *X1, int64_t n, int64_t x1_rs, int64_t x1
                             const void *w, int64_t w_rs, int64_t w_cs, int64_t t,
                             void *out, int64_t out_rs, int64_t out_cs, int dtype, void *stream);
 
+/* ---- conjugate-gradient iteration on device scalars ---------------------------
+ * flk_cg_update replaces the vector work of one iteration of the reference's multi-right-hand-side solver
+ * (falkon/optim/conjgrad.py:125-163: alpha = rsold / (sum(P * AP) + eps); X += P alpha; R -= AP alpha (or
+ * R = B - A X every cg_full_gradient_every iterations); rsnew = sum(R^2); converged = rsnew < tol^2, stop when
+ * every column has; P = R + P rsnew / (rsold + eps)), one workgroup per right-hand side, with the step lengths,
+ * residual norms and convergence flags kept on the device, so that the host need not wait for an iteration
+ * before it enqueues the next.  X, R, P, Q, B are m x t with the same element strides (rs, cs), one of them 1.
+ *   mode 0: whole iteration, Q = A P.
+ *   mode 1: step length and X += P alpha only, Q = A P; then, with Q = A X,
+ *   mode 2: R = B - Q and the rest of the iteration (the reference's full-gradient iterations, :133-138).
+ * rsold: t squared residual norms in the data dtype, set by the caller to sum(R^2) before the first iteration.
+ * state: flk_cg_state_ints(t) int32, zeroed by the caller before the first iteration: [0] becomes 1 once every
+ *   column has converged, and every later call then leaves X, R, P untouched (the reference's break, :143-145);
+ *   [1] counts the iterations applied; [2 .. 2+2t) are the columns' convergence flags of the last two iterations;
+ *   [2+2t .. 2+3t) marks columns that left the solve (differential != 0: a converged column is frozen at its
+ *   value, the reference's cg_differential_convergence, :113-161).
+ * iteration: index of the iteration (its parity selects the flag buffer); mode 1 and mode 2 of one iteration pass
+ *   the same value.  Sums are taken in a fixed order in double precision: results are reproducible. */
+int64_t flk_cg_state_ints(int64_t t);
+
+int flk_cg_update(int mode, void *X, void *R, void *P, const void *Q, const void *B, int64_t m, int64_t t,
+                  int64_t rs, int64_t cs, void *rsold, int32_t *state, int64_t iteration,
+                  double eps, double tol2, int differential, int dtype, void *stream);
+
 /* ---- explicit kernel matrix -------------------------------------------------
  * flk_gauss_fmm replaces falkon.mmv_ops.fmm.fmm for the dense Gaussian case
  *   (falkon/mmv_ops/fmm.py:699-708 -> :298-388 block loop -> distance_kernel.py:140-159):

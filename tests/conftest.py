@@ -41,11 +41,13 @@ def check_parity(got, ref_same_dtype, ref_f64, tol: float) -> None:
     """Parity of a GPU result with the reference-equivalent CPU path.
 
     ``ref_same_dtype`` is the CPU oracle run in the data's dtype, ``ref_f64`` the same path run in
-    fp64 on the same (exactly widened) inputs.  The GPU result must be within ``tol`` of the CPU
-    result in its own dtype; where the CPU fp32 path itself is further than tol/2 from its fp64 twin
-    (ill-conditioned sums: long fp32 accumulations, output columns that nearly cancel) two fp32
-    results cannot be expected to agree to ``tol``, and the GPU result must instead be at least as
-    close to the fp64 path as the CPU fp32 path is (factor 2 of slack).
+    fp64 on the same (exactly widened) inputs, both computed on the CPU.  The GPU result must be within
+    ``tol`` of the CPU result in its own dtype.  Where the CPU fp32 path itself is further than tol/2
+    from its fp64 twin (ill-conditioned sums: long fp32 accumulations, output columns that nearly
+    cancel) two fp32 results cannot be expected to agree to ``tol``; this is a relaxation of the
+    literal bar and it is bounded: the GPU result must then be at least as close to the fp64 CPU path
+    as the CPU fp32 path is (factor 2 of slack), and never further than ``10 * tol`` from it, however
+    far the CPU fp32 path has drifted.
     """
     e_ref = rel_err(ref_same_dtype, ref_f64)
     if e_ref < tol / 2:
@@ -53,4 +55,5 @@ def check_parity(got, ref_same_dtype, ref_f64, tol: float) -> None:
         assert e < tol, f"GPU vs CPU oracle: {e:.3e} >= {tol:.1e} (CPU fp32 vs fp64: {e_ref:.3e})"
     else:
         e = rel_err(got, ref_f64)
-        assert e < max(tol, 2 * e_ref), f"GPU vs fp64 oracle: {e:.3e}; CPU fp32 path vs fp64: {e_ref:.3e}"
+        bound = min(max(tol, 2 * e_ref), 10 * tol)
+        assert e < bound, f"GPU vs fp64 oracle: {e:.3e} >= {bound:.1e}; CPU fp32 path vs fp64: {e_ref:.3e}"

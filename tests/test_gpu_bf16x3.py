@@ -29,7 +29,7 @@ def test_products_vs_oracle(dev, d, t):
     n, m = 700 + 3 * d, 190 + d
     X, C, v, w = _data(n, m, d, t, seed=d + 100 * t)
     sigma = torch.tensor([0.9 * np.sqrt(d)], dtype=torch.float64)
-    k = GaussianKernel(sigma, opt=SPLIT)
+    k = GaussianKernel(sigma, opt=FalkonOptions(bf16x3_cross_term=True, many_rhs_stored_blocks=True))
     Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
     Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
     check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)
@@ -63,7 +63,7 @@ def test_lds_tiled_kernel_vs_oracle(dev, n, m, d, t):
     """Feature counts beyond 62 run the LDS-tiled kernel of the mode: both epilogues, ragged tiles."""
     X, C, v, w = _data(n, m, d, t, seed=n + d)
     sigma = torch.tensor([0.9 * np.sqrt(d)], dtype=torch.float64)
-    k = GaussianKernel(sigma, opt=SPLIT)
+    k = GaussianKernel(sigma, opt=FalkonOptions(bf16x3_cross_term=True, many_rhs_stored_blocks=True))
     Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
     Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
     check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)
@@ -229,7 +229,7 @@ def test_stored_block_route_in_the_mode(dev):
     n, m, d, t = 700, 300, 100, 40
     X, C, v, w = _data(n, m, d, t, seed=11)
     sigma = torch.tensor([0.9 * np.sqrt(d)], dtype=torch.float64)
-    k = GaussianKernel(sigma, opt=SPLIT)
+    k = GaussianKernel(sigma, opt=FalkonOptions(bf16x3_cross_term=True, many_rhs_stored_blocks=True))
     Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
     Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
     check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)

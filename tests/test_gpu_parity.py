@@ -113,8 +113,8 @@ def test_large_d_vs_oracle(dev, dtype, n, m, d, t):
     assert rel_err(got_mmv, mmv_ref.fmmv_ref(X, C, v, sigma)) < TOL[dtype]
     assert rel_err(got_dmmv, mmv_ref.fdmmv_ref(X, C, v, w, sigma)) < TOL[dtype]
     assert rel_err(got_mmv, brute.mmv_brute(X, C, sigma, v)) < 5 * TOL[dtype]
-    if t > 16:      # enough columns for the stored-block route: the product kernels' multi-pass route as well
-        kf = GaussianKernel(sigma, opt=FalkonOptions(never_store_kernel=True))
+    if t > 16:      # several passes of the product kernels above; the opt-in stored-block route as well
+        kf = GaussianKernel(sigma, opt=FalkonOptions(many_rhs_stored_blocks=True))
         assert rel_err(kf.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma)) < TOL[dtype]
         assert rel_err(kf.dmmv(Xg, Cg, vg, wg), mmv_ref.fdmmv_ref(X, C, v, w, sigma)) < TOL[dtype]
 
@@ -152,6 +152,18 @@ def test_per_dimension_sigma_fp32(dev):
     s32 = sigma.float()
     got1 = k1.dmmv((X / s32).to(dev), (C / s32).to(dev), v.to(dev), None)
     assert rel_err(got, got1) < 1e-5
+
+
+def test_sigma_changed_through_data_is_seen(dev):
+    """mmv, dmmv and the kernel matrix after ``sigma.data.fill_``: the results of a kernel built with the new value."""
+    X, C, v, w = (a.to(dev) for a in _rand(500, 7, 120, 2, torch.float32, seed=5))
+    k = GaussianKernel(2.0)
+    before = k.dmmv(X, C, v, w)
+    k.sigma.data.fill_(3.5)
+    fresh = GaussianKernel(3.5)
+    assert torch.equal(k.dmmv(X, C, v, w), fresh.dmmv(X, C, v, w)) and not torch.equal(before, fresh.dmmv(X, C, v, w))
+    assert torch.equal(k.mmv(X, C, v), fresh.mmv(X, C, v))
+    assert torch.equal(k(X, C), fresh(X, C))
 
 
 def test_wrong_sigma_length_raises(dev):
@@ -425,6 +437,35 @@ def test_many_right_hand_sides_small_d(dev, d, t):
     assert rel_err(got[:, [0, t - 1]], cols) < 5e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("t", [33, 64, 65, 128])
+@pytest.mark.parametrize("d", [9, 28, 40, 100])
+def test_many_right_hand_sides_stay_matrix_free(dev, dtype, d, t, monkeypatch):
+    """33 to 128 right-hand sides on the default route: several passes of the product kernels, no stored block of K
+    (the kernel-matrix entry point is never reached), parity with the CPU path, bit-identical repeats, and the same
+    numbers as the single-column kernels on the first and last column.  The shapes of the reference's own timing of
+    this case: falkon/benchmarks/timing_benchmarks/mmv_timings.py:48-127 (T = 10 .. 100)."""
+    import importlib
+    fmm_mod = importlib.import_module("falkon_amd.mmv_ops.fmm")
+
+    def refuse(*a, **k):
+        raise AssertionError("a kernel matrix was stored on the default route")
+    monkeypatch.setattr(fmm_mod, "gauss_fmm_native", refuse)
+    n, m = 700 + d, 257
+    X, C, v, w = _rand(n, d, m, t, dtype, seed=d * 1000 + t, scale=0.7)
+    sigma = 0.9 * np.sqrt(d)
+    k = GaussianKernel(sigma)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+    tol = TOL[dtype]
+    got_m, got_d = k.mmv(Xg, Cg, vg), k.dmmv(Xg, Cg, vg, wg)
+    check_parity(got_m, mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), tol)
+    check_parity(got_d, mmv_ref.fdmmv_ref(X, C, v, w, sigma), mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), tol)
+    assert torch.equal(got_d, k.dmmv(Xg, Cg, vg, wg))
+    cols = torch.cat([k.dmmv(Xg, Cg, vg[:, i:i + 1].contiguous(), wg[:, i:i + 1].contiguous()) for i in (0, t - 1)], 1)
+    assert rel_err(got_d[:, [0, t - 1]], cols) < (5e-6 if dtype == torch.float32 else 1e-12)
+
+
 @pytest.mark.parametrize("mode", ["f32", "f64", "bf16x3"])
 @pytest.mark.parametrize("d,t", [(8, 1), (28, 2), (28, 20), (40, 6), (100, 1), (100, 10)])
 def test_non_finite_rows_give_nan(dev, mode, d, t):
@@ -573,16 +614,17 @@ def test_packed_entry_points(dev, dtype, n, m, d, t):
 @pytest.mark.parametrize("n,m,d,t", [(700, 300, 100, 20), (300, 520, 784, 40), (2000, 333, 28, 130), (900, 257, 40, 70),
                                      (500, 129, 9, 200)])
 def test_many_right_hand_sides_through_stored_blocks(dev, dtype, n, m, d, t, monkeypatch):
-    """Enough right-hand sides that the drivers store blocks of K and contract them with library GEMMs (the
-    reference's own scheme, falkon/mmv_ops/fmmv.py:358-396,740-762): same tolerances against the CPU path, agreement
-    with the product kernels (``never_store_kernel=True``), several blocks (block size forced down), strided
+    """Opt-in ``many_rhs_stored_blocks``: with enough right-hand sides the drivers store blocks of K and contract them
+    with library GEMMs (the reference's own scheme, falkon/mmv_ops/fmmv.py:358-396,740-762): same tolerances against
+    the CPU path, agreement with the matrix-free default, several blocks (block size forced down), strided
     operands, ``out=``, host data, ``w = None``."""
     import importlib
     drv = importlib.import_module("falkon_amd.mmv_ops.fmmv")
-    assert drv._explicit_blocks_pay(d, t, dtype, FalkonOptions()) or dtype == torch.float64 and d <= 64 and t < 65
+    stored = FalkonOptions(many_rhs_stored_blocks=True)
+    assert drv._explicit_blocks_pay(d, t, dtype, stored) or dtype == torch.float64 and d <= 64 and t < 65
     X, C, v, w = _rand(n, d, m, t, dtype, seed=n + t, scale=0.6)
     sigma = 0.8 * np.sqrt(d)
-    k, k_free = GaussianKernel(sigma), GaussianKernel(sigma, opt=FalkonOptions(never_store_kernel=True))
+    k, k_free = GaussianKernel(sigma, opt=stored), GaussianKernel(sigma)
     Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
     Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
     tol = TOL[dtype]

@@ -109,6 +109,23 @@ def test_validate_sigma_and_kernel_object():
     torch.testing.assert_close(K, torch.exp(-0.5 * torch.cdist(X / s, C / s) ** 2), rtol=1e-10, atol=1e-12)
 
 
+def test_sigma_copy_follows_writes_through_data():
+    """The copy of sigma the kernels read is refreshed when sigma's values change, also through ``sigma.data``,
+    which leaves the tensor's version counter alone (manual hyper-parameter updates do that)."""
+    cpu = torch.device("cpu")
+    k = GaussianKernel(torch.tensor([1.0, 2.0, 3.0]))
+    first = k._sigma_on(cpu, torch.float32)
+    assert first.dtype == torch.float32 and first.tolist() == [1.0, 2.0, 3.0]
+    assert k._sigma_on(cpu, torch.float32) is first                    # unchanged values: the same copy
+    version = k.sigma._version
+    k.sigma.data.mul_(2.0)
+    assert k.sigma._version == version                                 # invisible to the version counter
+    assert k._sigma_on(cpu, torch.float32).tolist() == [2.0, 4.0, 6.0]
+    k.sigma.data.fill_(5.0)
+    assert k._sigma_on(cpu, torch.float64).tolist() == [5.0, 5.0, 5.0]
+    assert k._sigma_on(cpu, torch.float32).tolist() == [5.0, 5.0, 5.0]
+
+
 def test_dimension_and_dtype_checks_match_reference():
     """falkon/kernels/kernel.py:44-105."""
     k = GaussianKernel(1.0)
@@ -294,15 +311,18 @@ def test_stored_block_route_rules(monkeypatch):
     the blocks are, and the options that switch the route off or on."""
     import importlib
     drv = importlib.import_module("falkon_amd.mmv_ops.fmmv")
-    opt = FalkonOptions()
     f32, f64 = torch.float32, torch.float64
+    # off by default, whatever the number of right-hand sides: every product is matrix-free unless the caller opts in
+    assert not any(drv._explicit_blocks_pay(d, t, dt, FalkonOptions())
+                   for d in (9, 28, 100, 784) for t in (1, 17, 97, 1000, 10**4) for dt in (f32, f64))
+    opt = FalkonOptions(many_rhs_stored_blocks=True)
     # one pass of the product kernels: never; two passes beyond 64 features; four (fp32) / five (fp64) at small d
     assert not drv._explicit_blocks_pay(784, 16, f32, opt) and drv._explicit_blocks_pay(784, 17, f32, opt)
     assert not drv._explicit_blocks_pay(28, 96, f32, opt) and drv._explicit_blocks_pay(28, 97, f32, opt)
     assert not drv._explicit_blocks_pay(40, 64, f32, opt) and drv._explicit_blocks_pay(40, 65, f32, opt)
     assert not drv._explicit_blocks_pay(28, 64, f64, opt) and drv._explicit_blocks_pay(28, 65, f64, opt)
     assert drv._explicit_blocks_pay(100, 17, f64, opt)
-    assert not drv._explicit_blocks_pay(784, 1000, f32, FalkonOptions(never_store_kernel=True))
+    assert not drv._explicit_blocks_pay(784, 1000, f32, FalkonOptions(many_rhs_stored_blocks=True, never_store_kernel=True))
     # block rows: within the block size, within half of what the budget leaves, nothing below 32 rows
     monkeypatch.setattr(drv, "usable_gpu_memory", lambda dev, cap, slack, enough=float("inf"): 64 * 2**30)
     rows = drv._explicit_block_rows(10**6, 10_000, 784, 256, 4, None, opt, upload_bytes=0)
