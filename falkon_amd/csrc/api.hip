@@ -111,6 +111,10 @@ static void plan_register_resident(Plan &p, int64_t na_blocks, int64_t nb_blocks
     if (splits < 1) splits = 1;
     p.chunk = (na_blocks + splits - 1) / splits;
     if (p.chunk < 1) p.chunk = 1;
+    // even chunks for one right-hand side: the single-column fp32 kernel's loop handles two blocks per trip and
+    // processes the last block of an odd chunk twice (the second time against zeros), which then happens in the last
+    // chunk at most
+    if (t == 1 && p.chunk > 1 && (p.chunk & 1)) p.chunk += 1;
     p.splits = (int)((na_blocks + p.chunk - 1) / p.chunk);
     if (p.splits < 1) p.splits = 1;
     p.partials = p.splits;

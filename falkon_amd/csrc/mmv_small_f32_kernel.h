@@ -46,12 +46,15 @@ __device__ __forceinline__ void fetch_rowvals(RowVals<TT> &rv, const float *cons
     for (int c = 0; c < RowVals<TT>::C; c++) rv.x[c] = src[c][ab * 32];
 }
 
+// keep = 0 clears the right-hand side entries of the block (its kernel values then contribute nothing to the sums):
+// for the block that is processed a second time when a chunk holds an odd number of blocks.  Applied here and not
+// where the values are fetched, so that nothing touches the loaded registers before the tile step in between is done.
 template <int TT>
-__device__ __forceinline__ void stage_rowvals(const RowVals<TT> &rv, float *lds, int lane) {
+__device__ __forceinline__ void stage_rowvals(const RowVals<TT> &rv, float *lds, int lane, float keep = 1.0f) {
 #pragma unroll
     for (int c = 0; c < RowVals<TT>::C; c++) {
         int e = lane + 64 * c;
-        if (e < RowVals<TT>::N) lds[e] = rv.x[c];
+        if (e < RowVals<TT>::N) lds[e] = e >= 32 ? rv.x[c] * keep : rv.x[c];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -64,7 +67,15 @@ __device__ __forceinline__ void load_a(float (&a)[DP], const float *__restrict__
     for (int s = 0; s < DP; s++) a[s] = p[s * 32];
 }
 
-template <int DP, int FR, int TT, bool FOLD, int KF>
+// FOLD: the accumulators start from the A block's half norms alone (the output side's half norm arrives through the
+// MFMA chain, or, with RAW, is applied to the finished sums).  RAW (Gaussian only): the accumulator holds the exponent
+// without the output side's half norm; it can be positive, so the kernel value is the bare exp2, not clamped at 1.
+template <int KF, bool RAW> __device__ __forceinline__ float tile_value(float e) {
+    if constexpr (RAW) return __builtin_amdgcn_exp2f(e);
+    else return kernel_value<KF>(e);
+}
+
+template <int DP, int FR, int TT, bool FOLD, int KF, bool RAW = false, bool PIN = false>
 __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds, int h, const float (&breg)[FR][DP],
                                           const float (&hb)[FR], float (&o1)[FR][TT]) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -83,6 +94,9 @@ __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds
         for (int t = 0; t < TT; t++)
 #pragma unroll
             for (int g = 0; g < 4; g++) vec[t][g] = *(const floatx4 *)(lds + 32 + 32 * t + 8 * g + 4 * h);
+        // PIN (where there are registers to spare): keep these reads in front of the MFMA chain; the compiler
+        // would sink them to the epilogue, where each read then stalls the wave for the LDS latency
+        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < DP; s++)
 #pragma unroll
@@ -92,7 +106,7 @@ __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds
         for (int q = 0; q < FR; q++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                float k = kernel_value<KF>(acc[q][r]);
+                float k = tile_value<KF, RAW>(acc[q][r]);
 #pragma unroll
                 for (int t = 0; t < TT; t++) o1[q][t] = __builtin_fmaf(k, vec[t][r >> 2][r & 3], o1[q][t]);
             }
@@ -107,7 +121,7 @@ __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds
 #pragma unroll
         for (int q = 0; q < FR; q++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[q][r] = kernel_value<KF>(acc[q][r]);
+            for (int r = 0; r < 16; r++) acc[q][r] = tile_value<KF, RAW>(acc[q][r]);
         // Groups of up to four columns of one row group, software pipelined by hand: the reads of the
         // next group are issued, then a compiler memory fence pins them there, then the FMAs of the
         // current group run.  Without the fences the compiler moves all 4*TT LDS reads to the front
@@ -152,9 +166,103 @@ __device__ __forceinline__ void tile_step(const float (&a)[DP], const float *lds
     }
 }
 
+// The reduction loop of one wave over the A blocks a0 .. a1: streams the blocks (double buffered in registers, row
+// values through the wave's LDS stage) and accumulates into o1 / o2.  NOADD: the accumulators start from the A block's
+// half norms alone (see the kernel).
+template <int DP, int FR, int TT, bool NOADD, int KF, bool TWO_LEVEL, bool RAW>
+__device__ __forceinline__ void reduce_blocks(const float *__restrict__ PA, const float *const (&src)[RowVals<TT>::C],
+                                              int64_t a0, int64_t a1, int lane, int j, int h, float *lds0, float *lds1,
+                                              const float (&breg)[FR][DP], const float (&hb)[FR], float (&o1)[FR][TT],
+                                              float (&o2)[FR][TWO_LEVEL ? TT : 1]) {
+    using RV = RowVals<TT>;
+    float fa0[DP], fa1[DP];
+    RV rv;
+    if (a0 >= a1) return;
+    int since_flush = 0;
+    // One right-hand side and four resident blocks (the kernels of the single-column products at up to 32 features):
+    // a branch-free loop body with its phases pinned.  Measured on N = 1e6, M = 2e4, dfmmv: d = 28 19.95 -> 19.32 ms,
+    // d = 16 12.62 -> 12.29.  The other shapes keep the loop below (with two or four columns the pinned reads do
+    // not fit the registers; with two resident blocks it measured slower: d = 64 46.8 -> 51.3 ms).
+    if constexpr (TT == 1 && FR == 4) {
+        // Both tile steps of the body always run and every block's loads are issued unconditionally, one block ahead.
+        // (With loads or a tile step under a condition the compiler sinks the loads to their use, and at each wait
+        // has to assume that they may not have been issued, so it waits for the newest loads instead of the ones it
+        // needs.)  Past the end of the chunk the last block is loaded again: with an odd number of blocks it is
+        // processed twice, the second time against a right-hand side of zeros; the launch plans make the chunks
+        // even, so this happens in the last chunk at most.
+        // The scheduling barriers keep the phases of a step apart in the generated code: the loads of the next block
+        // are issued before the tile's arithmetic, and the staging of its row values, which has to wait for their
+        // load, stays behind the tile (hoisted to the front it waits out a full memory latency with nothing in flight).
+        const int64_t last = a1 - 1;
+        fetch_rowvals<TT>(rv, src, a0);
+        load_a<DP>(fa0, PA, a0, j, h);
+        stage_rowvals<TT>(rv, lds0, lane);
+        for (int64_t ab = a0; ab < a1; ab += 2) {
+            const bool second = ab + 1 < a1;
+            const int64_t n1 = second ? ab + 1 : last;
+            fetch_rowvals<TT>(rv, src, n1);    // first: staged right after this tile step
+            load_a<DP>(fa1, PA, n1, j, h);
+            __builtin_amdgcn_sched_barrier(0);
+            tile_step<DP, FR, TT, NOADD, KF, RAW, true>(fa0, lds0, h, breg, hb, o1);
+            __builtin_amdgcn_sched_barrier(0);
+            stage_rowvals<TT>(rv, lds1, lane, second ? 1.0f : 0.0f);
+            const int64_t n2 = ab + 2 < last ? ab + 2 : last;
+            fetch_rowvals<TT>(rv, src, n2);
+            load_a<DP>(fa0, PA, n2, j, h);
+            __builtin_amdgcn_sched_barrier(0);
+            tile_step<DP, FR, TT, NOADD, KF, RAW, true>(fa1, lds1, h, breg, hb, o1);
+            __builtin_amdgcn_sched_barrier(0);
+            stage_rowvals<TT>(rv, lds0, lane);
+            since_flush += 2;
+            if (TWO_LEVEL && since_flush >= kFlushEvery) {
+                since_flush = 0;
+#pragma unroll
+                for (int q = 0; q < FR; q++)
+#pragma unroll
+                    for (int t = 0; t < TT; t++) { o2[q][t] += o1[q][t]; o1[q][t] = 0.f; }
+            }
+        }
+    } else {
+        load_a<DP>(fa0, PA, a0, j, h);
+        fetch_rowvals<TT>(rv, src, a0);
+        stage_rowvals<TT>(rv, lds0, lane);
+        for (int64_t ab = a0; ab < a1; ab += 2) {
+            const bool has1 = ab + 1 < a1;
+            if (has1) { load_a<DP>(fa1, PA, ab + 1, j, h); fetch_rowvals<TT>(rv, src, ab + 1); }
+            tile_step<DP, FR, TT, NOADD, KF, RAW>(fa0, lds0, h, breg, hb, o1);
+            if (has1) {
+                stage_rowvals<TT>(rv, lds1, lane);
+                const bool has2 = ab + 2 < a1;
+                if (has2) { load_a<DP>(fa0, PA, ab + 2, j, h); fetch_rowvals<TT>(rv, src, ab + 2); }
+                tile_step<DP, FR, TT, NOADD, KF, RAW>(fa1, lds1, h, breg, hb, o1);
+                if (has2) stage_rowvals<TT>(rv, lds0, lane);
+            }
+            since_flush += 2;
+            if (TWO_LEVEL && since_flush >= kFlushEvery) {
+                since_flush = 0;
+#pragma unroll
+                for (int q = 0; q < FR; q++)
+#pragma unroll
+                    for (int t = 0; t < TT; t++) { o2[q][t] += o1[q][t]; o1[q][t] = 0.f; }
+            }
+        }
+    }
+}
+
+// Largest -hB (= half the squared norm of a scaled output row, in bits of the exponent) for which the Gaussian's
+// output-side half norm is taken out of the exponent: 2^(x.c + hA) <= 2^(-hB) then stays far below the fp32 range
+// (2^64 times the sum over the reduction rows of |vec| would have to overflow).
+constexpr float kFactorOutMaxBits = 64.0f;
+
 // FOLD (odd feature counts only): the one padding feature of the packed rows carries 1.0, and the
 // resident B fragment puts hB_j into that slot, so the MFMA chain adds hB_j by itself and the
 // accumulators start from the A block's half norms without any VALU add.
+// Even feature counts have no spare slot.  For the Gaussian the same adds (one per kernel value) are saved by
+// factoring the output row's half norm out of the sum: out_j = 2^hB_j * sum_i 2^(x_i.c_j + hA_i) vec_i, valid as long
+// as 2^(-hB_j) is nowhere near the fp32 range, which every wave checks on its own resident rows (kFactorOutMaxBits;
+// rows with a non-finite half norm fail the check) before it picks between the two loops.  The partial exponent
+// x.c + hA can be positive, so on that path a kernel value is not clamped entry by entry: where two points
+// coincide K is 1 to rounding (1 + 1e-6 at worst) instead of exactly 1.
 template <int DP, int FR, int TT, bool FOLD, int KF>
 __global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 registers per lane
     mmv_small_f32_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
@@ -165,6 +273,7 @@ __global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 r
     // caller's columns).
     using RV = RowVals<TT>;
     constexpr bool kTwoLevel = TT <= 4;   // long accumulator only where registers allow; wider TT uses short chunks
+    constexpr bool kCanFactorOut = !FOLD && KF == FLK_GAUSSIAN && TT <= 2;   // wider column chunks are out of registers with two loops
     __shared__ __attribute__((aligned(16))) float stage[kWavesPerWg][2][RV::N];
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
@@ -180,12 +289,14 @@ __global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 r
     // resident B fragments (blocks past the end re-read the last block; their results are not stored)
     float breg[FR][DP];
     float hb[FR];
+    [[maybe_unused]] bool small_norms = true;
 #pragma unroll
     for (int q = 0; q < FR; q++) {
         int64_t bb = bb0 + q < nb_blocks ? bb0 + q : nb_blocks - 1;
         load_a<DP>(breg[q], PB, bb, j, h);
         hb[q] = hB[bb * 32 + j];
         if (FOLD) breg[q][DP - 1] = h ? hb[q] : breg[q][DP - 1];   // feature 2*DP-1 lives in lane half 1, step DP-1
+        if constexpr (kCanFactorOut) small_norms = small_norms && hb[q] >= -kFactorOutMaxBits;   // false for NaN
     }
     // where this lane's staged dwords come from: element e = lane + 64c of [hn(32) | vec_0(32) | vec_1(32) ...]
     const float *src[RV::C];
@@ -201,44 +312,30 @@ __global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 r
 #pragma unroll
         for (int t = 0; t < TT; t++) { o1[q][t] = 0.f; if (kTwoLevel) o2[q][t] = 0.f; }
 
-    float fa0[DP], fa1[DP];
-    RV rv;
     float *lds0 = stage[wave][0], *lds1 = stage[wave][1];
-    if (a0 < a1) {
-        load_a<DP>(fa0, PA, a0, j, h);
-        fetch_rowvals<TT>(rv, src, a0);
-        stage_rowvals<TT>(rv, lds0, lane);
-    }
-    int since_flush = 0;
-    for (int64_t ab = a0; ab < a1; ab += 2) {
-        const bool has1 = ab + 1 < a1;
-        if (has1) { load_a<DP>(fa1, PA, ab + 1, j, h); fetch_rowvals<TT>(rv, src, ab + 1); }
-        tile_step<DP, FR, TT, FOLD, KF>(fa0, lds0, h, breg, hb, o1);
-        if (has1) {
-            stage_rowvals<TT>(rv, lds1, lane);
-            const bool has2 = ab + 2 < a1;
-            if (has2) { load_a<DP>(fa0, PA, ab + 2, j, h); fetch_rowvals<TT>(rv, src, ab + 2); }
-            tile_step<DP, FR, TT, FOLD, KF>(fa1, lds1, h, breg, hb, o1);
-            if (has2) stage_rowvals<TT>(rv, lds0, lane);
-        }
-        since_flush += 2;
-        if (kTwoLevel && since_flush >= kFlushEvery) {
-            since_flush = 0;
-#pragma unroll
-            for (int q = 0; q < FR; q++)
-#pragma unroll
-                for (int t = 0; t < TT; t++) { o2[q][t] += o1[q][t]; o1[q][t] = 0.f; }
-        }
+    [[maybe_unused]] bool factored = false;
+    if constexpr (kCanFactorOut) {
+        factored = __all(small_norms);      // wave-uniform
+        if (factored)
+            reduce_blocks<DP, FR, TT, true, KF, kTwoLevel, true>(PA, src, a0, a1, lane, j, h, lds0, lds1, breg, hb, o1, o2);
+        else
+            reduce_blocks<DP, FR, TT, FOLD, KF, kTwoLevel, false>(PA, src, a0, a1, lane, j, h, lds0, lds1, breg, hb, o1, o2);
+    } else {
+        reduce_blocks<DP, FR, TT, FOLD, KF, kTwoLevel, false>(PA, src, a0, a1, lane, j, h, lds0, lds1, breg, hb, o1, o2);
     }
 #pragma unroll
-    for (int q = 0; q < FR; q++)
+    for (int q = 0; q < FR; q++) {
+        [[maybe_unused]] float out_scale = 1.0f;
+        if constexpr (kCanFactorOut) out_scale = factored ? __builtin_amdgcn_exp2f(hb[q]) : 1.0f;
 #pragma unroll
         for (int t = 0; t < TT; t++) {
             float s = kTwoLevel ? o2[q][t] + o1[q][t] : o1[q][t];
             s += __shfl_xor(s, 32, 64);
+            if constexpr (kCanFactorOut) s *= out_scale;
             if (h == 0 && bb0 + q < nb_blocks && t < tcols)
                 partial[((int64_t)by * tcols + t) * nb_pad + (bb0 + q) * 32 + j] = s;
         }
+    }
 }
 
 
