@@ -49,7 +49,8 @@ inline double operand_scale(int kf) {
 // results below 2^-1021 flushed to zero, measured no faster.)
 __device__ __forceinline__ double exp2_nonpositive(double e) {
     constexpr double kRound = 6755399441055744.0;       // 1.5 * 2^52: adding it rounds to the nearest integer
-    e = fmax(e, -1100.0);
+    // (the bare instruction: the builtin would quieten a signalling NaN first, one more fp64 instruction per value)
+    asm("v_max_f64 %0, %1, %2" : "=v"(e) : "v"(e), "s"(-1100.0));
     const double t = e + kRound;
     const int n = (int)(unsigned)__double_as_longlong(t);  // the integer, in two's complement, is the low word
     const double f = e - (t - kRound);
@@ -68,6 +69,45 @@ __device__ __forceinline__ double exp2_nonpositive(double e) {
     return __builtin_ldexp(p, n);
 }
 
+// The same through a table: 2^e = 2^n * 2^(k/2048) * 2^f with N = rint(2048 e) = 2048 n + k (k the low 11 bits of
+// N, n = N >> 11) and |f| <= 2^-12, where the cubic Taylor polynomial of 2^f is exact to 3.4e-17.  tab[k] = 2^(k/2048)
+// lives in LDS (16 KB per workgroup, exp2_table_fill): ten fp64 and three 32-bit instructions in place of eighteen fp64
+// ones, and the LDS read runs beside the vector ALU.  For e <= 0 like exp2_nonpositive (a positive e up to 2^20 works
+// too); arguments below -1100 are raised to it.
+constexpr int kExpTableBits = 11;
+constexpr int kExpTableSize = 1 << kExpTableBits;
+
+// All threads of the workgroup call this once, followed by a workgroup barrier, before exp2_table is used.
+__device__ __forceinline__ void exp2_table_fill(double *tab, int tid, int nthreads) {
+    for (int k = tid; k < kExpTableSize; k += nthreads)
+        tab[k] = 2.0 * exp2_nonpositive((double)(k - kExpTableSize) * (1.0 / kExpTableSize));
+}
+
+__device__ __forceinline__ double exp2_table(double e, const double *tab) {
+    // adding 1.5 * 2^41 (ulp 2^-11) rounds e to the nearest multiple of 1/2048 and leaves N = rint(2048 e), in two's
+    // complement, in the low word of the sum; no multiplication is involved
+    constexpr double kRound = 3298534883328.0;               // 1.5 * 2^41
+    // (the instruction itself: the builtin would quieten a signalling NaN first, one more fp64 instruction per value)
+    double c;
+    asm("v_max_f64 %0, %1, %2" : "=v"(c) : "v"(e), "s"(-1100.0));
+    const double t = c + kRound;
+    const int N = (int)(unsigned)__double_as_longlong(t);
+    const double f = c - (t - kRound);                        // exact, |f| <= 2^-12
+    double p = fma(0x1.c6b08d704a0bfp-5, f, 0x1.ebfbdff82c58ep-3);   // ln2^3 / 6, ln2^2 / 2
+    p = fma(p, f, 0x1.62e42fefa39efp-1);                             // ln2
+    p = fma(p, f, 1.0);
+    return __builtin_ldexp(p * tab[N & (kExpTableSize - 1)], N >> kExpTableBits);
+}
+
+// How a kernel function evaluates 2^x in double precision: by polynomial, or from the table in LDS
+struct Exp2Poly {
+    __device__ __forceinline__ double operator()(double e) const { return exp2_nonpositive(e); }
+};
+struct Exp2Table {
+    const double *tab;
+    __device__ __forceinline__ double operator()(double e) const { return exp2_table(e, tab); }
+};
+
 template <int KF> struct KernelFn;
 
 // Gaussian: the median-of-three with 0 and 1 folds into the clamp bit of v_exp_f32, so the clamp is free
@@ -75,7 +115,11 @@ template <> struct KernelFn<FLK_GAUSSIAN> {
     static __device__ __forceinline__ float value(float e) {
         return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(e), 0.0f, 1.0f);
     }
-    static __device__ __forceinline__ double value(double e) { return exp2_nonpositive(fmin(e, 0.0)); }
+    template <class E> static __device__ __forceinline__ double value(double e, E ex) {
+        double c;    // min(e, 0) as the bare instruction (the builtin quietens signalling NaNs first: one more instruction)
+        asm("v_min_f64 %0, %1, 0" : "=v"(c) : "v"(e));
+        return ex(c);
+    }
 };
 
 // q = sqrt(max(-e, clamp)): the scaled distance, with the reference's clamp carried over to q^2
@@ -93,7 +137,9 @@ template <> struct KernelFn<FLK_LAPLACIAN> {
     static __device__ __forceinline__ float value(float e) {
         return __builtin_amdgcn_exp2f(-scaled_distance<FLK_LAPLACIAN>(e));
     }
-    static __device__ __forceinline__ double value(double e) { return exp2_nonpositive(-scaled_distance<FLK_LAPLACIAN>(e)); }
+    template <class E> static __device__ __forceinline__ double value(double e, E ex) {
+        return ex(-scaled_distance<FLK_LAPLACIAN>(e));
+    }
 };
 
 template <> struct KernelFn<FLK_LAPLACIAN_DU> {
@@ -102,9 +148,9 @@ template <> struct KernelFn<FLK_LAPLACIAN_DU> {
         const float k = __builtin_amdgcn_exp2f(-q) * ((float)kLog2e * __builtin_amdgcn_rcpf(q));
         return -e > (float)distance_clamp<FLK_LAPLACIAN_DU>() ? k : 0.0f;
     }
-    static __device__ __forceinline__ double value(double e) {
+    template <class E> static __device__ __forceinline__ double value(double e, E ex) {
         const double q = scaled_distance<FLK_LAPLACIAN_DU>(e);
-        return -e > distance_clamp<FLK_LAPLACIAN_DU>() ? exp2_nonpositive(-q) * kLog2e / q : 0.0;
+        return -e > distance_clamp<FLK_LAPLACIAN_DU>() ? ex(-q) * kLog2e / q : 0.0;
     }
 };
 
@@ -113,9 +159,9 @@ template <> struct KernelFn<FLK_MATERN32> {
         const float q = scaled_distance<FLK_MATERN32>(e);
         return __builtin_fmaf(q, (float)(1.0 / kLog2e), 1.0f) * __builtin_amdgcn_exp2f(-q);
     }
-    static __device__ __forceinline__ double value(double e) {
+    template <class E> static __device__ __forceinline__ double value(double e, E ex) {
         const double q = scaled_distance<FLK_MATERN32>(e);
-        return fma(q, 1.0 / kLog2e, 1.0) * exp2_nonpositive(-q);
+        return fma(q, 1.0 / kLog2e, 1.0) * ex(-q);
     }
 };
 
@@ -125,13 +171,17 @@ template <> struct KernelFn<FLK_MATERN52> {
         const float poly = __builtin_fmaf(q, __builtin_fmaf(q, (float)(1.0 / (3.0 * kLog2e * kLog2e)), (float)(1.0 / kLog2e)), 1.0f);
         return poly * __builtin_amdgcn_exp2f(-q);
     }
-    static __device__ __forceinline__ double value(double e) {
+    template <class E> static __device__ __forceinline__ double value(double e, E ex) {
         const double q = scaled_distance<FLK_MATERN52>(e);
-        return fma(q, fma(q, 1.0 / (3.0 * kLog2e * kLog2e), 1.0 / kLog2e), 1.0) * exp2_nonpositive(-q);
+        return fma(q, fma(q, 1.0 / (3.0 * kLog2e * kLog2e), 1.0 / kLog2e), 1.0) * ex(-q);
     }
 };
 
 template <int KF> __device__ __forceinline__ float kernel_value(float e) { return KernelFn<KF>::value(e); }
-template <int KF> __device__ __forceinline__ double kernel_value(double e) { return KernelFn<KF>::value(e); }
+template <int KF> __device__ __forceinline__ double kernel_value(double e) { return KernelFn<KF>::value(e, Exp2Poly{}); }
+// the same with 2^x read from the table in LDS (exp2_table_fill)
+template <int KF> __device__ __forceinline__ double kernel_value(double e, const double *tab) {
+    return KernelFn<KF>::value(e, Exp2Table{tab});
+}
 
 }  // namespace flk

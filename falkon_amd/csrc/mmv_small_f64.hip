@@ -43,14 +43,16 @@ __device__ __forceinline__ void load_afrag64(AFrag64<DP, TT> &f, const double *_
     for (int t = 0; t < TT; t++) f.vec[t] = *(const doublex4 *)(vecp + t * vec_ld + r0);
 }
 
-template <int DP, int FR, int TT>
+// RAW (Gaussian only): the output rows' half norms stay out of the exponent (they multiply the finished sums), so the
+// accumulators start from the A block's half norms alone and the kernel value is the bare 2^e, not clamped at 1.
+template <int DP, int FR, int TT, bool RAW>
 __device__ __forceinline__ void tile_step64(const AFrag64<DP, TT> &f, const double (&breg)[FR][DP],
-                                            const double (&hb)[FR], double (&o1)[FR][TT]) {
+                                            const double (&hb)[FR], double (&o1)[FR][TT], const double *exp_tab) {
     doublex4 acc[FR];
 #pragma unroll
     for (int c = 0; c < FR; c++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) acc[c][r] = f.hn[r] + hb[c];
+        for (int r = 0; r < 4; r++) acc[c][r] = RAW ? f.hn[r] : f.hn[r] + hb[c];
 #pragma unroll
     for (int s = 0; s < DP; s++)
 #pragma unroll
@@ -59,10 +61,42 @@ __device__ __forceinline__ void tile_step64(const AFrag64<DP, TT> &f, const doub
     for (int c = 0; c < FR; c++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            double k = kernel_value<FLK_KF>(acc[c][r]);
+            // (three and four columns leave room for one wave per SIMD only, and a lone wave cannot hide the table's
+            // LDS latency: those variants evaluate the polynomial; measured d = 28, T = 4: 16.2 ms against 18.8)
+            double k;
+            if constexpr (TT <= 2) k = RAW ? exp2_table(acc[c][r], exp_tab) : kernel_value<FLK_KF>(acc[c][r], exp_tab);
+            else k = RAW ? exp2_nonpositive(acc[c][r]) : kernel_value<FLK_KF>(acc[c][r]);
 #pragma unroll
             for (int t = 0; t < TT; t++) o1[c][t] = __builtin_fma(k, f.vec[t][r], o1[c][t]);
         }
+}
+
+// One wave's walk over the A blocks a0 .. a1 (double buffered in registers), accumulating into o1 / o2.
+template <int DP, int FR, int TT, bool RAW>
+__device__ __forceinline__ void reduce_blocks64(const double *__restrict__ PA, const double *__restrict__ hA,
+                                                const double *__restrict__ vecp, int64_t vec_ld, int64_t a0, int64_t a1,
+                                                int j, int q, const double (&breg)[FR][DP], const double (&hb)[FR],
+                                                double (&o1)[FR][TT], double (&o2)[FR][TT], const double *exp_tab) {
+    AFrag64<DP, TT> f0, f1;
+    if (a0 < a1) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, a0, j, q);
+    int since_flush = 0;
+    for (int64_t ab = a0; ab < a1; ab += 2) {
+        const bool has1 = ab + 1 < a1;
+        if (has1) load_afrag64<DP, TT>(f1, PA, hA, vecp, vec_ld, ab + 1, j, q);
+        tile_step64<DP, FR, TT, RAW>(f0, breg, hb, o1, exp_tab);
+        if (has1) {
+            if (ab + 2 < a1) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, ab + 2, j, q);
+            tile_step64<DP, FR, TT, RAW>(f1, breg, hb, o1, exp_tab);
+        }
+        since_flush += 2;
+        if (since_flush >= kFlushEvery64) {
+            since_flush = 0;
+#pragma unroll
+            for (int c = 0; c < FR; c++)
+#pragma unroll
+                for (int t = 0; t < TT; t++) { o2[c][t] += o1[c][t]; o1[c][t] = 0.0; }
+        }
+    }
 }
 
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
@@ -72,6 +106,12 @@ __global__ void __launch_bounds__(256)
                          int64_t vec_ld, const double *__restrict__ PB, const double *__restrict__ hB,
                          int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks, double *__restrict__ partial,
                          int64_t nb_pad, bool y_fastest) {
+    // gfx950 has no fp64 exponential: 2^(k/2048) from a table in LDS, filled here (kernel_fn.h)
+    __shared__ double exp_tab[TT <= 2 ? kExpTableSize : 1];
+    if constexpr (TT <= 2) {
+        exp2_table_fill(exp_tab, threadIdx.x, 256);
+        __syncthreads();
+    }
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
     const int lane = threadIdx.x & 63;
@@ -101,36 +141,35 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
         for (int t = 0; t < TT; t++) { o1[c][t] = 0.0; o2[c][t] = 0.0; }
 
-    AFrag64<DP, TT> f0, f1;
-    if (a0 < a1) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, a0, j, q);
-    int since_flush = 0;
-    for (int64_t ab = a0; ab < a1; ab += 2) {
-        const bool has1 = ab + 1 < a1;
-        if (has1) load_afrag64<DP, TT>(f1, PA, hA, vecp, vec_ld, ab + 1, j, q);
-        tile_step64<DP, FR, TT>(f0, breg, hb, o1);
-        if (has1) {
-            if (ab + 2 < a1) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, ab + 2, j, q);
-            tile_step64<DP, FR, TT>(f1, breg, hb, o1);
-        }
-        since_flush += 2;
-        if (since_flush >= kFlushEvery64) {
-            since_flush = 0;
+    // Gaussian: 2^hB_j is taken out of the sums, out_j = 2^hB_j sum_i 2^(x_i.c_j + hA_i) vec_i, which saves an add and
+    // the clamp per kernel value, as long as 2^(-hB_j) is nowhere near the fp64 range; every wave checks its own
+    // resident rows (rows with a non-finite half norm fail the check).  On that path a kernel value is not clamped
+    // entry by entry: where two points coincide K is 1 to rounding instead of exactly 1.
+    constexpr bool kCanFactorOut = KF == FLK_GAUSSIAN;
+    bool factored = false;
+    if constexpr (kCanFactorOut) {
+        bool small_norms = true;
 #pragma unroll
-            for (int c = 0; c < FR; c++)
-#pragma unroll
-                for (int t = 0; t < TT; t++) { o2[c][t] += o1[c][t]; o1[c][t] = 0.0; }
-        }
+        for (int c = 0; c < FR; c++) small_norms = small_norms && hb[c] >= -900.0;
+        factored = __all(small_norms);
     }
+    if (kCanFactorOut && factored)
+        reduce_blocks64<DP, FR, TT, true>(PA, hA, vecp, vec_ld, a0, a1, j, q, breg, hb, o1, o2, exp_tab);
+    else
+        reduce_blocks64<DP, FR, TT, false>(PA, hA, vecp, vec_ld, a0, a1, j, q, breg, hb, o1, o2, exp_tab);
 #pragma unroll
-    for (int c = 0; c < FR; c++)
+    for (int c = 0; c < FR; c++) {
+        const double out_scale = (kCanFactorOut && factored) ? exp2_nonpositive(hb[c]) : 1.0;
 #pragma unroll
         for (int t = 0; t < TT; t++) {
             double s = o2[c][t] + o1[c][t];
             s += __shfl_xor(s, 16, 64);
             s += __shfl_xor(s, 32, 64);
+            if (kCanFactorOut) s *= out_scale;
             if (q == 0 && bb0 + c < nb_blocks)
                 partial[((int64_t)by * TT + t) * nb_pad + (bb0 + c) * 16 + jrow] = s;
         }
+    }
 }
 
 // right-hand sides per pass of the FMA kernel above: four, except at 60 and 64 padded features, where its

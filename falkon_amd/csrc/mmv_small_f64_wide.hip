@@ -56,7 +56,7 @@ __device__ __forceinline__ void wide64_stage(const Wide64RowVals &rv, double *ld
 template <int DP, int FR, int KF>
 __device__ __forceinline__ void wide64_tile_step(const double (&a)[DP], const double *lds, int j, int q,
                                                  const double (&breg)[FR][DP], const double (&hb)[FR],
-                                                 doublex4 (&out2)[FR]) {
+                                                 doublex4 (&out2)[FR], const double *exp_tab) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const doublex4 hn = *(const doublex4 *)(lds + 4 * q);          // rows 4q .. 4q + 3 of the A block
     doublex4 acc[FR];
@@ -71,7 +71,7 @@ __device__ __forceinline__ void wide64_tile_step(const double (&a)[DP], const do
 #pragma unroll
     for (int c = 0; c < FR; c++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) acc[c][r] = kernel_value<KF>(acc[c][r]);
+        for (int r = 0; r < 4; r++) acc[c][r] = kernel_value<KF>(acc[c][r], exp_tab);
     const double *vb = lds + 16 + (4 * q) * kWide64Stride + j;     // vec[4q + r][t = j]
 #pragma unroll
     for (int r = 0; r < 4; r++) {
@@ -91,6 +91,10 @@ __global__ void __launch_bounds__(256, 2)
                               bool y_fastest) {
     // vecp must hold 16 planes (zeros beyond the caller's columns); the first tcols columns are stored
     __shared__ __attribute__((aligned(32))) double stage[kWide64Waves][2][kWide64Stage];
+    // gfx950 has no fp64 exponential: 2^(k/2048) from a table in LDS, filled here (kernel_fn.h)
+    __shared__ double exp_tab[kExpTableSize];
+    exp2_table_fill(exp_tab, threadIdx.x, 256);
+    __syncthreads();
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
     const int lane = threadIdx.x & 63;
@@ -98,7 +102,7 @@ __global__ void __launch_bounds__(256, 2)
     const int j = lane & 15, q = lane >> 4;
     const int jrow = 4 * (j & 3) + (j >> 2);  // matrix row (within its block) held at position j
     const int64_t bb0 = ((int64_t)bx * kWide64Waves + wave) * FR;
-    if (bb0 >= nb_blocks) return;             // whole wave idle; no workgroup barriers in this kernel
+    if (bb0 >= nb_blocks) return;             // whole wave idle; no workgroup barriers from here on
     const int64_t a0 = (int64_t)by * a_chunk_blocks;
     int64_t a1 = a0 + a_chunk_blocks;
     if (a1 > na_blocks) a1 = na_blocks;
@@ -128,12 +132,12 @@ __global__ void __launch_bounds__(256, 2)
     for (int64_t ab = a0; ab < a1; ab += 2) {
         const bool has1 = ab + 1 < a1;
         if (has1) { wide64_load_a<DP>(fa1, PA, ab + 1, j, q); wide64_fetch(rv, hA, vecp, vec_ld, ab + 1, lane); }
-        wide64_tile_step<DP, FR, KF>(fa0, lds0, j, q, breg, hb, out2);
+        wide64_tile_step<DP, FR, KF>(fa0, lds0, j, q, breg, hb, out2, exp_tab);
         if (has1) {
             wide64_stage(rv, lds1, lane);
             const bool has2 = ab + 2 < a1;
             if (has2) { wide64_load_a<DP>(fa0, PA, ab + 2, j, q); wide64_fetch(rv, hA, vecp, vec_ld, ab + 2, lane); }
-            wide64_tile_step<DP, FR, KF>(fa1, lds1, j, q, breg, hb, out2);
+            wide64_tile_step<DP, FR, KF>(fa1, lds1, j, q, breg, hb, out2, exp_tab);
             if (has2) wide64_stage(rv, lds0, lane);
         }
     }
