@@ -47,10 +47,22 @@ inline double operand_scale(int kf) {
 // 2^n and rounds results below 2^-1022 correctly.  Arguments below -1100 are raised to it (the result is 0 from
 // -1075 on), so that n always fits the low word.  (Scaling through the exponent field instead of v_ldexp_f64, with
 // results below 2^-1021 flushed to zero, measured no faster.)
+// max(e, about -1100) for the exponentials below, done on the high word as an unsigned integer (one 32-bit
+// instruction): among negative doubles a larger high word is a more negative number, so capping it at the high word
+// of -1100.0 raises everything below to [-1100.2, -1100], leaves the rest alone, and turns a negative NaN into -1100 too
+// (non-finite rows are handled through their half norms, not through the kernel values).  The fp64 maximum would
+// cost two instructions: the compiler has to quieten its operand first, as it does not know that an MFMA result
+// cannot be a signalling NaN.  (Inline assembly on an accumulator register is no way around that: the wait states
+// an MFMA result needs before a vector instruction may read it are not inserted for assembly.)
+__device__ __forceinline__ double raise_to_exp_range(double e) {
+    const unsigned long long bits = (unsigned long long)__double_as_longlong(e);
+    const unsigned hi = min((unsigned)(bits >> 32), 0xC0913000u);
+    return __longlong_as_double((long long)(((unsigned long long)hi << 32) | (bits & 0xffffffffull)));
+}
+
 __device__ __forceinline__ double exp2_nonpositive(double e) {
     constexpr double kRound = 6755399441055744.0;       // 1.5 * 2^52: adding it rounds to the nearest integer
-    // (the bare instruction: the builtin would quieten a signalling NaN first, one more fp64 instruction per value)
-    asm("v_max_f64 %0, %1, %2" : "=v"(e) : "v"(e), "s"(-1100.0));
+    e = raise_to_exp_range(e);
     const double t = e + kRound;
     const int n = (int)(unsigned)__double_as_longlong(t);  // the integer, in two's complement, is the low word
     const double f = e - (t - kRound);
@@ -83,29 +95,44 @@ __device__ __forceinline__ void exp2_table_fill(double *tab, int tid, int nthrea
         tab[k] = 2.0 * exp2_nonpositive((double)(k - kExpTableSize) * (1.0 / kExpTableSize));
 }
 
+template <bool ON_FMA = true>
 __device__ __forceinline__ double exp2_table(double e, const double *tab) {
     // adding 1.5 * 2^41 (ulp 2^-11) rounds e to the nearest multiple of 1/2048 and leaves N = rint(2048 e), in two's
     // complement, in the low word of the sum; no multiplication is involved
     constexpr double kRound = 3298534883328.0;               // 1.5 * 2^41
     // (the instruction itself: the builtin would quieten a signalling NaN first, one more fp64 instruction per value)
-    double c;
-    asm("v_max_f64 %0, %1, %2" : "=v"(c) : "v"(e), "s"(-1100.0));
+    const double c = raise_to_exp_range(e);
     const double t = c + kRound;
     const int N = (int)(unsigned)__double_as_longlong(t);
-    const double f = c - (t - kRound);                        // exact, |f| <= 2^-12
+    // ON_FMA: two of the additions and the product with the table entry are issued as v_fma_f64 (x * 1 + y,
+    // x * y + 0): on gfx950 that instruction measures 6.0 cycles per wave against 7.5 for v_add_f64 and 7.7 for
+    // v_mul_f64.  (They depend on t, so they come after the compiler's own first read of e, which carries the MFMA
+    // wait states.)  It pays where the MFMA chain is long enough to schedule around the fixed instructions (mmv at
+    // N = 5e5, M = 2e4: d = 28 12.5 -> 12.1 ms, but d = 9 7.6 -> 8.4): the callers choose.
+    double r, f, y;
+    if constexpr (ON_FMA) {
+        asm("v_fma_f64 %0, %1, 1.0, %2" : "=v"(r) : "v"(t), "s"(-kRound));
+        asm("v_fma_f64 %0, %1, -1.0, %2" : "=v"(f) : "v"(r), "v"(c));
+    } else {
+        r = t - kRound;
+        f = c - r;
+    }                                                                // f: exact, |f| <= 2^-12
     double p = fma(0x1.c6b08d704a0bfp-5, f, 0x1.ebfbdff82c58ep-3);   // ln2^3 / 6, ln2^2 / 2
     p = fma(p, f, 0x1.62e42fefa39efp-1);                             // ln2
     p = fma(p, f, 1.0);
-    return __builtin_ldexp(p * tab[N & (kExpTableSize - 1)], N >> kExpTableBits);
+    const double entry = tab[N & (kExpTableSize - 1)];
+    if constexpr (ON_FMA) asm("v_fma_f64 %0, %1, %2, 0" : "=v"(y) : "v"(p), "v"(entry));
+    else y = p * entry;
+    return __builtin_ldexp(y, N >> kExpTableBits);
 }
 
 // How a kernel function evaluates 2^x in double precision: by polynomial, or from the table in LDS
 struct Exp2Poly {
     __device__ __forceinline__ double operator()(double e) const { return exp2_nonpositive(e); }
 };
-struct Exp2Table {
+template <bool ON_FMA> struct Exp2Table {
     const double *tab;
-    __device__ __forceinline__ double operator()(double e) const { return exp2_table(e, tab); }
+    __device__ __forceinline__ double operator()(double e) const { return exp2_table<ON_FMA>(e, tab); }
 };
 
 template <int KF> struct KernelFn;
@@ -116,9 +143,7 @@ template <> struct KernelFn<FLK_GAUSSIAN> {
         return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(e), 0.0f, 1.0f);
     }
     template <class E> static __device__ __forceinline__ double value(double e, E ex) {
-        double c;    // min(e, 0) as the bare instruction (the builtin quietens signalling NaNs first: one more instruction)
-        asm("v_min_f64 %0, %1, 0" : "=v"(c) : "v"(e));
-        return ex(c);
+        return ex(fmin(e, 0.0));
     }
 };
 
@@ -180,8 +205,8 @@ template <> struct KernelFn<FLK_MATERN52> {
 template <int KF> __device__ __forceinline__ float kernel_value(float e) { return KernelFn<KF>::value(e); }
 template <int KF> __device__ __forceinline__ double kernel_value(double e) { return KernelFn<KF>::value(e, Exp2Poly{}); }
 // the same with 2^x read from the table in LDS (exp2_table_fill)
-template <int KF> __device__ __forceinline__ double kernel_value(double e, const double *tab) {
-    return KernelFn<KF>::value(e, Exp2Table{tab});
+template <int KF, bool ON_FMA = true> __device__ __forceinline__ double kernel_value(double e, const double *tab) {
+    return KernelFn<KF>::value(e, Exp2Table<ON_FMA>{tab});
 }
 
 }  // namespace flk

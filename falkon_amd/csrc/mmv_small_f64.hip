@@ -64,7 +64,8 @@ __device__ __forceinline__ void tile_step64(const AFrag64<DP, TT> &f, const doub
             // (three and four columns leave room for one wave per SIMD only, and a lone wave cannot hide the table's
             // LDS latency: those variants evaluate the polynomial; measured d = 28, T = 4: 16.2 ms against 18.8)
             double k;
-            if constexpr (TT <= 2) k = RAW ? exp2_table(acc[c][r], exp_tab) : kernel_value<FLK_KF>(acc[c][r], exp_tab);
+            if constexpr (TT <= 2)
+                k = RAW ? exp2_table<(DP > 4)>(acc[c][r], exp_tab) : kernel_value<FLK_KF, (DP > 4)>(acc[c][r], exp_tab);
             else k = RAW ? exp2_nonpositive(acc[c][r]) : kernel_value<FLK_KF>(acc[c][r]);
 #pragma unroll
             for (int t = 0; t < TT; t++) o1[c][t] = __builtin_fma(k, f.vec[t][r], o1[c][t]);

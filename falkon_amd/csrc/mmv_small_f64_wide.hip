@@ -71,7 +71,7 @@ __device__ __forceinline__ void wide64_tile_step(const double (&a)[DP], const do
 #pragma unroll
     for (int c = 0; c < FR; c++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) acc[c][r] = kernel_value<KF>(acc[c][r], exp_tab);
+        for (int r = 0; r < 4; r++) acc[c][r] = kernel_value<KF, (DP > 4)>(acc[c][r], exp_tab);
     const double *vb = lds + 16 + (4 * q) * kWide64Stride + j;     // vec[4q + r][t = j]
 #pragma unroll
     for (int r = 0; r < 4; r++) {
