@@ -91,6 +91,9 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     __shared__ __attribute__((aligned(32))) T ldsRow[kRowBuf];   // [hA | vec ...] of the A tile
 
     unsigned bx, by;
+    // (Banding the contracting mode as well was measured on N = 5e5, M = 1e4, d = 784: bytes fetched per launch
+    // 62 -> 93 GB, launch time unchanged at 60.8 ms: the re-reads come out of the Infinity Cache and do not bound
+    // the kernel, whose matrix pipe is 88 % busy.)
     if constexpr (kStore) xcd_remap_banded(bx, by);
     else xcd_remap(bx, by, y_fastest);
     const int tid = threadIdx.x;

@@ -65,8 +65,13 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     __shared__ __attribute__((aligned(32))) float ldsRow[kRowBuf];   // vec of the A tile
 
     unsigned bx, by;
+    // Where the reduction side is the big operand the contracting mode is banded too (8 output tiles x 8 reduction
+    // chunks per XCD instead of 64 output tiles on one chunk): the 256-row output tiles then stay in the XCD's L2.
+    // Measured on N = 5e5, M = 1e4, d = 784: bytes fetched per launch 68 -> 38 GB (mean of both passes); the launch
+    // time does not move (29.8 ms): the re-reads came out of the Infinity Cache.
     if constexpr (STORE) xcd_remap_banded(bx, by);
-    else xcd_remap(bx, by, y_fastest);
+    else if (y_fastest) xcd_remap(bx, by, true);
+    else xcd_remap_banded(bx, by);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform by construction: let the compiler know
