@@ -16,25 +16,33 @@ int FLK_CAT(launch_mmv_small_f32_fold_kf, FLK_KF)(const PackedView &A, const Pac
                                                   float *partial, hipStream_t st);
 
 // Columns per pass of the per-lane FMA kernels (must match the instantiations in launch_tt); calls with more
-// right-hand sides than that go to the 32-column kernel whose contraction runs on the matrix cores
+// right-hand sides than that go to the 32- or 64-column kernel whose contraction runs on the matrix cores
 // (mmv_small_f32_wide.hip: four resident blocks per wave up to 16 padded features, two beyond).
 static inline int fma_cols(int64_t dpad) {
     const int64_t dp = dpad / 2;
     return dp <= 7 ? 16 : dp <= 12 ? 12 : dp <= 16 ? 8 : 4;
 }
-constexpr int kWideColumns = 32;
+constexpr int kWideColumns = 32;       // one group of columns of the wide kernel
 constexpr int kWideMaxDpFr4 = 8;
+// The wide kernel takes two groups (64 columns) on one evaluation of K where the columns beyond 32 would need the wide
+// kernel again; up to fma_cols columns beyond 32, a 32-column pass and a pass of the FMA kernel are the faster pair.
+// Measured, dfmmv at N = 1e6, M = 2e4 (64-column kernel against two passes): d = 28: T = 64 69.1 ms against 86.1, T = 33
+// 67.9 against 62.2; d = 9: T = 64 54.6 against 58.2, T = 48 54.0 against 50.8; d = 64: T = 64 119 against 137.
+static inline bool two_groups(int64_t dpad, int64_t t) { return t > kWideColumns + fma_cols(dpad); }
 
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<float>() { return 2 * kMaxDpFr2; }
 template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad, int64_t t) {
+    if (two_groups(dpad, t)) return kWavesPerWg * ((dpad / 2) <= 16 ? 2 : 1);
     if (t > fma_cols(dpad)) return kWavesPerWg * ((dpad / 2) <= kWideMaxDpFr4 ? 4 : 2);
     return kWavesPerWg * ((dpad / 2) <= kMaxDpFr4 ? 4 : 2);
 }
 template <> int mmv_small_max_cols<float>(int64_t dpad, int64_t t) {
+    if (two_groups(dpad, t)) return 2 * kWideColumns;
     return t > fma_cols(dpad) ? kWideColumns : fma_cols(dpad);
 }
 template <> int mmv_small_width<float>(int64_t dpad, int tc) {
+    if (tc > kWideColumns) return 2 * kWideColumns;
     if (tc > fma_cols(dpad)) return kWideColumns;
     static const int widths[] = {1, 2, 3, 4, 6, 8, 12, 16};
     for (int w : widths) if (tc <= w) return w;

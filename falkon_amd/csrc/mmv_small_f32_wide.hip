@@ -1,4 +1,4 @@
-// Register-resident fp32 product kernel for many right-hand sides (up to 32 per pass), gfx950.
+// Register-resident fp32 product kernel for many right-hand sides (up to 32 or 64 per pass), gfx950.
 // Compiled once per kernel function (-DFLK_KF=0..4).
 //
 // Same walk as mmv_small_f32_kernel (a wave keeps FR blocks of 32 output rows in registers and streams blocks of 32
@@ -7,7 +7,9 @@
 // operand of an fp32 32x32x2 MFMA step (row i = 8*(s/4) + 4*(lane/32) + s%4 of the A block, column j = lane % 32),
 // so  out2[j][t] += sum_i K[i][j] vec[i][t]  is 16 more MFMAs per fragment whatever the number of columns, with
 // vec[i][t] (t = lane % 32) as the B operand.  Per-lane FMAs cost 16 per column and fragment: beyond eight columns
-// (four for the two-fragment kernels) this kernel is the cheaper one.
+// (four for the two-fragment kernels) this kernel is the cheaper one.  NC = 2 serves 64 columns per evaluation of K
+// (two groups of 32, 32 contraction MFMAs per fragment, two resident fragments per wave): between 33 and 64 columns
+// the cross term and the exponential are then computed once instead of twice.
 #include "mmv_small_f32_kernel.h"
 
 #ifndef FLK_KF
@@ -16,34 +18,43 @@
 
 namespace flk {
 
-constexpr int kWideCols = 32;
-constexpr int kWideStride = 33;                          // row stride of the staged vec values: conflict-free reads
-constexpr int kWideStage = 32 + 32 * kWideStride;        // hn(32) | vec[32 rows][33]
-constexpr int kWideFetch = 1 + kWideCols / 2;            // dwords a lane fetches per A block
+// NC groups of 32 columns: the staged values of an A block are hn(32) | vec[32 rows][32 NC + 1] (the odd row stride
+// makes the reads conflict free)
+template <int NC> struct WideGeo {
+    static constexpr int kCols = 32 * NC;
+    static constexpr int kStride = kCols + 1;
+    static constexpr int kStage = 32 + 32 * kStride;
+    static constexpr int kFetch = 1 + kCols / 2;         // dwords a lane fetches per A block
+};
+constexpr int kWideCols = 32;                            // of one group
+constexpr int kWideMaxGroups = 2;
 
-struct WideRowVals { float x[kWideFetch]; };
+template <int NC> struct WideRowVals { float x[WideGeo<NC>::kFetch]; };
 
-// lane l fetches hA[row l % 32] (lower half) and vec[row l % 32][2c + l / 32], c = 0..15: 128-byte runs of the planes
-__device__ __forceinline__ void wide_fetch(WideRowVals &rv, const float *__restrict__ hA, const float *__restrict__ vecp,
-                                           int64_t vec_ld, int64_t ab, int lane) {
+// lane l fetches hA[row l % 32] (lower half) and vec[row l % 32][2c + l / 32], c = 0..16 NC - 1: 128-byte runs of the planes
+template <int NC>
+__device__ __forceinline__ void wide_fetch(WideRowVals<NC> &rv, const float *__restrict__ hA,
+                                           const float *__restrict__ vecp, int64_t vec_ld, int64_t ab, int lane) {
     const int r = lane & 31, hh = lane >> 5;
     rv.x[0] = hA[ab * 32 + r];
 #pragma unroll
-    for (int c = 0; c < kWideCols / 2; c++) rv.x[1 + c] = vecp[(int64_t)(2 * c + hh) * vec_ld + ab * 32 + r];
+    for (int c = 0; c < WideGeo<NC>::kCols / 2; c++) rv.x[1 + c] = vecp[(int64_t)(2 * c + hh) * vec_ld + ab * 32 + r];
 }
-__device__ __forceinline__ void wide_stage(const WideRowVals &rv, float *lds, int lane) {
+template <int NC>
+__device__ __forceinline__ void wide_stage(const WideRowVals<NC> &rv, float *lds, int lane) {
     const int r = lane & 31, hh = lane >> 5;
     if (hh == 0) lds[r] = rv.x[0];
 #pragma unroll
-    for (int c = 0; c < kWideCols / 2; c++) lds[32 + r * kWideStride + 2 * c + hh] = rv.x[1 + c];
+    for (int c = 0; c < WideGeo<NC>::kCols / 2; c++) lds[32 + r * WideGeo<NC>::kStride + 2 * c + hh] = rv.x[1 + c];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 }
 
-template <int DP, int FR, bool FOLD, int KF>
+template <int DP, int FR, bool FOLD, int KF, int NC>
 __device__ __forceinline__ void wide_tile_step(const float (&a)[DP], const float *lds, int j, int h,
                                                const float (&breg)[FR][DP], const float (&hb)[FR],
-                                               floatx16 (&out2)[FR]) {
+                                               floatx16 (&out2)[FR][NC]) {
+    constexpr int kWideStride = WideGeo<NC>::kStride;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     floatx4 hn[4];
 #pragma unroll
@@ -64,26 +75,38 @@ __device__ __forceinline__ void wide_tile_step(const float (&a)[DP], const float
     // contraction on the matrix cores; the B operand is read one step ahead, fenced (otherwise every read is
     // hoisted to the front)
     const float *vb = lds + 32 + j;
-    float bval = vb[(4 * h) * kWideStride], bnext = 0.f;
+    float bval[NC], bnext[NC];
+#pragma unroll
+    for (int g = 0; g < NC; g++) { bval[g] = vb[(4 * h) * kWideStride + 32 * g]; bnext[g] = 0.f; }
 #pragma unroll
     for (int s2 = 0; s2 < 16; s2++) {
-        if (s2 + 1 < 16) bnext = vb[(8 * ((s2 + 1) >> 2) + 4 * h + ((s2 + 1) & 3)) * kWideStride];
+        if (s2 + 1 < 16) {
 #pragma unroll
-        for (int q = 0; q < FR; q++) out2[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(acc[q][s2], bval, out2[q], 0, 0, 0);
-        asm volatile("" : "+v"(bval) : "v"(vb) : "memory");
-        bval = bnext;
+            for (int g = 0; g < NC; g++)
+                bnext[g] = vb[(8 * ((s2 + 1) >> 2) + 4 * h + ((s2 + 1) & 3)) * kWideStride + 32 * g];
+        }
+#pragma unroll
+        for (int g = 0; g < NC; g++)
+#pragma unroll
+            for (int q = 0; q < FR; q++)
+                out2[q][g] = __builtin_amdgcn_mfma_f32_32x32x2f32(acc[q][s2], bval[g], out2[q][g], 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < NC; g++) {
+            asm volatile("" : "+v"(bval[g]) : "v"(vb) : "memory");
+            bval[g] = bnext[g];
+        }
     }
 }
 
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
-template <int DP, int FR, bool FOLD, int KF>
+template <int DP, int FR, bool FOLD, int KF, int NC>
 __global__ void __launch_bounds__(256, 2)
     mmv_small_f32_wide_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
                               int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB,
                               int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial,
                               int64_t nb_pad, int tcols, bool y_fastest) {
-    // vecp must hold 32 planes (zeros beyond the caller's columns); the first tcols columns are stored
-    __shared__ __attribute__((aligned(16))) float stage[kWavesPerWg][2][kWideStage];
+    // vecp must hold 32 NC planes (zeros beyond the caller's columns); the first tcols columns are stored
+    __shared__ __attribute__((aligned(16))) float stage[kWavesPerWg][2][WideGeo<NC>::kStage];
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
     const int lane = threadIdx.x & 63;
@@ -104,52 +127,57 @@ __global__ void __launch_bounds__(256, 2)
         hb[q] = hB[bb * 32 + j];
         if (FOLD) breg[q][DP - 1] = h ? hb[q] : breg[q][DP - 1];
     }
-    floatx16 out2[FR];
+    floatx16 out2[FR][NC];
 #pragma unroll
     for (int q = 0; q < FR; q++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) out2[q][r] = 0.f;
+        for (int g = 0; g < NC; g++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) out2[q][g][r] = 0.f;
 
     float fa0[DP], fa1[DP];
-    WideRowVals rv;
+    WideRowVals<NC> rv;
     float *lds0 = stage[wave][0], *lds1 = stage[wave][1];
     if (a0 < a1) {
         load_a<DP>(fa0, PA, a0, j, h);
-        wide_fetch(rv, hA, vecp, vec_ld, a0, lane);
-        wide_stage(rv, lds0, lane);
+        wide_fetch<NC>(rv, hA, vecp, vec_ld, a0, lane);
+        wide_stage<NC>(rv, lds0, lane);
     }
     for (int64_t ab = a0; ab < a1; ab += 2) {
         const bool has1 = ab + 1 < a1;
-        if (has1) { load_a<DP>(fa1, PA, ab + 1, j, h); wide_fetch(rv, hA, vecp, vec_ld, ab + 1, lane); }
-        wide_tile_step<DP, FR, FOLD, KF>(fa0, lds0, j, h, breg, hb, out2);
+        if (has1) { load_a<DP>(fa1, PA, ab + 1, j, h); wide_fetch<NC>(rv, hA, vecp, vec_ld, ab + 1, lane); }
+        wide_tile_step<DP, FR, FOLD, KF, NC>(fa0, lds0, j, h, breg, hb, out2);
         if (has1) {
-            wide_stage(rv, lds1, lane);
+            wide_stage<NC>(rv, lds1, lane);
             const bool has2 = ab + 2 < a1;
-            if (has2) { load_a<DP>(fa0, PA, ab + 2, j, h); wide_fetch(rv, hA, vecp, vec_ld, ab + 2, lane); }
-            wide_tile_step<DP, FR, FOLD, KF>(fa1, lds1, j, h, breg, hb, out2);
-            if (has2) wide_stage(rv, lds0, lane);
+            if (has2) { load_a<DP>(fa0, PA, ab + 2, j, h); wide_fetch<NC>(rv, hA, vecp, vec_ld, ab + 2, lane); }
+            wide_tile_step<DP, FR, FOLD, KF, NC>(fa1, lds1, j, h, breg, hb, out2);
+            if (has2) wide_stage<NC>(rv, lds0, lane);
         }
     }
     // lane = column t, registers = output rows (both lane halves hold different rows): no cross-lane step
-    if (j < tcols) {
 #pragma unroll
-        for (int q = 0; q < FR; q++) {
-            if (bb0 + q < nb_blocks) {
+    for (int g = 0; g < NC; g++) {
+        if (j + 32 * g < tcols) {
 #pragma unroll
-                for (int r = 0; r < 16; r++)
-                    partial[((int64_t)by * tcols + j) * nb_pad + (bb0 + q) * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] =
-                        out2[q][r];
+            for (int q = 0; q < FR; q++) {
+                if (bb0 + q < nb_blocks) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        partial[((int64_t)by * tcols + j + 32 * g) * nb_pad + (bb0 + q) * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] =
+                            out2[q][g][r];
+                }
             }
         }
     }
 }
 
-template <int DP, int FR, bool FOLD>
+template <int DP, int FR, bool FOLD, int NC = 1>
 static int launch_wide_one(const PackedView &A, const PackedView &B, const float *vecp, int64_t vec_ld, int tcols,
                            int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
     const int64_t per_wg = kWavesPerWg * FR;
     dim3 grid((unsigned)((B.nblk + per_wg - 1) / per_wg), (unsigned)splits);
-    hipLaunchKernelGGL((mmv_small_f32_wide_kernel<DP, FR, FOLD, FLK_KF>), grid, dim3(256), 0, st, (const float *)A.data,
+    hipLaunchKernelGGL((mmv_small_f32_wide_kernel<DP, FR, FOLD, FLK_KF, NC>), grid, dim3(256), 0, st, (const float *)A.data,
                        (const float *)A.hnorm, vecp, vec_ld, (const float *)B.data, (const float *)B.hnorm, A.nblk,
                        B.nblk, a_chunk_blocks, partial, B.npad, tcols, B.n > A.n);
     FLK_LAUNCH_CHECK("mmv_small_f32_wide_kernel");
@@ -159,9 +187,31 @@ static int launch_wide_one(const PackedView &A, const PackedView &B, const float
 int FLK_CAT(launch_mmv_small_f32_wide_kf, FLK_KF)(const PackedView &A, const PackedView &B, const float *vecp,
                                                   int64_t vec_ld, int tcols, int64_t a_chunk_blocks, int splits,
                                                   float *partial, hipStream_t st) {
-    if (tcols < 1 || tcols > kWideCols) return fail(FLK_EINVAL, "mmv_small wide: column chunk %d not in 1..32", tcols);
+    if (tcols < 1 || tcols > kWideCols * kWideMaxGroups)
+        return fail(FLK_EINVAL, "mmv_small wide: column chunk %d not in 1..64", tcols);
     const int dp = (int)(A.dpad / 2);
     const bool fold = f32_fold_applies(A.d);
+    if (tcols > kWideCols) {
+        // 33 to 64 columns: two groups of 32 on one evaluation of K; two resident fragments per wave up to 32 padded
+        // features, one beyond (registers: 64 output accumulators per fragment and 33 prefetched row values)
+#define FLK_WIDE2(DPV)                                                                                              \
+    case DPV:                                                                                                      \
+        return fold ? launch_wide_one<DPV, 2, true, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st) \
+                    : launch_wide_one<DPV, 2, false, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+#define FLK_WIDE2_PLAIN(DPV) \
+    case DPV: return launch_wide_one<DPV, 1, false, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+        switch (dp) {
+            FLK_WIDE2(1) FLK_WIDE2(2) FLK_WIDE2(3) FLK_WIDE2(4) FLK_WIDE2(5) FLK_WIDE2(6) FLK_WIDE2(7) FLK_WIDE2(8)
+            FLK_WIDE2(9) FLK_WIDE2(10) FLK_WIDE2(11) FLK_WIDE2(12) FLK_WIDE2(13) FLK_WIDE2(14) FLK_WIDE2(15) FLK_WIDE2(16)
+            FLK_WIDE2_PLAIN(17) FLK_WIDE2_PLAIN(18) FLK_WIDE2_PLAIN(19) FLK_WIDE2_PLAIN(20) FLK_WIDE2_PLAIN(21)
+            FLK_WIDE2_PLAIN(22) FLK_WIDE2_PLAIN(23) FLK_WIDE2_PLAIN(24) FLK_WIDE2_PLAIN(25) FLK_WIDE2_PLAIN(26)
+            FLK_WIDE2_PLAIN(27) FLK_WIDE2_PLAIN(28) FLK_WIDE2_PLAIN(29) FLK_WIDE2_PLAIN(30) FLK_WIDE2_PLAIN(31)
+            FLK_WIDE2_PLAIN(32)
+        }
+#undef FLK_WIDE2
+#undef FLK_WIDE2_PLAIN
+        return fail(FLK_EUNSUPPORTED, "mmv_small wide: padded feature count %lld not in 2..64", (long long)A.dpad);
+    }
 #define FLK_WIDE(DPV, FRV)                                                                                         \
     case DPV:                                                                                                      \
         return fold ? launch_wide_one<DPV, FRV, true>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st) \

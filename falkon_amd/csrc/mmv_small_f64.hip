@@ -184,8 +184,16 @@ constexpr int kMaxDp64Fr2 = 16;  // dpad <= 64
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<double>() { return 4 * kMaxDp64Fr2; }
 // more than four right-hand sides: the 16-column kernel of mmv_small_f64_wide.hip, which reads 16 planes
-template <> int mmv_small_max_cols<double>(int64_t dpad, int64_t t) { return t > fma_cols64(dpad) ? kWideCols64 : fma_cols64(dpad); }
-template <> int mmv_small_width<double>(int64_t dpad, int tc) { return tc > fma_cols64(dpad) ? kWideCols64 : tc; }
+// (beyond 16 columns two groups of 16 share one evaluation of K: 17 columns that way take less time than a
+// 16-column pass and a one-column pass, at every feature count)
+template <> int mmv_small_max_cols<double>(int64_t dpad, int64_t t) {
+    if (t > kWideCols64) return 2 * kWideCols64;
+    return t > fma_cols64(dpad) ? kWideCols64 : fma_cols64(dpad);
+}
+template <> int mmv_small_width<double>(int64_t dpad, int tc) {
+    if (tc > kWideCols64) return 2 * kWideCols64;
+    return tc > fma_cols64(dpad) ? kWideCols64 : tc;
+}
 template <> int mmv_small_b_blocks_per_wg<double>(int64_t dpad, int64_t t) {
     (void)t;
     return kWavesPerWg64 * ((dpad / 4) <= kMaxDp64Fr4 ? 4 : 2);

@@ -1,4 +1,4 @@
-// Register-resident fp64 product kernel for many right-hand sides (up to 16 per pass), gfx950.
+// Register-resident fp64 product kernel for many right-hand sides (up to 16 or 32 per pass), gfx950.
 // Compiled once per kernel function (-DFLK_KF=0..4).
 //
 // Same walk as mmv_small_f64_kernel (a wave keeps FR blocks of 16 output rows in registers and streams blocks of 16
@@ -10,6 +10,10 @@
 //   out2[position 4 r2 + q][t] += sum_i K[i][j] vec[i][t],
 // four more MFMAs per 16 x 16 tile whatever the number of columns, and register r2 of a lane ends up holding output
 // row 4 q + r2 of column t (positions map to rows as in the packed block), so there is no cross-lane step.
+// With NC = 2 a second group of 16 columns rides on the same kernel values (four more MFMAs per tile and group).
+// Measured, dfmmv at N = 5e5, M = 2e4: 32 columns in one pass against two passes of 16: d = 9 35.1 ms against 49.1,
+// d = 28 45.3 against 69.3, d = 64 69.2 against 116.7; 17 columns 35 / 45 / 69 ms against 39.1 / 58.9 / 106.6 for a
+// 16-column pass followed by a one-column pass.
 #include "flk_common.h"
 #include "kernel_fn.h"
 
@@ -22,12 +26,16 @@ namespace flk {
 typedef double doublex4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWide64Waves = 4;
-constexpr int kWide64Cols = 16;
-constexpr int kWide64Stride = 17;                           // row stride of the staged vec values
-constexpr int kWide64Stage = 16 + 16 * kWide64Stride;       // hn(16) | vec[16 rows][17]
-constexpr int kWide64Fetch = 1 + kWide64Cols / 4;           // doubles a lane fetches per A block
+constexpr int kWide64Cols = 16;                             // one group of columns; NC groups share an evaluation of K
+constexpr int kWide64MaxGroups = 2;
+template <int NC> struct Wide64Geo {
+    static constexpr int kCols = 16 * NC;
+    static constexpr int kStride = kCols + 1;               // row stride of the staged vec values
+    static constexpr int kStage = 16 + 16 * kStride;        // hn(16) | vec[16 rows][16 NC + 1]
+    static constexpr int kFetch = 1 + kCols / 4;            // doubles a lane fetches per A block
+};
 
-struct Wide64RowVals { double x[kWide64Fetch]; };
+template <int NC> struct Wide64RowVals { double x[Wide64Geo<NC>::kFetch]; };
 
 template <int DP>
 __device__ __forceinline__ void wide64_load_a(double (&a)[DP], const double *__restrict__ P, int64_t blk, int j, int q) {
@@ -36,27 +44,30 @@ __device__ __forceinline__ void wide64_load_a(double (&a)[DP], const double *__r
     for (int s = 0; s < DP; s++) a[s] = p[s * 16];
 }
 
-// lane l fetches hA[row l % 16] and vec[row l % 16][4c + l / 16], c = 0..3: 128-byte runs of the planes
-__device__ __forceinline__ void wide64_fetch(Wide64RowVals &rv, const double *__restrict__ hA,
+// lane l fetches hA[row l % 16] and vec[row l % 16][4c + l / 16], c = 0..4 NC - 1: 128-byte runs of the planes
+template <int NC>
+__device__ __forceinline__ void wide64_fetch(Wide64RowVals<NC> &rv, const double *__restrict__ hA,
                                              const double *__restrict__ vecp, int64_t vec_ld, int64_t ab, int lane) {
     const int r = lane & 15, hh = lane >> 4;
     rv.x[0] = hA[ab * 16 + r];
 #pragma unroll
-    for (int c = 0; c < kWide64Cols / 4; c++) rv.x[1 + c] = vecp[(int64_t)(4 * c + hh) * vec_ld + ab * 16 + r];
+    for (int c = 0; c < Wide64Geo<NC>::kCols / 4; c++) rv.x[1 + c] = vecp[(int64_t)(4 * c + hh) * vec_ld + ab * 16 + r];
 }
-__device__ __forceinline__ void wide64_stage(const Wide64RowVals &rv, double *lds, int lane) {
+template <int NC>
+__device__ __forceinline__ void wide64_stage(const Wide64RowVals<NC> &rv, double *lds, int lane) {
     const int r = lane & 15, hh = lane >> 4;
     if (hh == 0) lds[r] = rv.x[0];
 #pragma unroll
-    for (int c = 0; c < kWide64Cols / 4; c++) lds[16 + r * kWide64Stride + 4 * c + hh] = rv.x[1 + c];
+    for (int c = 0; c < Wide64Geo<NC>::kCols / 4; c++) lds[16 + r * Wide64Geo<NC>::kStride + 4 * c + hh] = rv.x[1 + c];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 }
 
-template <int DP, int FR, int KF>
+template <int DP, int FR, int KF, int NC>
 __device__ __forceinline__ void wide64_tile_step(const double (&a)[DP], const double *lds, int j, int q,
                                                  const double (&breg)[FR][DP], const double (&hb)[FR],
-                                                 doublex4 (&out2)[FR], const double *exp_tab) {
+                                                 doublex4 (&out2)[FR][NC], const double *exp_tab) {
+    constexpr int kWide64Stride = Wide64Geo<NC>::kStride;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const doublex4 hn = *(const doublex4 *)(lds + 4 * q);          // rows 4q .. 4q + 3 of the A block
     doublex4 acc[FR];
@@ -75,22 +86,26 @@ __device__ __forceinline__ void wide64_tile_step(const double (&a)[DP], const do
     const double *vb = lds + 16 + (4 * q) * kWide64Stride + j;     // vec[4q + r][t = j]
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        const double bval = vb[r * kWide64Stride];
 #pragma unroll
-        for (int c = 0; c < FR; c++) out2[c] = __builtin_amdgcn_mfma_f64_16x16x4f64(acc[c][r], bval, out2[c], 0, 0, 0);
+        for (int g = 0; g < NC; g++) {
+            const double bval = vb[r * kWide64Stride + 16 * g];
+#pragma unroll
+            for (int c = 0; c < FR; c++)
+                out2[c][g] = __builtin_amdgcn_mfma_f64_16x16x4f64(acc[c][r], bval, out2[c][g], 0, 0, 0);
+        }
     }
 }
 
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
-template <int DP, int FR, int KF>
+template <int DP, int FR, int KF, int NC>
 __global__ void __launch_bounds__(256, 2)
     mmv_small_f64_wide_kernel(const double *__restrict__ PA, const double *__restrict__ hA,
                               const double *__restrict__ vecp, int64_t vec_ld, const double *__restrict__ PB,
                               const double *__restrict__ hB, int64_t na_blocks, int64_t nb_blocks,
                               int64_t a_chunk_blocks, double *__restrict__ partial, int64_t nb_pad, int tcols,
                               bool y_fastest) {
-    // vecp must hold 16 planes (zeros beyond the caller's columns); the first tcols columns are stored
-    __shared__ __attribute__((aligned(32))) double stage[kWide64Waves][2][kWide64Stage];
+    // vecp must hold 16 NC planes (zeros beyond the caller's columns); the first tcols columns are stored
+    __shared__ __attribute__((aligned(32))) double stage[kWide64Waves][2][Wide64Geo<NC>::kStage];
     // gfx950 has no fp64 exponential: 2^(k/2048) from a table in LDS, filled here (kernel_fn.h)
     __shared__ double exp_tab[kExpTableSize];
     exp2_table_fill(exp_tab, threadIdx.x, 256);
@@ -115,47 +130,52 @@ __global__ void __launch_bounds__(256, 2)
         wide64_load_a<DP>(breg[c], PB, bb, j, q);
         hb[c] = hB[bb * 16 + jrow];
     }
-    doublex4 out2[FR];
+    doublex4 out2[FR][NC];
 #pragma unroll
     for (int c = 0; c < FR; c++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) out2[c][r] = 0.0;
+        for (int g = 0; g < NC; g++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) out2[c][g][r] = 0.0;
 
     double fa0[DP], fa1[DP];
-    Wide64RowVals rv;
+    Wide64RowVals<NC> rv;
     double *lds0 = stage[wave][0], *lds1 = stage[wave][1];
     if (a0 < a1) {
         wide64_load_a<DP>(fa0, PA, a0, j, q);
-        wide64_fetch(rv, hA, vecp, vec_ld, a0, lane);
-        wide64_stage(rv, lds0, lane);
+        wide64_fetch<NC>(rv, hA, vecp, vec_ld, a0, lane);
+        wide64_stage<NC>(rv, lds0, lane);
     }
     for (int64_t ab = a0; ab < a1; ab += 2) {
         const bool has1 = ab + 1 < a1;
-        if (has1) { wide64_load_a<DP>(fa1, PA, ab + 1, j, q); wide64_fetch(rv, hA, vecp, vec_ld, ab + 1, lane); }
-        wide64_tile_step<DP, FR, KF>(fa0, lds0, j, q, breg, hb, out2, exp_tab);
+        if (has1) { wide64_load_a<DP>(fa1, PA, ab + 1, j, q); wide64_fetch<NC>(rv, hA, vecp, vec_ld, ab + 1, lane); }
+        wide64_tile_step<DP, FR, KF, NC>(fa0, lds0, j, q, breg, hb, out2, exp_tab);
         if (has1) {
-            wide64_stage(rv, lds1, lane);
+            wide64_stage<NC>(rv, lds1, lane);
             const bool has2 = ab + 2 < a1;
-            if (has2) { wide64_load_a<DP>(fa0, PA, ab + 2, j, q); wide64_fetch(rv, hA, vecp, vec_ld, ab + 2, lane); }
-            wide64_tile_step<DP, FR, KF>(fa1, lds1, j, q, breg, hb, out2, exp_tab);
-            if (has2) wide64_stage(rv, lds0, lane);
+            if (has2) { wide64_load_a<DP>(fa0, PA, ab + 2, j, q); wide64_fetch<NC>(rv, hA, vecp, vec_ld, ab + 2, lane); }
+            wide64_tile_step<DP, FR, KF, NC>(fa1, lds1, j, q, breg, hb, out2, exp_tab);
+            if (has2) wide64_stage<NC>(rv, lds0, lane);
         }
     }
     // lane = column t = j, registers = output rows 4q .. 4q + 3 of each block
-    if (j < tcols) {
 #pragma unroll
-        for (int c = 0; c < FR; c++)
-            if (bb0 + c < nb_blocks)
-                *(doublex4 *)(&partial[((int64_t)by * tcols + j) * nb_pad + (bb0 + c) * 16 + 4 * q]) = out2[c];
+    for (int g = 0; g < NC; g++) {
+        if (j + 16 * g < tcols) {
+#pragma unroll
+            for (int c = 0; c < FR; c++)
+                if (bb0 + c < nb_blocks)
+                    *(doublex4 *)(&partial[((int64_t)by * tcols + j + 16 * g) * nb_pad + (bb0 + c) * 16 + 4 * q]) = out2[c][g];
+        }
     }
 }
 
-template <int DP, int FR>
+template <int DP, int FR, int NC>
 static int launch_wide64_one(const PackedView &A, const PackedView &B, const double *vecp, int64_t vec_ld, int tcols,
                              int64_t a_chunk_blocks, int splits, double *partial, hipStream_t st) {
     const int64_t per_wg = kWide64Waves * FR;
     dim3 grid((unsigned)((B.nblk + per_wg - 1) / per_wg), (unsigned)splits);
-    hipLaunchKernelGGL((mmv_small_f64_wide_kernel<DP, FR, FLK_KF>), grid, dim3(256), 0, st, (const double *)A.data,
+    hipLaunchKernelGGL((mmv_small_f64_wide_kernel<DP, FR, FLK_KF, NC>), grid, dim3(256), 0, st, (const double *)A.data,
                        (const double *)A.hnorm, vecp, vec_ld, (const double *)B.data, (const double *)B.hnorm, A.nblk,
                        B.nblk, a_chunk_blocks, partial, B.npad, tcols, B.n > A.n);
     FLK_LAUNCH_CHECK("mmv_small_f64_wide_kernel");
@@ -165,11 +185,15 @@ static int launch_wide64_one(const PackedView &A, const PackedView &B, const dou
 int FLK_CAT(launch_mmv_small_f64_wide_kf, FLK_KF)(const PackedView &A, const PackedView &B, const double *vecp,
                                                   int64_t vec_ld, int tcols, int64_t a_chunk_blocks, int splits,
                                                   double *partial, hipStream_t st) {
-    if (tcols < 1 || tcols > kWide64Cols) return fail(FLK_EINVAL, "mmv_small wide: column chunk %d not in 1..16", tcols);
+    if (tcols < 1 || tcols > kWide64Cols * kWide64MaxGroups)
+        return fail(FLK_EINVAL, "mmv_small wide: column chunk %d not in 1..32", tcols);
     if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_small: operands packed with different feature counts");
     const int dp = (int)(A.dpad / 4);
-#define FLK_WIDE64(DPV, FRV) \
-    case DPV: return launch_wide64_one<DPV, FRV>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+#define FLK_WIDE64(DPV, FRV)                                                                                         \
+    case DPV:                                                                                                       \
+        return tcols > kWide64Cols                                                                                  \
+                   ? launch_wide64_one<DPV, FRV, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st) \
+                   : launch_wide64_one<DPV, FRV, 1>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
     switch (dp) {
         FLK_WIDE64(1, 4) FLK_WIDE64(2, 4) FLK_WIDE64(3, 4) FLK_WIDE64(4, 4) FLK_WIDE64(5, 4) FLK_WIDE64(6, 4)
         FLK_WIDE64(7, 4) FLK_WIDE64(8, 4) FLK_WIDE64(9, 2) FLK_WIDE64(10, 2) FLK_WIDE64(11, 2) FLK_WIDE64(12, 2)

@@ -418,11 +418,12 @@ def test_host_rows_streamed_in_chunks(dev, monkeypatch, order, pinned):
 
 
 @pytest.mark.parametrize("d,t", [(3, 17), (3, 40), (9, 32), (15, 13), (16, 33), (17, 9), (28, 10), (28, 32), (31, 9),
-                                 (33, 5), (40, 12), (63, 7), (64, 33)])
+                                 (33, 5), (40, 12), (63, 7), (64, 33), (9, 50), (28, 47), (40, 37), (64, 100), (31, 64)])
 def test_many_right_hand_sides_small_d(dev, d, t):
     """More right-hand sides than the per-lane FMA kernels take in one pass: the 32-column register-resident kernel
     (contraction on the matrix cores), folded and plain operands, four and two resident blocks per wave, a second
-    pass for the columns beyond 32."""
+    pass for the columns beyond 32; its 64-column form (two groups of 32 on one evaluation of K) with a second group
+    that is partly filled, two and one resident blocks per wave, and a remainder pass after a full one."""
     n, m = 900 + d, 260 + t
     X, C, v, w = _rand(n, d, m, t, torch.float32, seed=d * 100 + t)
     k = GaussianKernel(0.9 * np.sqrt(d))
@@ -541,8 +542,8 @@ def test_non_finite_rows_give_nan(dev, mode, d, t):
                                  (64, 20)])
 def test_many_right_hand_sides_small_d_fp64(dev, d, t):
     """More than four right-hand sides at d <= 64 in fp64: the 16-column kernel whose contraction runs on the matrix
-    cores (one evaluation of K for 16 columns), including more columns than one pass holds and a last pass that is
-    narrow enough for the FMA kernel; 1e-11 against the CPU path, and the same numbers as column-by-column calls."""
+    cores (one evaluation of K for 16 columns) and its 32-column form (two groups of 16, the second one partly filled),
+    including more columns than one pass holds and a last pass that is narrow enough for the FMA kernel; 1e-11 against the CPU path, and the same numbers as column-by-column calls."""
     n, m = 900, 333
     X, C, v, w = _rand(n, d, m, t, torch.float64, seed=100 * d + t, scale=0.8)
     k = GaussianKernel(0.9 * np.sqrt(d) + 0.5)
