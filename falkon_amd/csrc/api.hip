@@ -67,6 +67,14 @@ constexpr int kMaxSplits = 4096;
 constexpr int64_t kL2ChunkBytes = 2 << 20;
 constexpr int64_t kL2PartialBytes = 128 << 20;
 constexpr int64_t kWideChunkBlocks = 64;  // column chunks wider than 4 accumulate in one fp32 level: keep the chunks short
+// A launch of fewer workgroups than this leaves compute units idle or unevenly loaded: its reduction chunks are then
+// chosen by the estimated makespan (all workgroups are resident at once, a compute unit works through the ones it was
+// given) instead of the rules for large problems; kTinyChunkBlocks is the shortest chunk that is worth a workgroup's
+// prologue and its partial result, whose cost is counted as kWgOverheadPercent / 100 of a block step.
+constexpr int64_t kComputeUnits = 256;
+constexpr int64_t kUnderfilledWgs = 4 * kComputeUnits;
+constexpr int64_t kTinyChunkBlocks = 2;
+constexpr int64_t kWgOverheadPercent = 50;
 
 struct Plan {
     bool large;            // LDS-tiled kernel (d beyond the register-resident kernel's range)
@@ -109,6 +117,24 @@ static void plan_register_resident(Plan &p, int64_t na_blocks, int64_t nb_blocks
     }
     if (splits > kMaxSplits) splits = kMaxSplits;
     if (splits < 1) splits = 1;
+    if (b_tiles * splits < kUnderfilledWgs && na_blocks > 0 && b_tiles > 0) {
+        // small problem: the split count with the shortest estimated makespan, at least the one chosen so far (the
+        // chunk caps above still hold); ties go to fewer splits
+        int64_t best = splits, best_cost = -1;
+        const int64_t most = na_blocks / kTinyChunkBlocks;
+        for (int64_t s = splits; s <= most && b_tiles * s <= 2 * kUnderfilledWgs; s++) {
+            int64_t c = (na_blocks + s - 1) / s;
+            if (t == 1 && c > 1 && (c & 1)) c += 1;
+            const int64_t wgs = b_tiles * ((na_blocks + c - 1) / c);
+            const int64_t deep = (wgs + kComputeUnits - 1) / kComputeUnits;     // workgroups on the busiest compute unit
+            // fp64: a second wave on a SIMD hides the latency of the exponential's table reads (measured, N = 2e4,
+            // M = 1e3, d = 8: 0.95 us per block step with one wave per SIMD, 0.60 with two or three); fp32: no gain
+            const int64_t per_block = (elem_bytes == 8 && deep >= 2) ? 65 : 100;
+            const int64_t cost = deep * (c * per_block + kWgOverheadPercent);
+            if (best_cost < 0 || cost < best_cost) { best = s; best_cost = cost; }
+        }
+        splits = best;
+    }
     p.chunk = (na_blocks + splits - 1) / splits;
     if (p.chunk < 1) p.chunk = 1;
     // even chunks for one right-hand side: the single-column fp32 kernel's loop handles two blocks per trip and
@@ -238,6 +264,27 @@ static int pack_impl(int kf, const void *X, int64_t n, int64_t d, int64_t rs, in
                              (T *)v.hnorm, v.dpad, v.nblk, one_pad, st);
 }
 
+// Prologue of a one-shot product in one launch: X1 packed into p1 (the output side of the first product), X2 into p2
+// and v, which multiplies the rows of X2, as planes in vp (zero_planes cleared planes after the t-th).
+template <typename T>
+static int pack_pair_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs, void *p1, const void *X2,
+                          int64_t m, int64_t x2_rs, int64_t x2_cs, void *p2, int64_t d, const void *sigma,
+                          int64_t n_sigma, const void *v, int64_t v_rs, int64_t v_cs, int64_t t, T *vp,
+                          int64_t zero_planes, hipStream_t st) {
+    int rc;
+    if ((rc = check_matrix("X", X1, n, d, x1_rs, x1_cs))) return rc;
+    if ((rc = check_matrix("X", X2, m, d, x2_rs, x2_cs))) return rc;
+    if (sigma == nullptr) return fail(FLK_EINVAL, "sigma: null pointer");
+    if (n_sigma != 1 && n_sigma != d)
+        return fail(FLK_EINVAL, "The size of sigma (%lld) must match the number of features (%lld) or be 1",
+                    (long long)n_sigma, (long long)d);
+    PackedView P1 = packed_view<T>(p1, n, d), P2 = packed_view<T>(p2, m, d);
+    const bool one_pad = sizeof(T) == 4 && f32_fold_applies(d);
+    return launch_pack_pair<T>((const T *)X1, n, x1_rs, x1_cs, (T *)P1.data, (T *)P1.hnorm, P1.nblk, (const T *)X2, m,
+                               x2_rs, x2_cs, (T *)P2.data, (T *)P2.hnorm, P2.nblk, d, (const T *)sigma, n_sigma,
+                               operand_scale(kf), P1.dpad, one_pad, (const T *)v, v_rs, v_cs, vp, t, zero_planes, st);
+}
+
 template <typename T>
 static int mmv_packed_impl(int kf, const void *pa, int64_t n_a, const void *pb, int64_t n_b, int64_t d, const void *vec,
                            int64_t vec_rs, int64_t vec_cs, int64_t t, const void *addend, int64_t add_rs,
@@ -293,10 +340,15 @@ static int fmmv_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x
     char *p = (char *)ws;
     void *px = p; p += packed_bytes<T>(n, d);
     void *pc = p; p += packed_bytes<T>(m, d);
-    if ((rc = pack_impl<T>(kf, X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
-    if ((rc = pack_impl<T>(kf, X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, packed_bytes<T>(m, d), st))) return rc;
-    return mmv_packed_impl<T>(kf, pc, m, px, n, d, v, v_rs, v_cs, t, nullptr, 0, 0, out, out_rs, out_cs, p,
-                              ws_bytes - (size_t)(p - (char *)ws), st);
+    T *vecp = (T *)p; p += planar_bytes<T>(m, n, d, t);
+    PackedView X = packed_view<T>(px, n, d), C = packed_view<T>(pc, m, d);
+    Plan plan = make_plan<T>(C.nblk, X.nblk, d, C.dpad, t);
+    if ((rc = pack_pair_impl<T>(kf, X1, n, x1_rs, x1_cs, px, X2, m, x2_rs, x2_cs, pc, d, sigma, n_sigma, v, v_rs, v_cs, t,
+                                vecp, zero_planes_needed<T>(plan, t), st)))
+        return rc;
+    if (n == 0 || t == 0) return FLK_OK;
+    return mmv_packed_planar<T>(kf, C, X, vecp, t, nullptr, 0, 0, (T *)out, out_rs, out_cs, false, (T *)p,
+                                ws_bytes - (size_t)(p - (char *)ws), st);
 }
 
 template <typename T>
@@ -323,13 +375,11 @@ static int fdmmv_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t 
     T *up = (T *)p; p += planar_bytes<T>(n, m, d, t);     // u multiplies the rows of X in K^T u
     T *partial = (T *)p;
     size_t partial_avail = ws_bytes - (size_t)(p - (char *)ws);
-    if ((rc = pack_impl<T>(kf, X1, n, d, x1_rs, x1_cs, sigma, n_sigma, px, packed_bytes<T>(n, d), st))) return rc;
-    if ((rc = pack_impl<T>(kf, X2, m, d, x2_rs, x2_cs, sigma, n_sigma, pc, packed_bytes<T>(m, d), st))) return rc;
     X = packed_view<T>(px, n, d);
     C = packed_view<T>(pc, m, d);
     Plan plan1 = make_plan<T>(C.nblk, X.nblk, d, C.dpad, t), plan2 = make_plan<T>(X.nblk, C.nblk, d, X.dpad, t);
-    if ((rc = launch_vec_planar<T>((const T *)v, m, t, v_rs, v_cs, vp, C.npad, zero_planes_needed<T>(plan1, t),
-                                   (const T *)C.hnorm, st)))
+    if ((rc = pack_pair_impl<T>(kf, X1, n, x1_rs, x1_cs, px, X2, m, x2_rs, x2_cs, pc, d, sigma, n_sigma, v, v_rs, v_cs, t,
+                                vp, zero_planes_needed<T>(plan1, t), st)))
         return rc;
     // u = K v + w, planar [t][X.npad] with zeroed padding (rows and the spare planes) so it can feed the
     // second product directly

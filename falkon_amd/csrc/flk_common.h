@@ -117,6 +117,14 @@ template <typename TI, typename T>   // TI: caller's element type, T: type of th
 int launch_pack(const TI *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const TI *sigma, int64_t n_sigma,
                 double scale, T *pdata, T *hnorm, int64_t dpad, int64_t nblk, bool one_pad, hipStream_t st);
 
+// One launch for the prologue of a one-shot product: packs the output-side operand (1) and the reduction-side operand
+// (2) and writes the planar copy vp[tcols + zero_planes][nblk2 * BLK] of the right-hand side v that multiplies the rows
+// of operand 2 (NaN in the rows whose half norm is not finite, as launch_vec_planar does); tcols = 0: no vector.
+template <typename T>
+int launch_pack_pair(const T *X1, int64_t n1, int64_t rs1, int64_t cs1, T *pdata1, T *hnorm1, int64_t nblk1, const T *X2,
+                     int64_t n2, int64_t rs2, int64_t cs2, T *pdata2, T *hnorm2, int64_t nblk2, int64_t d, const T *sigma,
+                     int64_t n_sigma, double scale, int64_t dpad, bool one_pad, const T *v, int64_t v_rs, int64_t v_cs,
+                     T *vp, int64_t tcols, int64_t zero_planes, hipStream_t st);
 
 // Non-finite data: a row holding a NaN or an infinity has a non-finite half norm.  The product kernels clamp the
 // kernel value (K <= 1, D^2 >= 1e-20), which turns such a row's NaN exponents into numbers; so that the result still

@@ -19,17 +19,16 @@ template <> __device__ __forceinline__ int block_pos<double>(int r) { return 4 *
 
 // TI is the caller's element type, T the type of the packed operand (T = double with TI = float serves
 // kernel matrices that are computed in double precision from single precision data).
+// Packs block blk of one operand; returns the block's half norm of row tid (threads tid < BLK; 0 for the others).
 template <typename TI, typename T>
-__global__ void __launch_bounds__(256) pack_kernel(const TI *__restrict__ X, int64_t n, int64_t d, int64_t rs,
-                                                   int64_t cs, const TI *__restrict__ sigma, int64_t n_sigma,
-                                                   double scale, T *__restrict__ pdata, T *__restrict__ hnorm,
-                                                   int64_t dpad, bool one_pad) {
+__device__ __forceinline__ T pack_block(int64_t blk, const TI *__restrict__ X, int64_t n, int64_t d, int64_t rs,
+                                        int64_t cs, const TI *__restrict__ sigma, int64_t n_sigma, double scale,
+                                        T *__restrict__ pdata, T *__restrict__ hnorm, int64_t dpad, bool one_pad) {
     constexpr int BLK = Geo<T>::BLK;
     constexpr int KT = 32;                       // features per LDS tile
     __shared__ T tile[BLK][KT + 1];
     __shared__ double nrm[BLK];
     const int tid = threadIdx.x;
-    const int64_t blk = blockIdx.x;
     const int64_t row0 = blk * BLK;
     if (tid < BLK) nrm[tid] = 0.0;
     const bool row_major = (cs == 1);
@@ -63,7 +62,20 @@ __global__ void __launch_bounds__(256) pack_kernel(const TI *__restrict__ X, int
             nrm[tid] += s;
         }
     }
-    if (tid < BLK) hnorm[row0 + tid] = (T)(-0.5 * nrm[tid]);
+    T h = T(0);
+    if (tid < BLK) {
+        h = (T)(-0.5 * nrm[tid]);
+        hnorm[row0 + tid] = h;
+    }
+    return h;
+}
+
+template <typename TI, typename T>
+__global__ void __launch_bounds__(256) pack_kernel(const TI *__restrict__ X, int64_t n, int64_t d, int64_t rs,
+                                                   int64_t cs, const TI *__restrict__ sigma, int64_t n_sigma,
+                                                   double scale, T *__restrict__ pdata, T *__restrict__ hnorm,
+                                                   int64_t dpad, bool one_pad) {
+    pack_block<TI, T>(blockIdx.x, X, n, d, rs, cs, sigma, n_sigma, scale, pdata, hnorm, dpad, one_pad);
 }
 
 template <typename TI, typename T>
@@ -103,6 +115,69 @@ __global__ void __launch_bounds__(256) vec_planar_kernel(const T *__restrict__ v
     if (row_half_norm && i < n && t < tcols && !finite_value(row_half_norm[i])) val = quiet_nan<T>();
     vp[t * npad + i] = val;
 }
+
+// ---------------------------------------------------------------------------
+// The whole prologue of a one-shot product in one launch: workgroups 0 .. nblk1 - 1 pack the output-side operand,
+// the others the reduction-side operand, and each of those also writes its BLK rows of the planar right-hand side
+// (it holds the rows' half norms, which decide where the vector becomes NaN).  Small products are bound by their
+// launches: three launches fewer than pack + pack + vec_planar.
+// ---------------------------------------------------------------------------
+template <typename T>
+struct PackArgs {
+    const T *X;
+    int64_t n, rs, cs;
+    T *pdata, *hnorm;
+    int64_t nblk;
+};
+template <typename T>
+__global__ void __launch_bounds__(256) pack_pair_kernel(PackArgs<T> out_side, PackArgs<T> red_side, int64_t d,
+                                                        const T *__restrict__ sigma, int64_t n_sigma, double scale,
+                                                        int64_t dpad, bool one_pad, const T *__restrict__ v,
+                                                        int64_t v_rs, int64_t v_cs, T *__restrict__ vp, int64_t tcols,
+                                                        int64_t planes) {
+    constexpr int BLK = Geo<T>::BLK;
+    __shared__ T hrow[BLK];
+    int64_t blk = blockIdx.x;
+    if (blk < out_side.nblk) {
+        pack_block<T, T>(blk, out_side.X, out_side.n, d, out_side.rs, out_side.cs, sigma, n_sigma, scale, out_side.pdata,
+                         out_side.hnorm, dpad, one_pad);
+        return;
+    }
+    blk -= out_side.nblk;
+    const T h = pack_block<T, T>(blk, red_side.X, red_side.n, d, red_side.rs, red_side.cs, sigma, n_sigma, scale,
+                                 red_side.pdata, red_side.hnorm, dpad, one_pad);
+    const int tid = threadIdx.x;
+    if (tid < BLK) hrow[tid] = h;
+    __syncthreads();
+    const int64_t npad = red_side.nblk * BLK;
+    for (int64_t e = tid; e < planes * BLK; e += 256) {
+        const int r = (int)(e % BLK);
+        const int64_t t = e / BLK, i = blk * BLK + r;
+        T val = (i < red_side.n && t < tcols) ? v[i * v_rs + t * v_cs] : T(0);
+        if (i < red_side.n && t < tcols && !finite_value(hrow[r])) val = quiet_nan<T>();
+        vp[t * npad + i] = val;
+    }
+}
+template <typename T>
+int launch_pack_pair(const T *X1, int64_t n1, int64_t rs1, int64_t cs1, T *pdata1, T *hnorm1, int64_t nblk1, const T *X2,
+                     int64_t n2, int64_t rs2, int64_t cs2, T *pdata2, T *hnorm2, int64_t nblk2, int64_t d, const T *sigma,
+                     int64_t n_sigma, double scale, int64_t dpad, bool one_pad, const T *v, int64_t v_rs, int64_t v_cs,
+                     T *vp, int64_t tcols, int64_t zero_planes, hipStream_t st) {
+    if (nblk1 + nblk2 == 0) return FLK_OK;
+    PackArgs<T> a{X1, n1, rs1, cs1, pdata1, hnorm1, nblk1}, b{X2, n2, rs2, cs2, pdata2, hnorm2, nblk2};
+    hipLaunchKernelGGL(pack_pair_kernel<T>, dim3((unsigned)(nblk1 + nblk2)), dim3(256), 0, st, a, b, d, sigma, n_sigma,
+                       scale, dpad, one_pad, v, v_rs, v_cs, vp, tcols, tcols > 0 ? tcols + zero_planes : 0);
+    FLK_LAUNCH_CHECK("pack_pair_kernel");
+    return FLK_OK;
+}
+template int launch_pack_pair<float>(const float *, int64_t, int64_t, int64_t, float *, float *, int64_t, const float *,
+                                     int64_t, int64_t, int64_t, float *, float *, int64_t, int64_t, const float *, int64_t,
+                                     double, int64_t, bool, const float *, int64_t, int64_t, float *, int64_t, int64_t,
+                                     hipStream_t);
+template int launch_pack_pair<double>(const double *, int64_t, int64_t, int64_t, double *, double *, int64_t,
+                                      const double *, int64_t, int64_t, int64_t, double *, double *, int64_t, int64_t,
+                                      const double *, int64_t, double, int64_t, bool, const double *, int64_t, int64_t,
+                                      double *, int64_t, int64_t, hipStream_t);
 
 template <typename T>
 __global__ void __launch_bounds__(256) zero_fill_kernel(T *__restrict__ p, int64_t count) {

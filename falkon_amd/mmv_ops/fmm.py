@@ -16,8 +16,8 @@ import torch
 from .. import _backend
 from ..options import BaseOptions
 from ..utils.helpers import sizeof_dtype
-from .fmmv import (_DTYPE_CODE, _arith_code, _check_dtype, _compute_device, _kernel_fn, _mat, _on, _rows_that_fit,
-                   _stream_handle)
+from .fmmv import (_DTYPE_CODE, _arith_code, _check_dtype, _compute_device, _current, _kernel_fn, _mat, _on,
+                   _rows_that_fit, _stream_handle)
 from .utils import check_contiguity, create_output_mat, usable_gpu_memory
 
 __all__ = ("fmm", "gauss_fmm_native")
@@ -36,7 +36,7 @@ def gauss_fmm_native(X1, X2, sigma_dev, out, compute_f64: bool, kernel_fn: int =
     p1, _, r1, c1 = _mat(X1)
     p2, _, r2, c2 = _mat(X2)
     po, _, ro, co = _mat(out)
-    with torch.cuda.device(X1.device):
+    with _current(X1.device):
         rc = lib.flk_kernel_fmm(kernel_fn, p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
                                 po, ro, co, code, int(compute_f64), ws.data_ptr(), ws_bytes,
                                 _stream_handle(X1.device))

@@ -10,6 +10,7 @@ resident; split the rows of X1 only if the packed operands do not fit".
 There is no CPU computation in this module.
 """
 import math
+import contextlib
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -29,8 +30,22 @@ def _mat(t: torch.Tensor) -> Tuple[int, int, int, int]:
     return t.data_ptr(), t.shape[0], t.stride(0), t.stride(1)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_handle(dev: torch.device) -> int:
+    """The HIP stream torch currently works on, as an integer handle."""
+    if _raw_stream is not None and dev.index is not None:
+        return _raw_stream(dev.index)                      # the same handle without building a Stream object
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _current(dev: torch.device):
+    """Context that makes ``dev`` the current GPU; nothing to enter or leave when it already is (a small call's
+    host time is a few tens of microseconds, and torch's device guard object costs several of them)."""
+    if dev.index is None or torch.cuda.current_device() == dev.index:
+        return contextlib.nullcontext()
+    return torch.cuda.device(dev)
 
 
 def _arith_code(dtype: torch.dtype, opt: Optional[BaseOptions]) -> int:
@@ -53,7 +68,7 @@ def gauss_fmmv_native(X1, X2, sigma_dev, v, out, kernel_fn: int = _backend.FLK_G
     p2, _, r2, c2 = _mat(X2)
     pv, _, rv, cv = _mat(v)
     po, _, ro, co = _mat(out)
-    with torch.cuda.device(X1.device):
+    with _current(X1.device):
         rc = lib.flk_kernel_fmmv(kernel_fn, p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
                                  pv, rv, cv, t, po, ro, co, code, ws.data_ptr(), ws_bytes, _stream_handle(X1.device))
     _backend.raise_for_status(rc, "flk_kernel_fmmv")
@@ -73,7 +88,7 @@ def gauss_fdmmv_native(X1, X2, sigma_dev, v, w, out, kernel_fn: int = _backend.F
     pv, _, rv, cv = _mat(v)
     pw, rw, cw = (w.data_ptr(), w.stride(0), w.stride(1)) if w is not None else (None, 0, 0)
     po, _, ro, co = _mat(out)
-    with torch.cuda.device(X1.device):
+    with _current(X1.device):
         rc = lib.flk_kernel_fdmmv(kernel_fn, p1, n, r1, c1, p2, m, r2, c2, d, sigma_dev.data_ptr(), sigma_dev.numel(),
                                   pv, rv, cv, pw, rw, cw, t, po, ro, co, code, ws.data_ptr(), ws_bytes,
                                   _stream_handle(X1.device))
@@ -106,12 +121,22 @@ def _reject_block_kwargs(kwargs_m1, kwargs_m2):
         raise TypeError("The Gaussian kernel takes no per-block keyword tensors (kwargs_m1 / kwargs_m2)")
 
 
+_gpu_seen = False
+
+
+def _gpu_present() -> bool:
+    global _gpu_seen
+    if not _gpu_seen:
+        _gpu_seen = torch.cuda.is_available()          # asked again on every call only while the answer is no
+    return _gpu_seen
+
+
 def _compute_device(opt: BaseOptions, data_devs) -> torch.device:
     """The GPU to compute on; mirrors the reference's device choice (fmmv.py:906,1038) minus its CPU branch."""
     if opt.use_cpu:
         raise RuntimeError("falkon_amd has no CPU compute path: `use_cpu=True` cannot be honoured "
                            "(the MI355X kernels are the only implementation)")
-    if not torch.cuda.is_available():
+    if not _gpu_present():
         raise RuntimeError("falkon_amd needs a ROCm GPU (MI355X); torch.cuda.is_available() is False")
     cuda_devs = {d for d in data_devs if d.type == "cuda"}
     if len(cuda_devs) > 1:

@@ -47,6 +47,7 @@ class ConjugateGradient:
     # ------------------------------------------------------------------ GPU tensors
     def _solve_on_device(self, X0, B, mmv, max_iter, callback) -> torch.Tensor:
         from . import _backend
+        from .mmv_ops.fmmv import _current, _stream_handle
         lib = _backend.load()
         started = time.time()
         dev, (m, t) = B.device, B.shape
@@ -77,10 +78,10 @@ class ConjugateGradient:
 
         def update(mode, q, it):
             q = same_layout(q)
-            with torch.cuda.device(dev):
+            with _current(dev):
                 rc = lib.flk_cg_update(mode, sol.data_ptr(), resid.data_ptr(), direction.data_ptr(), q.data_ptr(),
                                        B.data_ptr(), m, t, rs, cs, rsold.data_ptr(), state.data_ptr(), it, eps, tol2,
-                                       differential, code, torch.cuda.current_stream(dev).cuda_stream)
+                                       differential, code, _stream_handle(dev))
             _backend.raise_for_status(rc, "flk_cg_update")
 
         def iteration(it):
