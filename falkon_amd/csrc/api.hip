@@ -157,7 +157,7 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
                                (int64_t)sizeof(T));
     } else {
         const int64_t a_tiles = (na_blocks + mmv_large_a_tile_blocks<T>() - 1) / mmv_large_a_tile_blocks<T>();
-        const int64_t b_tiles = (nb_blocks + mmv_large_b_tile_blocks<T>() - 1) / mmv_large_b_tile_blocks<T>();
+        const int64_t b_tiles = (nb_blocks + mmv_large_b_tile_blocks<T>(t) - 1) / mmv_large_b_tile_blocks<T>(t);
         int64_t splits = (kTargetWgsLarge + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
         if (splits > a_tiles) splits = a_tiles;
         if (splits > kMaxSplits) splits = kMaxSplits;
@@ -167,7 +167,7 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
         p.splits = (int)((a_tiles + p.chunk - 1) / p.chunk);
         if (p.splits < 1) p.splits = 1;
         p.partials = p.splits * mmv_large_partials_per_split<T>();
-        p.col_chunk = mmv_large_max_cols<T>();
+        p.col_chunk = mmv_large_max_cols<T>(t);
     }
     return p;
 }
@@ -176,7 +176,7 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
 // that many planes of the planar right-hand side, so the planes past the caller's columns must be zero.
 template <typename T>
 static int instantiated_cols(const Plan &p, int tc) {
-    static const int large[] = {1, 2, 4, 8, 16};     // the 8-column instantiation exists in fp64 only
+    static const int large[] = {1, 2, 4, 8, 16, 32, 64};     // 8 columns: an instantiation of fp64 only; 64: of fp32 only
     if (p.large) {
         for (int w : large) if (tc <= w && (w != 8 || sizeof(T) == 8)) return w;
         return tc;

@@ -161,9 +161,9 @@ constexpr int64_t kColPad = 31;
 // LDS-tiled ("large d") product kernel: any padded feature count, up to mmv_large_max_cols columns per pass.
 // Writes splits * mmv_large_partials_per_split partial results.
 template <typename T> int mmv_large_a_tile_blocks();
-template <typename T> int mmv_large_b_tile_blocks();
+template <typename T> int mmv_large_b_tile_blocks(int64_t t);   // output blocks per workgroup with t columns in all
 template <typename T> int mmv_large_partials_per_split();
-template <typename T> int mmv_large_max_cols();
+template <typename T> int mmv_large_max_cols(int64_t t);   // columns per pass when there are t in all
 
 // The kernels that evaluate K are compiled once per kernel function (the same source with -DFLK_KF=0..4,
 // FLK_GAUSSIAN .. FLK_LAPLACIAN_DU): launchers carry the function in their name, and the helpers below pick one.

@@ -13,6 +13,12 @@
 //
 // Waves are arranged WVA (A) x WVB (B); waves with the same wb produce partial sums for the same
 // output rows and simply write separate partials (they count as extra splits for the reduction).
+//
+// Right-hand sides per pass: up to 4 (fp32) / 8 (fp64) are contracted with per-lane FMAs; beyond, a second MFMA takes
+// the kernel values in the accumulator registers as its A operand and a 16-column (fp32 also 32-column) slice of vec
+// as its B operand, and up to 64 columns ride on one evaluation of K as two groups of 32 (fp32) or four of 16 (fp64).
+// Measured, dfmmv at N = 5e5, M = 1e4, d = 784: fp32 T = 16 123.4 ms, 32 132.2, 64 149.0 (four passes of 16: 494);
+// fp64 T = 16 258.9, 32 262.7, 64 287.1 (1036).  N = 5e5, M = 2e4, d = 100: fp32 47.0 / 50.6 / 84.4, fp64 89.2 / 97.9 / 131.8.
 #include <type_traits>
 
 #include "flk_common.h"
@@ -69,7 +75,7 @@ template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC, int TT, in
 __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   // two waves per SIMD either way
     mmv_large_kernel(const T *__restrict__ PA, const T *__restrict__ hA, const T *__restrict__ vecp, int64_t vec_ld,
                      int tcols, const T *__restrict__ PB, const T *__restrict__ hB, int64_t na_blocks,
-                     int64_t nb_blocks, int64_t dpad, int last_steps, int64_t a_tiles_per_chunk,
+                     int64_t nb_blocks, int64_t dpad, int n_chunks_used, int last_steps, int64_t a_tiles_per_chunk,
                      T *__restrict__ partial, int64_t nb_pad, bool y_fastest, void *__restrict__ kout = nullptr,
                      int64_t kout_ld = 0, int64_t n_a = 0, int64_t n_b = 0) {
     constexpr bool kStore = !std::is_void<O>::value;
@@ -84,9 +90,16 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     __shared__ __attribute__((aligned(16))) T ldsB[2][G::B_ELEMS];
     // More than four (fp32) / eight (fp64) columns: the contraction against vec runs on the MFMA as well (a second,
     // small GEMM whose A operand are the kernel values sitting in the accumulator registers, see the epilogue), with vec staged
-    // as [row][16 columns] at a stride of 17 elements.  Fewer columns: per-lane FMAs, vec staged planar.
+    // as [row][16 or 32 columns] at an odd stride.  Fewer columns: per-lane FMAs, vec staged planar.
+    // fp32: the 32x32x2 step has room for 32 columns (lane % 32), fp64's 16x16x4 for 16.
     constexpr bool kMfmaEpi = TT > kLargeFmaCols<T>;
-    constexpr int kVecStride = 17;
+    // More columns than one step holds: NC groups of columns ride on the same kernel values (one more contraction
+    // per group, NC times the output accumulators).
+    constexpr int kGroupCols = (sizeof(T) == 4 && TT > 16) ? 32 : 16;
+    constexpr int NC = (kMfmaEpi && TT > kGroupCols) ? TT / kGroupCols : 1;
+    constexpr int kEpiCols = kGroupCols * NC;
+    static_assert(TT <= kEpiCols || !kMfmaEpi, "columns per pass must be a whole number of column groups");
+    constexpr int kVecStride = kEpiCols + 1;
     constexpr int kRowBuf = kMfmaEpi ? G::A_ROWS * (1 + kVecStride) : (1 + TT) * G::A_ROWS;
     __shared__ __attribute__((aligned(32))) T ldsRow[kRowBuf];   // [hA | vec ...] of the A tile
 
@@ -106,7 +119,9 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     const int64_t at0 = (int64_t)by * a_tiles_per_chunk;
     int64_t at1 = at0 + a_tiles_per_chunk;
     if (at1 > a_tiles) at1 = a_tiles;
-    const int64_t n_chunks = DPsteps / KC;     // dpad is a whole number of chunks
+    // chunks of KC steps that hold features of the data; the last of them stops after last_steps steps (dpad is padded
+    // to whole chunks of kLargeKChunk steps: what lies past the data is zero and is never read)
+    const int64_t n_chunks = n_chunks_used;
 
     // half norms of this lane's output rows
     T hb[WB_FR];
@@ -117,7 +132,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         hb[q] = hB[bb * TR::BLK + TR::out_row(j)];
     }
     T out[WB_FR][kMfmaEpi ? 1 : TT];          // per-lane FMA path: out[q][t] for this lane's output row
-    acc_t out2[kMfmaEpi ? WB_FR : 1];         // MFMA path: lane = column t, registers = output rows
+    acc_t out2[kMfmaEpi ? WB_FR : 1][NC];     // MFMA path: lane = column t (of every group), registers = output rows
 #pragma unroll
     for (int q = 0; q < WB_FR; q++)
 #pragma unroll
@@ -125,7 +140,9 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
     for (int q = 0; q < (kMfmaEpi ? WB_FR : 1); q++)
 #pragma unroll
-        for (int r = 0; r < TR::ACCN; r++) out2[q][r] = T(0);
+        for (int g = 0; g < NC; g++)
+#pragma unroll
+            for (int r = 0; r < TR::ACCN; r++) out2[q][g][r] = T(0);
 
     for (int64_t at = at0; at < at1; at++) {
         const int64_t ablk0 = at * G::NAB;
@@ -158,7 +175,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         // are issued before anything waits, and the barrier that protects ldsRow and the stages from the
         // previous tile's epilogue comes after them, so one memory round trip covers the whole prologue.
         fetch(0);
-        constexpr int kRowVals = (1 + (kMfmaEpi ? 16 : TT)) * G::A_ROWS;
+        constexpr int kRowVals = (1 + (kMfmaEpi ? kEpiCols : TT)) * G::A_ROWS;
         constexpr int kRowValsPerThread = (kRowVals + kLThreads - 1) / kLThreads;
         T rowv[kRowValsPerThread];
 #pragma unroll
@@ -339,22 +356,36 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             }
             // out2[q][j-rows][t] += sum_i K[i][j] vec[i][t]: accumulator register s of a lane is exactly the MFMA
             // A operand of step s (row i = acc_row(s, lg), column j = lane), so K needs no data movement; the
-            // B operand is vec[acc_row(s, lg)][t] with t = lane % 16 (columns past 16 are never stored).
-            const int tl = j & 15;
+            // B operand is vec[acc_row(s, lg)][t] with t = lane % kGroupCols (+ kGroupCols per further group; fp32 lanes
+            // 16 .. 31 repeat the columns 0 .. 15 in the 16-column form and are never stored).
+            const int tl = j & (kGroupCols - 1);
             const T *vb = &ldsRow[G::A_ROWS + tl];
             // one read ahead, fenced like the feature loop (otherwise all reads are hoisted and spilled)
-            T bval = vb[((wa * WA_FR) * TR::BLK + TR::acc_row(0, lg)) * kVecStride], bnext = T(0);
+            T bval[NC], bnext[NC];
+#pragma unroll
+            for (int g = 0; g < NC; g++) {
+                bval[g] = vb[((wa * WA_FR) * TR::BLK + TR::acc_row(0, lg)) * kVecStride + g * kGroupCols];
+                bnext[g] = T(0);
+            }
 #pragma unroll
             for (int p = 0; p < WA_FR; p++) {
                 const int rbase = (wa * WA_FR + p) * TR::BLK;
 #pragma unroll
                 for (int s2 = 0; s2 < TR::ACCN; s2++) {
-                    if (s2 + 1 < TR::ACCN) bnext = vb[(rbase + TR::acc_row(s2 + 1, lg)) * kVecStride];
-                    else if (p + 1 < WA_FR) bnext = vb[(rbase + TR::BLK + TR::acc_row(0, lg)) * kVecStride];
 #pragma unroll
-                    for (int q = 0; q < WB_FR; q++) out2[q] = TR::mfma(acc[p][q][s2], bval, out2[q]);
-                    asm volatile("" : "+v"(bval) : "v"(vb) : "memory");
-                    bval = bnext;
+                    for (int g = 0; g < NC; g++) {
+                        if (s2 + 1 < TR::ACCN) bnext[g] = vb[(rbase + TR::acc_row(s2 + 1, lg)) * kVecStride + g * kGroupCols];
+                        else if (p + 1 < WA_FR) bnext[g] = vb[(rbase + TR::BLK + TR::acc_row(0, lg)) * kVecStride + g * kGroupCols];
+                    }
+#pragma unroll
+                    for (int g = 0; g < NC; g++)
+#pragma unroll
+                        for (int q = 0; q < WB_FR; q++) out2[q][g] = TR::mfma(acc[p][q][s2], bval[g], out2[q][g]);
+#pragma unroll
+                    for (int g = 0; g < NC; g++) {
+                        asm volatile("" : "+v"(bval[g]) : "v"(vb) : "memory");
+                        bval[g] = bnext[g];
+                    }
                 }
             }
         }
@@ -364,16 +395,20 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         // nothing left to write
     } else if constexpr (kMfmaEpi) {
         // lane = column t (both lane groups hold different output rows): no cross-lane step
-        const int tl = j & 15;
-        if (j < 16 && tl < tcols) {
+        const int tl = j & (kGroupCols - 1);
 #pragma unroll
-            for (int q = 0; q < WB_FR; q++) {
-                const int64_t bb = bblk0 + wb * WB_FR + q;
-                if (bb < nb_blocks) {
+        for (int g = 0; g < NC; g++) {
+            const int col = tl + g * kGroupCols;
+            if (j < kGroupCols && col < tcols) {
 #pragma unroll
-                    for (int r = 0; r < TR::ACCN; r++)
-                        partial[(((int64_t)by * kLWavesA + wa) * tcols + tl) * nb_pad + bb * TR::BLK +
-                                TR::acc_row(r, lg)] = out2[q][r];
+                for (int q = 0; q < WB_FR; q++) {
+                    const int64_t bb = bblk0 + wb * WB_FR + q;
+                    if (bb < nb_blocks) {
+#pragma unroll
+                        for (int r = 0; r < TR::ACCN; r++)
+                            partial[(((int64_t)by * kLWavesA + wa) * tcols + col) * nb_pad + bb * TR::BLK +
+                                    TR::acc_row(r, lg)] = out2[q][g][r];
+                    }
                 }
             }
         }
@@ -404,36 +439,51 @@ template <> struct LCfg<float>  { static constexpr int WVA = 2, WVB = 2, WA_FR =
 // fp64: 8 waves (2 x 4), one workgroup per CU; tile 128 (A) x 128 (B) rows.
 template <> struct LCfg<double> { static constexpr int WVA = 2, WVB = 4, WA_FR = 4, WB_FR = 2, KC = 8; };
 
+// fp32 with 17 .. 32 columns: the row values of an A tile take 34 KB of LDS, two workgroups with the 48 KB of feature
+// stages each no longer fit a CU; 8 waves (2 x 4) on a 256 x 256 tile, one workgroup per CU.
+struct LCfgWide32 { static constexpr int WVA = 2, WVB = 4, WA_FR = 4, WB_FR = 2, KC = 8; };
+// fp64 with 17 .. 32 columns (two groups of 16): the row values take 35 KB; feature stages of four steps instead of eight
+// (64 KB instead of 128) make room for them.
+struct LCfgWide64 { static constexpr int WVA = 2, WVB = 4, WA_FR = 4, WB_FR = 2, KC = 4; };
+
 constexpr int kLargeMaxCols = 16;
 #if FLK_KF == FLK_GAUSSIAN   // the tile geometry is the same for every kernel function: defined once
 template <typename T> int mmv_large_a_tile_blocks() { return LCfg<T>::WVA * LCfg<T>::WA_FR; }
-template <typename T> int mmv_large_b_tile_blocks() { return LCfg<T>::WVB * LCfg<T>::WB_FR; }
+template <typename T> int mmv_large_b_tile_blocks(int64_t t) {
+    if (sizeof(T) == 4 && t > kLargeMaxCols) return LCfgWide32::WVB * LCfgWide32::WB_FR;
+    return LCfg<T>::WVB * LCfg<T>::WB_FR;
+}
 template <typename T> int mmv_large_partials_per_split() { return LCfg<T>::WVA; }
-template <> int mmv_large_max_cols<float>() { return kLargeMaxCols; }
-template <> int mmv_large_max_cols<double>() { return kLargeMaxCols; }
+template <typename T> int mmv_large_max_cols(int64_t t) {
+    return t > 2 * kLargeMaxCols ? 4 * kLargeMaxCols : t > kLargeMaxCols ? 2 * kLargeMaxCols : kLargeMaxCols;
+}
+template int mmv_large_max_cols<float>(int64_t);
+template int mmv_large_max_cols<double>(int64_t);
 template int mmv_large_a_tile_blocks<float>();
 template int mmv_large_a_tile_blocks<double>();
-template int mmv_large_b_tile_blocks<float>();
-template int mmv_large_b_tile_blocks<double>();
+template int mmv_large_b_tile_blocks<float>(int64_t);
+template int mmv_large_b_tile_blocks<double>(int64_t);
 template int mmv_large_partials_per_split<float>();
 template int mmv_large_partials_per_split<double>();
 #endif
 
-template <typename T, int TT>
+template <typename T, int TT, typename C = LCfg<T>>
 static int launch_large_tt(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
                            int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
-    typedef LCfg<T> C;
     const int64_t nbb = C::WVB * C::WB_FR;
     dim3 grid((unsigned)((B.nblk + nbb - 1) / nbb), (unsigned)splits);
-    // MFMA steps of the last feature chunk that hold features of the data (the rest of the chunk is zero padding)
+    // feature chunks that hold features of the data, and the MFMA steps of the last of them that do
     const int64_t chunk_features = (int64_t)C::KC * LTraits<T>::KG;
-    const int64_t tail = A.d - (A.dpad / chunk_features - 1) * chunk_features;
+    const int64_t n_chunks = (A.d + chunk_features - 1) / chunk_features;
+    const int64_t tail = A.d - (n_chunks - 1) * chunk_features;
     const int last_steps = (int)((tail + LTraits<T>::KG - 1) / LTraits<T>::KG);
-    if (last_steps < 1 || last_steps > C::KC) return fail(FLK_EINVAL, "mmv_large: operand padding does not match d");
+    if (n_chunks < 1 || n_chunks * chunk_features > A.dpad || last_steps < 1 || last_steps > C::KC)
+        return fail(FLK_EINVAL, "mmv_large: operand padding does not match d");
     hipLaunchKernelGGL((mmv_large_kernel<T, C::WVA, C::WVB, C::WA_FR, C::WB_FR, C::KC, TT, FLK_KF>), grid,
                        dim3(64 * C::WVA * C::WVB), 0, st,
                        (const T *)A.data, (const T *)A.hnorm, vecp, vec_ld, tcols, (const T *)B.data,
-                       (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, last_steps, a_tiles_per_chunk, partial, B.npad, B.n > A.n);
+                       (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, (int)n_chunks, last_steps, a_tiles_per_chunk, partial, B.npad,
+                       B.n > A.n);
     FLK_LAUNCH_CHECK("mmv_large_kernel");
     return FLK_OK;
 }
@@ -456,7 +506,8 @@ int FLK_CAT(launch_fmm_large_kf, FLK_KF)(const PackedView &A, const PackedView &
         return fail(FLK_EINVAL, "fmm: operand padding does not match the LDS-tiled kernel");
     hipLaunchKernelGGL((mmv_large_kernel<T, C::WVA, C::WVB, C::WA_FR, C::WB_FR, C::KC, 1, FLK_KF, O>), grid,
                        dim3(64 * C::WVA * C::WVB), 0, st, (const T *)A.data, (const T *)A.hnorm, (const T *)nullptr,
-                       (int64_t)0, 0, (const T *)B.data, (const T *)B.hnorm, A.nblk, B.nblk, A.dpad, last_steps, per_wg,
+                       (int64_t)0, 0, (const T *)B.data, (const T *)B.hnorm, A.nblk, B.nblk, A.dpad,
+                       (int)(A.dpad / chunk_features), last_steps, per_wg,
                        (T *)nullptr, B.npad, B.n > A.n, (void *)out, ld, A.n, B.n);
     FLK_LAUNCH_CHECK("mmv_large_kernel (kernel matrix)");
     return FLK_OK;
@@ -473,8 +524,19 @@ int FLK_CAT(launch_mmv_large_kf, FLK_KF)(const PackedView &A, const PackedView &
                                          int tcols, int64_t a_tiles_per_chunk, int splits, T *partial,
                                          hipStream_t st) {
     if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_large: operands packed with different feature counts");
-    if (tcols < 1 || tcols > kLargeMaxCols)
-        return fail(FLK_EINVAL, "mmv_large: column chunk %d not in 1..%d", tcols, kLargeMaxCols);
+    const int most = 4 * kLargeMaxCols;
+    if (tcols < 1 || tcols > most) return fail(FLK_EINVAL, "mmv_large: column chunk %d not in 1..%d", tcols, most);
+    if (tcols > kLargeMaxCols) {
+        if constexpr (sizeof(T) == 4) {
+            if (tcols > 2 * kLargeMaxCols)
+                return launch_large_tt<T, 64, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+            return launch_large_tt<T, 32, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+        } else {
+            if (tcols > 2 * kLargeMaxCols)
+                return launch_large_tt<T, 64, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+            return launch_large_tt<T, 32, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+        }
+    }
     if (tcols == 1) return launch_large_tt<T, 1>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols == 2) return launch_large_tt<T, 2>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols <= 4) return launch_large_tt<T, 4>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);

@@ -101,9 +101,15 @@ def test_reference_fixture_fp64(dev, order, sig):
     (333, 520, 300, 7),
     (257, 129, 70, 8),      # eight columns (per-lane FMAs in fp64), a last feature chunk that is mostly padding
     (130, 300, 97, 9),      # one real feature in the last chunk
+    (400, 300, 784, 32),    # 17 .. 32 columns in one pass: the full width of the fp32 step, two groups of 16 in fp64
+    (260, 300, 97, 24),     # ... partly filled, with whole feature chunks of padding behind the data (fp64: chunks of 16)
+    (150, 520, 131, 48),    # 33 .. 64 columns in one pass: column groups on one evaluation of K, the last one half full
+    (300, 200, 70, 64),
+    (280, 150, 200, 70),    # a 64-column pass and a narrow one
 ])
 def test_large_d_vs_oracle(dev, dtype, n, m, d, t):
-    """d > 64 runs the LDS-tiled kernel; same tolerances against the blocked CPU oracle."""
+    """d > 64 runs the LDS-tiled kernel (up to 64 right-hand sides per pass); same tolerances against the blocked CPU
+    oracle."""
     X, C, v, w = _rand(n, d, m, t, dtype, seed=n + d, scale=0.5)
     sigma = 0.6 * np.sqrt(d)
     k = GaussianKernel(sigma)
