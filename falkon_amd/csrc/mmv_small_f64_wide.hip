@@ -13,7 +13,9 @@
 // With NC = 2 a second group of 16 columns rides on the same kernel values (four more MFMAs per tile and group).
 // Measured, dfmmv at N = 5e5, M = 2e4: 32 columns in one pass against two passes of 16: d = 9 35.1 ms against 49.1,
 // d = 28 45.3 against 69.3, d = 64 69.2 against 116.7; 17 columns 35 / 45 / 69 ms against 39.1 / 58.9 / 106.6 for a
-// 16-column pass followed by a one-column pass.
+// 16-column pass followed by a one-column pass.  (Four groups, 64 columns, were measured and not kept: their 68 KB of
+// staged row values leave one workgroup per CU, and with half the resident blocks T = 64 took 71.1 / 81.7 / 143.8 ms
+// against 70.0 / 90.5 / 138.6 for two passes of 32, T = 33 80.5 at d = 28 against 69.5.)
 #include "flk_common.h"
 #include "kernel_fn.h"
 
