@@ -306,22 +306,20 @@ class _KernelMmvFn(torch.autograd.Function):
 _EXPLICIT_BLOCK_BYTES = 8 * 2**30          # size of a stored block of K, memory permitting
 
 
-def _columns_per_pass(d: int, dtype: torch.dtype) -> int:
-    """Right-hand sides one evaluation of K serves in the product kernels."""
-    return 16 if d > 64 or dtype == torch.float64 else 32
-
-
-def _explicit_blocks_pay(d: int, t: int, dtype: torch.dtype, opt: BaseOptions) -> bool:
+def _explicit_blocks_pay(d: int, t: int, dtype: torch.dtype, opt: BaseOptions, two_products: bool = False) -> bool:
     """Whether the caller opted into stored blocks of K (``many_rhs_stored_blocks``) and t right-hand sides are
-    enough passes of the product kernels for them to be the faster route."""
+    enough for them to be the faster route.  The product kernels serve up to 64 columns (32 in fp64 up to 64 features)
+    with one evaluation of K; ``two_products`` (``dmmv``) evaluates K twice on the matrix-free route and once on this
+    one.  Break-even measured at N = 5e5, M = 2e4 (d = 784: N = 2.5e5, M = 1e4) for d = 9, 28, 64, 100, 784 and
+    T = 17 ... 256; e.g. fp32 d = 28: mmv T = 64 17.8 ms matrix-free against 23.0 stored, T = 96 28.8 / 27.1;
+    dmmv T = 64 34.8 / 33.1, T = 128 69.5 / 49.3; fp64 d = 100: dmmv T = 64 131.8 / 151.5, T = 96 229.5 / 151.7."""
     if getattr(opt, "never_store_kernel", False) or not getattr(opt, "many_rhs_stored_blocks", False):
         return False
-    passes = -(-t // _columns_per_pass(d, dtype))
-    if d > 64:
-        return passes >= 2
     if dtype == torch.float64:
-        return passes >= 5
-    return passes >= (4 if d <= 32 else 3)
+        least = (96, 64) if d <= 64 else (64, 64) if d <= 256 else (64, 16)
+    else:
+        least = (96, 64) if d <= 32 else (64, 32) if d <= 64 else (32, 16)
+    return t > least[1 if two_products else 0]
 
 
 def _block_leading_dim(M: int, sz: int) -> int:
@@ -479,7 +477,7 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
         # (opt-in beyond 64 features whatever T: a stored block costs about one pass of the product kernel there,
         # and K^T(K v + w) then needs K once instead of twice; C4: 122 -> 69 ms.  Off by default: the path is
         # specified as one that never materialises K.)
-        stored = _explicit_blocks_pay(D, T, X1.dtype, opt) or (
+        stored = _explicit_blocks_pay(D, T, X1.dtype, opt, two_products=True) or (
             getattr(opt, "dmmv_stored_blocks", False) and D > 64 and not getattr(opt, "never_store_kernel", False))
         if N > 0 and M > 0 and stored:
             if _fdmmv_explicit(X1, X2, v, w, out, sigma_dev, kernel_fn, dev, opt):

@@ -646,7 +646,7 @@ def test_packed_entry_points(dev, dtype, n, m, d, t):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-@pytest.mark.parametrize("n,m,d,t", [(700, 300, 100, 20), (300, 520, 784, 40), (2000, 333, 28, 130), (900, 257, 40, 70),
+@pytest.mark.parametrize("n,m,d,t", [(700, 300, 100, 70), (300, 520, 784, 40), (2000, 333, 28, 130), (900, 257, 40, 100),
                                      (500, 129, 9, 200)])
 def test_many_right_hand_sides_through_stored_blocks(dev, dtype, n, m, d, t, monkeypatch):
     """Opt-in ``many_rhs_stored_blocks``: with enough right-hand sides the drivers store blocks of K and contract them
@@ -656,7 +656,8 @@ def test_many_right_hand_sides_through_stored_blocks(dev, dtype, n, m, d, t, mon
     import importlib
     drv = importlib.import_module("falkon_amd.mmv_ops.fmmv")
     stored = FalkonOptions(many_rhs_stored_blocks=True)
-    assert drv._explicit_blocks_pay(d, t, dtype, stored) or dtype == torch.float64 and d <= 64 and t < 65
+    assert drv._explicit_blocks_pay(d, t, dtype, stored, two_products=True)
+    assert drv._explicit_blocks_pay(d, t, dtype, stored) or (dtype == torch.float64 and d == 784)
     X, C, v, w = _rand(n, d, m, t, dtype, seed=n + t, scale=0.6)
     sigma = 0.8 * np.sqrt(d)
     k, k_free = GaussianKernel(sigma, opt=stored), GaussianKernel(sigma)

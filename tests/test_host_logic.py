@@ -316,12 +316,17 @@ def test_stored_block_route_rules(monkeypatch):
     assert not any(drv._explicit_blocks_pay(d, t, dt, FalkonOptions())
                    for d in (9, 28, 100, 784) for t in (1, 17, 97, 1000, 10**4) for dt in (f32, f64))
     opt = FalkonOptions(many_rhs_stored_blocks=True)
-    # one pass of the product kernels: never; two passes beyond 64 features; four (fp32) / five (fp64) at small d
-    assert not drv._explicit_blocks_pay(784, 16, f32, opt) and drv._explicit_blocks_pay(784, 17, f32, opt)
-    assert not drv._explicit_blocks_pay(28, 96, f32, opt) and drv._explicit_blocks_pay(28, 97, f32, opt)
-    assert not drv._explicit_blocks_pay(40, 64, f32, opt) and drv._explicit_blocks_pay(40, 65, f32, opt)
-    assert not drv._explicit_blocks_pay(28, 64, f64, opt) and drv._explicit_blocks_pay(28, 65, f64, opt)
-    assert drv._explicit_blocks_pay(100, 17, f64, opt)
+    # from the measured break-even on: later for one product than for the two of dmmv (which evaluates K twice on the
+    # matrix-free route), later at small d and in fp64, where an evaluation of K is cheap next to storing it
+    pays = drv._explicit_blocks_pay
+    assert not pays(784, 32, f32, opt) and pays(784, 33, f32, opt)
+    assert not pays(784, 16, f32, opt, two_products=True) and pays(784, 17, f32, opt, two_products=True)
+    assert not pays(28, 96, f32, opt) and pays(28, 97, f32, opt)
+    assert not pays(28, 64, f32, opt, two_products=True) and pays(28, 65, f32, opt, two_products=True)
+    assert not pays(40, 64, f32, opt) and pays(40, 65, f32, opt) and pays(40, 33, f32, opt, two_products=True)
+    assert not pays(28, 96, f64, opt) and pays(28, 97, f64, opt) and pays(28, 65, f64, opt, two_products=True)
+    assert not pays(100, 64, f64, opt, two_products=True) and pays(100, 65, f64, opt, two_products=True)
+    assert pays(784, 17, f64, opt, two_products=True) and not pays(784, 64, f64, opt) and pays(784, 65, f64, opt)
     assert not drv._explicit_blocks_pay(784, 1000, f32, FalkonOptions(many_rhs_stored_blocks=True, never_store_kernel=True))
     # block rows: within the block size, within half of what the budget leaves, nothing below 32 rows
     monkeypatch.setattr(drv, "usable_gpu_memory", lambda dev, cap, slack, enough=float("inf"): 64 * 2**30)
