@@ -180,6 +180,77 @@ def cpu_baseline(X, C, sigma, v, w, gpu_out_fn, rows, time_rows, reps, kernel_na
     return base
 
 
+def run_c1(args, lib):
+    """Configuration 1 (N = 20 000, d = 8, M = 1 000, one right-hand side, fp64 fmmv): a launch-bound call.  Reports the
+    time of a call the host waits for, the rate of calls issued back to back, the product kernel's share, and the
+    result against the whole CPU path (the case is small enough to run it in full)."""
+    from falkon_amd import GaussianKernel, _backend
+    dev = torch.device("cuda:0")
+    N, d, M, T = 20_000, 8, 1_000, 1
+    rng = np.random.default_rng(1001)                # draw order X, idx, v
+    X = torch.from_numpy(rng.standard_normal((N, d)))
+    C = X[torch.from_numpy(rng.choice(N, size=M, replace=False))].contiguous()
+    v = torch.from_numpy(rng.standard_normal((M, T)))
+    tdt = torch.float64 if args.dtype == "f64" else torch.float32
+    X, C, v = X.to(tdt), C.to(tdt), v.to(tdt)
+    Xg, Cg, vg = X.to(dev), C.to(dev), v.to(dev)
+    kernel = GaussianKernel(2.0)
+    out = torch.empty(N, T, dtype=tdt, device=dev)
+    for _ in range(max(args.warmup, 20)):
+        kernel.mmv(Xg, Cg, vg, out=out)
+    torch.cuda.synchronize()
+    waits = []
+    for _ in range(200):
+        t0 = time.perf_counter()
+        kernel.mmv(Xg, Cg, vg, out=out)
+        torch.cuda.synchronize()
+        waits.append(time.perf_counter() - t0)
+    steps = max(args.steps, 1000)
+    lib.flk_kernel_timing_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        kernel.mmv(Xg, Cg, vg, out=out)
+    host = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    tot_ms, launches = ctypes.c_double(), ctypes.c_int64()
+    _backend.raise_for_status(lib.flk_kernel_timing_read(ctypes.byref(tot_ms), ctypes.byref(launches)), "flk_kernel_timing_read")
+    lib.flk_kernel_timing_enable(0)
+    kern_ms = tot_ms.value / max(launches.value, 1)
+    flop = N * M * (2 * d + 4 + 2 * T)
+    peak = FP64_PEAK_TFLOPS if tdt == torch.float64 else FP32_PEAK_TFLOPS
+    res = {
+        "metric": f"fmmv kernel-entries/sec (N*M*T/s) {'fp64' if tdt == torch.float64 else 'fp32'}, 1 MI355X",
+        "value": N * M * T / (elapsed / steps), "unit": "kernel entries/s", "n_gpus": 1, "steps": steps,
+        "warmup": max(args.warmup, 20), "ms_per_step": elapsed / steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f64" if tdt == torch.float64 else "f32", "data": "synthetic",
+        "config": {"workload": f"C1: gaussian fmmv K v, N={N}, d={d}, M={M}, T={T}, sigma=2, "
+                               f"{'fp64' if tdt == torch.float64 else 'fp32'}, inputs resident in HBM, packing included in "
+                               "every call, calls issued back to back"},
+        "latency_us_per_waited_call": {"median": float(np.median(waits)) * 1e6, "min": min(waits) * 1e6},
+        "host_us_per_call": host / steps * 1e6,
+        "roofline": {"bound": "mfma", "achieved": flop / (kern_ms * 1e-3) / 1e12 if kern_ms > 0 else 0.0, "peak": peak,
+                     "unit": "TFLOP/s", "frac": flop / (kern_ms * 1e-3) / 1e12 / peak if kern_ms > 0 else 0.0,
+                     "traffic": None, "kernel": product_kernel_name(d, T, "f64" if tdt == torch.float64 else "f32"),
+                     "launches_per_step": launches.value / steps, "avg_launch_ms": kern_ms, "flop_per_launch": flop,
+                     "note": "launch-bound: 79 000 tiles of 16 x 16 fill the chip for a few block steps only"},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import mmv_ref                      # checker only; never on the product path
+        for _ in range(2):
+            ref = mmv_ref.fmmv_ref(X, C, v, 2.0)
+        ts = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            ref = mmv_ref.fmmv_ref(X, C, v, 2.0)
+            ts.append(time.perf_counter() - t0)
+        res["cpu_baseline"] = {"value": N * M * T / float(np.median(ts)), "unit": "kernel entries/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": "the whole of C1, 2 warm-ups + 5 repetitions, median",
+                               "rel_err_gpu_vs_cpu": _rel(out.cpu(), ref)}
+    return res
+
+
 def make_c5(N, Nts, seed=1005, d=28):
     """Train/test rows and +-1 labels y = sign(sin(x.a) + 0.3 eps), a ~ N(0, I/d); draw order X, Xts, a, eps, eps_ts."""
     rng = np.random.default_rng(seed)
@@ -283,10 +354,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS) + ["C5"])
+    ap.add_argument("--workload", default="C2", choices=["C1"] + sorted(WORKLOADS) + ["C5"])
     ap.add_argument("--c5-n", type=int, default=2_000_000, help="training rows of the C5 workload")
     ap.add_argument("--c5-m", type=int, default=50_000, help="centres of the C5 workload")
-    ap.add_argument("--dtype", default="f32", choices=["f32", "f64"], help="arithmetic type (the headline is f32)")
+    ap.add_argument("--dtype", default=None, choices=["f32", "f64"],
+                    help="arithmetic type (default: f32, the headline; f64 for C1, which is an fp64 configuration)")
     ap.add_argument("--op", default="dmmv", choices=["dmmv", "mmv"],
                     help="dmmv = K^T(Kv+w), the headline; mmv = K v only (one launch per step)")
     ap.add_argument("--kernel", default="gaussian", choices=["gaussian", "laplacian", "matern32", "matern52"],
@@ -310,6 +382,8 @@ def main():
                     help="only run a plain device copy of BYTES bytes five times (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
+    if args.dtype is None:
+        args.dtype = "f64" if args.workload == "C1" else "f32"
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only; --gpus must be 1 "
               "(sharding would split the rows of X and end with one M x T all-reduce; it is not built)",
@@ -339,6 +413,9 @@ def main():
                                 "laplacian": (lambda s: LaplacianKernel(s, opt=kopt), "laplacian"),
                                 "matern32": (lambda s: MaternKernel(s, 1.5, opt=kopt), "1.5-matern"),
                                 "matern52": (lambda s: MaternKernel(s, 2.5, opt=kopt), "2.5-matern")}[args.kernel]
+    if args.workload == "C1":
+        print(json.dumps(run_c1(args, lib)), flush=True)
+        return
     if args.workload == "C5":
         print(json.dumps(run_c5(args, lib)), flush=True)
         return
