@@ -186,17 +186,22 @@ template <> int64_t mmv_small_max_d<double>() { return 4 * kMaxDp64Fr2; }
 // more than four right-hand sides: the 16-column kernel of mmv_small_f64_wide.hip, which reads 16 planes
 // (beyond 16 columns two groups of 16 share one evaluation of K: 17 columns that way take less time than a
 // 16-column pass and a one-column pass, at every feature count)
+// (four groups where the columns beyond 32 would need the wide kernel again; up to fma_cols64 columns beyond 32, a
+// 32-column pass and a pass of the FMA kernel are the faster pair: d = 9, T = 33: 49.6 ms against 56.8)
+static inline bool four_groups64(int64_t dpad, int64_t t) { return t > 2 * kWideCols64 + fma_cols64(dpad); }
 template <> int mmv_small_max_cols<double>(int64_t dpad, int64_t t) {
+    if (four_groups64(dpad, t)) return 4 * kWideCols64;
     if (t > kWideCols64) return 2 * kWideCols64;
     return t > fma_cols64(dpad) ? kWideCols64 : fma_cols64(dpad);
 }
 template <> int mmv_small_width<double>(int64_t dpad, int tc) {
+    if (tc > 2 * kWideCols64) return 4 * kWideCols64;
     if (tc > kWideCols64) return 2 * kWideCols64;
     return tc > fma_cols64(dpad) ? kWideCols64 : tc;
 }
 template <> int mmv_small_b_blocks_per_wg<double>(int64_t dpad, int64_t t) {
-    (void)t;
-    return kWavesPerWg64 * ((dpad / 4) <= kMaxDp64Fr4 ? 4 : 2);
+    const int fr = (dpad / 4) <= kMaxDp64Fr4 ? 4 : 2;
+    return kWavesPerWg64 * (four_groups64(dpad, t) ? fr / 2 : fr);   // four column groups: half the resident blocks
 }
 #endif
 

@@ -13,9 +13,10 @@
 // With NC = 2 a second group of 16 columns rides on the same kernel values (four more MFMAs per tile and group).
 // Measured, dfmmv at N = 5e5, M = 2e4: 32 columns in one pass against two passes of 16: d = 9 35.1 ms against 49.1,
 // d = 28 45.3 against 69.3, d = 64 69.2 against 116.7; 17 columns 35 / 45 / 69 ms against 39.1 / 58.9 / 106.6 for a
-// 16-column pass followed by a one-column pass.  (Four groups, 64 columns, were measured and not kept: their 68 KB of
-// staged row values leave one workgroup per CU, and with half the resident blocks T = 64 took 71.1 / 81.7 / 143.8 ms
-// against 70.0 / 90.5 / 138.6 for two passes of 32, T = 33 80.5 at d = 28 against 69.5.)
+// 16-column pass followed by a one-column pass.  With NC = 4 (33 to 64 columns) the resident
+// blocks per wave are halved (registers: 16 output accumulators per block and group) and the staged row values are
+// single-buffered, so that two workgroups still fit a CU: T = 64 58.1 / 68.3 / 108.4 ms against 70.0 / 90.5 / 138.6 for
+// two passes of 32.
 #include "flk_common.h"
 #include "kernel_fn.h"
 
@@ -29,7 +30,7 @@ typedef double doublex4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWide64Waves = 4;
 constexpr int kWide64Cols = 16;                             // one group of columns; NC groups share an evaluation of K
-constexpr int kWide64MaxGroups = 2;
+constexpr int kWide64MaxGroups = 4;
 template <int NC> struct Wide64Geo {
     static constexpr int kCols = 16 * NC;
     static constexpr int kStride = kCols + 1;               // row stride of the staged vec values
@@ -107,7 +108,10 @@ __global__ void __launch_bounds__(256, 2)
                               int64_t a_chunk_blocks, double *__restrict__ partial, int64_t nb_pad, int tcols,
                               bool y_fastest) {
     // vecp must hold 16 NC planes (zeros beyond the caller's columns); the first tcols columns are stored
-    __shared__ __attribute__((aligned(32))) double stage[kWide64Waves][2][Wide64Geo<NC>::kStage];
+    // (a wave's stage is written after the tile step that read it and before the next one, in program order, so one
+    // buffer is enough; with four column groups two of them would leave room for one workgroup per CU only)
+    constexpr int kBufs = NC >= 4 ? 1 : 2;
+    __shared__ __attribute__((aligned(32))) double stage[kWide64Waves][kBufs][Wide64Geo<NC>::kStage];
     // gfx950 has no fp64 exponential: 2^(k/2048) from a table in LDS, filled here (kernel_fn.h)
     __shared__ double exp_tab[kExpTableSize];
     exp2_table_fill(exp_tab, threadIdx.x, 256);
@@ -142,7 +146,7 @@ __global__ void __launch_bounds__(256, 2)
 
     double fa0[DP], fa1[DP];
     Wide64RowVals<NC> rv;
-    double *lds0 = stage[wave][0], *lds1 = stage[wave][1];
+    double *lds0 = stage[wave][0], *lds1 = stage[wave][kBufs - 1];
     if (a0 < a1) {
         wide64_load_a<DP>(fa0, PA, a0, j, q);
         wide64_fetch<NC>(rv, hA, vecp, vec_ld, a0, lane);
@@ -188,13 +192,15 @@ int FLK_CAT(launch_mmv_small_f64_wide_kf, FLK_KF)(const PackedView &A, const Pac
                                                   int64_t vec_ld, int tcols, int64_t a_chunk_blocks, int splits,
                                                   double *partial, hipStream_t st) {
     if (tcols < 1 || tcols > kWide64Cols * kWide64MaxGroups)
-        return fail(FLK_EINVAL, "mmv_small wide: column chunk %d not in 1..32", tcols);
+        return fail(FLK_EINVAL, "mmv_small wide: column chunk %d not in 1..64", tcols);
     if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_small: operands packed with different feature counts");
     const int dp = (int)(A.dpad / 4);
-#define FLK_WIDE64(DPV, FRV)                                                                                         \
-    case DPV:                                                                                                       \
-        return tcols > kWide64Cols                                                                                  \
-                   ? launch_wide64_one<DPV, FRV, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st) \
+#define FLK_WIDE64(DPV, FRV)                                                                                             \
+    case DPV:                                                                                                           \
+        if (tcols > 2 * kWide64Cols)                                                                                    \
+            return launch_wide64_one<DPV, (FRV) / 2, 4>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st); \
+        return tcols > kWide64Cols                                                                                      \
+                   ? launch_wide64_one<DPV, FRV, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)     \
                    : launch_wide64_one<DPV, FRV, 1>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
     switch (dp) {
         FLK_WIDE64(1, 4) FLK_WIDE64(2, 4) FLK_WIDE64(3, 4) FLK_WIDE64(4, 4) FLK_WIDE64(5, 4) FLK_WIDE64(6, 4)

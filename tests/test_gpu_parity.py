@@ -545,10 +545,11 @@ def test_non_finite_rows_give_nan(dev, mode, d, t):
 
 
 @pytest.mark.parametrize("d,t", [(1, 5), (3, 16), (9, 7), (12, 40), (28, 29), (32, 9), (33, 17), (50, 6), (64, 16), (61, 4),
-                                 (64, 20)])
+                                 (64, 20), (12, 70), (28, 50), (40, 64), (64, 37)])
 def test_many_right_hand_sides_small_d_fp64(dev, d, t):
     """More than four right-hand sides at d <= 64 in fp64: the 16-column kernel whose contraction runs on the matrix
-    cores (one evaluation of K for 16 columns) and its 32-column form (two groups of 16, the second one partly filled),
+    cores (one evaluation of K for 16 columns) and its 32- and 64-column forms (two / four groups of 16, the last one partly
+    filled; half the resident blocks per wave with four groups),
     including more columns than one pass holds and a last pass that is narrow enough for the FMA kernel; 1e-11 against the CPU path, and the same numbers as column-by-column calls."""
     n, m = 900, 333
     X, C, v, w = _rand(n, d, m, t, torch.float64, seed=100 * d + t, scale=0.8)
