@@ -309,14 +309,15 @@ _EXPLICIT_BLOCK_BYTES = 8 * 2**30          # size of a stored block of K, memory
 def _explicit_blocks_pay(d: int, t: int, dtype: torch.dtype, opt: BaseOptions, two_products: bool = False) -> bool:
     """Whether the caller opted into stored blocks of K (``many_rhs_stored_blocks``) and t right-hand sides are
     enough for them to be the faster route.  The product kernels serve up to 64 columns with one evaluation of K
-    (the break-even below was measured when fp64 up to 64 features still took 32); ``two_products`` (``dmmv``) evaluates K twice on the matrix-free route and once on this
+    (for fp64 up to 32 features the break-even is placed from the 64-column kernel's times: d = 28, T = 128:
+    137 ms matrix-free against 134 stored for dmmv, 68 against 74 for mmv); ``two_products`` (``dmmv``) evaluates K twice on the matrix-free route and once on this
     one.  Break-even measured at N = 5e5, M = 2e4 (d = 784: N = 2.5e5, M = 1e4) for d = 9, 28, 64, 100, 784 and
     T = 17 ... 256; e.g. fp32 d = 28: mmv T = 64 17.8 ms matrix-free against 23.0 stored, T = 96 28.8 / 27.1;
     dmmv T = 64 34.8 / 33.1, T = 128 69.5 / 49.3; fp64 d = 100: dmmv T = 64 131.8 / 151.5, T = 96 229.5 / 151.7."""
     if getattr(opt, "never_store_kernel", False) or not getattr(opt, "many_rhs_stored_blocks", False):
         return False
     if dtype == torch.float64:
-        least = (96, 64) if d <= 64 else (64, 64) if d <= 256 else (64, 16)
+        least = (128, 128) if d <= 32 else (96, 64) if d <= 64 else (64, 64) if d <= 256 else (64, 16)
     else:
         least = (96, 64) if d <= 32 else (64, 32) if d <= 64 else (32, 16)
     return t > least[1 if two_products else 0]

@@ -324,7 +324,8 @@ def test_stored_block_route_rules(monkeypatch):
     assert not pays(28, 96, f32, opt) and pays(28, 97, f32, opt)
     assert not pays(28, 64, f32, opt, two_products=True) and pays(28, 65, f32, opt, two_products=True)
     assert not pays(40, 64, f32, opt) and pays(40, 65, f32, opt) and pays(40, 33, f32, opt, two_products=True)
-    assert not pays(28, 96, f64, opt) and pays(28, 97, f64, opt) and pays(28, 65, f64, opt, two_products=True)
+    assert not pays(28, 128, f64, opt) and pays(28, 129, f64, opt) and pays(28, 129, f64, opt, two_products=True)
+    assert not pays(40, 96, f64, opt) and pays(40, 97, f64, opt) and pays(40, 65, f64, opt, two_products=True)
     assert not pays(100, 64, f64, opt, two_products=True) and pays(100, 65, f64, opt, two_products=True)
     assert pays(784, 17, f64, opt, two_products=True) and not pays(784, 64, f64, opt) and pays(784, 65, f64, opt)
     assert not drv._explicit_blocks_pay(784, 1000, f32, FalkonOptions(many_rhs_stored_blocks=True, never_store_kernel=True))
