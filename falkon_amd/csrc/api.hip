@@ -98,8 +98,8 @@ static void plan_register_resident(Plan &p, int64_t na_blocks, int64_t nb_blocks
     if (max_splits < 1) max_splits = 1;
     if (splits > max_splits) splits = max_splits;
     p.col_chunk = col_chunk;
-    if (t > 4 && p.col_chunk > 4) {
-        int64_t want = (na_blocks + kWideChunkBlocks - 1) / kWideChunkBlocks;
+    if (t > 4 && p.col_chunk > 4 && elem_bytes == 4) {     // (fp64 sums need no such cap: C2's shape with 64 columns
+        int64_t want = (na_blocks + kWideChunkBlocks - 1) / kWideChunkBlocks;   // would write 10 GB of partial sums)
         if (splits < want) splits = want;
     }
     // a reduction chunk is streamed by every output tile that shares it: keep it within half of one XCD's
