@@ -137,6 +137,40 @@ def test_config4_full_size(dev, dtype, bf16x3):
     _full_size_checks(dev, "C4", dtype, n_rows=2000, n_centres=32, bf16x3=bf16x3)
 
 
+@pytest.mark.parametrize("name,dtype,t", [("C2", torch.float32, 64), ("C2", torch.float32, 40), ("C2", torch.float64, 64),
+                                          ("C4", torch.float32, 64), ("C4", torch.float64, 64), ("C4", torch.float32, 24)],
+                         ids=["C2-fp32-64", "C2-fp32-40", "C2-fp64-64", "C4-fp32-64", "C4-fp64-64", "C4-fp32-24"])
+def test_many_columns_full_size(dev, name, dtype, t):
+    """The matrices of configurations 2 and 4 with 24 to 64 right-hand sides (one evaluation of K serves them all): rows of
+    K v against the CPU oracle, the adjoint identity in every column, and sampled columns of K^T (K v + w) against the
+    single-column kernels, which the tests above check at this size."""
+    X, C, sigma, _, _ = inputs.make_config(name, dtype=dtype)
+    N, M = X.shape[0], C.shape[0]
+    tol = TOL[dtype]
+    g = np.random.default_rng(11)
+    v = torch.from_numpy(g.standard_normal((M, t))).to(dtype)
+    w = torch.from_numpy(g.standard_normal((N, t))).to(dtype)
+    k = GaussianKernel(sigma)
+    Xg, Cg, vg, wg = X.to(dev), C.to(dev), v.to(dev), w.to(dev)
+    u = k.mmv(Xg, Cg, vg)
+    out = k.dmmv(Xg, Cg, vg, wg)
+    assert u.shape == (N, t) and out.shape == (M, t) and bool(torch.isfinite(out).all())
+    rows = torch.from_numpy(np.sort(g.choice(N, 1000, replace=False)))
+    Xs = X[rows].contiguous()
+    check_parity(u[rows.to(dev)], mmv_ref.fmmv_ref(Xs, C, v, sigma),
+                 mmv_ref.fmmv_ref(Xs.double(), C.double(), v.double(), sigma), tol)
+    z = torch.from_numpy(g.standard_normal((N, t))).to(dtype).to(dev)
+    ktz = k.mmv(Cg, Xg, z)
+    lhs, rhs = (z.double() * u.double()).sum(0), (ktz.double() * vg.double()).sum(0)
+    scale = z.double().norm(dim=0) * u.double().norm(dim=0)
+    assert float(((lhs - rhs).abs() / scale).max()) < tol
+    cols = sorted(c for c in {0, 15, 16, 31, 32, t - 1} if c < t)
+    for c in cols:
+        one = k.dmmv(Xg, Cg, vg[:, c:c + 1].contiguous(), wg[:, c:c + 1].contiguous())
+        assert rel_err(out[:, c:c + 1], one) < tol, c
+    assert torch.equal(out, k.dmmv(Xg, Cg, vg, wg))
+
+
 @pytest.mark.parametrize("bf16x3", [False, True], ids=["fp32-mfma", "bf16x3"])
 def test_kernel_matrix_large_square(dev, bf16x3):
     """K(A, A) for 30 000 rows of 256 features, evaluated in fp32 (3.6 GB): properties no sample can miss — a unit
