@@ -24,16 +24,20 @@ static inline int fma_cols(int64_t dpad) {
 }
 constexpr int kWideColumns = 32;       // one group of columns of the wide kernel
 constexpr int kWideMaxDpFr4 = 8;
-// The wide kernel takes two groups (64 columns) on one evaluation of K where the columns beyond 32 would need the wide
-// kernel again; up to fma_cols columns beyond 32, a 32-column pass and a pass of the FMA kernel are the faster pair.
-// Measured, dfmmv at N = 1e6, M = 2e4 (64-column kernel against two passes): d = 28: T = 64 69.1 ms against 86.1, T = 33
-// 67.9 against 62.2; d = 9: T = 64 54.6 against 58.2, T = 48 54.0 against 50.8; d = 64: T = 64 119 against 137.
-static inline bool two_groups(int64_t dpad, int64_t t) { return t > kWideColumns + fma_cols(dpad); }
+// The wide kernel takes two groups (64 columns) on one evaluation of K unless the few columns beyond 32 are cheaper as a
+// pass of the FMA kernel behind a 32-column pass.  Measured, dfmmv at N = 1e6, M = 2e4: 64-column kernel (any 33 to
+// 64 columns) d = 9 / 16 / 28 / 40 / 64: 47.2 / 51.5 / 59.1 / 67.3 / 84.3 ms; 32-column pass 27.1 / 31.3 / 39.4 / 46.3 /
+// 60.8; one-column pass 8.7 / 12.3 / 19.2 / 29.9 / 46.8, 16 columns at d = 9 21.7.
+static inline int cheap_extra_cols(int64_t dpad) {
+    const int64_t dp = dpad / 2;
+    return dp <= 5 ? 12 : dp <= 8 ? 8 : dp <= 12 ? 3 : 0;
+}
+static inline bool two_groups(int64_t dpad, int64_t t) { return t > kWideColumns + cheap_extra_cols(dpad); }
 
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<float>() { return 2 * kMaxDpFr2; }
 template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad, int64_t t) {
-    if (two_groups(dpad, t)) return kWavesPerWg * ((dpad / 2) <= 16 ? 2 : 1);
+    if (two_groups(dpad, t)) return kWavesPerWg * 2;
     if (t > fma_cols(dpad)) return kWavesPerWg * ((dpad / 2) <= kWideMaxDpFr4 ? 4 : 2);
     return kWavesPerWg * ((dpad / 2) <= kMaxDpFr4 ? 4 : 2);
 }

@@ -24,30 +24,39 @@ template <int NC> struct WideGeo {
     static constexpr int kCols = 32 * NC;
     static constexpr int kStride = kCols + 1;
     static constexpr int kStage = 32 + 32 * kStride;
-    static constexpr int kFetch = 1 + kCols / 2;         // dwords a lane fetches per A block
+    static constexpr int kFetch = 1 + kCols / 8;         // dwords a thread fetches per A block
 };
 constexpr int kWideCols = 32;                            // of one group
 constexpr int kWideMaxGroups = 2;
 
 template <int NC> struct WideRowVals { float x[WideGeo<NC>::kFetch]; };
 
-// lane l fetches hA[row l % 32] (lower half) and vec[row l % 32][2c + l / 32], c = 0..16 NC - 1: 128-byte runs of the planes
+// The row values of an A block (half norms and right-hand side entries) are the same for the four waves of a
+// workgroup, which walk the same reduction chunk: the workgroup fetches them once, thread t the half norm of row
+// t % 32 and the entries vec[row t % 32][t / 32 + 8 c], c = 0 .. 4 NC - 1 (128-byte runs of the planes), and stages
+// them in one LDS buffer that every wave reads its MFMA operands from.  (With a private copy per wave the 16 NC + 1
+// loads per lane and block cost 9 % of the launch: N = 1e6, M = 2e4, d = 28, 32 columns, 21.3 ms against 19.4 with
+// those loads removed.)
 template <int NC>
 __device__ __forceinline__ void wide_fetch(WideRowVals<NC> &rv, const float *__restrict__ hA,
-                                           const float *__restrict__ vecp, int64_t vec_ld, int64_t ab, int lane) {
-    const int r = lane & 31, hh = lane >> 5;
+                                           const float *__restrict__ vecp, int64_t vec_ld, int64_t ab, int tid) {
+    const int r = tid & 31, p0 = tid >> 5;
     rv.x[0] = hA[ab * 32 + r];
 #pragma unroll
-    for (int c = 0; c < WideGeo<NC>::kCols / 2; c++) rv.x[1 + c] = vecp[(int64_t)(2 * c + hh) * vec_ld + ab * 32 + r];
+    for (int c = 0; c < WideGeo<NC>::kCols / 8; c++) rv.x[1 + c] = vecp[(int64_t)(p0 + 8 * c) * vec_ld + ab * 32 + r];
 }
 template <int NC>
-__device__ __forceinline__ void wide_stage(const WideRowVals<NC> &rv, float *lds, int lane) {
-    const int r = lane & 31, hh = lane >> 5;
-    if (hh == 0) lds[r] = rv.x[0];
+__device__ __forceinline__ void wide_stage(const WideRowVals<NC> &rv, float *lds, int tid) {
+    const int r = tid & 31, p0 = tid >> 5;
+    if (p0 == 0) lds[r] = rv.x[0];
 #pragma unroll
-    for (int c = 0; c < WideGeo<NC>::kCols / 2; c++) lds[32 + r * WideGeo<NC>::kStride + 2 * c + hh] = rv.x[1 + c];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    for (int c = 0; c < WideGeo<NC>::kCols / 8; c++) lds[32 + r * WideGeo<NC>::kStride + p0 + 8 * c] = rv.x[1 + c];
+}
+// Workgroup barrier that drains the wave's LDS traffic only (not its global loads, which are meant to stay in flight)
+__device__ __forceinline__ void wide_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 }
 
 template <int DP, int FR, bool FOLD, int KF, int NC>
@@ -55,7 +64,6 @@ __device__ __forceinline__ void wide_tile_step(const float (&a)[DP], const float
                                                const float (&breg)[FR][DP], const float (&hb)[FR],
                                                floatx16 (&out2)[FR][NC]) {
     constexpr int kWideStride = WideGeo<NC>::kStride;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     floatx4 hn[4];
 #pragma unroll
     for (int g = 0; g < 4; g++) hn[g] = *(const floatx4 *)(lds + 8 * g + 4 * h);
@@ -72,6 +80,9 @@ __device__ __forceinline__ void wide_tile_step(const float (&a)[DP], const float
     for (int q = 0; q < FR; q++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[q][r] = kernel_value<KF>(acc[q][r]);
+    // All kernel values first, then the contraction: left alone the compiler sinks every v_exp_f32 to just in front of
+    // the MFMA that consumes it, and each of those MFMAs then waits for the exponential's result.
+    __builtin_amdgcn_sched_barrier(0);
     // contraction on the matrix cores; the B operand is read one step ahead, fenced (otherwise every read is
     // hoisted to the front)
     const float *vb = lds + 32 + j;
@@ -106,14 +117,15 @@ __global__ void __launch_bounds__(256, 2)
                               int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial,
                               int64_t nb_pad, int tcols, bool y_fastest) {
     // vecp must hold 32 NC planes (zeros beyond the caller's columns); the first tcols columns are stored
-    __shared__ __attribute__((aligned(16))) float stage[kWavesPerWg][2][WideGeo<NC>::kStage];
+    __shared__ __attribute__((aligned(16))) float stage[2][WideGeo<NC>::kStage];   // shared by the four waves
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
     const int j = lane & 31, h = lane >> 5;
+    // (a wave whose blocks all lie past the end keeps going on the last block, for the barriers; it stores nothing)
     const int64_t bb0 = ((int64_t)bx * kWavesPerWg + wave) * FR;
-    if (bb0 >= nb_blocks) return;  // whole wave idle; no barriers in this kernel
     const int64_t a0 = (int64_t)by * a_chunk_blocks;
     int64_t a1 = a0 + a_chunk_blocks;
     if (a1 > na_blocks) a1 = na_blocks;
@@ -137,23 +149,28 @@ __global__ void __launch_bounds__(256, 2)
 
     float fa0[DP], fa1[DP];
     WideRowVals<NC> rv;
-    float *lds0 = stage[wave][0], *lds1 = stage[wave][1];
+    float *lds0 = stage[0], *lds1 = stage[1];
     if (a0 < a1) {
         load_a<DP>(fa0, PA, a0, j, h);
-        wide_fetch<NC>(rv, hA, vecp, vec_ld, a0, lane);
-        wide_stage<NC>(rv, lds0, lane);
+        wide_fetch<NC>(rv, hA, vecp, vec_ld, a0, tid);
+        wide_stage<NC>(rv, lds0, tid);
     }
+    wide_barrier();
+    // One barrier per A block: a stage is written after the barrier that follows its last reader and read after the
+    // barrier that follows its writers.  The conditions are the same for every wave of the workgroup.
     for (int64_t ab = a0; ab < a1; ab += 2) {
         const bool has1 = ab + 1 < a1;
-        if (has1) { load_a<DP>(fa1, PA, ab + 1, j, h); wide_fetch<NC>(rv, hA, vecp, vec_ld, ab + 1, lane); }
+        if (has1) { load_a<DP>(fa1, PA, ab + 1, j, h); wide_fetch<NC>(rv, hA, vecp, vec_ld, ab + 1, tid); }
         wide_tile_step<DP, FR, FOLD, KF, NC>(fa0, lds0, j, h, breg, hb, out2);
+        if (has1) wide_stage<NC>(rv, lds1, tid);
+        wide_barrier();
         if (has1) {
-            wide_stage<NC>(rv, lds1, lane);
             const bool has2 = ab + 2 < a1;
-            if (has2) { load_a<DP>(fa0, PA, ab + 2, j, h); wide_fetch<NC>(rv, hA, vecp, vec_ld, ab + 2, lane); }
+            if (has2) { load_a<DP>(fa0, PA, ab + 2, j, h); wide_fetch<NC>(rv, hA, vecp, vec_ld, ab + 2, tid); }
             wide_tile_step<DP, FR, FOLD, KF, NC>(fa1, lds1, j, h, breg, hb, out2);
-            if (has2) wide_stage<NC>(rv, lds0, lane);
+            if (has2) wide_stage<NC>(rv, lds0, tid);
         }
+        wide_barrier();
     }
     // lane = column t, registers = output rows (both lane halves hold different rows): no cross-lane step
 #pragma unroll
@@ -192,14 +209,15 @@ int FLK_CAT(launch_mmv_small_f32_wide_kf, FLK_KF)(const PackedView &A, const Pac
     const int dp = (int)(A.dpad / 2);
     const bool fold = f32_fold_applies(A.d);
     if (tcols > kWideCols) {
-        // 33 to 64 columns: two groups of 32 on one evaluation of K; two resident fragments per wave up to 32 padded
-        // features, one beyond (registers: 64 output accumulators per fragment and 33 prefetched row values)
+        // 33 to 64 columns: two groups of 32 on one evaluation of K; two resident fragments per wave (64 output
+        // accumulators per fragment; from 56 padded features on a few registers spill, which still beats one fragment:
+        // d = 64, 64 columns: 84.3 ms per dfmmv against 84.9, d = 40: 67.3 against 73.8)
 #define FLK_WIDE2(DPV)                                                                                              \
     case DPV:                                                                                                      \
         return fold ? launch_wide_one<DPV, 2, true, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st) \
                     : launch_wide_one<DPV, 2, false, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
 #define FLK_WIDE2_PLAIN(DPV) \
-    case DPV: return launch_wide_one<DPV, 1, false, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+    case DPV: return launch_wide_one<DPV, 2, false, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
         switch (dp) {
             FLK_WIDE2(1) FLK_WIDE2(2) FLK_WIDE2(3) FLK_WIDE2(4) FLK_WIDE2(5) FLK_WIDE2(6) FLK_WIDE2(7) FLK_WIDE2(8)
             FLK_WIDE2(9) FLK_WIDE2(10) FLK_WIDE2(11) FLK_WIDE2(12) FLK_WIDE2(13) FLK_WIDE2(14) FLK_WIDE2(15) FLK_WIDE2(16)

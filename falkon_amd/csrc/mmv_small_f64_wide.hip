@@ -14,9 +14,7 @@
 // Measured, dfmmv at N = 5e5, M = 2e4: 32 columns in one pass against two passes of 16: d = 9 35.1 ms against 49.1,
 // d = 28 45.3 against 69.3, d = 64 69.2 against 116.7; 17 columns 35 / 45 / 69 ms against 39.1 / 58.9 / 106.6 for a
 // 16-column pass followed by a one-column pass.  With NC = 4 (33 to 64 columns) the resident
-// blocks per wave are halved (registers: 16 output accumulators per block and group) and the staged row values are
-// single-buffered, so that two workgroups still fit a CU: T = 64 58.1 / 68.3 / 108.4 ms against 70.0 / 90.5 / 138.6 for
-// two passes of 32.
+// blocks per wave are halved (registers: 16 output accumulators per block and group).
 #include "flk_common.h"
 #include "kernel_fn.h"
 
@@ -35,7 +33,8 @@ template <int NC> struct Wide64Geo {
     static constexpr int kCols = 16 * NC;
     static constexpr int kStride = kCols + 1;               // row stride of the staged vec values
     static constexpr int kStage = 16 + 16 * kStride;        // hn(16) | vec[16 rows][16 NC + 1]
-    static constexpr int kFetch = 1 + kCols / 4;            // doubles a lane fetches per A block
+    static constexpr bool kShared = NC >= 4;                // one stage per workgroup instead of one per wave (below)
+    static constexpr int kFetch = kShared ? 1 + NC : 1 + kCols / 4;   // doubles a thread fetches per A block
 };
 
 template <int NC> struct Wide64RowVals { double x[Wide64Geo<NC>::kFetch]; };
@@ -64,6 +63,35 @@ __device__ __forceinline__ void wide64_stage(const Wide64RowVals<NC> &rv, double
     for (int c = 0; c < Wide64Geo<NC>::kCols / 4; c++) lds[16 + r * Wide64Geo<NC>::kStride + 4 * c + hh] = rv.x[1 + c];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+}
+
+// The row values of an A block (half norms and right-hand side entries) are the same for the four waves of a
+// workgroup, which walk the same reduction chunk: the workgroup fetches them once, thread t the half norm of row
+// t % 16 and the entries vec[row t % 16][t / 16 + 16 c], c = 0 .. NC - 1 (128-byte runs of the planes), and stages
+// them in one LDS buffer that every wave reads its MFMA operands from, at the price of a workgroup barrier per A block.
+// Used with four column groups, where a private copy per wave costs 17 loads per lane and block (dfmmv at N = 5e5,
+// M = 2e4, 64 columns: d = 40 85.9 -> 75.8 ms, d = 64 105.1 -> 98.6); with one or two groups the private copies are as
+// fast or faster (16 columns, d = 64: 58.4 ms against 61.2) and stay.
+template <int NC>
+__device__ __forceinline__ void wide64_fetch_wg(Wide64RowVals<NC> &rv, const double *__restrict__ hA,
+                                             const double *__restrict__ vecp, int64_t vec_ld, int64_t ab, int tid) {
+    const int r = tid & 15, p0 = tid >> 4;
+    rv.x[0] = hA[ab * 16 + r];
+#pragma unroll
+    for (int c = 0; c < NC; c++) rv.x[1 + c] = vecp[(int64_t)(p0 + 16 * c) * vec_ld + ab * 16 + r];
+}
+template <int NC>
+__device__ __forceinline__ void wide64_stage_wg(const Wide64RowVals<NC> &rv, double *lds, int tid) {
+    const int r = tid & 15, p0 = tid >> 4;
+    if (p0 == 0) lds[r] = rv.x[0];
+#pragma unroll
+    for (int c = 0; c < NC; c++) lds[16 + r * Wide64Geo<NC>::kStride + p0 + 16 * c] = rv.x[1 + c];
+}
+// Workgroup barrier that drains the wave's LDS traffic only (not its global loads, which are meant to stay in flight)
+__device__ __forceinline__ void wide64_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 }
 
 template <int DP, int FR, int KF, int NC>
@@ -108,22 +136,23 @@ __global__ void __launch_bounds__(256, 2)
                               int64_t a_chunk_blocks, double *__restrict__ partial, int64_t nb_pad, int tcols,
                               bool y_fastest) {
     // vecp must hold 16 NC planes (zeros beyond the caller's columns); the first tcols columns are stored
-    // (a wave's stage is written after the tile step that read it and before the next one, in program order, so one
-    // buffer is enough; with four column groups two of them would leave room for one workgroup per CU only)
-    constexpr int kBufs = NC >= 4 ? 1 : 2;
-    __shared__ __attribute__((aligned(32))) double stage[kWide64Waves][kBufs][Wide64Geo<NC>::kStage];
+    constexpr bool kShared = Wide64Geo<NC>::kShared;
+    __shared__ __attribute__((aligned(32))) double stage[kShared ? 1 : kWide64Waves][2][Wide64Geo<NC>::kStage];
     // gfx950 has no fp64 exponential: 2^(k/2048) from a table in LDS, filled here (kernel_fn.h)
     __shared__ double exp_tab[kExpTableSize];
     exp2_table_fill(exp_tab, threadIdx.x, 256);
     __syncthreads();
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
     const int j = lane & 15, q = lane >> 4;
     const int jrow = 4 * (j & 3) + (j >> 2);  // matrix row (within its block) held at position j
     const int64_t bb0 = ((int64_t)bx * kWide64Waves + wave) * FR;
-    if (bb0 >= nb_blocks) return;             // whole wave idle; no workgroup barriers from here on
+    // private stages: a wave whose blocks all lie past the end leaves (no workgroup barriers from here on); shared
+    // stage: it keeps going on the last block, for the barriers, and stores nothing
+    if (!kShared && bb0 >= nb_blocks) return;
     const int64_t a0 = (int64_t)by * a_chunk_blocks;
     int64_t a1 = a0 + a_chunk_blocks;
     if (a1 > na_blocks) a1 = na_blocks;
@@ -146,22 +175,47 @@ __global__ void __launch_bounds__(256, 2)
 
     double fa0[DP], fa1[DP];
     Wide64RowVals<NC> rv;
-    double *lds0 = stage[wave][0], *lds1 = stage[wave][kBufs - 1];
-    if (a0 < a1) {
-        wide64_load_a<DP>(fa0, PA, a0, j, q);
-        wide64_fetch<NC>(rv, hA, vecp, vec_ld, a0, lane);
-        wide64_stage<NC>(rv, lds0, lane);
-    }
-    for (int64_t ab = a0; ab < a1; ab += 2) {
-        const bool has1 = ab + 1 < a1;
-        if (has1) { wide64_load_a<DP>(fa1, PA, ab + 1, j, q); wide64_fetch<NC>(rv, hA, vecp, vec_ld, ab + 1, lane); }
-        wide64_tile_step<DP, FR, KF, NC>(fa0, lds0, j, q, breg, hb, out2, exp_tab);
-        if (has1) {
-            wide64_stage<NC>(rv, lds1, lane);
-            const bool has2 = ab + 2 < a1;
-            if (has2) { wide64_load_a<DP>(fa0, PA, ab + 2, j, q); wide64_fetch<NC>(rv, hA, vecp, vec_ld, ab + 2, lane); }
-            wide64_tile_step<DP, FR, KF, NC>(fa1, lds1, j, q, breg, hb, out2, exp_tab);
-            if (has2) wide64_stage<NC>(rv, lds0, lane);
+    double *lds0 = stage[kShared ? 0 : wave][0], *lds1 = stage[kShared ? 0 : wave][1];
+    if constexpr (kShared) {
+        if (a0 < a1) {
+            wide64_load_a<DP>(fa0, PA, a0, j, q);
+            wide64_fetch_wg<NC>(rv, hA, vecp, vec_ld, a0, tid);
+            wide64_stage_wg<NC>(rv, lds0, tid);
+        }
+        wide64_barrier();
+        // One barrier per A block: a stage is written after the barrier that follows its last reader and read after
+        // the barrier that follows its writers.  The conditions are the same for every wave of the workgroup.
+        for (int64_t ab = a0; ab < a1; ab += 2) {
+            const bool has1 = ab + 1 < a1;
+            if (has1) { wide64_load_a<DP>(fa1, PA, ab + 1, j, q); wide64_fetch_wg<NC>(rv, hA, vecp, vec_ld, ab + 1, tid); }
+            wide64_tile_step<DP, FR, KF, NC>(fa0, lds0, j, q, breg, hb, out2, exp_tab);
+            if (has1) wide64_stage_wg<NC>(rv, lds1, tid);
+            wide64_barrier();
+            if (has1) {
+                const bool has2 = ab + 2 < a1;
+                if (has2) { wide64_load_a<DP>(fa0, PA, ab + 2, j, q); wide64_fetch_wg<NC>(rv, hA, vecp, vec_ld, ab + 2, tid); }
+                wide64_tile_step<DP, FR, KF, NC>(fa1, lds1, j, q, breg, hb, out2, exp_tab);
+                if (has2) wide64_stage_wg<NC>(rv, lds0, tid);
+            }
+            wide64_barrier();
+        }
+    } else {
+        if (a0 < a1) {
+            wide64_load_a<DP>(fa0, PA, a0, j, q);
+            wide64_fetch<NC>(rv, hA, vecp, vec_ld, a0, lane);
+            wide64_stage<NC>(rv, lds0, lane);
+        }
+        for (int64_t ab = a0; ab < a1; ab += 2) {
+            const bool has1 = ab + 1 < a1;
+            if (has1) { wide64_load_a<DP>(fa1, PA, ab + 1, j, q); wide64_fetch<NC>(rv, hA, vecp, vec_ld, ab + 1, lane); }
+            wide64_tile_step<DP, FR, KF, NC>(fa0, lds0, j, q, breg, hb, out2, exp_tab);
+            if (has1) {
+                wide64_stage<NC>(rv, lds1, lane);
+                const bool has2 = ab + 2 < a1;
+                if (has2) { wide64_load_a<DP>(fa0, PA, ab + 2, j, q); wide64_fetch<NC>(rv, hA, vecp, vec_ld, ab + 2, lane); }
+                wide64_tile_step<DP, FR, KF, NC>(fa1, lds1, j, q, breg, hb, out2, exp_tab);
+                if (has2) wide64_stage<NC>(rv, lds0, lane);
+            }
         }
     }
     // lane = column t = j, registers = output rows 4q .. 4q + 3 of each block
