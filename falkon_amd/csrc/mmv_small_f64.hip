@@ -181,6 +181,11 @@ constexpr int kWideCols64 = 16;  // of the kernel that contracts on the matrix c
 constexpr int kMaxDp64Fr4 = 8;   // dpad <= 32
 constexpr int kMaxDp64Fr2 = 16;  // dpad <= 64
 
+// resident blocks per wave of the FMA kernel with tt columns (fr: the single-column kernel's count)
+constexpr int fr64_for(int dp, int fr, int tt) {
+    return fr == 4 && ((tt == 2 && dp >= 2) || (tt == 3 && dp >= 6) || (tt >= 4 && dp >= 5)) ? 2 : fr;
+}
+
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<double>() { return 4 * kMaxDp64Fr2; }
 // more than four right-hand sides: the 16-column kernel of mmv_small_f64_wide.hip, which reads 16 planes
@@ -201,6 +206,7 @@ template <> int mmv_small_width<double>(int64_t dpad, int tc) {
 }
 template <> int mmv_small_b_blocks_per_wg<double>(int64_t dpad, int64_t t) {
     const int fr = (dpad / 4) <= kMaxDp64Fr4 ? 4 : 2;
+    if (t >= 2 && t <= fma_cols64(dpad)) return kWavesPerWg64 * fr64_for((int)(dpad / 4), fr, (int)t);
     return kWavesPerWg64 * (four_groups64(dpad, t) ? fr / 2 : fr);   // four column groups: half the resident blocks
 }
 #endif
@@ -220,11 +226,17 @@ static int launch_one64(const PackedView &A, const PackedView &B, const double *
 template <int DP, int FR>
 static int launch_tt64(int tt, const PackedView &A, const PackedView &B, const double *vecp, int64_t vec_ld,
                        int64_t a_chunk_blocks, int splits, double *partial, hipStream_t st) {
+    // With more than one column the four-block variants need more than 256 registers and run one wave per SIMD, which
+    // leaves the latency of the exponential's table reads and of the MFMA results exposed: two resident blocks (two or
+    // three waves per SIMD) are faster from 8 features on with two columns, from 24 on with three and from 20 on with four.  Measured,
+    // dfmmv at N = 5e5, M = 2e4, four blocks -> two: T = 2: d = 16 20.5 -> 18.1 ms, d = 28 29.6 -> 24.8, d = 32 35.6 ->
+    // 29.4 (d = 4: 11.4 -> 11.6, kept at four); T = 4: d = 28 30.4 -> 28.9 (d = 16: 21.3 -> 22.5, kept at four).
+    constexpr int kFr2 = fr64_for(DP, FR, 2), kFr3 = fr64_for(DP, FR, 3), kFr4 = fr64_for(DP, FR, 4);
     switch (tt) {
         case 1: return launch_one64<DP, FR, 1>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
-        case 2: return launch_one64<DP, FR, 2>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
-        case 3: return launch_one64<DP, FR, 3>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
-        case 4: return launch_one64<DP, FR, 4>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 2: return launch_one64<DP, kFr2, 2>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 3: return launch_one64<DP, kFr3, 3>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 4: return launch_one64<DP, kFr4, 4>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
     }
     return fail(FLK_EINVAL, "mmv_small: column chunk %d not in 1..4", tt);
 }
