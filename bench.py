@@ -79,7 +79,7 @@ def product_kernel_name(d, T, dtype):
         steps = (d + 1) // 2
         fma_cols = 16 if steps <= 7 else 12 if steps <= 12 else 8 if steps <= 16 else 4
         return "mmv_small_f32_wide_kernel" if T > fma_cols else "mmv_small_f32_kernel"
-    return "mmv_small_f64_wide_kernel" if T > (3 if d > 56 else 4) else "mmv_small_f64_kernel"
+    return "mmv_small_f64_wide_kernel" if T > (3 if d > 52 else 4) else "mmv_small_f64_kernel"
 
 
 def make_inputs(name, rhs=0):

@@ -273,7 +273,10 @@ __global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 r
     // caller's columns).
     using RV = RowVals<TT>;
     constexpr bool kTwoLevel = TT <= 4;   // long accumulator only where registers allow; wider TT uses short chunks
-    constexpr bool kCanFactorOut = !FOLD && KF == FLK_GAUSSIAN && TT <= 2;   // wider column chunks are out of registers with two loops
+    // (wider column chunks are out of registers with two loops; with two resident blocks per wave, beyond 32 features,
+    // the kernel with both loops measured slower than the plain one: d = 64, one column, 46.8 ms per dfmmv at N = 1e6,
+    // M = 2e4 against 42.9, d = 40 32.9 against 27.8)
+    constexpr bool kCanFactorOut = !FOLD && KF == FLK_GAUSSIAN && TT <= 2 && FR == 4;
     __shared__ __attribute__((aligned(16))) float stage[kWavesPerWg][2][RV::N];
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);

@@ -176,7 +176,7 @@ __global__ void __launch_bounds__(256)
 // right-hand sides per pass of the FMA kernel above: four, except at 60 and 64 padded features, where its
 // four-column variant is out of registers (d = 64, N = 5e5, M = 2e4: 37.4 ms against 29.5 for the 16-column kernel;
 // three columns 25.5)
-inline int fma_cols64(int64_t dpad) { return dpad >= 60 ? 3 : 4; }
+inline int fma_cols64(int64_t dpad) { return dpad >= 56 ? 3 : 4; }   // (d = 56, four columns: 54.1 ms against 52.2)
 constexpr int kWideCols64 = 16;  // of the kernel that contracts on the matrix cores
 constexpr int kMaxDp64Fr4 = 8;   // dpad <= 32
 constexpr int kMaxDp64Fr2 = 16;  // dpad <= 64
