@@ -352,8 +352,8 @@ def run_c5(args, lib):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default 50; C5, whose step is a whole fit: 2)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 3; C5: 1)")
     ap.add_argument("--workload", default="C2", choices=["C1"] + sorted(WORKLOADS) + ["C5"])
     ap.add_argument("--c5-n", type=int, default=2_000_000, help="training rows of the C5 workload")
     ap.add_argument("--c5-m", type=int, default=50_000, help="centres of the C5 workload")
@@ -384,6 +384,10 @@ def main():
     args = ap.parse_args()
     if args.dtype is None:
         args.dtype = "f64" if args.workload == "C1" else "f32"
+    if args.steps is None:
+        args.steps = 2 if args.workload == "C5" else 50
+    if args.warmup is None:
+        args.warmup = 1 if args.workload == "C5" else 3
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only; --gpus must be 1 "
               "(sharding would split the rows of X and end with one M x T all-reduce; it is not built)",
