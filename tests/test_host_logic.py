@@ -336,3 +336,40 @@ def test_stored_block_route_rules(monkeypatch):
     assert drv._explicit_block_rows(500, 10_000, 784, 256, 4, None, opt, upload_bytes=0) == 500
     monkeypatch.setattr(drv, "usable_gpu_memory", lambda dev, cap, slack, enough=float("inf"): 2**20)
     assert drv._explicit_block_rows(10**6, 10_000, 784, 256, 4, None, opt, upload_bytes=0) == 0
+
+
+def test_memory_budget_reuses_a_recent_driver_report(monkeypatch):
+    """``usable_gpu_memory`` (falkon/mmv_ops/utils.py:47-58): ``slack * min(free, max_gpu_mem)``.  The driver's report is
+    asked for again unless a call needs at most an eighth of what it said within the last 50 ms; the value handed to
+    such a call is a lower bound that still covers it."""
+    import importlib
+    utils = importlib.import_module("falkon_amd.mmv_ops.utils")
+    calls = []
+
+    def report(dev):
+        calls.append(dev)
+        return 80 * 2**30, 288 * 2**30
+    monkeypatch.setattr(torch.cuda, "mem_get_info", report)
+    monkeypatch.setattr(torch.cuda, "memory_reserved", lambda dev: 0)
+    monkeypatch.setattr(torch.cuda, "memory_allocated", lambda dev: 0)
+    utils._recent_free.clear()
+    dev = torch.device("cuda", 0)
+    big = utils.usable_gpu_memory(dev, float("inf"), 0.9, enough=2**30)
+    assert len(calls) == 1 and big == pytest.approx(0.9 * 80 * 2**30)
+    small = utils.usable_gpu_memory(dev, float("inf"), 0.9, enough=2**30)          # 8 GiB <= 72 GiB: the report is reused
+    assert len(calls) == 1 and 2**30 <= small <= big
+    assert utils.usable_gpu_memory(dev, 2**29, 0.9, enough=2**30) == pytest.approx(0.9 * 2**29)   # the cap still binds
+    assert len(calls) == 1
+    utils.usable_gpu_memory(dev, float("inf"), 0.9, enough=20 * 2**30)             # too large a share: asked again
+    assert len(calls) == 2
+    monkeypatch.setattr(utils, "_FREE_MEMORY_TTL", 0.0)
+    utils.usable_gpu_memory(dev, float("inf"), 0.9, enough=2**20)                  # too old: asked again
+    assert len(calls) == 3
+    utils._recent_free.clear()
+
+
+def test_bench_defaults_by_workload():
+    """The C5 workload's step is a whole fit: it defaults to few of them; the others keep 50 timed steps."""
+    import ast
+    src = open(os.path.join(os.path.dirname(__file__), "..", "bench.py")).read()
+    assert 'args.steps = 2 if args.workload == "C5" else 50' in src and ast.parse(src)
