@@ -174,6 +174,10 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         // Prologue of an A tile.  All global loads (first feature chunk, then the per-row values hA and vec)
         // are issued before anything waits, and the barrier that protects ldsRow and the stages from the
         // previous tile's epilogue comes after them, so one memory round trip covers the whole prologue.
+        // (Loading the next tile's first chunk and row values during this tile's last chunk and epilogue, into the
+        // then idle prefetch registers, was measured over d = 65 .. 1000 and 1 .. 64 columns: 1 to 2 % faster up to four
+        // columns, 4 to 15 % slower with the MFMA epilogue below 200 features, whose 17 to 33 row values per thread then
+        // spill; not kept.)
         fetch(0);
         constexpr int kRowVals = (1 + (kMfmaEpi ? kEpiCols : TT)) * G::A_ROWS;
         constexpr int kRowValsPerThread = (kRowVals + kLThreads - 1) / kLThreads;
