@@ -173,17 +173,23 @@ __global__ void __launch_bounds__(256)
     }
 }
 
-// right-hand sides per pass of the FMA kernel above: four, except at 60 and 64 padded features, where its
-// four-column variant is out of registers (d = 64, N = 5e5, M = 2e4: 37.4 ms against 29.5 for the 16-column kernel;
-// three columns 25.5)
-inline int fma_cols64(int64_t dpad) { return dpad >= 56 ? 3 : 4; }   // (d = 56, four columns: 54.1 ms against 52.2)
+// right-hand sides per pass of the FMA kernel above: four, except from 52 padded features on, where its
+// four-column variant is out of registers and runs one wave per SIMD (dfmmv at N = 5e5, M = 2e4, four columns against
+// the 16-column kernel: d = 52 56.3 ms against 49.9, d = 56 54.1 against 52.2, d = 64 56.6 against 49.0 for three)
+inline int fma_cols64(int64_t dpad) { return dpad >= 52 ? 3 : 4; }
 constexpr int kWideCols64 = 16;  // of the kernel that contracts on the matrix cores
 constexpr int kMaxDp64Fr4 = 8;   // dpad <= 32
 constexpr int kMaxDp64Fr2 = 16;  // dpad <= 64
 
 // resident blocks per wave of the FMA kernel with tt columns (fr: the single-column kernel's count)
 constexpr int fr64_for(int dp, int fr, int tt) {
-    return fr == 4 && ((tt == 2 && dp >= 2) || (tt == 3 && dp >= 6) || (tt >= 4 && dp >= 5)) ? 2 : fr;
+    if (fr != 4) return fr;
+    // the other kernel functions' longer epilogues push two more four-block variants past 256 registers (one wave per
+    // SIMD): Matern 3/2 and 5/2 with one column at 25 .. 28 features (d = 28: 44.5 ms per dfmmv at N = 5e5, M = 2e4
+    // against 39.2 for the two-column kernel, which runs two blocks), and four columns at 13 .. 16 features
+    if (FLK_KF != FLK_GAUSSIAN && tt == 4 && dp == 4) return 2;
+    if ((FLK_KF == FLK_MATERN32 || FLK_KF == FLK_MATERN52) && tt == 1 && dp == 7) return 2;
+    return ((tt == 2 && dp >= 2) || (tt == 3 && dp >= 6) || (tt >= 4 && dp >= 5)) ? 2 : fr;
 }
 
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
@@ -231,9 +237,9 @@ static int launch_tt64(int tt, const PackedView &A, const PackedView &B, const d
     // three waves per SIMD) are faster from 8 features on with two columns, from 24 on with three and from 20 on with four.  Measured,
     // dfmmv at N = 5e5, M = 2e4, four blocks -> two: T = 2: d = 16 20.5 -> 18.1 ms, d = 28 29.6 -> 24.8, d = 32 35.6 ->
     // 29.4 (d = 4: 11.4 -> 11.6, kept at four); T = 4: d = 28 30.4 -> 28.9 (d = 16: 21.3 -> 22.5, kept at four).
-    constexpr int kFr2 = fr64_for(DP, FR, 2), kFr3 = fr64_for(DP, FR, 3), kFr4 = fr64_for(DP, FR, 4);
+    constexpr int kFr1 = fr64_for(DP, FR, 1), kFr2 = fr64_for(DP, FR, 2), kFr3 = fr64_for(DP, FR, 3), kFr4 = fr64_for(DP, FR, 4);
     switch (tt) {
-        case 1: return launch_one64<DP, FR, 1>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
+        case 1: return launch_one64<DP, kFr1, 1>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
         case 2: return launch_one64<DP, kFr2, 2>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
         case 3: return launch_one64<DP, kFr3, 3>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
         case 4: return launch_one64<DP, kFr4, 4>(A, B, vecp, vec_ld, a_chunk_blocks, splits, partial, st);
