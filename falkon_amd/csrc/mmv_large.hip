@@ -182,15 +182,22 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         constexpr int kRowVals = (1 + (kMfmaEpi ? kEpiCols : TT)) * G::A_ROWS;
         constexpr int kRowValsPerThread = (kRowVals + kLThreads - 1) / kLThreads;
         T rowv[kRowValsPerThread];
+        // A wave's 64 values belong to one vector (hA or one column of vec): its number is made a scalar, so that the
+        // column's offset and the test against tcols are scalar work.  (The leading dimension goes through an empty asm
+        // in every tile: otherwise the compiler forms one pointer per row value ahead of the tile loop, up to 33 of
+        // them, and keeps them in scratch memory.)
+        static_assert(G::A_ROWS % 64 == 0 && kLThreads % 64 == 0, "a wave's row values must belong to one vector");
+        int64_t vld = vec_ld;
+        asm volatile("" : "+s"(vld));
 #pragma unroll
         for (int c = 0; c < kRowValsPerThread; c++) {
             const int e = tid + c * kLThreads;
-            const int which = e / G::A_ROWS, r = e % G::A_ROWS;
+            const int which = __builtin_amdgcn_readfirstlane(e / G::A_ROWS), r = e % G::A_ROWS;
             const int64_t row = ablk0 * TR::BLK + r;
             T val = T(0);                      // rows past n_a carry zero weight
             if (e < kRowVals && row < na_blocks * TR::BLK) {
                 if (which == 0) val = hA[row];
-                else if (which - 1 < tcols) val = vecp[(int64_t)(which - 1) * vec_ld + row];
+                else if (which - 1 < tcols) val = vecp[(int64_t)(which - 1) * vld + row];
             }
             rowv[c] = val;
         }
@@ -198,7 +205,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
         for (int c = 0; c < kRowValsPerThread; c++) {
             const int e = tid + c * kLThreads;
-            const int which = e / G::A_ROWS, r = e % G::A_ROWS;
+            const int which = __builtin_amdgcn_readfirstlane(e / G::A_ROWS), r = e % G::A_ROWS;
             if (e < kRowVals) {
                 if (!kMfmaEpi || which == 0) ldsRow[e] = rowv[c];
                 else ldsRow[G::A_ROWS + r * kVecStride + (which - 1)] = rowv[c];
@@ -363,31 +370,41 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             // B operand is vec[acc_row(s, lg)][t] with t = lane % kGroupCols (+ kGroupCols per further group; fp32 lanes
             // 16 .. 31 repeat the columns 0 .. 15 in the 16-column form and are never stored).
             const int tl = j & (kGroupCols - 1);
-            const T *vb = &ldsRow[G::A_ROWS + tl];
+            // index of this lane's first B value (step 0 of its wave row's first block); every other read lies a
+            // compile-time constant further on
+            const int lane_idx = G::A_ROWS + tl + ((wa * WA_FR) * TR::BLK + TR::acc_row(0, lg)) * kVecStride;
             // one read ahead, fenced like the feature loop (otherwise all reads are hoisted and spilled)
             T bval[NC], bnext[NC];
 #pragma unroll
             for (int g = 0; g < NC; g++) {
-                bval[g] = vb[((wa * WA_FR) * TR::BLK + TR::acc_row(0, lg)) * kVecStride + g * kGroupCols];
+                bval[g] = ldsRow[lane_idx + g * kGroupCols];
                 bnext[g] = T(0);
             }
 #pragma unroll
             for (int p = 0; p < WA_FR; p++) {
-                const int rbase = (wa * WA_FR + p) * TR::BLK;
 #pragma unroll
                 for (int s2 = 0; s2 < TR::ACCN; s2++) {
+                    // the lane's offset goes through an empty asm before every read: the rows lie further apart than the
+                    // offset field of a paired LDS read reaches, and from an offset it can see through the compiler
+                    // forms one address register per read, keeps all of them live across the tile loop (60 with 64
+                    // columns) and reloads them from scratch memory between the MFMAs; this way each address is one
+                    // addition next to its read
+                    int off = lane_idx * (int)sizeof(T);       // in bytes: no shift left between the asm and the read
+                    asm volatile("" : "+v"(off));
+                    const T *lane_row = (const T *)((const char *)ldsRow + off);
+                    const bool more = s2 + 1 < TR::ACCN || p + 1 < WA_FR;
+                    const int step = s2 + 1 < TR::ACCN ? p * TR::BLK + TR::acc_row(s2 + 1, 0) - TR::acc_row(0, 0)
+                                                       : (p + 1) * TR::BLK;
 #pragma unroll
-                    for (int g = 0; g < NC; g++) {
-                        if (s2 + 1 < TR::ACCN) bnext[g] = vb[(rbase + TR::acc_row(s2 + 1, lg)) * kVecStride + g * kGroupCols];
-                        else if (p + 1 < WA_FR) bnext[g] = vb[(rbase + TR::BLK + TR::acc_row(0, lg)) * kVecStride + g * kGroupCols];
-                    }
+                    for (int g = 0; g < NC; g++)
+                        if (more) bnext[g] = lane_row[step * kVecStride + g * kGroupCols];
 #pragma unroll
                     for (int g = 0; g < NC; g++)
 #pragma unroll
                         for (int q = 0; q < WB_FR; q++) out2[q][g] = TR::mfma(acc[p][q][s2], bval[g], out2[q][g]);
 #pragma unroll
                     for (int g = 0; g < NC; g++) {
-                        asm volatile("" : "+v"(bval[g]) : "v"(vb) : "memory");
+                        asm volatile("" : "+v"(bval[g]) : "v"(&ldsRow[0]) : "memory");
                         bval[g] = bnext[g];
                     }
                 }

@@ -102,7 +102,7 @@ __device__ __forceinline__ void reduce_blocks64(const double *__restrict__ PA, c
 
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
 template <int DP, int FR, int TT, int KF>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
     mmv_small_f64_kernel(const double *__restrict__ PA, const double *__restrict__ hA, const double *__restrict__ vecp,
                          int64_t vec_ld, const double *__restrict__ PB, const double *__restrict__ hB,
                          int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks, double *__restrict__ partial,
@@ -184,10 +184,8 @@ constexpr int kMaxDp64Fr2 = 16;  // dpad <= 64
 // resident blocks per wave of the FMA kernel with tt columns (fr: the single-column kernel's count)
 constexpr int fr64_for(int dp, int fr, int tt) {
     if (fr != 4) return fr;
-    // the other kernel functions' longer epilogues push two more four-block variants past 256 registers (one wave per
-    // SIMD): Matern 3/2 and 5/2 with one column at 25 .. 28 features (d = 28: 44.5 ms per dfmmv at N = 5e5, M = 2e4
-    // against 39.2 for the two-column kernel, which runs two blocks), and four columns at 13 .. 16 features
-    if (FLK_KF != FLK_GAUSSIAN && tt == 4 && dp == 4) return 2;
+    // Matern 3/2 and 5/2 with one column at 25 .. 28 features: the four-block variant does not fit 256 registers
+    // (two blocks, dfmmv at N = 5e5, M = 2e4, d = 28: 44.5 -> 40.0 ms)
     if ((FLK_KF == FLK_MATERN32 || FLK_KF == FLK_MATERN52) && tt == 1 && dp == 7) return 2;
     return ((tt == 2 && dp >= 2) || (tt == 3 && dp >= 6) || (tt >= 4 && dp >= 5)) ? 2 : fr;
 }
