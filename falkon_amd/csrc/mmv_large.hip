@@ -187,12 +187,15 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         // in every tile: otherwise the compiler forms one pointer per row value ahead of the tile loop, up to 33 of
         // them, and keeps them in scratch memory.)
         static_assert(G::A_ROWS % 64 == 0 && kLThreads % 64 == 0, "a wave's row values must belong to one vector");
+        // (not for fp64 with 32 columns, measured: C4's shape 260.7 ms per dfmmv against 265.4 with, where 16 columns take
+        // 251.5 against 260.1 and 64 columns 279.1 against 283.6)
+        constexpr bool kScalarWhich = sizeof(T) == 4 || TT != 32;
         int64_t vld = vec_ld;
-        asm volatile("" : "+s"(vld));
+        if constexpr (kScalarWhich) asm volatile("" : "+s"(vld));
 #pragma unroll
         for (int c = 0; c < kRowValsPerThread; c++) {
             const int e = tid + c * kLThreads;
-            const int which = __builtin_amdgcn_readfirstlane(e / G::A_ROWS), r = e % G::A_ROWS;
+            const int which = kScalarWhich ? __builtin_amdgcn_readfirstlane(e / G::A_ROWS) : e / G::A_ROWS, r = e % G::A_ROWS;
             const int64_t row = ablk0 * TR::BLK + r;
             T val = T(0);                      // rows past n_a carry zero weight
             if (e < kRowVals && row < na_blocks * TR::BLK) {
@@ -205,7 +208,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
         for (int c = 0; c < kRowValsPerThread; c++) {
             const int e = tid + c * kLThreads;
-            const int which = __builtin_amdgcn_readfirstlane(e / G::A_ROWS), r = e % G::A_ROWS;
+            const int which = kScalarWhich ? __builtin_amdgcn_readfirstlane(e / G::A_ROWS) : e / G::A_ROWS, r = e % G::A_ROWS;
             if (e < kRowVals) {
                 if (!kMfmaEpi || which == 0) ldsRow[e] = rowv[c];
                 else ldsRow[G::A_ROWS + r * kVecStride + (which - 1)] = rowv[c];
