@@ -98,6 +98,9 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     constexpr int kGroupCols = (sizeof(T) == 4 && TT > 16) ? 32 : 16;
     constexpr int NC = (kMfmaEpi && TT > kGroupCols) ? TT / kGroupCols : 1;
     constexpr int kEpiCols = kGroupCols * NC;
+    // fp32 with up to 16 columns: the four-block 16x16x1 step contracts them in half the cycles of a 32x32x2 step that
+    // would leave half of its columns unused (see the epilogue)
+    constexpr bool kHalf16 = kMfmaEpi && sizeof(T) == 4 && kGroupCols == 16;
     static_assert(TT <= kEpiCols || !kMfmaEpi, "columns per pass must be a whole number of column groups");
     constexpr int kVecStride = kEpiCols + 1;
     constexpr int kRowBuf = kMfmaEpi ? G::A_ROWS * (1 + kVecStride) : (1 + TT) * G::A_ROWS;
@@ -370,8 +373,12 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             }
             // out2[q][j-rows][t] += sum_i K[i][j] vec[i][t]: accumulator register s of a lane is exactly the MFMA
             // A operand of step s (row i = acc_row(s, lg), column j = lane), so K needs no data movement; the
-            // B operand is vec[acc_row(s, lg)][t] with t = lane % kGroupCols (+ kGroupCols per further group; fp32 lanes
-            // 16 .. 31 repeat the columns 0 .. 15 in the 16-column form and are never stored).
+            // B operand is vec[acc_row(s, lg)][t] with t = lane % kGroupCols (+ kGroupCols per further group).
+            // The 16-column fp32 form uses the four-block 16x16x1 step instead: with the same A operand, block
+            // b = lane / 16 holds the output rows 16 (b & 1) .. + 15 against the row of lane half b >> 1, its B operand is
+            // vec[acc_row(s, lg)][t = lane % 16], which is what the lanes of that quarter read, and it accumulates in
+            // registers 4 b .. 4 b + 3 (output row 16 (b & 1) + 4 (lane / 16) + r, column lane % 16); blocks b and
+            // b + 2 are partial sums of the same outputs, added at the store.
             const int tl = j & (kGroupCols - 1);
             // index of this lane's first B value (step 0 of its wave row's first block); every other read lies a
             // compile-time constant further on
@@ -406,7 +413,11 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
                     for (int g = 0; g < NC; g++)
 #pragma unroll
-                        for (int q = 0; q < WB_FR; q++) out2[q][g] = TR::mfma(acc[p][q][s2], bval[g], out2[q][g]);
+                        for (int q = 0; q < WB_FR; q++) {
+                            if constexpr (kHalf16)
+                                out2[q][g] = __builtin_amdgcn_mfma_f32_16x16x1f32(acc[p][q][s2], bval[g], out2[q][g], 0, 0, 0);
+                            else out2[q][g] = TR::mfma(acc[p][q][s2], bval[g], out2[q][g]);
+                        }
 #pragma unroll
                     for (int g = 0; g < NC; g++) {
                         asm volatile("" : "+v"(bval[g]) : "v"(&ldsRow[0]) : "memory");
@@ -419,6 +430,22 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 
     if constexpr (kStore) {
         // nothing left to write
+    } else if constexpr (kHalf16) {
+        const int tl = lane & 15, mq = lane >> 4;
+        if (tl < tcols) {
+#pragma unroll
+            for (int q = 0; q < WB_FR; q++) {
+                const int64_t bb = bblk0 + wb * WB_FR + q;
+                if (bb < nb_blocks) {
+#pragma unroll
+                    for (int b = 0; b < 2; b++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            partial[(((int64_t)by * kLWavesA + wa) * tcols + tl) * nb_pad + bb * TR::BLK + 16 * b + 4 * mq + r] =
+                                out2[q][0][4 * b + r] + out2[q][0][4 * (b + 2) + r];
+                }
+            }
+        }
     } else if constexpr (kMfmaEpi) {
         // lane = column t (both lane groups hold different output rows): no cross-lane step
         const int tl = j & (kGroupCols - 1);

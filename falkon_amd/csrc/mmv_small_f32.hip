@@ -16,12 +16,12 @@ int FLK_CAT(launch_mmv_small_f32_fold_kf, FLK_KF)(const PackedView &A, const Pac
                                                   float *partial, hipStream_t st);
 
 // Columns per pass of the per-lane FMA kernels (must match the instantiations in launch_tt); calls with more
-// right-hand sides than that go to the 32- or 64-column kernel whose contraction runs on the matrix cores
-// (mmv_small_f32_wide.hip: four resident blocks per wave up to 16 padded features, two beyond).
-static inline int fma_cols(int64_t dpad) {
-    const int64_t dp = dpad / 2;
-    return dp <= 7 ? 16 : dp <= 12 ? 12 : dp <= 16 ? 8 : 4;
-}
+// right-hand sides than that go to the kernel whose contraction runs on the matrix cores (mmv_small_f32_wide.hip:
+// 16, 32 or 64 columns per pass; four resident blocks per wave up to 16 padded features, two beyond).  Measured
+// against its 16-column form, dfmmv at N = 5e5, M = 2e4, 9 to 12 columns: d = 9 9.3 ms on the FMA kernel against 8.9,
+// d = 16 11.3 against 11.0, d = 24 14.1 against 13.4 (and 13 to 16 columns at d = 9: 10.9 against 9.0); eight columns:
+// d = 9 7.8 against 8.9, d = 28 13.3 against 14.7.
+static inline int fma_cols(int64_t dpad) { return dpad / 2 <= 16 ? 8 : 4; }
 constexpr int kWideColumns = 32;       // one group of columns of the wide kernel
 constexpr int kWideMaxDpFr4 = 8;
 // The wide kernel takes two groups (64 columns) on one evaluation of K unless the few columns beyond 32 are cheaper as a
@@ -47,8 +47,8 @@ template <> int mmv_small_max_cols<float>(int64_t dpad, int64_t t) {
 }
 template <> int mmv_small_width<float>(int64_t dpad, int tc) {
     if (tc > kWideColumns) return 2 * kWideColumns;
-    if (tc > fma_cols(dpad)) return kWideColumns;
-    static const int widths[] = {1, 2, 3, 4, 6, 8, 12, 16};
+    if (tc > fma_cols(dpad)) return tc > kWideColumns / 2 ? kWideColumns : kWideColumns / 2;   // the wide kernel's 16-column form
+    static const int widths[] = {1, 2, 3, 4, 6, 8};
     for (int w : widths) if (tc <= w) return w;
     return tc;
 }

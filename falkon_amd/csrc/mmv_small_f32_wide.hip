@@ -18,15 +18,17 @@
 
 namespace flk {
 
-// NC groups of 32 columns: the staged values of an A block are hn(32) | vec[32 rows][32 NC + 1] (the odd row stride
+// NC groups of 32 columns: the staged values of an A block are hn(32) | vec[32 rows][columns + 1] (the odd row stride
 // makes the reads conflict free)
+// (NC = 0 stands for the 16-column form: one half group)
 template <int NC> struct WideGeo {
-    static constexpr int kCols = 32 * NC;
+    static constexpr int kCols = NC == 0 ? 16 : 32 * NC;
     static constexpr int kStride = kCols + 1;
     static constexpr int kStage = 32 + 32 * kStride;
     static constexpr int kFetch = 1 + kCols / 8;         // dwords a thread fetches per A block
 };
 constexpr int kWideCols = 32;                            // of one group
+constexpr int kWideHalfCols = 16;                        // of the 16-column form
 constexpr int kWideMaxGroups = 2;
 
 template <int NC> struct WideRowVals { float x[WideGeo<NC>::kFetch]; };
@@ -62,7 +64,7 @@ __device__ __forceinline__ void wide_barrier() {
 template <int DP, int FR, bool FOLD, int KF, int NC>
 __device__ __forceinline__ void wide_tile_step(const float (&a)[DP], const float *lds, int j, int h,
                                                const float (&breg)[FR][DP], const float (&hb)[FR],
-                                               floatx16 (&out2)[FR][NC]) {
+                                               floatx16 (&out2)[FR][NC == 0 ? 1 : NC]) {
     constexpr int kWideStride = WideGeo<NC>::kStride;
     floatx4 hn[4];
 #pragma unroll
@@ -85,26 +87,46 @@ __device__ __forceinline__ void wide_tile_step(const float (&a)[DP], const float
     __builtin_amdgcn_sched_barrier(0);
     // contraction on the matrix cores; the B operand is read one step ahead, fenced (otherwise every read is
     // hoisted to the front)
-    const float *vb = lds + 32 + j;
-    float bval[NC], bnext[NC];
+    if constexpr (NC == 0) {
+        // Up to 16 columns: the four-block 16x16x1 step, half the cycles of a 32x32x2 step that would leave half of its
+        // columns unused.  Its blocks are the lane quarters: as A operand, register s2 of lane l is K[i][j] with
+        // j = l % 32 and i the row of step s2 in lane half h, i.e. block b = l / 16 holds the output rows 16 (b & 1) ..
+        // + 15 against row i of half b >> 1; the B operand of block b is vec[that row][t = l % 16], which is what the
+        // lanes of that quarter read.  Block b accumulates in registers 4 b .. 4 b + 3 (output row 16 (b & 1) +
+        // 4 (lane / 16) + r, column lane % 16): blocks b and b + 2 are partial sums of the same outputs.
+        const float *vb = lds + 32 + (j & 15);
+        float bval = vb[(4 * h) * kWideStride], bnext = 0.f;
 #pragma unroll
-    for (int g = 0; g < NC; g++) { bval[g] = vb[(4 * h) * kWideStride + 32 * g]; bnext[g] = 0.f; }
-#pragma unroll
-    for (int s2 = 0; s2 < 16; s2++) {
-        if (s2 + 1 < 16) {
-#pragma unroll
-            for (int g = 0; g < NC; g++)
-                bnext[g] = vb[(8 * ((s2 + 1) >> 2) + 4 * h + ((s2 + 1) & 3)) * kWideStride + 32 * g];
-        }
-#pragma unroll
-        for (int g = 0; g < NC; g++)
+        for (int s2 = 0; s2 < 16; s2++) {
+            if (s2 + 1 < 16) bnext = vb[(8 * ((s2 + 1) >> 2) + 4 * h + ((s2 + 1) & 3)) * kWideStride];
 #pragma unroll
             for (int q = 0; q < FR; q++)
-                out2[q][g] = __builtin_amdgcn_mfma_f32_32x32x2f32(acc[q][s2], bval[g], out2[q][g], 0, 0, 0);
+                out2[q][0] = __builtin_amdgcn_mfma_f32_16x16x1f32(acc[q][s2], bval, out2[q][0], 0, 0, 0);
+            asm volatile("" : "+v"(bval) : "v"(vb) : "memory");
+            bval = bnext;
+        }
+    } else {
+        const float *vb = lds + 32 + j;
+        float bval[NC], bnext[NC];
 #pragma unroll
-        for (int g = 0; g < NC; g++) {
-            asm volatile("" : "+v"(bval[g]) : "v"(vb) : "memory");
-            bval[g] = bnext[g];
+        for (int g = 0; g < NC; g++) { bval[g] = vb[(4 * h) * kWideStride + 32 * g]; bnext[g] = 0.f; }
+#pragma unroll
+        for (int s2 = 0; s2 < 16; s2++) {
+            if (s2 + 1 < 16) {
+#pragma unroll
+                for (int g = 0; g < NC; g++)
+                    bnext[g] = vb[(8 * ((s2 + 1) >> 2) + 4 * h + ((s2 + 1) & 3)) * kWideStride + 32 * g];
+            }
+#pragma unroll
+            for (int g = 0; g < NC; g++)
+#pragma unroll
+                for (int q = 0; q < FR; q++)
+                    out2[q][g] = __builtin_amdgcn_mfma_f32_32x32x2f32(acc[q][s2], bval[g], out2[q][g], 0, 0, 0);
+#pragma unroll
+            for (int g = 0; g < NC; g++) {
+                asm volatile("" : "+v"(bval[g]) : "v"(vb) : "memory");
+                bval[g] = bnext[g];
+            }
         }
     }
 }
@@ -116,7 +138,7 @@ __global__ void __launch_bounds__(256, 2)
                               int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB,
                               int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial,
                               int64_t nb_pad, int tcols, bool y_fastest) {
-    // vecp must hold 32 NC planes (zeros beyond the caller's columns); the first tcols columns are stored
+    // vecp must hold 32 NC planes (16 for NC = 0; zeros beyond the caller's columns); the first tcols columns are stored
     __shared__ __attribute__((aligned(16))) float stage[2][WideGeo<NC>::kStage];   // shared by the four waves
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
@@ -139,11 +161,12 @@ __global__ void __launch_bounds__(256, 2)
         hb[q] = hB[bb * 32 + j];
         if (FOLD) breg[q][DP - 1] = h ? hb[q] : breg[q][DP - 1];
     }
-    floatx16 out2[FR][NC];
+    constexpr int kGroups = NC == 0 ? 1 : NC;
+    floatx16 out2[FR][kGroups];
 #pragma unroll
     for (int q = 0; q < FR; q++)
 #pragma unroll
-        for (int g = 0; g < NC; g++)
+        for (int g = 0; g < kGroups; g++)
 #pragma unroll
             for (int r = 0; r < 16; r++) out2[q][g][r] = 0.f;
 
@@ -172,17 +195,35 @@ __global__ void __launch_bounds__(256, 2)
         }
         wide_barrier();
     }
-    // lane = column t, registers = output rows (both lane halves hold different rows): no cross-lane step
-#pragma unroll
-    for (int g = 0; g < NC; g++) {
-        if (j + 32 * g < tcols) {
+    if constexpr (NC == 0) {
+        // lane = column t = lane % 16; registers 4 b + r and 4 (b + 2) + r together are output row 16 b + 4 (lane / 16) + r
+        const int t = lane & 15, mq = lane >> 4;
+        if (t < tcols) {
 #pragma unroll
             for (int q = 0; q < FR; q++) {
                 if (bb0 + q < nb_blocks) {
 #pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        partial[((int64_t)by * tcols + j + 32 * g) * nb_pad + (bb0 + q) * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] =
-                            out2[q][g][r];
+                    for (int b = 0; b < 2; b++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            partial[((int64_t)by * tcols + t) * nb_pad + (bb0 + q) * 32 + 16 * b + 4 * mq + r] =
+                                out2[q][0][4 * b + r] + out2[q][0][4 * (b + 2) + r];
+                }
+            }
+        }
+    } else {
+        // lane = column t, registers = output rows (both lane halves hold different rows): no cross-lane step
+#pragma unroll
+        for (int g = 0; g < NC; g++) {
+            if (j + 32 * g < tcols) {
+#pragma unroll
+                for (int q = 0; q < FR; q++) {
+                    if (bb0 + q < nb_blocks) {
+#pragma unroll
+                        for (int r = 0; r < 16; r++)
+                            partial[((int64_t)by * tcols + j + 32 * g) * nb_pad + (bb0 + q) * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] =
+                                out2[q][g][r];
+                    }
                 }
             }
         }
@@ -230,12 +271,15 @@ int FLK_CAT(launch_mmv_small_f32_wide_kf, FLK_KF)(const PackedView &A, const Pac
 #undef FLK_WIDE2_PLAIN
         return fail(FLK_EUNSUPPORTED, "mmv_small wide: padded feature count %lld not in 2..64", (long long)A.dpad);
     }
-#define FLK_WIDE(DPV, FRV)                                                                                         \
-    case DPV:                                                                                                      \
-        return fold ? launch_wide_one<DPV, FRV, true>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st) \
-                    : launch_wide_one<DPV, FRV, false>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+    // up to 16 columns: the 16-column form (vecp holds 16 planes); 17 to 32: one group of 32
+    const bool half = tcols <= kWideHalfCols;
+#define FLK_WIDE_ONE(DPV, FRV, FOLDV)                                                                              \
+    (half ? launch_wide_one<DPV, FRV, FOLDV, 0>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)     \
+          : launch_wide_one<DPV, FRV, FOLDV, 1>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st))
+#define FLK_WIDE(DPV, FRV) \
+    case DPV: return fold ? FLK_WIDE_ONE(DPV, FRV, true) : FLK_WIDE_ONE(DPV, FRV, false);
 #define FLK_WIDE_PLAIN(DPV, FRV) \
-    case DPV: return launch_wide_one<DPV, FRV, false>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+    case DPV: return FLK_WIDE_ONE(DPV, FRV, false);
     switch (dp) {
         FLK_WIDE(1, 4) FLK_WIDE(2, 4) FLK_WIDE(3, 4) FLK_WIDE(4, 4) FLK_WIDE(5, 4) FLK_WIDE(6, 4) FLK_WIDE(7, 4)
         FLK_WIDE(8, 4) FLK_WIDE(9, 2) FLK_WIDE(10, 2) FLK_WIDE(11, 2) FLK_WIDE(12, 2) FLK_WIDE(13, 2) FLK_WIDE(14, 2)
@@ -247,6 +291,7 @@ int FLK_CAT(launch_mmv_small_f32_wide_kf, FLK_KF)(const PackedView &A, const Pac
     }
 #undef FLK_WIDE
 #undef FLK_WIDE_PLAIN
+#undef FLK_WIDE_ONE
     return fail(FLK_EUNSUPPORTED, "mmv_small wide: padded feature count %lld not in 2..64", (long long)A.dpad);
 }
 

@@ -289,9 +289,13 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                 for (int q = 0; q < WB_FR; q++)
 #pragma unroll
                     for (int r = 0; r < 16; r++) acc[p][q][r] = kernel_value<KF>(acc[p][q][r]);
-            // out2[q][j-rows][t] += sum_i K[i][j] vec[i][t]: accumulator register s2 of a lane is exactly the fp32
-            // MFMA A operand of step s2 (row i = acc_row(s2, lg), column j = lane % 32); the B operand is
-            // vec[acc_row(s2, lg)][t] with t = lane % 16 (columns past 16 are never stored)
+            // out2[q][j-rows][t] += sum_i K[i][j] vec[i][t] with the four-block fp32 16x16x1 step (half the cycles of a
+            // 32x32x2 step, which would leave 16 of its 32 columns unused): as its A operand, accumulator register s2
+            // of lane l is K[i][j] with i = acc_row(s2, lg), j = l % 32, so block b = l / 16 holds the output rows
+            // 16 (b & 1) .. + 15 against the row of lane half b >> 1; its B operand is vec[acc_row(s2, lg)][t = l % 16],
+            // which is what the lanes of that quarter read.  Block b accumulates in registers 4 b .. 4 b + 3 (output
+            // row 16 (b & 1) + 4 (lane / 16) + r, column lane % 16): blocks b and b + 2 are partial sums of the same
+            // outputs, added at the store.
             const float *vb = &ldsRow[j & 15];
             // one read ahead, fenced (otherwise all reads are hoisted to the front and spilled)
             float bval = vb[((wa * WA_FR) * 32 + TR::acc_row(0, lg)) * kVecStride], bnext = 0.f;
@@ -303,7 +307,8 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                     if (s2 + 1 < 16) bnext = vb[(rbase + TR::acc_row(s2 + 1, lg)) * kVecStride];
                     else if (p + 1 < WA_FR) bnext = vb[(rbase + 32 + TR::acc_row(0, lg)) * kVecStride];
 #pragma unroll
-                    for (int q = 0; q < WB_FR; q++) out2[q] = TR::mfma(acc[p][q][s2], bval, out2[q]);
+                    for (int q = 0; q < WB_FR; q++)
+                        out2[q] = __builtin_amdgcn_mfma_f32_16x16x1f32(acc[p][q][s2], bval, out2[q], 0, 0, 0);
                     asm volatile("" : "+v"(bval) : "v"(vb) : "memory");
                     bval = bnext;
                 }
@@ -314,16 +319,18 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     if constexpr (STORE) {
         // nothing left to write
     } else if constexpr (kMfmaEpi) {
-        const int tl = j & 15;
-        if (j < 16 && tl < tcols) {
+        const int tl = lane & 15, mq = lane >> 4;
+        if (tl < tcols) {
 #pragma unroll
             for (int q = 0; q < WB_FR; q++) {
                 const int64_t bb = bblk0 + wb * WB_FR + q;
                 if (bb < nb_blocks) {
 #pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        partial[(((int64_t)by * WVA + wa) * tcols + tl) * nb_pad + bb * 32 + TR::acc_row(r, lg)] =
-                            out2[q][r];
+                    for (int b = 0; b < 2; b++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            partial[(((int64_t)by * WVA + wa) * tcols + tl) * nb_pad + bb * 32 + 16 * b + 4 * mq + r] =
+                                out2[q][4 * b + r] + out2[q][4 * (b + 2) + r];
                 }
             }
         }
