@@ -432,26 +432,24 @@ static int fmm_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1
 // ---------------------------------------------------------------------------
 constexpr int64_t kTargetWgsSplitLarge = 8192;  // one 512-thread workgroup per CU: 32 rounds
 
-// Where the bf16x3 kernels are the faster route to the same result.  Measured at N = 1e6, M = 2e4, dfmmv, against the
-// fp32 MFMA kernels.  d = 28: 1 right-hand side 10.9 ms against 20.2, 2: 11.7 against 21.1, 3 or 4: 14.3 against
-// 22.4 / 22.7 (register-resident kernel, up to four columns per pass); 5: 2 x 14.3 against 24.4 (the fp32 kernels
-// contract up to eight columns per pass with per-lane FMAs up to 32 features); 9: 34.8 against 41.9, 16: 35.0 against
-// 42.2 (LDS-tiled kernel, sixteen columns per pass on the matrix cores, against the fp32 kernel that contracts 32);
-// 17: 50.0 against 42.2, 32: 70.1 against 43.0.  d = 40 / 60, where the fp32 FMA kernels take four columns per pass:
-// 4: 18.4 / 24.3 against 29.9 / 48.0, 5: 49.9 / 64.4 for the fp32 32-column kernel, i.e. two passes of the
-// register-resident bf16x3 kernel are the faster route for 5 to 8 columns.  So: every feature count beyond the
-// register-resident kernels; at small feature counts 1 to 4 and 9 to 16 right-hand sides, and 5 to 8 beyond 32
-// features; otherwise the fp32 MFMA kernels serve the mode.
+// Where the bf16x3 kernels are the faster route to the same result.  Measured at N = 5e5, M = 2e4, dfmmv, against the
+// fp32 MFMA kernels.  Up to four right-hand sides (register-resident kernel, up to four columns per pass): d = 9 / 28 /
+// 60, 4 columns: 5.0 / 7.3 / 12.5 ms against 6.2 / 11.3 / 21.6.  5 to 16 (LDS-tiled kernel, sixteen columns per pass on
+// the matrix cores; the fp32 kernels contract 8 or 16 columns with narrow MFMA steps): d = 9 / 16 / 28 / 32: 11.4 / 13.5 /
+// 13.4 / 15.6 against 6.7 / 8.8 / 12.3 / 13.5 with 5 columns and 8.8 / 11.0 / 14.6 / 15.9 with 9; d = 40 / 48 / 60: 15.7 /
+// 17.8 / 17.9 against 16.8 / 19.0 / 23.6 with 5 columns and 18.4 / 20.7 / 25.0 with 9 (two passes of the register-resident
+// kernel for 5 to 8 columns: 17.8 / 22.2 / 23.2).  17 and more: the fp32 kernels contract 32 or 64 columns per pass.  So:
+// every feature count beyond the register-resident kernels; at small feature counts 1 to 4 right-hand sides, 5 to 16
+// beyond 32 features and 9 to 16 from 25 features on; otherwise the fp32 MFMA kernels serve the mode.
 static bool split_applies(int64_t d, int64_t t) {
-    return d > kSplitMaxD || t <= kSplitMaxCols || (t <= 2 * kSplitMaxCols && d > 32) || (t > 8 && t <= 16);
+    return d > kSplitMaxD || t <= kSplitMaxCols || (t <= 16 && d > 32) || (t > 8 && t <= 16 && d > 24);
 }
 
 static Plan make_plan_split(int64_t na_blocks, int64_t nb_blocks, int64_t ks, int64_t t) {
     Plan p;
-    // up to four right-hand sides per pass the register-resident kernel (two passes for five to eight); beyond that
-    // (see split_applies) the LDS-tiled kernel,
+    // up to four right-hand sides the register-resident kernel; beyond that (see split_applies) the LDS-tiled kernel,
     // whose epilogue contracts sixteen columns per pass on the matrix cores, also for small feature counts
-    if (ks * 16 <= kSplitMaxD + 2 && t <= 2 * kSplitMaxCols) {
+    if (ks * 16 <= kSplitMaxD + 2 && t <= kSplitMaxCols) {
         plan_register_resident(p, na_blocks, nb_blocks, split_b_blocks_per_wg(ks, t), ks * 3 * 64 * 16, 32, kSplitMaxCols,
                                t, (int64_t)sizeof(float));
         return p;

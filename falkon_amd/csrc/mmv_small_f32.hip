@@ -17,11 +17,12 @@ int FLK_CAT(launch_mmv_small_f32_fold_kf, FLK_KF)(const PackedView &A, const Pac
 
 // Columns per pass of the per-lane FMA kernels (must match the instantiations in launch_tt); calls with more
 // right-hand sides than that go to the kernel whose contraction runs on the matrix cores (mmv_small_f32_wide.hip:
-// 16, 32 or 64 columns per pass; four resident blocks per wave up to 16 padded features, two beyond).  Measured
-// against its 16-column form, dfmmv at N = 5e5, M = 2e4, 9 to 12 columns: d = 9 9.3 ms on the FMA kernel against 8.9,
-// d = 16 11.3 against 11.0, d = 24 14.1 against 13.4 (and 13 to 16 columns at d = 9: 10.9 against 9.0); eight columns:
-// d = 9 7.8 against 8.9, d = 28 13.3 against 14.7.
-static inline int fma_cols(int64_t dpad) { return dpad / 2 <= 16 ? 8 : 4; }
+// 8, 16, 32 or 64 columns per pass; four resident blocks per wave up to 16 padded features, two beyond).  Measured,
+// dfmmv at N = 5e5, M = 2e4, FMA kernel against the 8-column form (which costs the same for 3 to 8 columns):
+// d = 9: 4 columns 6.2 ms against 6.6, 5 columns 7.0 against 6.7, 8 columns 8.1 against 6.8; d = 16: 8.2 / 8.9 / 9.9 against
+// 8.7 / 8.8 / 8.9; d = 28: 5 and 6 columns 12.4 against 12.8, 8 columns 13.4 against 12.8; d = 40 (two resident blocks):
+// 4 columns 15.5 against 17.0, 5 to 8 columns on the 16-column form 18.4 against 16.9.
+static inline int fma_cols(int64_t dpad) { return dpad / 2 > 8 && dpad / 2 <= 16 ? 6 : 4; }
 constexpr int kWideColumns = 32;       // one group of columns of the wide kernel
 constexpr int kWideMaxDpFr4 = 8;
 // The wide kernel takes two groups (64 columns) on one evaluation of K unless the few columns beyond 32 are cheaper as a
@@ -47,8 +48,9 @@ template <> int mmv_small_max_cols<float>(int64_t dpad, int64_t t) {
 }
 template <> int mmv_small_width<float>(int64_t dpad, int tc) {
     if (tc > kWideColumns) return 2 * kWideColumns;
-    if (tc > fma_cols(dpad)) return tc > kWideColumns / 2 ? kWideColumns : kWideColumns / 2;   // the wide kernel's 16-column form
-    static const int widths[] = {1, 2, 3, 4, 6, 8};
+    if (tc > fma_cols(dpad))      // the wide kernel's 32-, 16- and 8-column forms
+        return tc > kWideColumns / 2 ? kWideColumns : tc > kWideColumns / 4 ? kWideColumns / 2 : kWideColumns / 4;
+    static const int widths[] = {1, 2, 3, 4, 6};
     for (int w : widths) if (tc <= w) return w;
     return tc;
 }

@@ -20,15 +20,29 @@ namespace flk {
 
 // NC groups of 32 columns: the staged values of an A block are hn(32) | vec[32 rows][columns + 1] (the odd row stride
 // makes the reads conflict free)
-// (NC = 0 stands for the 16-column form: one half group)
+// (NC = 0 stands for the 16-column form, one half group, and NC = -1 for the 8-column form)
 template <int NC> struct WideGeo {
-    static constexpr int kCols = NC == 0 ? 16 : 32 * NC;
+    static constexpr int kCols = NC == -1 ? 8 : NC == 0 ? 16 : 32 * NC;
     static constexpr int kStride = kCols + 1;
     static constexpr int kStage = 32 + 32 * kStride;
     static constexpr int kFetch = 1 + kCols / 8;         // dwords a thread fetches per A block
 };
 constexpr int kWideCols = 32;                            // of one group
 constexpr int kWideHalfCols = 16;                        // of the 16-column form
+constexpr int kWideNarrowCols = 8;                       // of the 8-column form
+
+// Output accumulators of a resident block: one 16-register set per group of 32 columns (one for the 16-column form);
+// the 8-column form keeps two sets of four registers (columns 0 .. 3 and 4 .. 7)
+template <int NC> struct WideOut {
+    typedef floatx16 type;
+    static constexpr int kSets = NC == 0 ? 1 : NC;
+    static constexpr int kRegs = 16;
+};
+template <> struct WideOut<-1> {
+    typedef floatx4 type;
+    static constexpr int kSets = 2;
+    static constexpr int kRegs = 4;
+};
 constexpr int kWideMaxGroups = 2;
 
 template <int NC> struct WideRowVals { float x[WideGeo<NC>::kFetch]; };
@@ -64,7 +78,7 @@ __device__ __forceinline__ void wide_barrier() {
 template <int DP, int FR, bool FOLD, int KF, int NC>
 __device__ __forceinline__ void wide_tile_step(const float (&a)[DP], const float *lds, int j, int h,
                                                const float (&breg)[FR][DP], const float (&hb)[FR],
-                                               floatx16 (&out2)[FR][NC == 0 ? 1 : NC]) {
+                                               typename WideOut<NC>::type (&out2)[FR][WideOut<NC>::kSets]) {
     constexpr int kWideStride = WideGeo<NC>::kStride;
     floatx4 hn[4];
 #pragma unroll
@@ -87,7 +101,34 @@ __device__ __forceinline__ void wide_tile_step(const float (&a)[DP], const float
     __builtin_amdgcn_sched_barrier(0);
     // contraction on the matrix cores; the B operand is read one step ahead, fenced (otherwise every read is
     // hoisted to the front)
-    if constexpr (NC == 0) {
+    if constexpr (NC == -1) {
+        // Up to 8 columns: two 16-block 4x4x1 steps (8 cycles each; the 16x16x1 step below takes 32, 16 per-lane FMAs per
+        // column 64).  As A operand, register s2 of lane l is K[i][j] with j = l % 32 and i the row of step s2 in lane
+        // half h: block b = l / 4 holds the output rows 4 (b % 8) .. + 3 against that row of half b / 8.  The B operand
+        // of block b is vec[that row][4 u + l % 4] for the column set u, and output (row 4 (b % 8) + r, column
+        // 4 u + l % 4) accumulates in register r of set u in lane l: the two lane halves hold partial sums of the
+        // same outputs, added at the store.
+        const float *vb = lds + 32 + (j & 3);
+        float bval[2] = {vb[(4 * h) * kWideStride], vb[(4 * h) * kWideStride + 4]}, bnext[2] = {0.f, 0.f};
+#pragma unroll
+        for (int s2 = 0; s2 < 16; s2++) {
+            if (s2 + 1 < 16) {
+#pragma unroll
+                for (int u = 0; u < 2; u++)
+                    bnext[u] = vb[(8 * ((s2 + 1) >> 2) + 4 * h + ((s2 + 1) & 3)) * kWideStride + 4 * u];
+            }
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int q = 0; q < FR; q++)
+                    out2[q][u] = __builtin_amdgcn_mfma_f32_4x4x1f32(acc[q][s2], bval[u], out2[q][u], 0, 0, 0);
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                asm volatile("" : "+v"(bval[u]) : "v"(vb) : "memory");
+                bval[u] = bnext[u];
+            }
+        }
+    } else if constexpr (NC == 0) {
         // Up to 16 columns: the four-block 16x16x1 step, half the cycles of a 32x32x2 step that would leave half of its
         // columns unused.  Its blocks are the lane quarters: as A operand, register s2 of lane l is K[i][j] with
         // j = l % 32 and i the row of step s2 in lane half h, i.e. block b = l / 16 holds the output rows 16 (b & 1) ..
@@ -138,7 +179,8 @@ __global__ void __launch_bounds__(256, 2)
                               int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB,
                               int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial,
                               int64_t nb_pad, int tcols, bool y_fastest) {
-    // vecp must hold 32 NC planes (16 for NC = 0; zeros beyond the caller's columns); the first tcols columns are stored
+    // vecp must hold 32 NC planes (16 for NC = 0, 8 for NC = -1; zeros beyond the caller's columns); the first tcols
+    // columns are stored
     __shared__ __attribute__((aligned(16))) float stage[2][WideGeo<NC>::kStage];   // shared by the four waves
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
@@ -161,14 +203,13 @@ __global__ void __launch_bounds__(256, 2)
         hb[q] = hB[bb * 32 + j];
         if (FOLD) breg[q][DP - 1] = h ? hb[q] : breg[q][DP - 1];
     }
-    constexpr int kGroups = NC == 0 ? 1 : NC;
-    floatx16 out2[FR][kGroups];
+    typename WideOut<NC>::type out2[FR][WideOut<NC>::kSets];
 #pragma unroll
     for (int q = 0; q < FR; q++)
 #pragma unroll
-        for (int g = 0; g < kGroups; g++)
+        for (int g = 0; g < WideOut<NC>::kSets; g++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) out2[q][g][r] = 0.f;
+            for (int r = 0; r < WideOut<NC>::kRegs; r++) out2[q][g][r] = 0.f;
 
     float fa0[DP], fa1[DP];
     WideRowVals<NC> rv;
@@ -195,7 +236,20 @@ __global__ void __launch_bounds__(256, 2)
         }
         wide_barrier();
     }
-    if constexpr (NC == 0) {
+    if constexpr (NC == -1) {
+        // lane l and lane l + 32 hold partial sums of output rows 4 ((l / 4) % 8) + r, column 4 u + l % 4
+        const int t4 = lane & 3, jb = 4 * ((lane >> 2) & 7);
+#pragma unroll
+        for (int q = 0; q < FR; q++)
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float sum = out2[q][u][r] + __shfl_xor(out2[q][u][r], 32);
+                    if (lane < 32 && 4 * u + t4 < tcols && bb0 + q < nb_blocks)
+                        partial[((int64_t)by * tcols + 4 * u + t4) * nb_pad + (bb0 + q) * 32 + jb + r] = sum;
+                }
+    } else if constexpr (NC == 0) {
         // lane = column t = lane % 16; registers 4 b + r and 4 (b + 2) + r together are output row 16 b + 4 (lane / 16) + r
         const int t = lane & 15, mq = lane >> 4;
         if (t < tcols) {
@@ -271,11 +325,13 @@ int FLK_CAT(launch_mmv_small_f32_wide_kf, FLK_KF)(const PackedView &A, const Pac
 #undef FLK_WIDE2_PLAIN
         return fail(FLK_EUNSUPPORTED, "mmv_small wide: padded feature count %lld not in 2..64", (long long)A.dpad);
     }
-    // up to 16 columns: the 16-column form (vecp holds 16 planes); 17 to 32: one group of 32
-    const bool half = tcols <= kWideHalfCols;
+    // up to 8 columns: the 8-column form (vecp holds 8 planes); up to 16: the 16-column form (16 planes); 17 to 32: one
+    // group of 32
+    const bool half = tcols <= kWideHalfCols, narrow = tcols <= kWideNarrowCols;
 #define FLK_WIDE_ONE(DPV, FRV, FOLDV)                                                                              \
-    (half ? launch_wide_one<DPV, FRV, FOLDV, 0>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)     \
-          : launch_wide_one<DPV, FRV, FOLDV, 1>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st))
+    (narrow ? launch_wide_one<DPV, FRV, FOLDV, -1>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)  \
+     : half ? launch_wide_one<DPV, FRV, FOLDV, 0>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)   \
+            : launch_wide_one<DPV, FRV, FOLDV, 1>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st))
 #define FLK_WIDE(DPV, FRV) \
     case DPV: return fold ? FLK_WIDE_ONE(DPV, FRV, true) : FLK_WIDE_ONE(DPV, FRV, false);
 #define FLK_WIDE_PLAIN(DPV, FRV) \
