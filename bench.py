@@ -26,7 +26,7 @@ FP64_PEAK_TFLOPS = 78.6    # MI355X fp64 matrix peak = fp64 vector peak
 BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 
 
-def split_roofline(pairs, d, kern_ms, algorithmic_flop, traffic=None):
+def split_roofline(pairs, d, kern_ms, algorithmic_flop, traffic=None, pairs_cols=1):
     """Roofline of the bf16x3 product kernel: it executes 6 partial products over the features padded to whole
     k-steps of 16 (two of them carry the half norms), on the bf16 matrix cores."""
     ksteps = (d + 2 + 15) // 16
@@ -34,7 +34,7 @@ def split_roofline(pairs, d, kern_ms, algorithmic_flop, traffic=None):
     achieved = executed / (kern_ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": achieved / BF16_PEAK_TFLOPS, "traffic": traffic,
-            "kernel": "mmv_split_kernel" if d <= 62 else "mmv_split_large_kernel",
+            "kernel": "mmv_split_kernel" if d <= 62 and pairs_cols <= 4 else "mmv_split_large_kernel",
             "avg_launch_ms": kern_ms, "flop_per_launch": executed,
             "note": "achieved = bf16 MFMA flops the kernel executes (6 partial products, padded features); "
                     "algorithmic fp32 flops per launch and their rate are given beside it",
@@ -77,9 +77,15 @@ def product_kernel_name(d, T, dtype):
         return "mmv_large_kernel"
     if dtype == "f32":
         steps = (d + 1) // 2
-        fma_cols = 16 if steps <= 7 else 12 if steps <= 12 else 8 if steps <= 16 else 4
+        fma_cols = 6 if 8 < steps <= 16 else 4
         return "mmv_small_f32_wide_kernel" if T > fma_cols else "mmv_small_f32_kernel"
-    return "mmv_small_f64_wide_kernel" if T > (3 if d > 52 else 4) else "mmv_small_f64_kernel"
+    return "mmv_small_f64_wide_kernel" if T > (3 if d > 48 else 4) else "mmv_small_f64_kernel"
+
+
+def split_kernels_serve(d, T):
+    """Whether the bf16x3 kernels serve a call of the bf16x3 mode with d features and T right-hand sides, or the fp32
+    kernels do (split_applies in csrc/api.hip)."""
+    return d > 62 or T <= 4 or (T <= 16 and d > 32) or (8 < T <= 16 and d > 24)
 
 
 def make_inputs(name, rhs=0):
@@ -517,8 +523,8 @@ def main():
             res["roofline"].update(achieved=executed / (elapsed / args.steps) / 1e12, peak=BF16_PEAK_TFLOPS,
                                    frac=executed / (elapsed / args.steps) / 1e12 / BF16_PEAK_TFLOPS,
                                    algorithmic_frac_of_fp32_peak=once)
-    if split and launches.value > 0:
-        res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch, traffic),
+    if split and launches.value > 0 and split_kernels_serve(d, T):
+        res["roofline"] = dict(split_roofline(N * M, d, kern_ms, flop_per_launch, traffic, pairs_cols=T),
                                launches_per_step=launches.value / args.steps, traffic_source=traffic_src)
     if not split and args.dtype == "f32" and args.kernel == "gaussian" and not args.no_cpu_baseline:
         # not the headline: the same step with the opt-in bf16x3 cross term (fp32 data and results, the cross term
