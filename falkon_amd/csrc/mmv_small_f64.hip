@@ -195,19 +195,18 @@ template <> int64_t mmv_small_max_d<double>() { return 4 * kMaxDp64Fr2; }
 // more than four right-hand sides: the 16-column kernel of mmv_small_f64_wide.hip, which reads 16 planes
 // (beyond 16 columns two groups of 16 share one evaluation of K: 17 columns that way take less time than a
 // 16-column pass and a one-column pass, at every feature count)
-// (four groups unless the few columns beyond 32 are cheaper as a pass of the FMA kernel behind a 32-column pass, which
-// holds at small feature counts only.  Measured, dfmmv at N = 5e5, M = 2e4, the pair against the 64-column form:
-// d = 4, T = 36: 46.1 ms against 48.2; d = 9, T = 33 / 34 / 36: 49.2 / 50.2 / 54.2 against 52.9; d = 16, T = 34: 55.2
-// against 56.0; d = 28, T = 33: 69.2 against 65.7; d = 64: 115.0 against 98.7)
-static inline int cheap_extra_cols64(int64_t dpad) { return dpad <= 8 ? 4 : dpad <= 16 ? 2 : 0; }
-static inline bool four_groups64(int64_t dpad, int64_t t) { return t > 2 * kWideCols64 + cheap_extra_cols64(dpad); }
+// (beyond 32 columns three or four groups share one evaluation of K, with half the resident blocks.  A 32-column pass
+// followed by a pass of the FMA kernel for one to four more columns is never the faster pair: dfmmv at N = 5e5, M = 2e4,
+// d = 9, T = 33: 49.5 ms against 43.6 for the three-group form, d = 28: 69.2 against 54.1)
+static inline bool four_groups64(int64_t dpad, int64_t t) { (void)dpad; return t > 2 * kWideCols64; }
 template <> int mmv_small_max_cols<double>(int64_t dpad, int64_t t) {
     if (four_groups64(dpad, t)) return 4 * kWideCols64;
     if (t > kWideCols64) return 2 * kWideCols64;
     return t > fma_cols64(dpad) ? kWideCols64 : fma_cols64(dpad);
 }
 template <> int mmv_small_width<double>(int64_t dpad, int tc) {
-    if (tc > 2 * kWideCols64) return 4 * kWideCols64;
+    if (tc > 3 * kWideCols64) return 4 * kWideCols64;
+    if (tc > 2 * kWideCols64) return 3 * kWideCols64;     // 33 to 48 columns: three groups
     if (tc > kWideCols64) return 2 * kWideCols64;
     return tc > fma_cols64(dpad) ? kWideCols64 : tc;
 }

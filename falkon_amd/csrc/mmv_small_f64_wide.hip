@@ -33,7 +33,7 @@ template <int NC> struct Wide64Geo {
     static constexpr int kCols = 16 * NC;
     static constexpr int kStride = kCols + 1;               // row stride of the staged vec values
     static constexpr int kStage = 16 + 16 * kStride;        // hn(16) | vec[16 rows][16 NC + 1]
-    static constexpr bool kShared = NC >= 4;                // one stage per workgroup instead of one per wave (below)
+    static constexpr bool kShared = NC >= 3;                // one stage per workgroup instead of one per wave (below)
     static constexpr int kFetch = kShared ? 1 + NC : 1 + kCols / 4;   // doubles a thread fetches per A block
 };
 
@@ -251,8 +251,10 @@ int FLK_CAT(launch_mmv_small_f64_wide_kf, FLK_KF)(const PackedView &A, const Pac
     const int dp = (int)(A.dpad / 4);
 #define FLK_WIDE64(DPV, FRV)                                                                                             \
     case DPV:                                                                                                           \
-        if (tcols > 2 * kWide64Cols)                                                                                    \
+        if (tcols > 3 * kWide64Cols)                                                                                    \
             return launch_wide64_one<DPV, (FRV) / 2, 4>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st); \
+        if (tcols > 2 * kWide64Cols)                                                                                    \
+            return launch_wide64_one<DPV, (FRV) / 2, 3>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st); \
         return tcols > kWide64Cols                                                                                      \
                    ? launch_wide64_one<DPV, FRV, 2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)     \
                    : launch_wide64_one<DPV, FRV, 1>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);

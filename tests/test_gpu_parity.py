@@ -547,7 +547,7 @@ def test_non_finite_rows_give_nan(dev, mode, d, t):
 
 
 @pytest.mark.parametrize("d,t", [(1, 5), (3, 16), (9, 7), (12, 40), (28, 29), (32, 9), (33, 17), (50, 6), (64, 16), (61, 4),
-                                 (64, 20), (12, 70), (28, 50), (40, 64), (64, 37)])
+                                 (64, 20), (12, 70), (28, 50), (40, 64), (64, 37), (28, 48), (9, 33)])
 def test_many_right_hand_sides_small_d_fp64(dev, d, t):
     """More than four right-hand sides at d <= 64 in fp64: the 16-column kernel whose contraction runs on the matrix
     cores (one evaluation of K for 16 columns) and its 32- and 64-column forms (two / four groups of 16, the last one partly
