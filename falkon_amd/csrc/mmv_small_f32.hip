@@ -17,39 +17,26 @@ int FLK_CAT(launch_mmv_small_f32_fold_kf, FLK_KF)(const PackedView &A, const Pac
 
 // Columns per pass of the per-lane FMA kernels (must match the instantiations in launch_tt); calls with more
 // right-hand sides than that go to the kernel whose contraction runs on the matrix cores (mmv_small_f32_wide.hip:
-// 8, 16, 32 or 64 columns per pass; four resident blocks per wave up to 16 padded features, two beyond).  Measured,
+// 8 to 64 columns per pass in steps of 8; wide_form_cols, wide_blocks_per_wave in mmv_small_f32_kernel.h).  Measured,
 // dfmmv at N = 5e5, M = 2e4, FMA kernel against the 8-column form (which costs the same for 3 to 8 columns):
 // d = 9: 4 columns 6.2 ms against 6.6, 5 columns 7.0 against 6.7, 8 columns 8.1 against 6.8; d = 16: 8.2 / 8.9 / 9.9 against
 // 8.7 / 8.8 / 8.9; d = 28: 5 and 6 columns 12.4 against 12.8, 8 columns 13.4 against 12.8; d = 40 (two resident blocks):
 // 4 columns 15.5 against 17.0, 5 to 8 columns on the 16-column form 18.4 against 16.9.
 static inline int fma_cols(int64_t dpad) { return dpad / 2 > 8 && dpad / 2 <= 16 ? 6 : 4; }
-constexpr int kWideColumns = 32;       // one group of columns of the wide kernel
-constexpr int kWideMaxDpFr4 = 8;
-// The wide kernel takes two groups (64 columns) on one evaluation of K unless the few columns beyond 32 are cheaper as a
-// pass of the FMA kernel behind a 32-column pass.  Measured, dfmmv at N = 1e6, M = 2e4: 64-column kernel (any 33 to
-// 64 columns) d = 9 / 16 / 28 / 40 / 64: 47.2 / 51.5 / 59.1 / 67.3 / 84.3 ms; 32-column pass 27.1 / 31.3 / 39.4 / 46.3 /
-// 60.8; one-column pass 8.7 / 12.3 / 19.2 / 29.9 / 46.8, 16 columns at d = 9 21.7.
-static inline int cheap_extra_cols(int64_t dpad) {
-    const int64_t dp = dpad / 2;
-    return dp <= 5 ? 12 : dp <= 8 ? 8 : dp <= 12 ? 3 : 0;
-}
-static inline bool two_groups(int64_t dpad, int64_t t) { return t > kWideColumns + cheap_extra_cols(dpad); }
+constexpr int kWideMaxColumns = 64;    // per pass of the wide kernel
 
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<float>() { return 2 * kMaxDpFr2; }
 template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad, int64_t t) {
-    if (two_groups(dpad, t)) return kWavesPerWg * 2;
-    if (t > fma_cols(dpad)) return kWavesPerWg * ((dpad / 2) <= kWideMaxDpFr4 ? 4 : 2);
+    if (t > fma_cols(dpad))
+        return kWavesPerWg * wide_blocks_per_wave((int)(dpad / 2), wide_form_cols((int)(t < kWideMaxColumns ? t : kWideMaxColumns)));
     return kWavesPerWg * ((dpad / 2) <= kMaxDpFr4 ? 4 : 2);
 }
 template <> int mmv_small_max_cols<float>(int64_t dpad, int64_t t) {
-    if (two_groups(dpad, t)) return 2 * kWideColumns;
-    return t > fma_cols(dpad) ? kWideColumns : fma_cols(dpad);
+    return t > fma_cols(dpad) ? kWideMaxColumns : fma_cols(dpad);
 }
 template <> int mmv_small_width<float>(int64_t dpad, int tc) {
-    if (tc > kWideColumns) return 2 * kWideColumns;
-    if (tc > fma_cols(dpad))      // the wide kernel's 32-, 16- and 8-column forms
-        return tc > kWideColumns / 2 ? kWideColumns : tc > kWideColumns / 4 ? kWideColumns / 2 : kWideColumns / 4;
+    if (tc > fma_cols(dpad)) return wide_form_cols(tc);
     static const int widths[] = {1, 2, 3, 4, 6};
     for (int w : widths) if (tc <= w) return w;
     return tc;

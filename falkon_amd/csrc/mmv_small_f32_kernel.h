@@ -25,6 +25,16 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWavesPerWg = 4;
+
+// Forms of the kernel that contracts on the matrix cores (mmv_small_f32_wide.hip): columns per pass that serve tcols
+// right-hand sides, and resident blocks per wave of a form: four up to 16 padded features where a block has 16 output
+// accumulators or fewer (8, 16 and 32 columns), two otherwise (registers)
+constexpr int wide_form_cols(int tcols) {
+    return tcols <= 8 ? 8 : tcols <= 16 ? 16 : tcols <= 24 ? 24 : tcols <= 32 ? 32 : tcols <= 40 ? 40 : tcols <= 48 ? 48 : 64;
+}
+constexpr int wide_blocks_per_wave(int dp, int cols) {
+    return dp <= 8 && (cols == 8 || cols == 16 || cols == 32) ? 4 : 2;
+}
 constexpr int kFlushEvery = 16;  // A blocks between flushes of the short accumulator
 
 // Per-row quantities of an A block (half norms and right-hand side entries) reach the lanes through

@@ -425,12 +425,12 @@ def test_host_rows_streamed_in_chunks(dev, monkeypatch, order, pinned):
 
 @pytest.mark.parametrize("d,t", [(3, 17), (3, 40), (9, 32), (15, 13), (16, 33), (17, 9), (28, 10), (28, 32), (31, 9),
                                  (33, 5), (40, 12), (63, 7), (64, 33), (9, 50), (28, 47), (40, 37), (64, 100), (31, 64),
-                                 (3, 9), (9, 16), (64, 16), (9, 44)])
+                                 (3, 9), (9, 16), (64, 16), (9, 44), (28, 20), (64, 24), (16, 39), (40, 48), (57, 41)])
 def test_many_right_hand_sides_small_d(dev, d, t):
     """More right-hand sides than the per-lane FMA kernels take in one pass: the register-resident kernel whose
-    contraction runs on the matrix cores, in its 16-column form (9 to 16 columns, from 5 on beyond 32 features; also as
-    the remainder pass behind a 32-column one) and its 32-column form, folded and plain operands, four and two
-    resident blocks per wave, a second pass for the columns beyond 32; its 64-column form (two groups of 32 on one evaluation of K) with a second group
+    contraction runs on the matrix cores, in every form (8 to 64 columns per pass: groups of 32 columns on the
+    32x32x2 step, a group of 16 on the four-block 16x16x1 step, a group of 8 on two 16-block 4x4x1 steps, and their
+    combinations), folded and plain operands, four and two resident blocks per wave, a second pass beyond 64 columns; its 64-column form (two groups of 32 on one evaluation of K) with a second group
     that is partly filled, two and one resident blocks per wave, and a remainder pass after a full one."""
     n, m = 900 + d, 260 + t
     X, C, v, w = _rand(n, d, m, t, torch.float32, seed=d * 100 + t)
