@@ -589,8 +589,10 @@ int FLK_CAT(launch_mmv_large_kf, FLK_KF)(const PackedView &A, const PackedView &
                 return launch_large_tt<T, 64, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
             return launch_large_tt<T, 32, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
         } else {
-            if (tcols > 2 * kLargeMaxCols)
+            if (tcols > 3 * kLargeMaxCols)
                 return launch_large_tt<T, 64, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+            if (tcols > 2 * kLargeMaxCols)       // 33 to 48 columns: three groups of 16
+                return launch_large_tt<T, 48, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
             return launch_large_tt<T, 32, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
         }
     }
