@@ -176,9 +176,9 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
 // that many planes of the planar right-hand side, so the planes past the caller's columns must be zero.
 template <typename T>
 static int instantiated_cols(const Plan &p, int tc) {
-    static const int large[] = {1, 2, 4, 8, 16, 32, 48, 64};     // 8 and 48 columns: instantiations of fp64 only
+    static const int large[] = {1, 2, 4, 8, 16, 32, 48, 64};     // 8 columns: an instantiation of fp64 only
     if (p.large) {
-        for (int w : large) if (tc <= w && ((w != 8 && w != 48) || sizeof(T) == 8)) return w;
+        for (int w : large) if (tc <= w && (w != 8 || sizeof(T) == 8)) return w;
         return tc;
     }
     return mmv_small_width<T>(p.dpad, tc);

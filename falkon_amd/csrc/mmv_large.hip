@@ -96,8 +96,10 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     // More columns than one step holds: NC groups of columns ride on the same kernel values (one more contraction
     // per group, NC times the output accumulators).
     constexpr int kGroupCols = (sizeof(T) == 4 && TT > 16) ? 32 : 16;
-    constexpr int NC = (kMfmaEpi && TT > kGroupCols) ? TT / kGroupCols : 1;
-    constexpr int kEpiCols = kGroupCols * NC;
+    // fp32 with 48 columns: a group of 32 and, as the second group, 16 columns on the four-block 16x16x1 step
+    constexpr bool kTail16 = kMfmaEpi && sizeof(T) == 4 && TT == 48;
+    constexpr int NC = kTail16 ? 2 : (kMfmaEpi && TT > kGroupCols) ? TT / kGroupCols : 1;
+    constexpr int kEpiCols = kTail16 ? 48 : kGroupCols * NC;
     // fp32 with up to 16 columns: the four-block 16x16x1 step contracts them in half the cycles of a 32x32x2 step that
     // would leave half of its columns unused (see the epilogue)
     constexpr bool kHalf16 = kMfmaEpi && sizeof(T) == 4 && kGroupCols == 16;
@@ -384,10 +386,12 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
             // compile-time constant further on
             const int lane_idx = G::A_ROWS + tl + ((wa * WA_FR) * TR::BLK + TR::acc_row(0, lg)) * kVecStride;
             // one read ahead, fenced like the feature loop (otherwise all reads are hoisted and spilled)
+            // (the 16-column group behind a group of 32: its lanes 16 .. 31 read the columns of lanes 0 .. 15)
+            const int tail_adj = kTail16 ? (j & 16) : 0;
             T bval[NC], bnext[NC];
 #pragma unroll
             for (int g = 0; g < NC; g++) {
-                bval[g] = ldsRow[lane_idx + g * kGroupCols];
+                bval[g] = ldsRow[lane_idx + g * kGroupCols - (kTail16 && g == 1 ? tail_adj : 0)];
                 bnext[g] = T(0);
             }
 #pragma unroll
@@ -409,14 +413,18 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                                                        : (p + 1) * TR::BLK;
 #pragma unroll
                     for (int g = 0; g < NC; g++)
-                        if (more) bnext[g] = lane_row[step * kVecStride + g * kGroupCols];
+                        if (more) bnext[g] = lane_row[step * kVecStride + g * kGroupCols - (kTail16 && g == 1 ? tail_adj : 0)];
 #pragma unroll
                     for (int g = 0; g < NC; g++)
 #pragma unroll
                         for (int q = 0; q < WB_FR; q++) {
-                            if constexpr (kHalf16)
-                                out2[q][g] = __builtin_amdgcn_mfma_f32_16x16x1f32(acc[p][q][s2], bval[g], out2[q][g], 0, 0, 0);
-                            else out2[q][g] = TR::mfma(acc[p][q][s2], bval[g], out2[q][g]);
+                            if constexpr (kHalf16 || kTail16) {
+                                if (kHalf16 || g == 1)
+                                    out2[q][g] = __builtin_amdgcn_mfma_f32_16x16x1f32(acc[p][q][s2], bval[g], out2[q][g], 0, 0, 0);
+                                else out2[q][g] = TR::mfma(acc[p][q][s2], bval[g], out2[q][g]);
+                            } else {
+                                out2[q][g] = TR::mfma(acc[p][q][s2], bval[g], out2[q][g]);
+                            }
                         }
 #pragma unroll
                     for (int g = 0; g < NC; g++) {
@@ -430,27 +438,31 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 
     if constexpr (kStore) {
         // nothing left to write
-    } else if constexpr (kHalf16) {
-        const int tl = lane & 15, mq = lane >> 4;
-        if (tl < tcols) {
+    } else if constexpr (kMfmaEpi) {
+        if constexpr (kHalf16 || kTail16) {
+            // the group on the 16x16x1 step: registers 4 b + r and 4 (b + 2) + r together are output row
+            // 16 b + 4 (lane / 16) + r of column lane % 16 (behind the 32 columns of the first group, if there is one)
+            constexpr int g16 = kTail16 ? 1 : 0;
+            const int col = (kTail16 ? kGroupCols : 0) + (lane & 15), mq = lane >> 4;
+            if (col < tcols) {
 #pragma unroll
-            for (int q = 0; q < WB_FR; q++) {
-                const int64_t bb = bblk0 + wb * WB_FR + q;
-                if (bb < nb_blocks) {
+                for (int q = 0; q < WB_FR; q++) {
+                    const int64_t bb = bblk0 + wb * WB_FR + q;
+                    if (bb < nb_blocks) {
 #pragma unroll
-                    for (int b = 0; b < 2; b++)
+                        for (int b = 0; b < 2; b++)
 #pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            partial[(((int64_t)by * kLWavesA + wa) * tcols + tl) * nb_pad + bb * TR::BLK + 16 * b + 4 * mq + r] =
-                                out2[q][0][4 * b + r] + out2[q][0][4 * (b + 2) + r];
+                            for (int r = 0; r < 4; r++)
+                                partial[(((int64_t)by * kLWavesA + wa) * tcols + col) * nb_pad + bb * TR::BLK + 16 * b + 4 * mq + r] =
+                                    out2[q][g16][4 * b + r] + out2[q][g16][4 * (b + 2) + r];
+                    }
                 }
             }
         }
-    } else if constexpr (kMfmaEpi) {
         // lane = column t (both lane groups hold different output rows): no cross-lane step
         const int tl = j & (kGroupCols - 1);
 #pragma unroll
-        for (int g = 0; g < NC; g++) {
+        for (int g = 0; g < (kHalf16 ? 0 : kTail16 ? 1 : NC); g++) {
             const int col = tl + g * kGroupCols;
             if (j < kGroupCols && col < tcols) {
 #pragma unroll
@@ -585,8 +597,10 @@ int FLK_CAT(launch_mmv_large_kf, FLK_KF)(const PackedView &A, const PackedView &
     if (tcols < 1 || tcols > most) return fail(FLK_EINVAL, "mmv_large: column chunk %d not in 1..%d", tcols, most);
     if (tcols > kLargeMaxCols) {
         if constexpr (sizeof(T) == 4) {
-            if (tcols > 2 * kLargeMaxCols)
+            if (tcols > 3 * kLargeMaxCols)
                 return launch_large_tt<T, 64, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+            if (tcols > 2 * kLargeMaxCols)       // 33 to 48 columns: a group of 32 and a group of 16
+                return launch_large_tt<T, 48, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
             return launch_large_tt<T, 32, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
         } else {
             if (tcols > 3 * kLargeMaxCols)
