@@ -19,7 +19,7 @@ OBJ_DIR = os.path.join(_HERE, "build")
 # (Gaussian, Laplacian, Matern 3/2, Matern 5/2, the Laplacian's derivative weight).
 KERNEL_FNS = (0, 1, 2, 3, 4)
 PER_KERNEL_FN = ["mmv_small_f32.hip", "mmv_small_f32_fold.hip", "mmv_small_f32_wide.hip", "mmv_small_f64.hip", "mmv_small_f64_wide.hip", "mmv_large.hip", "fmm.hip",
-                 "mmv_split.hip", "mmv_split_large.hip"]
+                 "mmv_split.hip", "mmv_split_wide.hip", "mmv_split_large.hip"]
 SOURCES = [("api.hip", None), ("pack.hip", None), ("pack_split.hip", None), ("cg.hip", None)] + [(src, kf) for kf in KERNEL_FNS for src in PER_KERNEL_FN]
 
 HIPCC_FLAGS = [

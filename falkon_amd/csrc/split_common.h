@@ -23,6 +23,15 @@ constexpr int kSplitMaxCols = 4;            // its right-hand sides per pass
 
 inline int64_t split_ksteps(int64_t d) { return (d + 2 + 15) / 16; }
 
+// The register-resident kernel for many right-hand sides (mmv_split_wide.hip): up to two k-steps, passes of 8 to 64
+// columns (the forms of mmv_wide_common.h), two resident blocks per wave
+constexpr int64_t kSplitWideMaxD = 30;
+constexpr int kSplitWideMaxCols = 64;
+constexpr int kSplitWideBlocksPerWave = 2;
+constexpr int split_wide_form_cols(int tcols) {
+    return tcols <= 8 ? 8 : tcols <= 16 ? 16 : tcols <= 24 ? 24 : tcols <= 32 ? 32 : tcols <= 40 ? 40 : tcols <= 48 ? 48 : 64;
+}
+
 struct SplitView {
     const void *data;    // [nblk][ks][3][64] x 16 bytes
     const float *hnorm;  // [npad] half norms in fp32 (the kernels use the split copy inside data; this one tells
@@ -60,6 +69,8 @@ int split_large_max_cols();
 #define FLK_DECLARE_SPLIT_KF(KF)                                                                              \
     int launch_mmv_split_kf##KF(const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld,    \
                                 int tcols, int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st); \
+    int launch_mmv_split_wide_kf##KF(const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld, \
+                                     int tcols, int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st); \
     int launch_mmv_split_large_kf##KF(const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld, \
                                       int tcols, int64_t a_tiles_per_chunk, int splits, float *partial,        \
                                       hipStream_t st);                                                         \
@@ -74,6 +85,13 @@ FLK_DECLARE_SPLIT_KF(4)
 inline int launch_mmv_split(int kf, const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld, int tcols,
                             int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
 #define FLK_CALL(KF) launch_mmv_split_kf##KF(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)
+    FLK_SWITCH_KF(kf, FLK_CALL)
+#undef FLK_CALL
+}
+
+inline int launch_mmv_split_wide(int kf, const SplitView &A, const SplitView &B, const float *vecp, int64_t vec_ld,
+                                 int tcols, int64_t a_chunk_blocks, int splits, float *partial, hipStream_t st) {
+#define FLK_CALL(KF) launch_mmv_split_wide_kf##KF(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st)
     FLK_SWITCH_KF(kf, FLK_CALL)
 #undef FLK_CALL
 }

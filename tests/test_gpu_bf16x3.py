@@ -39,6 +39,28 @@ def test_products_vs_oracle(dev, d, t):
                  mmv_ref.fdmmv_ref(Xd, Cd, vd, None, sigma), 1e-5)
 
 
+@pytest.mark.parametrize("d", [9, 14, 28, 30])
+@pytest.mark.parametrize("t", [7, 16, 17, 24, 33, 48, 64, 70])
+def test_many_right_hand_sides_on_the_register_resident_kernel(dev, d, t):
+    """Five and more right-hand sides at up to 30 features: the bf16x3 chain for the cross term, the contraction of
+    8 to 64 columns per pass on the fp32 matrix-core steps (every form, a second pass beyond 64 columns); repeatable
+    bit for bit, Fortran-ordered operands included."""
+    n, m = 650 + 5 * d, 300 + t
+    X, C, v, w = _data(n, m, d, t, seed=3 * d + 7 * t)
+    sigma = torch.tensor([0.9 * np.sqrt(d)], dtype=torch.float64)
+    k = GaussianKernel(sigma, opt=SPLIT)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+    check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)
+    got = k.dmmv(Xg, Cg, vg, wg)
+    check_parity(got, mmv_ref.fdmmv_ref(X, C, v, w, sigma), mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), 1e-5)
+    f = lambda a: a.T.contiguous().T                                                      # noqa: E731
+    assert torch.equal(k.dmmv(f(Xg), f(Cg), f(vg), f(wg)), got)
+    # the same numbers as the fp32 kernels give, to rounding
+    plain = GaussianKernel(sigma).dmmv(Xg, Cg, vg, wg)
+    assert rel_err(got, plain) < 5e-6
+
+
 def test_layouts_sigma_per_dimension_and_repeatability(dev):
     X, C, v, w = _data(1500, 333, 11, 2, seed=7)
     sigma = torch.from_numpy(np.random.default_rng(3).uniform(1.0, 4.0, 11))
