@@ -35,7 +35,7 @@ def split_roofline(pairs, d, kern_ms, algorithmic_flop, traffic=None, pairs_cols
     return {"bound": "mfma", "achieved": achieved, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": achieved / BF16_PEAK_TFLOPS, "traffic": traffic,
             "kernel": ("mmv_split_kernel" if d <= 62 and pairs_cols <= 4 else
-                       "mmv_split_wide_kernel" if d <= 30 else "mmv_split_large_kernel"),
+                       "mmv_split_wide_kernel" if d <= 62 else "mmv_split_large_kernel"),
             "avg_launch_ms": kern_ms, "flop_per_launch": executed,
             "note": "achieved = bf16 MFMA flops the kernel executes (6 partial products, padded features); "
                     "algorithmic fp32 flops per launch and their rate are given beside it",
@@ -86,11 +86,7 @@ def product_kernel_name(d, T, dtype):
 def split_kernels_serve(d, T):
     """Whether the bf16x3 kernels serve a call of the bf16x3 mode with d features and T right-hand sides, or the fp32
     kernels do (split_applies in csrc/api.hip)."""
-    if d > 62 or T <= 4:
-        return True
-    if d <= 30:
-        return d > 8 or T <= 16
-    return (T <= 16 and d > 32) or (8 < T <= 16 and d > 24)
+    return d > 62 or T <= 4 or d > 8 or T <= 16
 
 
 def make_inputs(name, rhs=0):

@@ -441,27 +441,26 @@ constexpr int64_t kTargetWgsSplitLarge = 8192;  // one 512-thread workgroup per 
 // kernel for 5 to 8 columns: 17.8 / 22.2 / 23.2).  17 and more: the fp32 kernels contract 32 or 64 columns per pass.  So:
 // every feature count beyond the register-resident kernels; at small feature counts 1 to 4 right-hand sides, 5 to 16
 // beyond 32 features and 9 to 16 from 25 features on; otherwise the fp32 MFMA kernels serve the mode.
-// Up to kSplitWideMaxD features the register-resident bf16x3 kernel for many right-hand sides (mmv_split_wide.hip)
-// serves the column counts beyond four.  N = 5e5, M = 2e4, 8 / 16 / 32 / 64 columns against the fp32 kernels: d = 28
-// 8.3 / 10.4 / 14.7 / 25.3 ms against 12.4 / 15.1 / 19.9 / 29.4; d = 9 5.8 / 7.9 / 12.6 / 23.0 against 6.9 / 9.0 / 13.8 / 23.9;
-// d = 4 5.6 / 7.7 / 12.6 / 23.0 against 5.7 / 7.8 / 12.4 / 22.1 (the fp32 kernels keep four resident blocks per wave there):
-// below 9 features up to 16 columns only.
+// The register-resident bf16x3 kernel for many right-hand sides (mmv_split_wide.hip) serves the column counts beyond
+// four at every feature count of the register-resident kernels.  N = 5e5, M = 2e4, 8 / 16 / 32 / 64 columns against the fp32
+// kernels: d = 28 8.3 / 10.4 / 14.7 / 25.3 ms against 12.4 / 15.1 / 19.9 / 29.4; d = 56 13.5 / 15.7 / 19.7 / 30.2 against 21.7 /
+// 23.5 / 28.3 / 38.0 (and 17.9 for up to 16 columns on the LDS-tiled bf16x3 kernel); d = 9 5.8 / 7.9 / 12.6 / 23.0 against
+// 6.9 / 9.0 / 13.8 / 23.9; d = 4 5.6 / 7.7 / 12.6 / 23.0 against 5.7 / 7.8 / 12.4 / 22.1 (the fp32 kernels keep four resident blocks
+// per wave there): below 9 features up to 16 columns only, the fp32 kernels beyond.
 static bool split_applies(int64_t d, int64_t t) {
     if (d > kSplitMaxD || t <= kSplitMaxCols) return true;
-    if (d <= kSplitWideMaxD) return d > 8 || t <= 16;
-    return (t <= 16 && d > 32) || (t > 8 && t <= 16 && d > 24);
+    return d > 8 || t <= 16;
 }
 
 static Plan make_plan_split(int64_t na_blocks, int64_t nb_blocks, int64_t ks, int64_t t) {
     Plan p;
-    // up to four right-hand sides the register-resident kernel; beyond that (see split_applies) the LDS-tiled kernel,
-    // whose epilogue contracts sixteen columns per pass on the matrix cores, also for small feature counts
+    // up to four right-hand sides the register-resident kernel with per-lane FMAs
     if (ks * 16 <= kSplitMaxD + 2 && t <= kSplitMaxCols) {
         plan_register_resident(p, na_blocks, nb_blocks, split_b_blocks_per_wg(ks, t), ks * 3 * 64 * 16, 32, kSplitMaxCols,
                                t, (int64_t)sizeof(float));
         return p;
     }
-    // more right-hand sides at up to two k-steps: the register-resident kernel that contracts on the matrix cores
+    // more right-hand sides: the register-resident kernel that contracts on the matrix cores
     if (ks * 16 <= kSplitWideMaxD + 2) {
         plan_register_resident(p, na_blocks, nb_blocks, 4 * kSplitWideBlocksPerWave, ks * 3 * 64 * 16, 32,
                                kSplitWideMaxCols, t, (int64_t)sizeof(float));

@@ -1,5 +1,5 @@
 // Register-resident kernel-vector product of the bf16x3 mode for many right-hand sides (5 to 64 per pass), fp32 data,
-// up to 30 features (two k-steps), gfx950.  Compiled once per kernel function (-DFLK_KF=0..4).
+// up to 62 features (four k-steps), gfx950.  Compiled once per kernel function (-DFLK_KF=0..4).
 //
 //   partial[split][t][b] = sum_{a in chunk(split)} K(A_a, B_b) * vec[a,t]
 //
@@ -158,7 +158,7 @@ static int launch_split_wide_ks(const SplitView &A, const SplitView &B, const fl
     case COLSV:                                                                                                     \
         return launch_split_wide_one<KS, kSplitWideBlocksPerWave, COLSV>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, \
                                                                          splits, partial, st);
-    switch (split_wide_form_cols(tcols)) {
+    switch (split_wide_form_cols(tcols, KS)) {
         FLK_SPLIT_WIDE_FORM(8) FLK_SPLIT_WIDE_FORM(16) FLK_SPLIT_WIDE_FORM(24) FLK_SPLIT_WIDE_FORM(32)
         FLK_SPLIT_WIDE_FORM(40) FLK_SPLIT_WIDE_FORM(48) FLK_SPLIT_WIDE_FORM(64)
     }
@@ -175,6 +175,8 @@ int FLK_CAT(launch_mmv_split_wide_kf, FLK_KF)(const SplitView &A, const SplitVie
     switch (A.ks) {
         case 1: return launch_split_wide_ks<1>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
         case 2: return launch_split_wide_ks<2>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+        case 3: return launch_split_wide_ks<3>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
+        case 4: return launch_split_wide_ks<4>(A, B, vecp, vec_ld, tcols, a_chunk_blocks, splits, partial, st);
     }
     return fail(FLK_EUNSUPPORTED, "mmv_split wide: %lld features (more than %lld)", (long long)A.d,
                 (long long)kSplitWideMaxD);

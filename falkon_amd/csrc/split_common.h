@@ -23,13 +23,15 @@ constexpr int kSplitMaxCols = 4;            // its right-hand sides per pass
 
 inline int64_t split_ksteps(int64_t d) { return (d + 2 + 15) / 16; }
 
-// The register-resident kernel for many right-hand sides (mmv_split_wide.hip): up to two k-steps, passes of 8 to 64
-// columns (the forms of mmv_wide_common.h), two resident blocks per wave
-constexpr int64_t kSplitWideMaxD = 30;
+// The register-resident kernel for many right-hand sides (mmv_split_wide.hip): passes of 8 to 64 columns (the forms of
+// mmv_wide_common.h), two resident blocks per wave.  (With four k-steps the forms beyond 16 output accumulators per
+// block spill some registers; the 24-column form is then slower than the 32-column one: d = 56, N = 5e5, M = 2e4,
+// 20.2 ms against 19.7.)
+constexpr int64_t kSplitWideMaxD = kSplitMaxD;
 constexpr int kSplitWideMaxCols = 64;
 constexpr int kSplitWideBlocksPerWave = 2;
-constexpr int split_wide_form_cols(int tcols) {
-    return tcols <= 8 ? 8 : tcols <= 16 ? 16 : tcols <= 24 ? 24 : tcols <= 32 ? 32 : tcols <= 40 ? 40 : tcols <= 48 ? 48 : 64;
+constexpr int split_wide_form_cols(int tcols, int ks) {
+    return tcols <= 8 ? 8 : tcols <= 16 ? 16 : tcols <= 24 && ks < 4 ? 24 : tcols <= 32 ? 32 : tcols <= 40 ? 40 : tcols <= 48 ? 48 : 64;
 }
 
 struct SplitView {
