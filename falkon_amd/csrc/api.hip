@@ -447,8 +447,13 @@ constexpr int64_t kTargetWgsSplitLarge = 8192;  // one 512-thread workgroup per 
 // 23.5 / 28.3 / 38.0 (and 17.9 for up to 16 columns on the LDS-tiled bf16x3 kernel); d = 9 5.8 / 7.9 / 12.6 / 23.0 against
 // 6.9 / 9.0 / 13.8 / 23.9; d = 4 5.6 / 7.7 / 12.6 / 23.0 against 5.7 / 7.8 / 12.4 / 22.1 (the fp32 kernels keep four resident blocks
 // per wave there): below 9 features up to 16 columns only, the fp32 kernels beyond.
+// Beyond the register-resident kernels the LDS-tiled bf16x3 kernel contracts 16 columns per pass and the fp32 one up to 64:
+// one pass always wins (N = 2.5e5, M = 2e4, 16 columns: d = 63 / 100 / 300 10.6 / 13.5 / 30.7 ms against 12.8 / 20.3 / 49.3), two
+// passes only where the cross term dominates (17 columns: 18.6 / 24.5 / 58.5 against 14.7 / 24.0 / 54.3; N = 5e5, M = 1e4,
+// d = 784: 113 against 130, and 32 columns 116 against 129), more never (d = 784, 64 columns: 231 against 138).
 static bool split_applies(int64_t d, int64_t t) {
-    if (d > kSplitMaxD || t <= kSplitMaxCols) return true;
+    if (t <= kSplitMaxCols) return true;
+    if (d > kSplitMaxD) return t <= 16 || (t <= 32 && d >= 512);
     return d > 8 || t <= 16;
 }
 
