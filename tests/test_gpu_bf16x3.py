@@ -40,10 +40,11 @@ def test_products_vs_oracle(dev, d, t):
 
 
 @pytest.mark.parametrize("d", [9, 14, 28, 30, 31, 46, 47, 62])
-@pytest.mark.parametrize("t", [7, 16, 17, 24, 33, 48, 64, 70])
+@pytest.mark.parametrize("t", [7, 16, 17, 24, 33, 48, 64, 66, 70])
 def test_many_right_hand_sides_on_the_register_resident_kernel(dev, d, t):
     """Five and more right-hand sides at up to 62 features (one to four k-steps): the bf16x3 chain for the cross term, the contraction of
-    8 to 64 columns per pass on the fp32 matrix-core steps (every form, a second pass beyond 64 columns); repeatable
+    8 to 64 columns per pass on the fp32 matrix-core steps (every form, a second pass beyond 64 columns, which the
+    per-lane FMA kernel takes when it has four columns or fewer); repeatable
     bit for bit, Fortran-ordered operands included."""
     n, m = 650 + 5 * d, 300 + t
     X, C, v, w = _data(n, m, d, t, seed=3 * d + 7 * t)
