@@ -24,14 +24,16 @@ constexpr int kSplitMaxCols = 4;            // its right-hand sides per pass
 inline int64_t split_ksteps(int64_t d) { return (d + 2 + 15) / 16; }
 
 // The register-resident kernel for many right-hand sides (mmv_split_wide.hip): passes of 8 to 64 columns (the forms of
-// mmv_wide_common.h), two resident blocks per wave.  (With four k-steps the forms beyond 16 output accumulators per
-// block spill some registers; the 24-column form is then slower than the 32-column one: d = 56, N = 5e5, M = 2e4,
-// 20.2 ms against 19.7.)
+// mmv_wide_common.h), two resident blocks per wave.  Passes of 32 and 64 columns contract on the bf16 matrix cores up to
+// three k-steps (with four the 64-column pass is out of registers that way: d = 56, N = 5e5, M = 2e4, 36.4 ms against
+// 30.2 on the fp32 steps), which makes them cheaper than the 24- and, up to two k-steps, the 48-column pass on the fp32
+// steps: d = 28, 24 / 32 columns 14.0 / 13.8 ms, 48 / 64 columns 20.8 / 19.6; d = 40 (three k-steps) 48 / 64: 23.1 / 23.7.
 constexpr int64_t kSplitWideMaxD = kSplitMaxD;
 constexpr int kSplitWideMaxCols = 64;
 constexpr int kSplitWideBlocksPerWave = 2;
+constexpr bool split_wide_bf16_contraction(int cols, int ks) { return (cols == 32 || cols == 64) && ks <= 3; }
 constexpr int split_wide_form_cols(int tcols, int ks) {
-    return tcols <= 8 ? 8 : tcols <= 16 ? 16 : tcols <= 24 && ks < 4 ? 24 : tcols <= 32 ? 32 : tcols <= 40 ? 40 : tcols <= 48 ? 48 : 64;
+    return tcols <= 8 ? 8 : tcols <= 16 ? 16 : tcols <= 32 ? 32 : tcols <= 40 ? 40 : tcols <= 48 && ks >= 3 ? 48 : 64;
 }
 
 struct SplitView {
