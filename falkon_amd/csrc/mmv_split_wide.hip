@@ -57,8 +57,8 @@ __device__ __forceinline__ void split_wide_stage(const SplitWideRowVals<COLS> &r
 
 // ---------------------------------------------------------------------------
 // Contraction on the bf16 matrix cores (passes of 32 and 64 columns).  The kernel values and the right-hand sides are
-// split three ways like the data (x = hi + mid + lo, bfloat16 pieces by truncation: the subtractions are exact and
-// the pieces carry 24 bits together), and K v is accumulated from the same six partial products as the cross term.
+// split three ways like the data (x = hi + mid + lo, bfloat16 pieces, see split3_pair), and K v is accumulated from the
+// same six partial products as the cross term.
 // Register s of a lane holds K[i][j] with i = 8 (s / 4) + 4 h + s % 4: the eight registers 8 c .. 8 c + 7 of a lane are
 // the k values of a 32x32x16 step c for the lane's output row j, so the A operand is those eight values packed; the B
 // operand is vec[the same eight rows][t = lane % 32], which the stage holds as one 16-byte piece per (group, piece,
@@ -68,14 +68,23 @@ template <int COLS> struct SplitWideBf16Geo {
     static constexpr int kGroups = COLS / 32;
     static constexpr int kStageDw = kGroups * 3 * 2 * 2 * 32 * 4;      // dwords: [group][piece][step][half][column][8 bf16]
 };
-__device__ __forceinline__ void trunc_split3(float x, unsigned &hi, unsigned &mid, unsigned &lo) {
-    hi = __float_as_uint(x) & 0xffff0000u;
-    const float r1 = x - __uint_as_float(hi);
-    mid = __float_as_uint(r1) & 0xffff0000u;
-    lo = __float_as_uint(r1 - __uint_as_float(mid)) & 0xffff0000u;
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+// (x, y) = hi + mid + lo, each piece the pair of bfloat16 numbers nearest to what the previous pieces leave (the
+// subtractions are exact), x in the low half of the words: v_cvt_pk_bf16_f32 rounds to nearest even, as the packing of
+// the data does.  (Pieces by truncation would carry the same 24 bits, but the partial products that are dropped are then
+// eight times larger and all of one sign: a column whose terms cancel 200-fold came out at 2.3e-5 instead of 1.6e-6.)
+__device__ __forceinline__ void split3_pair(float x, float y, unsigned (&piece)[3]) {
+    floatx2 r = {x, y};
+#pragma unroll
+    for (int p = 0; p < 3; p++) {
+        piece[p] = __builtin_bit_cast(unsigned, __builtin_convertvector(r, bf16x2));
+        if (p < 2) {
+            r[0] -= __uint_as_float(piece[p] << 16);
+            r[1] -= __uint_as_float(piece[p] & 0xffff0000u);
+        }
+    }
 }
-// the upper halves of two words as one word (a in the low half)
-__device__ __forceinline__ unsigned pack_hi16(unsigned a, unsigned b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
 
 template <int COLS>
 __device__ __forceinline__ void split_wide_stage_bf16(const SplitWideRowVals<COLS> &rv, unsigned short *lds, int tid) {
@@ -83,13 +92,16 @@ __device__ __forceinline__ void split_wide_stage_bf16(const SplitWideRowVals<COL
     // row r = 16 c + 8 e1 + 4 h + e0 is element e = 4 e1 + e0 of step c in lane half h
     const int c = r >> 4, e = 4 * ((r >> 3) & 1) + (r & 3), h = (r >> 2) & 1;
 #pragma unroll
-    for (int cc = 0; cc < COLS / 8; cc++) {
-        const int col = p0 + 8 * cc, g = col >> 5, t = col & 31;
+    for (int cc = 0; cc < COLS / 8; cc += 2) {
         unsigned piece[3];
-        trunc_split3(rv.x[cc], piece[0], piece[1], piece[2]);
+        split3_pair(rv.x[cc], rv.x[cc + 1], piece);
 #pragma unroll
-        for (int p = 0; p < 3; p++)
-            lds[((((g * 3 + p) * 2 + c) * 2 + h) * 32 + t) * 8 + e] = (unsigned short)(piece[p] >> 16);
+        for (int u = 0; u < 2; u++) {
+            const int col = p0 + 8 * (cc + u), g = col >> 5, t = col & 31;
+#pragma unroll
+            for (int p = 0; p < 3; p++)
+                lds[((((g * 3 + p) * 2 + c) * 2 + h) * 32 + t) * 8 + e] = (unsigned short)(u ? piece[p] >> 16 : piece[p] & 0xffffu);
+        }
     }
 }
 
@@ -106,11 +118,10 @@ __device__ __forceinline__ void wide_contract_bf16(const floatx16 (&acc)[FR], co
         for (int q = 0; q < FR; q++) {
 #pragma unroll
             for (int e2 = 0; e2 < 4; e2++) {
-                unsigned x[3], y[3];
-                trunc_split3(acc[q][8 * c + 2 * e2], x[0], x[1], x[2]);
-                trunc_split3(acc[q][8 * c + 2 * e2 + 1], y[0], y[1], y[2]);
+                unsigned piece[3];
+                split3_pair(acc[q][8 * c + 2 * e2], acc[q][8 * c + 2 * e2 + 1], piece);
 #pragma unroll
-                for (int p = 0; p < 3; p++) a[q][p][e2] = pack_hi16(x[p], y[p]);
+                for (int p = 0; p < 3; p++) a[q][p][e2] = piece[p];
             }
         }
 #pragma unroll
