@@ -86,11 +86,13 @@ def product_kernel_name(d, T, dtype):
 def split_kernels_serve(d, T):
     """Whether the bf16x3 kernels serve a call of the bf16x3 mode with d features and T right-hand sides, or the fp32
     kernels do (split_applies in csrc/api.hip)."""
+    if d <= 4:
+        return False
     if T <= 4:
         return True
     if d > 62:
         return T <= 16 or (T <= 32 and d >= 512)
-    return d > 8 or T <= 16
+    return d > 8 or (T <= 16 and d > 5)
 
 
 def make_inputs(name, rhs=0):

@@ -451,10 +451,13 @@ constexpr int64_t kTargetWgsSplitLarge = 8192;  // one 512-thread workgroup per 
 // one pass always wins (N = 2.5e5, M = 2e4, 16 columns: d = 63 / 100 / 300 10.6 / 13.5 / 30.7 ms against 12.8 / 20.3 / 49.3), two
 // passes only where the cross term dominates (17 columns: 18.6 / 24.5 / 58.5 against 14.7 / 24.0 / 54.3; N = 5e5, M = 1e4,
 // d = 784: 113 against 130, and 32 columns 116 against 129), more never (d = 784, 64 columns: 231 against 138).
+// Up to four features the fp32 kernels are the faster ones at every column count (their cross term is one or two MFMA steps;
+// one right-hand side at d = 2 / 4 / 5 / 6: 2.6 / 3.0 / 3.8 / 3.7 ms against 3.4 / 3.5 / 3.5 / 3.6).
 static bool split_applies(int64_t d, int64_t t) {
+    if (d <= 4) return false;
     if (t <= kSplitMaxCols) return true;
     if (d > kSplitMaxD) return t <= 16 || (t <= 32 && d >= 512);
-    return d > 8 || t <= 16;
+    return d > 8 || (t <= 16 && d > 5);
 }
 
 static Plan make_plan_split(int64_t na_blocks, int64_t nb_blocks, int64_t ks, int64_t t) {
