@@ -184,14 +184,14 @@ def test_degenerate_shapes(dev, d):
         assert rel_err(got, mmv_ref.fdmmv_ref(X[:n], C[:m], v[:m], w[:n], k.sigma)) < 1e-5
 
 
-@pytest.mark.parametrize("d", [28, 200])
-def test_dmmv_replays_from_a_hip_graph(dev, d):
+@pytest.mark.parametrize("d,t", [(28, 2), (200, 2), (28, 40), (200, 12)])
+def test_dmmv_replays_from_a_hip_graph(dev, d, t):
     """As for the fp32 kernels: nothing is allocated, cleared with a memset or synchronised, so a call can be captured
-    into a HIP graph; every replay reproduces the eager result bit for bit."""
-    X, C, v, w = _data(20_000, 1_200, d, 2, seed=21)
+    into a HIP graph; every replay reproduces the eager result bit for bit.  With few and with many right-hand sides."""
+    X, C, v, w = _data(20_000, 1_200, d, t, seed=21)
     k = GaussianKernel(0.7 * np.sqrt(d), opt=SPLIT)
     Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
-    out = torch.empty(1_200, 2, device=dev)
+    out = torch.empty(1_200, t, device=dev)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -203,8 +203,8 @@ def test_dmmv_replays_from_a_hip_graph(dev, d):
         k.dmmv(Xg, Cg, vg, wg, out=out)
     g = np.random.default_rng(5)
     for _ in range(3):
-        vg.copy_(torch.from_numpy(g.standard_normal((1_200, 2)).astype(np.float32)))
-        wg.copy_(torch.from_numpy(g.standard_normal((20_000, 2)).astype(np.float32)))
+        vg.copy_(torch.from_numpy(g.standard_normal((1_200, t)).astype(np.float32)))
+        wg.copy_(torch.from_numpy(g.standard_normal((20_000, t)).astype(np.float32)))
         graph.replay()
         torch.cuda.synchronize()
         replayed = out.clone()

@@ -362,14 +362,16 @@ def test_strided_views_and_column_order(dev):
         k.mmv(big[::2, ::2][:, :6], C.to(dev)[:, :6].contiguous(), v.to(dev))
 
 
-def test_dmmv_replays_from_a_hip_graph(dev):
+@pytest.mark.parametrize("t", [2, 20, 70])
+def test_dmmv_replays_from_a_hip_graph(dev, t):
     """The library allocates nothing, clears memory with kernels and never synchronises, so a dmmv call can be
     captured into a HIP graph (e.g. a whole CG iteration).  Every replay, with the program's own eager work and
-    synchronisations in between, must reproduce the eager result bit for bit."""
-    X, C, v, w = _rand(30_000, 28, 1_500, 2, torch.float32, seed=21)
+    synchronisations in between, must reproduce the eager result bit for bit.  Two right-hand sides run on the
+    FMA kernel, 20 on the many-column kernel, 70 in two column chunks."""
+    X, C, v, w = _rand(30_000, 28, 1_500, t, torch.float32, seed=21)
     k = GaussianKernel(3.8)
     Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
-    out = torch.empty(1_500, 2, device=dev)
+    out = torch.empty(1_500, t, device=dev)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -381,8 +383,8 @@ def test_dmmv_replays_from_a_hip_graph(dev):
         k.dmmv(Xg, Cg, vg, wg, out=out)
     g = np.random.default_rng(5)
     for _ in range(4):
-        vg.copy_(torch.from_numpy(g.standard_normal((1_500, 2)).astype(np.float32)))
-        wg.copy_(torch.from_numpy(g.standard_normal((30_000, 2)).astype(np.float32)))
+        vg.copy_(torch.from_numpy(g.standard_normal((1_500, t)).astype(np.float32)))
+        wg.copy_(torch.from_numpy(g.standard_normal((30_000, t)).astype(np.float32)))
         graph.replay()
         torch.cuda.synchronize()
         replayed = out.clone()
