@@ -20,7 +20,11 @@ OBJ_DIR = os.path.join(_HERE, "build")
 KERNEL_FNS = (0, 1, 2, 3, 4)
 PER_KERNEL_FN = ["mmv_small_f32.hip", "mmv_small_f32_fold.hip", "mmv_small_f32_wide.hip", "mmv_small_f64.hip", "mmv_small_f64_wide.hip", "mmv_large.hip", "fmm.hip",
                  "mmv_split.hip", "mmv_split_wide.hip", "mmv_split_large.hip"]
-SOURCES = [("api.hip", None), ("pack.hip", None), ("pack_split.hip", None), ("cg.hip", None)] + [(src, kf) for kf in KERNEL_FNS for src in PER_KERNEL_FN]
+# Longest compiles first (the many-column fp32 kernel takes as long as all the other sources of its kernel function
+# together), so that the parallel build does not end on one of them running alone.
+SOURCES = [(src, kf) for src in PER_KERNEL_FN for kf in KERNEL_FNS]
+SOURCES.sort(key=lambda job: {"mmv_small_f32_wide.hip": 0, "mmv_small_f32.hip": 1, "mmv_small_f32_fold.hip": 2}.get(job[0], 3))
+SOURCES += [("api.hip", None), ("pack.hip", None), ("pack_split.hip", None), ("cg.hip", None)]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
