@@ -91,7 +91,7 @@ def split_kernels_serve(d, T):
     if T <= 4:
         return True
     if d > 62:
-        return T <= 16 or (T <= 32 and d >= 512)
+        return True
     return d > 8 or (T <= 16 and d > 5)
 
 

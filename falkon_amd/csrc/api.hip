@@ -447,16 +447,17 @@ constexpr int64_t kTargetWgsSplitLarge = 8192;  // one 512-thread workgroup per 
 // 23.5 / 28.3 / 38.0 (and 17.9 for up to 16 columns on the LDS-tiled bf16x3 kernel); d = 9 5.8 / 7.9 / 12.6 / 23.0 against
 // 6.9 / 9.0 / 13.8 / 23.9; d = 4 5.6 / 7.7 / 12.6 / 23.0 against 5.7 / 7.8 / 12.4 / 22.1 (the fp32 kernels keep four resident blocks
 // per wave there): below 9 features up to 16 columns only, the fp32 kernels beyond.
-// Beyond the register-resident kernels the LDS-tiled bf16x3 kernel contracts 16 columns per pass and the fp32 one up to 64:
-// one pass always wins (N = 2.5e5, M = 2e4, 16 columns: d = 63 / 100 / 300 10.6 / 13.5 / 30.7 ms against 12.8 / 20.3 / 49.3), two
-// passes only where the cross term dominates (17 columns: 18.6 / 24.5 / 58.5 against 14.7 / 24.0 / 54.3; N = 5e5, M = 1e4,
-// d = 784: 113 against 130, and 32 columns 116 against 129), more never (d = 784, 64 columns: 231 against 138).
+// Beyond the register-resident kernels the LDS-tiled bf16x3 kernel contracts 16, 32 or 64 columns per pass, as the fp32
+// one does, and its cross term is the shorter one at every column count (N = 2.5e5, M = 2e4, 16 / 32 / 64 columns: d = 63
+// 10.8 / 13.5 / 19.1 ms against 12.8 / 15.2 / 21.3, d = 100 13.6 / 16.3 / 21.5 against 20.3 / 24.4 / 32.2, d = 300 30.6 / 34.2 /
+// 39.6 against 49.2 / 54.5 / 62.8; N = 5e5, M = 1e4, d = 784: 73.1 / 82.2 / 87.1 against 120.3 / 129.3 / 138.3; the one
+// exception found, 33 to 40 columns just beyond 62 features, is 18.3 against 17.5).
 // Up to four features the fp32 kernels are the faster ones at every column count (their cross term is one or two MFMA steps;
 // one right-hand side at d = 2 / 4 / 5 / 6: 2.6 / 3.0 / 3.8 / 3.7 ms against 3.4 / 3.5 / 3.5 / 3.6).
 static bool split_applies(int64_t d, int64_t t) {
     if (d <= 4) return false;
     if (t <= kSplitMaxCols) return true;
-    if (d > kSplitMaxD) return t <= 16 || (t <= 32 && d >= 512);
+    if (d > kSplitMaxD) return true;
     return d > 8 || (t <= 16 && d > 5);
 }
 

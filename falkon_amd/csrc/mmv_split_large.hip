@@ -1,6 +1,6 @@
 // LDS-tiled kernel-vector product of the bf16x3 mode (see split_common.h), fp32 data, gfx950: feature counts beyond
-// the register-resident kernel, and more than four right-hand sides at any feature count (its epilogue contracts
-// sixteen columns per pass on the matrix cores).  Compiled once per kernel function (-DFLK_KF=0..4).
+// the register-resident kernels (its epilogue contracts up to 64 columns per pass on the matrix cores).
+// Compiled once per kernel function (-DFLK_KF=0..4).
 //
 //   partial[split'][t][b] = sum_{a in chunk} K(A_a, B_b) * vec[a,t]
 //
@@ -11,7 +11,9 @@
 // accumulators and issues the six partial products of each pair with v_mfma_f32_32x32x16_bf16.  The half norms
 // ride in the last two features (the B side swaps the pair when it reads its operands), so after the last k-step
 // the accumulators hold the exponent.  Epilogue as in the fp32 LDS-tiled kernel: per-lane FMAs for up to four
-// right-hand sides, a second small fp32 MFMA contraction (accumulator registers as the A operand) beyond that.
+// right-hand sides, a second small fp32 MFMA contraction (accumulator registers as the A operand) beyond that: 16
+// columns per pass with the 16x16x1 step, 32 or 64 with one or two groups of 32x32x2 steps.  The right-hand sides of
+// the tile then take the room of the third operand stage (two stages, filled one k-step ahead).
 #include "kernel_fn.h"
 #include "mfma_traits.h"
 #include "split_common.h"
@@ -56,9 +58,12 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     // a stage is copied in units of one piece of one block (64 lanes x 16 bytes = one direct-to-LDS load of a wave)
     constexpr int kUnits = (NAB + NBB) * 3, kUnitsPerWave = kUnits / kWaves;
     static_assert(kUnits % kWaves == 0, "the units of a stage must split evenly over the waves");
-    constexpr int kStages = 3;     // k-steps in LDS: one in use, the others in flight
+    // k-steps in LDS: one in use, the others in flight.  Passes of 32 and 64 columns give the third stage's room to
+    // the right-hand sides of the tile (64 columns: 2 x 48 KB of operands + 64 KB, all of the CU's LDS).
     constexpr bool kMfmaEpi = TT > 4;
-    constexpr int kVecStride = 16;
+    constexpr int kGroups32 = TT / 32;                            // groups of 32 columns (32x32x2 steps)
+    constexpr int kStages = kGroups32 ? 2 : 3;
+    constexpr int kVecStride = kGroups32 ? TT : 16;
     constexpr int kRowBuf = kMfmaEpi ? A_ROWS * kVecStride : TT * A_ROWS;
     __shared__ __attribute__((aligned(16))) uintx4 ldsA[kStages][A_VECS];
     __shared__ __attribute__((aligned(16))) uintx4 ldsB[kStages][B_VECS];
@@ -84,15 +89,20 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     if (at1 > a_tiles) at1 = a_tiles;
 
     float out[WB_FR][kMfmaEpi ? 1 : TT];          // per-lane FMA path: out[q][t] for this lane's output row
-    floatx16 out2[kMfmaEpi ? WB_FR : 1];          // MFMA path: lane = column t, registers = output rows
+    constexpr int kOut2 = kMfmaEpi ? WB_FR * (kGroups32 ? kGroups32 : 1) : 1;
+    floatx16 out2[kOut2];                         // MFMA path: lane = column t, registers = output rows; [q][group]
 #pragma unroll
     for (int q = 0; q < WB_FR; q++)
 #pragma unroll
         for (int t = 0; t < (kMfmaEpi ? 1 : TT); t++) out[q][t] = 0.f;
 #pragma unroll
-    for (int q = 0; q < (kMfmaEpi ? WB_FR : 1); q++)
+    for (int q = 0; q < kOut2; q++)
 #pragma unroll
         for (int r = 0; r < 16; r++) out2[q][r] = 0.f;
+    // Slot of (row r of the tile, column c) in ldsRow.  With 32 or 64 columns the column index is swizzled with the row
+    // so that neither the writers (consecutive rows of one column) nor the readers (32 consecutive columns of one
+    // row) meet in one bank.
+    auto vec_slot = [](int r, int c) { return r * kVecStride + (kGroups32 ? (c ^ (r & (kVecStride - 1))) : c); };
 
     // The stages are filled by direct global-to-LDS loads (global_load_lds_dwordx4: lane l of the issuing wave
     // writes its 16 bytes at the wave-uniform LDS address + 16 l, which is the packed order), three k-steps deep,
@@ -146,26 +156,38 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         // the tile's right-hand side values: loaded, then written to ldsRow once every wave has left the previous
         // tile's epilogue (the loads complete behind the two stages already in flight, so nothing is outstanding
         // when the k-steps start)
-        constexpr int kRowVals = (kMfmaEpi ? 16 : TT) * A_ROWS;
+        constexpr int kRowVals = (kMfmaEpi ? kVecStride : TT) * A_ROWS;
         constexpr int kRowValsPerThread = (kRowVals + kThreads - 1) / kThreads;
+        // value c of a thread: column tid / A_ROWS + c * kColStep of row tid % A_ROWS; the column step is the same for
+        // every thread, so that the addresses differ by multiples of a wave-uniform stride (worked out per thread
+        // they are 2 x kRowValsPerThread registers that the compiler keeps across the tile loop)
+        static_assert(kThreads % A_ROWS == 0, "a thread's values must lie in one row of the tile");
+        constexpr int kColStep = kThreads / A_ROWS;
         float rowv[kRowValsPerThread];
+        {
+            const int col0 = tid / A_ROWS;
+            const int64_t row = ablk0 * 32 + tid % A_ROWS;
+            const bool row_ok = row < na_blocks * 32;     // rows past n_a carry zero weight
+            const float *src = vecp + (int64_t)col0 * vec_ld + row;
 #pragma unroll
-        for (int c = 0; c < kRowValsPerThread; c++) {
-            const int e = tid + c * kThreads;
-            const int which = e / A_ROWS, r = e % A_ROWS;
-            const int64_t row = ablk0 * 32 + r;
-            float val = 0.f;                      // rows past n_a carry zero weight
-            if (e < kRowVals && row < na_blocks * 32 && which < tcols) val = vecp[(int64_t)which * vec_ld + row];
-            rowv[c] = val;
+            for (int c = 0; c < kRowValsPerThread; c++) {
+                const int which = col0 + c * kColStep;
+                float val = 0.f;
+                if (tid + c * kThreads < kRowVals && row_ok && which < tcols) val = src[(int64_t)(c * kColStep) * vec_ld];
+                rowv[c] = val;
+            }
         }
         wg_barrier();
+        {
+            // (opaque, so that the swizzled slots are worked out here and not kept in registers across the tile loop)
+            int r = tid % A_ROWS, col0 = tid / A_ROWS;
+            asm volatile("" : "+v"(r), "+v"(col0));
 #pragma unroll
-        for (int c = 0; c < kRowValsPerThread; c++) {
-            const int e = tid + c * kThreads;
-            const int which = e / A_ROWS, r = e % A_ROWS;
-            if (e < kRowVals) {
-                if (!kMfmaEpi) ldsRow[e] = rowv[c];
-                else ldsRow[r * kVecStride + which] = rowv[c];
+            for (int c = 0; c < kRowValsPerThread; c++) {
+                if (tid + c * kThreads < kRowVals) {
+                    if (!kMfmaEpi) ldsRow[tid + c * kThreads] = rowv[c];
+                    else ldsRow[vec_slot(r, col0 + c * kColStep)] = rowv[c];
+                }
             }
         }
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -282,6 +304,48 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                     }
                 }
             }
+        } else if constexpr (kGroups32 > 0) {
+            // 32 columns per group with the 32x32x2 step: accumulator register s2 of lane l is K[i][j] with i =
+            // acc_row(s2, lg), j = l % 32, i.e. its A operand for the pair of rows (lg = 0, 1); the B operand is
+            // vec[acc_row(s2, lg)][32 g + l % 32]; a lane ends up with column 32 g + l % 32 of output rows acc_row(r, lg).
+            // The lane's part of the slot (vec_slot with r = 32 (wa WA_FR + p) + acc_row(s2, lg) and c = 32 g + j) is
+            // kept opaque: computed in the open, the compiler works out all 64 or 128 read addresses in front of the
+            // tile loop and spills them.
+            int lane_off = (wa * WA_FR * 32 + 4 * lg) * kVecStride, lane_col = j ^ (4 * lg);
+            asm volatile("" : "+v"(lane_off), "+v"(lane_col));
+            auto read_vec = [&](int p, int s2, int g) {
+                const int rc = p * 32 + 8 * (s2 >> 2) + (s2 & 3);      // the row without the lane's part (a constant)
+                return ldsRow[lane_off + rc * kVecStride + ((32 * g + lane_col) ^ (rc & (kVecStride - 1)))];
+            };
+#pragma unroll
+            for (int p = 0; p < WA_FR; p++) {
+#pragma unroll
+                for (int q = 0; q < WB_FR; q++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[p][q][r] = kernel_value<KF>(acc[p][q][r]);
+                float bval[kGroups32], bnext[kGroups32];
+#pragma unroll
+                for (int g = 0; g < kGroups32; g++) bval[g] = read_vec(p, 0, g);
+#pragma unroll
+                for (int s2 = 0; s2 < 16; s2++) {
+                    if (s2 + 1 < 16) {
+#pragma unroll
+                        for (int g = 0; g < kGroups32; g++) bnext[g] = read_vec(p, s2 + 1, g);
+                    }
+#pragma unroll
+                    for (int g = 0; g < kGroups32; g++)
+#pragma unroll
+                        for (int q = 0; q < WB_FR; q++)
+                            out2[q * kGroups32 + g] = __builtin_amdgcn_mfma_f32_32x32x2f32(acc[p][q][s2], bval[g],
+                                                                                           out2[q * kGroups32 + g], 0, 0, 0);
+                    // one read ahead, fenced (otherwise all reads are hoisted to the front and spilled)
+#pragma unroll
+                    for (int g = 0; g < kGroups32; g++) {
+                        asm volatile("" : "+v"(bval[g]) : : "memory");
+                        bval[g] = bnext[g];
+                    }
+                }
+            }
         } else {
 #pragma unroll
             for (int p = 0; p < WA_FR; p++)
@@ -318,6 +382,23 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 
     if constexpr (STORE) {
         // nothing left to write
+    } else if constexpr (kGroups32 > 0) {
+#pragma unroll
+        for (int g = 0; g < kGroups32; g++) {
+            const int t = 32 * g + j;
+            if (t < tcols) {
+#pragma unroll
+                for (int q = 0; q < WB_FR; q++) {
+                    const int64_t bb = bblk0 + wb * WB_FR + q;
+                    if (bb < nb_blocks) {
+#pragma unroll
+                        for (int r = 0; r < 16; r++)
+                            partial[(((int64_t)by * WVA + wa) * tcols + t) * nb_pad + bb * 32 + TR::acc_row(r, lg)] =
+                                out2[q * kGroups32 + g][r];
+                    }
+                }
+            }
+        }
     } else if constexpr (kMfmaEpi) {
         const int tl = lane & 15, mq = lane >> 4;
         if (tl < tcols) {
@@ -358,7 +439,7 @@ constexpr int kSLWavesA = 2, kSLWavesB = 4, kSLFragsA = 4, kSLFragsB = 2;
 int split_large_a_tile_blocks() { return kSLWavesA * kSLFragsA; }
 int split_large_b_tile_blocks() { return kSLWavesB * kSLFragsB; }
 int split_large_partials_per_split() { return kSLWavesA; }
-int split_large_max_cols() { return 16; }
+int split_large_max_cols() { return 64; }
 #endif
 
 template <int TT>
@@ -399,11 +480,13 @@ int FLK_CAT(launch_mmv_split_large_kf, FLK_KF)(const SplitView &A, const SplitVi
                                                float *partial, hipStream_t st) {
     if (A.ks != B.ks || A.d != B.d)
         return fail(FLK_EINVAL, "mmv_split_large: operands packed with different feature counts");
-    if (tcols < 1 || tcols > 16) return fail(FLK_EINVAL, "mmv_split_large: column chunk %d not in 1..16", tcols);
+    if (tcols < 1 || tcols > 64) return fail(FLK_EINVAL, "mmv_split_large: column chunk %d not in 1..64", tcols);
     if (tcols == 1) return launch_split_large_tt<1>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols == 2) return launch_split_large_tt<2>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
     if (tcols <= 4) return launch_split_large_tt<4>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
-    return launch_split_large_tt<16>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    if (tcols <= 16) return launch_split_large_tt<16>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    if (tcols <= 32) return launch_split_large_tt<32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    return launch_split_large_tt<64>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
 }
 
 }  // namespace flk

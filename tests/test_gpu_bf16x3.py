@@ -80,6 +80,34 @@ def test_layouts_sigma_per_dimension_and_repeatability(dev):
     assert torch.equal(k.dmmv(X, C, v, w).to(dev), ref)
 
 
+@pytest.mark.parametrize("d", [63, 100, 300])
+@pytest.mark.parametrize("t", [17, 32, 33, 48, 64, 65, 100])
+def test_many_right_hand_sides_on_the_lds_tiled_kernel(dev, d, t):
+    """Beyond 62 features the LDS-tiled kernel of the mode takes up to 64 columns per pass: 16 with the 16x16x1 step, 32
+    and 64 with one or two groups of 32x32x2 steps (their right-hand sides swizzled in LDS, two operand stages instead
+    of three), a second pass beyond 64 columns; ragged tiles on both sides, several reduction tiles per workgroup,
+    Fortran-ordered operands, repeatable bit for bit."""
+    n, m = 900 + 3 * d + t, 280 + t
+    X, C, v, w = _data(n, m, d, t, seed=5 * d + 11 * t)
+    sigma = torch.tensor([0.9 * np.sqrt(d)], dtype=torch.float64)
+    k = GaussianKernel(sigma, opt=SPLIT)
+    Xg, Cg, vg, wg = (a.to(dev) for a in (X, C, v, w))
+    Xd, Cd, vd, wd = (a.double() for a in (X, C, v, w))
+    check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)
+    got = k.dmmv(Xg, Cg, vg, wg)
+    check_parity(got, mmv_ref.fdmmv_ref(X, C, v, w, sigma), mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), 1e-5)
+    f = lambda a: a.T.contiguous().T                                                      # noqa: E731
+    assert torch.equal(k.dmmv(f(Xg), f(Cg), f(vg), f(wg)), got)
+    plain = GaussianKernel(sigma).dmmv(Xg, Cg, vg, wg)
+    assert rel_err(got, plain) < 5e-6
+    # fewer rows than one tile on either side.  (With so few rows of X single output columns are one cancelling sum
+    # times a vector, whatever kernel computes them: the error is taken over the whole result here.)
+    for nn, mm in ((40, m), (n, 1)):
+        g1 = k.dmmv(Xg[:nn], Cg[:mm], vg[:mm], wg[:nn]).cpu().double()
+        r1 = mmv_ref.fdmmv_ref(Xd[:nn], Cd[:mm], vd[:mm], wd[:nn], sigma)
+        assert float((g1 - r1).norm() / r1.norm()) < 1e-5
+
+
 @pytest.mark.parametrize("n,m,d,t", [(400, 150, 63, 2), (300, 257, 65, 1), (129, 64, 200, 10), (64, 300, 784, 5),
                                      (700, 129, 100, 4), (513, 260, 130, 16), (260, 513, 96, 17)])
 def test_lds_tiled_kernel_vs_oracle(dev, n, m, d, t):
@@ -184,7 +212,7 @@ def test_degenerate_shapes(dev, d):
         assert rel_err(got, mmv_ref.fdmmv_ref(X[:n], C[:m], v[:m], w[:n], k.sigma)) < 1e-5
 
 
-@pytest.mark.parametrize("d,t", [(28, 2), (200, 2), (28, 40), (200, 12)])
+@pytest.mark.parametrize("d,t", [(28, 2), (200, 2), (28, 40), (200, 12), (200, 40)])
 def test_dmmv_replays_from_a_hip_graph(dev, d, t):
     """As for the fp32 kernels: nothing is allocated, cleared with a memset or synchronised, so a call can be captured
     into a HIP graph; every replay reproduces the eager result bit for bit.  With few and with many right-hand sides."""
