@@ -54,7 +54,7 @@ template <typename T, int WVA, int WVB, int WA_FR, int WB_FR, int KC> struct LGe
 // KG s .. KG s + KG - 1 (lane group lg takes feature KG s + lg), so a step's operands are adjacent rows of the
 // packed block and the zero padding past d sits in the last steps of the last chunk, which the kernel skips.
 // The packed feature count is a whole number of chunks (padded_features), so there is no feature tail to mask.
-template <typename T, int KC>
+template <typename T, int KC, bool SCALAR_BLK = false>
 __device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t blk0, int64_t nblk, int64_t dpad,
                                               int64_t s0, int vi) {
     typedef LTraits<T> TR;
@@ -62,7 +62,13 @@ __device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t b
     const int jv = vi % VPB;
     const int lg = (vi / VPB) % TR::KG;
     const int s = (vi / (VPB * TR::KG)) % KC;
-    const int blk = vi / (VPB * TR::KG * KC);
+    // A block's vectors of a chunk are a whole number of waves: the block is the same for the 64 lanes.  SCALAR_BLK
+    // says so to the compiler, which then keeps the blocks' base addresses in scalar registers.  That pays where the
+    // vector registers are short (the fp32 passes of 48 and 64 columns otherwise reload spilled addresses in every
+    // chunk: N = 5e5, M = 1e4, d = 784, 64 columns 138.3 -> 135.9 ms, d = 300 at N = 2.5e5, M = 2e4 62.8 -> 61.2) and costs
+    // elsewhere (16 columns at d = 784: 120.0 -> 126.8 ms, fp64 248.6 -> 269.1).
+    static_assert((VPB * TR::KG * KC) % 64 == 0, "a wave's vectors must belong to one block");
+    const int blk = SCALAR_BLK ? __builtin_amdgcn_readfirstlane(vi / (VPB * TR::KG * KC)) : vi / (VPB * TR::KG * KC);
     int64_t b = blk0 + blk;
     if (b >= nblk) b = nblk - 1;                 // past the end: any valid block (its rows get zero weight / are not stored)
     return P + (b * dpad + (s0 + s) * TR::KG + lg) * TR::BLK + jv * TR::VPL;
@@ -160,14 +166,15 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                 for (int r = 0; r < TR::ACCN; r++) acc[p][q][r] = T(0);
 
         V16 ra[G::A_VPT], rb[G::B_VPT];
+        constexpr bool kScalarBlk = sizeof(T) == 4 && TT >= 48;
         auto fetch = [&](int64_t chunk) {
             const int64_t s0 = chunk * KC;
 #pragma unroll
             for (int c = 0; c < G::A_VPT; c++)
-                ra[c] = *(const V16 *)stage_src<T, KC>(PA, ablk0, na_blocks, dpad, s0, tid + c * kLThreads);
+                ra[c] = *(const V16 *)stage_src<T, KC, kScalarBlk>(PA, ablk0, na_blocks, dpad, s0, tid + c * kLThreads);
 #pragma unroll
             for (int c = 0; c < G::B_VPT; c++)
-                rb[c] = *(const V16 *)stage_src<T, KC>(PB, bblk0, nb_blocks, dpad, s0, tid + c * kLThreads);
+                rb[c] = *(const V16 *)stage_src<T, KC, kScalarBlk>(PB, bblk0, nb_blocks, dpad, s0, tid + c * kLThreads);
         };
         auto commit = [&](int buf) {
 #pragma unroll
