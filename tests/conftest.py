@@ -57,3 +57,15 @@ def check_parity(got, ref_same_dtype, ref_f64, tol: float) -> None:
         e = rel_err(got, ref_f64)
         bound = min(max(tol, 2 * e_ref), 10 * tol)
         assert e < bound, f"GPU vs fp64 oracle: {e:.3e} >= {bound:.1e}; CPU fp32 path vs fp64: {e_ref:.3e}"
+
+
+def scaled_err(got, ref_f64, scale) -> float:
+    """Worst column of ``|got - ref| / |scale|`` (norm-wise), where ``scale`` is the same product formed
+    from the absolute values of its terms: the error measured against the size of what was summed rather
+    than against a result that may have cancelled.  A backward-stable fp32 summation stays at a small
+    multiple of 6e-8 here however strongly a column cancels; an accumulation that loses digits does not."""
+    a = torch.as_tensor(got).detach().double().cpu()
+    e = torch.as_tensor(ref_f64).detach().double().cpu()
+    s = torch.as_tensor(scale).detach().double().cpu()
+    a, e, s = a.reshape(e.shape[0], -1), e.reshape(e.shape[0], -1), s.reshape(e.shape[0], -1)
+    return float(((a - e).norm(dim=0) / s.norm(dim=0).clamp_min(1e-300)).max())
