@@ -881,6 +881,32 @@ int flk_cg_update(int mode, void *X, void *R, void *P, const void *Q, const void
     return fail(FLK_EINVAL, "unknown dtype %d", dtype);
 }
 
+int64_t flk_tri_solve_work_elems(int64_t m, int64_t t, int64_t block) {
+    if (m < 0 || t < 0 || block < 1) return 0;
+    return tri_solve_work_elems(m, t, block);
+}
+
+int flk_tri_solve(int dtype, int transposed, const void *L, int64_t m, int64_t ld, int row_major, const void *dinv,
+                  const void *dinv_t, int64_t block, const void *b, int64_t ldb, void *x, int64_t ldx, int64_t t,
+                  void *work, void *stream) {
+    g_err[0] = 0;
+    if (m < 0 || t < 0) return fail(FLK_EINVAL, "flk_tri_solve: negative size");
+    if (m == 0 || t == 0) return FLK_OK;
+    if (block < 4 || block % 4 != 0) return fail(FLK_EINVAL, "flk_tri_solve: block size %lld (a positive multiple of 4)", (long long)block);
+    if (ld < m || ldb < m || ldx < m) return fail(FLK_EINVAL, "flk_tri_solve: leading dimension below m");
+    if (!L || !dinv || !dinv_t || !b || !x || !work) return fail(FLK_EINVAL, "flk_tri_solve: null pointer");
+    if (x == b || work == b || work == x) return fail(FLK_EINVAL, "flk_tri_solve: b, x and work must be distinct buffers");
+    if (t > 4) return fail(FLK_EUNSUPPORTED, "flk_tri_solve: %lld right-hand sides (1 .. 4 per call)", (long long)t);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == FLK_F32)
+        return launch_tri_solve<float>((const float *)L, m, ld, row_major, (const float *)dinv, (const float *)dinv_t, block,
+                                       transposed, (const float *)b, ldb, (float *)x, ldx, t, (float *)work, st);
+    if (dtype == FLK_F64)
+        return launch_tri_solve<double>((const double *)L, m, ld, row_major, (const double *)dinv, (const double *)dinv_t,
+                                        block, transposed, (const double *)b, ldb, (double *)x, ldx, t, (double *)work, st);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
 size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype, int compute_f64) {
     if (n < 0 || m < 0 || d < 1 || d > flk_max_d(dtype) || !known_dtype(dtype, true)) return 0;
     if (fmm_split_applies(d, dtype, compute_f64)) return split_packed_bytes(n, d) + split_packed_bytes(m, d);

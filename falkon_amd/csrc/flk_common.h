@@ -112,6 +112,12 @@ int fail(int code, const char *fmt, ...);
             return ::flk::fail(FLK_EHIP, "launch of %s failed: %s", name, hipGetErrorString(e__)); \
     } while (0)
 
+// Blocked triangular solve with a resident factor and the inverses of its diagonal blocks (trsv.hip)
+int64_t tri_solve_work_elems(int64_t m, int64_t t, int64_t block);
+template <typename T>
+int launch_tri_solve(const T *L, int64_t m, int64_t ld, int row_major, const T *dinv, const T *dinv_t, int64_t block,
+                     int transposed, const T *b, int64_t ldb, T *x, int64_t ldx, int64_t t, T *work, hipStream_t st);
+
 // launchers implemented in the .hip files -------------------------------------
 template <typename TI, typename T>   // TI: caller's element type, T: type of the packed operand
 int launch_pack(const TI *X, int64_t n, int64_t d, int64_t rs, int64_t cs, const TI *sigma, int64_t n_sigma,

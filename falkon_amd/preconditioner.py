@@ -11,7 +11,10 @@ right-hand sides, where a library ``trsm`` runs far below the memory roofline (M
 per solve against 2 ms for a matrix-vector product over the same factor).  ``_BlockedTriangular`` does
 the solve by blocks instead: the diagonal blocks are inverted once when the factor is built, and a
 solve is then a chain of small matrix products with those inverses and matrix-vector products over
-the row panels of the factor, each element of which is read once.
+the row panels of the factor, each element of which is read once.  For a device-resident factor and up to
+four right-hand sides those products are the library's own kernels (``flk_tri_solve``, csrc/trsv.hip: two
+launches per diagonal block, the triangle streamed once at 5 TB/s, fixed summation order); host tensors and
+wider right-hand sides take the same chain in torch ops.
 """
 from typing import Optional
 
@@ -96,16 +99,57 @@ class _BlockedTriangular:
         M = L.shape[0]
         self.row_major = M < 2 or L.stride(1) == 1
         self.dinv, self.panels = [], []
-        for k0, k1 in self.bounds:
+        self._stack = self._stack_t = None
+        if not self.bounds:
+            return
+        block = self.bounds[0][1] - self.bounds[0][0]
+        # the inverted diagonal blocks, block k at [k] with leading dimension `block` (zero beyond a smaller last
+        # block), and their transposes: the layout flk_tri_solve reads; the torch path uses views of the same memory
+        self._stack = torch.zeros(len(self.bounds), block, block, dtype=L.dtype, device=L.device)
+        for k, (k0, k1) in enumerate(self.bounds):
             eye = torch.eye(k1 - k0, dtype=L.dtype, device=L.device)
-            self.dinv.append(torch.linalg.solve_triangular(L[k0:k1, k0:k1], eye, upper=False))
+            self._stack[k, :k1 - k0, :k1 - k0] = torch.linalg.solve_triangular(L[k0:k1, k0:k1], eye, upper=False).tril_()
+            self.dinv.append(self._stack[k, :k1 - k0, :k1 - k0])
             # views with unit column stride: L[k, :k] (row-major L) or (L^T)[k, k+1:] (column-major L)
             self.panels.append(L[k0:k1, :k0] if self.row_major else L[k1:, k0:k1].T)
+        if L.is_cuda:
+            self._stack_t = self._stack.transpose(1, 2).contiguous()
 
     def to(self, device):
         self.L = self.L.to(device)
         self._build()
         return self
+
+    NATIVE_MAX_RHS = 4
+
+    def _native_applies(self, b: torch.Tensor) -> bool:
+        """The library's solve (``flk_tri_solve``: two launches per diagonal block, every element of the factor read
+        once at streaming rate) serves device-resident fp32 / fp64 factors with up to four right-hand sides; the
+        torch-op path below serves host tensors and wider right-hand sides."""
+        L = self.L
+        return (self._stack_t is not None and self._stack.shape[1] % 4 == 0 and b.is_cuda and b.device == L.device
+                and b.dtype == L.dtype
+                and L.dtype in (torch.float32, torch.float64) and b.dim() == 2 and 1 <= b.shape[1] <= self.NATIVE_MAX_RHS
+                and (L.stride(1) == 1 or L.stride(0) == 1))
+
+    def _solve_native(self, b: torch.Tensor, transposed: bool) -> torch.Tensor:
+        from . import _backend
+        from .mmv_ops.fmmv import _current, _stream_handle
+        lib = _backend.load()
+        L = self.L
+        m, t = b.shape
+        cols = b.T.contiguous()                     # [t][m]: one contiguous column per right-hand side
+        ld = L.stride(0) if self.row_major else L.stride(1)
+        block = self._stack.shape[1]
+        x = torch.empty_like(cols)
+        work = torch.empty(int(lib.flk_tri_solve_work_elems(m, t, block)), dtype=L.dtype, device=L.device)
+        code = _backend.FLK_F32 if L.dtype == torch.float32 else _backend.FLK_F64
+        with _current(L.device):
+            rc = lib.flk_tri_solve(code, int(transposed), L.data_ptr(), m, ld, int(self.row_major), self._stack.data_ptr(),
+                                   self._stack_t.data_ptr(), block, cols.data_ptr(), m, x.data_ptr(), m, t, work.data_ptr(),
+                                   _stream_handle(L.device))
+        _backend.raise_for_status(rc, "flk_tri_solve")
+        return x.view(m, 1) if t == 1 else x.T
 
     @staticmethod
     def _as_columns(b: torch.Tensor):
@@ -143,12 +187,16 @@ class _BlockedTriangular:
         """x with L x = b."""
         if not self.bounds:
             return torch.linalg.solve_triangular(self.L, b, upper=False)
+        if self._native_applies(b):
+            return self._solve_native(b, transposed=False)
         return self._substitute(b, transposed=False)
 
     def solve_t(self, b: torch.Tensor) -> torch.Tensor:
         """x with L^T x = b."""
         if not self.bounds:
             return torch.linalg.solve_triangular(self.L.T, b, upper=True)
+        if self._native_applies(b):
+            return self._solve_native(b, transposed=True)
         return self._substitute(b, transposed=True)
 
 

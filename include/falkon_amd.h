@@ -190,6 +190,27 @@ int flk_cg_update(int mode, void *X, void *R, void *P, const void *Q, const void
                   int64_t rs, int64_t cs, void *rsold, int32_t *state, int64_t iteration,
                   double eps, double tol2, int differential, int dtype, void *stream);
 
+/* ---- triangular solves of the preconditioner ----------------------------------
+ * flk_tri_solve replaces the triangular solves with the preconditioner's two Cholesky factors that every
+ * conjugate-gradient iteration performs (falkon/preconditioner/flk_preconditioner.py:166-256: invA, invAt, invT,
+ * invTt, there the library's trsm; falkon/optim/conjgrad.py:242-256 is the caller) for 1 .. 4 right-hand sides.
+ *   L: m x m lower-triangular factor, element (i, j) at L[i*ld + j] (row_major != 0) or L[i + j*ld]; only the
+ *      part below the diagonal blocks is read.
+ *   dinv, dinv_t: inverses of the diagonal blocks L[k*block .. , k*block ..] and the transposes of those inverses,
+ *      block k at + k*block*block elements, row-major with leading dimension `block` (a smaller last block keeps
+ *      that leading dimension); the caller computes them once per factor.  block: a multiple of 4.
+ *   transposed == 0 solves L x = b, otherwise L^T x = b.
+ *   b, x: t columns of m elements each, column c at + c*ldb, + c*ldx; work: flk_tri_solve_work_elems(m, t, block)
+ *      elements of the data dtype (partial sums of the panel products); three distinct buffers.
+ * A solve reads the triangle once (two launches per diagonal block: a panel product over long contiguous rows and
+ * the product with the inverted block), sums in a fixed order in double precision (reproducible), takes no
+ * workspace beyond `work` and does not synchronise. */
+int64_t flk_tri_solve_work_elems(int64_t m, int64_t t, int64_t block);
+
+int flk_tri_solve(int dtype, int transposed, const void *L, int64_t m, int64_t ld, int row_major,
+                  const void *dinv, const void *dinv_t, int64_t block,
+                  const void *b, int64_t ldb, void *x, int64_t ldx, int64_t t, void *work, void *stream);
+
 /* ---- explicit kernel matrix -------------------------------------------------
  * flk_gauss_fmm replaces falkon.mmv_ops.fmm.fmm for the dense Gaussian case
  *   (falkon/mmv_ops/fmm.py:699-708 -> :298-388 block loop -> distance_kernel.py:140-159):
