@@ -56,15 +56,17 @@ __device__ __forceinline__ void fetch_rowvals(RowVals<TT> &rv, const float *cons
     for (int c = 0; c < RowVals<TT>::C; c++) rv.x[c] = src[c][ab * 32];
 }
 
-// keep = 0 clears the right-hand side entries of the block (its kernel values then contribute nothing to the sums):
-// for the block that is processed a second time when a chunk holds an odd number of blocks.  Applied here and not
+// keep = false clears the right-hand side entries of the block (its kernel values then contribute nothing to the
+// sums): for the block that is processed a second time when a chunk holds an odd number of blocks.  A bit mask, not a
+// product with zero: an infinite entry of the right-hand side must not turn into NaN there.  Applied here and not
 // where the values are fetched, so that nothing touches the loaded registers before the tile step in between is done.
 template <int TT>
-__device__ __forceinline__ void stage_rowvals(const RowVals<TT> &rv, float *lds, int lane, float keep = 1.0f) {
+__device__ __forceinline__ void stage_rowvals(const RowVals<TT> &rv, float *lds, int lane, bool keep = true) {
+    const unsigned mask = keep ? 0xffffffffu : 0u;
 #pragma unroll
     for (int c = 0; c < RowVals<TT>::C; c++) {
         int e = lane + 64 * c;
-        if (e < RowVals<TT>::N) lds[e] = e >= 32 ? rv.x[c] * keep : rv.x[c];
+        if (e < RowVals<TT>::N) lds[e] = e >= 32 ? __uint_as_float(__float_as_uint(rv.x[c]) & mask) : rv.x[c];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -215,7 +217,7 @@ __device__ __forceinline__ void reduce_blocks(const float *__restrict__ PA, cons
             __builtin_amdgcn_sched_barrier(0);
             tile_step<DP, FR, TT, NOADD, KF, RAW, true>(fa0, lds0, h, breg, hb, o1);
             __builtin_amdgcn_sched_barrier(0);
-            stage_rowvals<TT>(rv, lds1, lane, second ? 1.0f : 0.0f);
+            stage_rowvals<TT>(rv, lds1, lane, second);
             const int64_t n2 = ab + 2 < last ? ab + 2 : last;
             fetch_rowvals<TT>(rv, src, n2);
             load_a<DP>(fa0, PA, n2, j, h);

@@ -18,7 +18,7 @@ import torch
 from .. import _backend
 from ..options import BaseOptions
 from ..utils.helpers import sizeof_dtype
-from .utils import check_contiguity, create_output_mat, usable_gpu_memory
+from .utils import check_contiguity, create_output_mat, retry_with_fresh_memory_report, usable_gpu_memory
 
 __all__ = ("fmmv", "fdmmv", "gauss_fmmv_native", "gauss_fdmmv_native")
 
@@ -397,7 +397,7 @@ def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optio
     kernel_params = list(kernel.diff_params.values())
     if any(t.requires_grad for t in [X1, X2, v] + kernel_params):
         return _KernelMmvFn.apply(kernel, opt, out, X1, X2, v, *kernel_params)
-    return _fmmv_run(X1, X2, v, kernel, kernel_fn, out, opt, cached_sigma=True)
+    return retry_with_fresh_memory_report(lambda: _fmmv_run(X1, X2, v, kernel, kernel_fn, out, opt, cached_sigma=True))
 
 
 def _fmmv_run(X1, X2, v, kernel, kernel_fn: int, out, opt: BaseOptions, cached_sigma: bool) -> torch.Tensor:
@@ -453,6 +453,11 @@ def fdmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, w: Optional[torch
 
     ``v`` is required (the reference reads ``v.shape`` unconditionally, fmmv.py:1035-1041); ``w`` may be None.
     """
+    return retry_with_fresh_memory_report(
+        lambda: _fdmmv_run(X1, X2, v, w, kernel, out, differentiable, opt, kwargs_m1, kwargs_m2))
+
+
+def _fdmmv_run(X1, X2, v, w, kernel, out, differentiable, opt, kwargs_m1, kwargs_m2) -> torch.Tensor:
     opt = opt if opt is not None else BaseOptions()
     if differentiable:
         raise NotImplementedError(

@@ -10,7 +10,7 @@ import torch
 
 from ..utils.tensor_helpers import create_C, create_fortran, create_same_stride, is_contig
 
-__all__ = ("check_contiguity", "create_output_mat", "usable_gpu_memory")
+__all__ = ("check_contiguity", "create_output_mat", "usable_gpu_memory", "retry_with_fresh_memory_report")
 
 
 def check_contiguity(*args: Tuple[Optional[torch.Tensor], str]) -> None:
@@ -42,8 +42,12 @@ def create_output_mat(out: Optional[torch.Tensor], data_devs: Sequence[torch.dev
 
 # Asking the driver for the free memory takes longer (about 12 microseconds) than the host side of everything else in
 # a small product, so a call that needs at most 1/8 of what the driver reported within the last 50 ms reuses that
-# report; the value returned is then a lower bound (1/8 of it), which such a call fits by construction.
+# report; the value returned is then 1/8 of it, which such a call fits unless somebody allocated seven eighths of the
+# free memory in between.  Reading the allocator's counters to notice that would cost more than the report itself, so
+# the drivers guard the other end instead: a product that runs out of memory on a plan made from a reused report is
+# planned again from a fresh one (retry_with_fresh_memory_report).
 _recent_free = {}
+_reused = set()        # devices whose last budget came from a reused report
 _FREE_MEMORY_TTL = 0.05
 _SMALL_CALL_MARGIN = 8.0
 
@@ -60,7 +64,9 @@ def usable_gpu_memory(dev: torch.device, max_gpu_mem: float, slack: float, enoug
     seen = _recent_free.get(key)
     now = time.monotonic()
     if seen is not None and now - seen[1] < _FREE_MEMORY_TTL and _SMALL_CALL_MARGIN * enough <= seen[0] * slack:
+        _reused.add(key)
         return min(seen[0] * slack / _SMALL_CALL_MARGIN, max_gpu_mem * slack)
+    _reused.discard(key)
     free, _total = torch.cuda.mem_get_info(dev)
     _recent_free[key] = (free, now)
     usable = min(free * slack, max_gpu_mem * slack)
@@ -72,3 +78,16 @@ def usable_gpu_memory(dev: torch.device, max_gpu_mem: float, slack: float, enoug
         raise MemoryError(f"Usable memory on device {dev} is less than 0. Either there is no free memory "
                           f"available, or the `max_gpu_mem` setting is too low.")
     return usable
+
+
+def retry_with_fresh_memory_report(run):
+    """``run()``; if it runs out of device memory on a plan that was made from a reused free-memory report, forget the
+    reports and run it once more (the second plan asks the driver, sees what is really free and splits the rows)."""
+    try:
+        return run()
+    except torch.cuda.OutOfMemoryError:
+        if not _reused:
+            raise
+        _reused.clear()
+        _recent_free.clear()
+        return run()

@@ -29,14 +29,18 @@ class ConjugateGradient:
     ``CHECK_EVERY`` iterations (every iteration when a callback wants the solution), so iterations are enqueued
     without waiting for each other.  Once every column has converged the remaining launches of that window leave the
     solution untouched: the result is the one the reference's ``break`` gives.  With ``cg_capture_graph`` every kind
-    of iteration is captured once into a HIP graph (operator and update together) and replayed.  Host tensors run
-    the same iteration in torch ops."""
+    of iteration is captured once into a HIP graph (operator and update together) and replayed; the row-block plan
+    and workspace sizes of the operator are those of the capture, an operator that cannot be captured makes the
+    solve continue eagerly with a warning, and host-resident operands switch replay off.  Differential convergence
+    freezes a converged column but still passes it through the operator: unlike the reference, which shrinks its
+    matrices (:113-161), it saves no operator work here.  Host tensors run the same iteration in torch ops."""
 
     CHECK_EVERY = 5
 
     def __init__(self, opt: Optional[ConjugateGradientOptions] = None):
         self.params = opt if opt is not None else ConjugateGradientOptions()
         self.num_iter = None
+        self.capture_ok = True      # set to False by a caller whose operator touches host-resident data
 
     def solve(self, X0: Optional[torch.Tensor], B: torch.Tensor, mmv: Callable[[torch.Tensor], torch.Tensor],
               max_iter: int, callback: Optional[Callable[[int, torch.Tensor, float], None]] = None) -> torch.Tensor:
@@ -51,7 +55,9 @@ class ConjugateGradient:
         lib = _backend.load()
         started = time.time()
         dev, (m, t) = B.device, B.shape
-        if 1 not in B.stride() and m > 1 and t > 1:
+        # work buffers take B's strides, so B has to be dense: row-major or column-major as it is, anything else (a
+        # slice with a leading dimension, an expanded view whose columns alias each other) as a row-major copy
+        if not (B.is_contiguous() or B.T.is_contiguous()):
             B = B.contiguous()
         strides = B.stride()
 
@@ -92,7 +98,9 @@ class ConjugateGradient:
                 update(2, mmv(sol), it)
 
         graphs, pool = {}, None
-        use_graph = bool(getattr(self.params, "cg_capture_graph", False))
+        # replay needs an operator that only enqueues device work on device-resident data (a host-resident operand
+        # would put pageable uploads into the capture): the caller says so through `capture_ok`
+        use_graph = bool(getattr(self.params, "cg_capture_graph", False)) and self.capture_ok
         every = 1 if callback is not None else self.CHECK_EVERY
         elapsed = time.time() - started
         applied = 0
@@ -103,10 +111,22 @@ class ConjugateGradient:
                 if key not in graphs:
                     g = torch.cuda.CUDAGraph()
                     pool = torch.cuda.graph_pool_handle() if pool is None else pool
-                    with torch.cuda.graph(g, pool=pool):
-                        iteration(it)
-                    graphs[key] = g
-                graphs[key].replay()
+                    try:
+                        with torch.cuda.graph(g, pool=pool):
+                            iteration(it)
+                        graphs[key] = g
+                    except Exception as exc:            # noqa: BLE001 -- an operator that cannot be captured
+                        # (it waits for the device, or allocates outside the pool): the capture has ended with the
+                        # context manager; nothing of this iteration has run, so the solve goes on eagerly from here
+                        import warnings
+                        warnings.warn(f"cg_capture_graph: the iteration could not be captured ({exc!r}); "
+                                      "continuing without graph replay")
+                        use_graph = False
+                        graphs.pop(key, None)
+                if use_graph:
+                    graphs[key].replay()
+                else:
+                    iteration(it)
             else:
                 iteration(it)
             applied = it + 1
@@ -236,6 +256,7 @@ class FalkonConjugateGradient:
             operator = functools.partial(self.weighted_falkon_mmv, penalty=_lambda, X=X, M=M, y_weights=y_weights, n=n)
         else:
             operator = functools.partial(self.falkon_mmv, penalty=_lambda, X=X, M=M, n=n)
+        self.optimizer.capture_ok = bool(X.is_cuda and M.is_cuda and Y.is_cuda)
         kty = self.stored_knm.T @ y_over_n if self.stored_knm is not None else self.kernel.mmv(M, X, y_over_n, opt=self.params)
         rhs = self.preconditioner.apply_t(kty)                                                # B^T K_nm^T (W) y / n
         return self.optimizer.solve(initial_solution, rhs, operator, max_iter, callback)

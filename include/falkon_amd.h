@@ -150,8 +150,11 @@ int flk_gauss_fdmmv(const void *X1, int64_t n, int64_t x1_rs, int64_t x1_cs,
  * flk_gauss_fdmmv_noalloc has no counterpart in the reference.  It is flk_gauss_fdmmv without the workspace
  * argument, for callers that cannot obtain device memory at the call: code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc.  The workspace is an array of FLK_NOALLOC_SCRATCH_BYTES
- * bytes that is part of the library's device code: every GPU the library runs on holds its own copy from the
- * first call on it until the process ends.  The call allocates and frees nothing and enqueues the same kernels
+ * bytes that is part of the library's device code: every GPU on which the library's device code is loaded (by the
+ * first flk_* call of any kind that launches there) holds its own copy from then until the process ends, whether
+ * or not this entry point is ever called.  The array's device address is looked up on the first call of this entry
+ * point on a GPU: make that first call outside a graph capture (the tests capture after one eager call).
+ * The call allocates and frees nothing and enqueues the same kernels
  * as flk_gauss_fdmmv, so the results are bit-identical to it.  A problem whose
  * flk_gauss_fdmmv_workspace_bytes(n, m, d, t, dtype) exceeds FLK_NOALLOC_SCRATCH_BYTES is refused with
  * FLK_ENOMEM and a message naming both sizes.  All calls on one GPU share that GPU's array: two calls whose

@@ -192,3 +192,83 @@ def _conjgrad_problem64():
     Y = torch.from_numpy(inputs.gen_random(N, 1, np.float64, F=False, seed=9))
     idx = np.random.default_rng(2).choice(N, M, replace=False)
     return X, Y, X[idx].clone(), 100.0, 10.0
+
+
+@pytest.mark.gpu
+def test_right_hand_sides_that_are_no_dense_matrix(dev):
+    """Work buffers take the right-hand side's strides: an expanded view (columns aliasing each other) or a column
+    slice of a wider matrix must be solved as a dense copy, column for column like their dense twins."""
+    A, B = _spd(150, 3, seed=5)
+    Ag = A.to(dev)
+    opt = FalkonOptions(cg_tolerance=1e-9)
+    one = B[:, :1].to(dev)
+    expanded = one.expand(150, 3)
+    assert expanded.stride() == (1, 0)
+    wide = torch.zeros(150, 7, dtype=torch.float64, device=dev)
+    wide[:, 2:5] = B.to(dev)
+    sliced = wide[:, 2:5]
+    assert not sliced.is_contiguous() and not sliced.T.is_contiguous()
+    with torch.inference_mode():
+        Xe = ConjugateGradient(opt).solve(None, expanded, lambda v: Ag @ v, 300)
+        Xs = ConjugateGradient(opt).solve(None, sliced, lambda v: Ag @ v, 300)
+    exact = torch.linalg.solve(A, B)
+    assert rel_err(Xs, exact) < 1e-8
+    assert rel_err(Xe, exact[:, :1].expand(150, 3)) < 1e-8
+    assert wide[:, :2].abs().max() == 0 and wide[:, 5:].abs().max() == 0        # nothing written beside the slice
+
+
+@pytest.mark.gpu
+def test_graph_replay_with_a_callback(dev):
+    """Graph replay together with a callback (the host then looks at the flags after every iteration): the callback
+    sees the same iterates as in the eager solve, and the solution is the same."""
+    A, B = _spd(250, 2, seed=6)
+    Ag, Bg = A.to(dev), B.to(dev)
+    seen = {}
+    for graph in (False, True):
+        opt = FalkonOptions(cg_tolerance=1e-9, cg_capture_graph=graph)
+        trace = []
+        with torch.inference_mode():
+            X = ConjugateGradient(opt).solve(None, Bg.clone(), lambda v: Ag @ v, 60,
+                                             callback=lambda it, sol, t: trace.append((it, sol.clone())))
+        seen[graph] = (X, trace)
+    (Xe, te), (Xg, tg) = seen[False], seen[True]
+    assert len(te) == len(tg) > 5 and [i for i, _ in te] == [i for i, _ in tg]
+    for (_, a), (_, b) in zip(te, tg):
+        assert rel_err(b, a) < 1e-12
+    assert rel_err(Xg, Xe) < 1e-12 and rel_err(Ag @ Xg, Bg) < 1e-8
+
+
+@pytest.mark.gpu
+def test_an_operator_that_cannot_be_captured_falls_back_to_eager_iterations():
+    """An operator that waits for the device cannot be recorded into a graph: the solve warns, goes on eagerly and
+    returns the eager result.  Run in a process of its own, so that a capture that fails cannot touch the state of the
+    other tests' device context."""
+    import subprocess
+    import sys
+    code = r'''
+import warnings, numpy as np, torch
+from falkon_amd import FalkonOptions
+from falkon_amd.optim import ConjugateGradient
+g = np.random.default_rng(8)
+Q = g.standard_normal((120, 120))
+A = torch.from_numpy(Q @ Q.T + 120 * np.eye(120)).cuda()
+B = torch.from_numpy(g.standard_normal((120, 2))).cuda()
+def waiting_operator(v):
+    out = A @ v
+    float(out[0, 0])            # a host wait: not allowed while a stream is capturing
+    return out
+with torch.inference_mode():
+    want = ConjugateGradient(FalkonOptions(cg_tolerance=1e-9)).solve(None, B.clone(), lambda v: A @ v, 100)
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        got = ConjugateGradient(FalkonOptions(cg_tolerance=1e-9, cg_capture_graph=True)).solve(None, B.clone(), waiting_operator, 100)
+torch.cuda.synchronize()
+assert any("could not be captured" in str(w.message) for w in caught), [str(w.message) for w in caught]
+err = float((got - want).norm() / want.norm())
+assert err < 1e-10, err
+print("fallback ok", err)
+'''
+    import os
+    env = dict(os.environ, PYTHONPATH=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=240, env=env)
+    assert res.returncode == 0 and "fallback ok" in res.stdout, res.stdout + res.stderr

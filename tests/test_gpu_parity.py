@@ -705,3 +705,36 @@ def test_dmmv_stored_blocks_option(dev, dtype):
         assert rel_err(got, GaussianKernel(sigma).dmmv(Xg, Cg, vg, wg)) < TOL[dtype]
     X, C, v, w = (a.to(dev) for a in _rand(500, 28, 200, 2, dtype, seed=1))
     assert torch.equal(GaussianKernel(3.0, opt=opt).dmmv(X, C, v, w), GaussianKernel(3.0).dmmv(X, C, v, w))
+
+
+@pytest.mark.parametrize("d", [9, 28])
+@pytest.mark.parametrize("blocks", [1, 5, 37])
+def test_odd_reduction_blocks_single_column_and_coincident_points(dev, d, blocks):
+    """One right-hand side in fp32 with an odd number of 32-row blocks on the reduction side (the single-column loop
+    walks two blocks per trip and handles the last block of an odd chunk a second time against zeros), the centres
+    being rows of X, so that kernel values of exactly 1 occur (the reference clamps the squared distance at 1e-20,
+    falkon/kernels/distance_kernel.py:100, i.e. K <= 1): parity with the CPU path, K <= 1 to rounding, and an
+    infinite entry of v in the repeated block gives infinities, not NaN."""
+    m = 32 * blocks
+    X, _, v, w = _rand(1500, d, m, 1, torch.float32, seed=40 + blocks)
+    C = X[:m].clone()
+    sigma = float(d) ** 0.5
+    k = GaussianKernel(sigma)
+    Xg, Cg, vg, wg = X.to(dev), C.to(dev), v.to(dev), w.to(dev)
+    Xd, Cd, vd, wd = X.double(), C.double(), v.double(), w.double()
+    check_parity(k.mmv(Xg, Cg, vg), mmv_ref.fmmv_ref(X, C, v, sigma), mmv_ref.fmmv_ref(Xd, Cd, vd, sigma), 1e-5)
+    check_parity(k.dmmv(Xg, Cg, vg, wg), mmv_ref.fdmmv_ref(X, C, v, w, sigma), mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma), 1e-5)
+    # a column of K through a unit vector: the entry of the coincident pair is 1 (to rounding on the factored path)
+    for j in (0, m - 1):
+        unit = torch.zeros(m, 1)
+        unit[j] = 1.0
+        col = k.mmv(Xg, Cg, unit.to(dev)).cpu()
+        assert abs(float(col[j]) - 1.0) <= 2e-6 and float(col.max()) <= 1.0 + 2e-6
+        want = torch.from_numpy(brute.gaussian_brute(X, C[j:j + 1], sigma))
+        assert float((col.double() - want).abs().max()) < 2e-6
+    # an infinite right-hand side entry in the last block
+    vi = v.clone()
+    vi[m - 1] = float("inf")
+    got = k.mmv(Xg, Cg, vi.to(dev)).cpu()
+    ref = mmv_ref.fmmv_ref(X, C, vi, sigma)
+    assert torch.isinf(ref).all() and torch.equal(torch.isinf(got), torch.isinf(ref)) and not torch.isnan(got).any()

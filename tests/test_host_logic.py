@@ -366,6 +366,37 @@ def test_memory_budget_reuses_a_recent_driver_report(monkeypatch):
     utils.usable_gpu_memory(dev, float("inf"), 0.9, enough=2**20)                  # too old: asked again
     assert len(calls) == 3
     utils._recent_free.clear()
+    utils._reused.clear()
+
+
+def test_out_of_memory_on_a_reused_report_is_planned_again(monkeypatch):
+    """A plan made from a reused free-memory report can be stale (somebody allocated in between): a product that runs
+    out of memory on such a plan runs once more on a fresh report; one that was planned on a fresh report fails."""
+    import importlib
+    utils = importlib.import_module("falkon_amd.mmv_ops.utils")
+    calls, runs = [], []
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda dev: (calls.append(dev), (80 * 2**30, 288 * 2**30))[1])
+    utils._recent_free.clear()
+    utils._reused.clear()
+    dev = torch.device("cuda", 0)
+
+    def product():
+        runs.append(utils.usable_gpu_memory(dev, float("inf"), 0.9, enough=2**30))
+        if len(runs) == 2:                                       # the plan from the reused report does not fit
+            raise torch.cuda.OutOfMemoryError("simulated")
+        return len(runs)
+
+    assert utils.retry_with_fresh_memory_report(product) == 1 and len(calls) == 1
+    assert utils.retry_with_fresh_memory_report(product) == 3    # second run reused the report, failed, ran again
+    assert len(calls) == 2 and runs[2] == pytest.approx(0.9 * 80 * 2**30)
+
+    def always_fails():
+        utils.usable_gpu_memory(dev, float("inf"), 0.9, enough=70 * 2**30)     # too large a share: a fresh report
+        raise torch.cuda.OutOfMemoryError("simulated")
+    with pytest.raises(torch.cuda.OutOfMemoryError):
+        utils.retry_with_fresh_memory_report(always_fails)
+    utils._recent_free.clear()
+    utils._reused.clear()
 
 
 def test_bench_defaults_by_workload():

@@ -34,14 +34,16 @@ def _call(lib, name, X, C, sigma, v, w, out, code, stream, workspace=None):
     return getattr(lib, name)(*args, stream)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, "bf16x3"])
 def test_noalloc_equals_fdmmv_on_consecutive_calls(dev, dtype):
     """Two calls in a row, the second on a smaller problem (different blocking, the first call's packed operands and
     partial sums still in the array): each equals ``flk_gauss_fdmmv`` bit for bit and the CPU oracle to tolerance; no
     device memory is allocated through torch during the calls."""
     from falkon_amd import _backend
     lib = _backend.load()
-    code = _backend.FLK_F32 if dtype == torch.float32 else _backend.FLK_F64
+    # "bf16x3": fp32 data with the cross term on the bf16 matrix cores (dtype code FLK_F32_BF16X3)
+    code = {torch.float32: _backend.FLK_F32, torch.float64: _backend.FLK_F64, "bf16x3": _backend.FLK_F32_BF16X3}[dtype]
+    dtype = torch.float32 if dtype == "bf16x3" else dtype
     tol = 1e-5 if dtype == torch.float32 else 1e-11
     stream = torch.cuda.current_stream(dev).cuda_stream
     sigma = torch.tensor([2.5], dtype=dtype, device=dev)
@@ -68,6 +70,40 @@ def test_noalloc_equals_fdmmv_on_consecutive_calls(dev, dtype):
         assert torch.equal(got, want), f"case {i}: not bit-identical to flk_gauss_fdmmv"
         exp = mmv_ref.fdmmv_ref(X.cpu(), C.cpu(), v.cpu(), w.cpu() if w is not None else None, sigma.cpu())
         assert rel_err(got, exp) < tol, f"case {i}"
+
+
+def test_noalloc_captured_into_a_graph_and_replayed(dev):
+    """What the entry point is for: after one eager call (which looks the array's address up) the call is captured
+    into a HIP graph and replayed several times with other work and synchronisations in between; every replay gives
+    the eager result bit for bit, also after the inputs have changed in place."""
+    from falkon_amd import _backend
+    lib = _backend.load()
+    code = _backend.FLK_F32
+    sigma = torch.tensor([2.5], device=dev)
+    X, C, v, w = _inputs(20_000, 1_500, 28, 2, torch.float32, 7, dev)
+    want = torch.empty(1_500, 2, device=dev)
+    got = torch.empty_like(want)
+    eager = torch.cuda.current_stream(dev).cuda_stream
+    _backend.raise_for_status(_call(lib, "flk_gauss_fdmmv_noalloc", X, C, sigma, v, w, want, code, eager), "eager call")
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = _call(lib, "flk_gauss_fdmmv_noalloc", X, C, sigma, v, w, got, code, side.cuda_stream)
+    _backend.raise_for_status(rc, "captured call")
+    for rep in range(4):
+        got.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {rep}"
+        # other work of the program between the replays: a different problem through the same array, new inputs
+        X2, C2, v2, w2 = _inputs(3_000, 200, 9, 1, torch.float32, 50 + rep, dev)
+        tmp = torch.empty(200, 1, device=dev)
+        _backend.raise_for_status(_call(lib, "flk_gauss_fdmmv_noalloc", X2, C2, sigma, v2, w2, tmp, code, eager), "between")
+        v.mul_(1.25)
+        _backend.raise_for_status(_call(lib, "flk_gauss_fdmmv_noalloc", X, C, sigma, v, w, want, code, eager), "eager call")
+        torch.cuda.synchronize()
 
 
 def test_noalloc_rejects_problems_beyond_the_array(dev):
