@@ -9,8 +9,11 @@
 // the accumulator registers are the A operand of fp32 32x32x2, 16x16x1 and 4x4x1 steps whose B operand comes from a
 // stage of the A block's right-hand sides that the four waves of the workgroup share.  The bf16 chains run on the
 // matrix cores beside the fp32 instructions (the exponentials and the fp32 contraction steps of the other wave of the
-// SIMD), so a pass costs about what its exponentials and its contraction cost.  Passes of 32 and 64 columns contract on
-// the bf16 matrix cores as well (wide_contract_bf16 below).
+// SIMD), so a pass costs about what its exponentials and its contraction cost.  The contraction itself stays on the
+// fp32 steps at every width: done on the bf16 matrix cores as well (kernel values and right-hand sides split three
+// ways) it was a third faster at 32 and 64 columns, but a column whose terms cancel came out a digit further from the
+// fp64 result than with the fp32 steps (1.4e-5 against 1.6e-6 for a 200-fold cancellation), which is not the accuracy
+// this mode promises.
 #include "kernel_fn.h"
 #include "split_common.h"
 #include "mmv_wide_common.h"
@@ -55,91 +58,6 @@ __device__ __forceinline__ void split_wide_stage(const SplitWideRowVals<COLS> &r
     for (int c = 0; c < COLS / 8; c++) lds[32 + r * WideGeo<COLS>::kStride + p0 + 8 * c] = rv.x[c];
 }
 
-// ---------------------------------------------------------------------------
-// Contraction on the bf16 matrix cores (passes of 32 and 64 columns).  The kernel values and the right-hand sides are
-// split three ways like the data (x = hi + mid + lo, bfloat16 pieces, see split3_pair), and K v is accumulated from the
-// same six partial products as the cross term.
-// Register s of a lane holds K[i][j] with i = 8 (s / 4) + 4 h + s % 4: the eight registers 8 c .. 8 c + 7 of a lane are
-// the k values of a 32x32x16 step c for the lane's output row j, so the A operand is those eight values packed; the B
-// operand is vec[the same eight rows][t = lane % 32], which the stage holds as one 16-byte piece per (group, piece,
-// step, lane half, column).
-// ---------------------------------------------------------------------------
-template <int COLS> struct SplitWideBf16Geo {
-    static constexpr int kGroups = COLS / 32;
-    static constexpr int kStageDw = kGroups * 3 * 2 * 2 * 32 * 4;      // dwords: [group][piece][step][half][column][8 bf16]
-};
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-// (x, y) = hi + mid + lo, each piece the pair of bfloat16 numbers nearest to what the previous pieces leave (the
-// subtractions are exact), x in the low half of the words: v_cvt_pk_bf16_f32 rounds to nearest even, as the packing of
-// the data does.  (Pieces by truncation would carry the same 24 bits, but the partial products that are dropped are then
-// eight times larger and all of one sign: a column whose terms cancel 200-fold came out at 2.3e-5 instead of 1.6e-6.)
-__device__ __forceinline__ void split3_pair(float x, float y, unsigned (&piece)[3]) {
-    floatx2 r = {x, y};
-#pragma unroll
-    for (int p = 0; p < 3; p++) {
-        piece[p] = __builtin_bit_cast(unsigned, __builtin_convertvector(r, bf16x2));
-        if (p < 2) {
-            r[0] -= __uint_as_float(piece[p] << 16);
-            r[1] -= __uint_as_float(piece[p] & 0xffff0000u);
-        }
-    }
-}
-
-template <int COLS>
-__device__ __forceinline__ void split_wide_stage_bf16(const SplitWideRowVals<COLS> &rv, unsigned short *lds, int tid) {
-    const int r = tid & 31, p0 = tid >> 5;
-    // row r = 16 c + 8 e1 + 4 h + e0 is element e = 4 e1 + e0 of step c in lane half h
-    const int c = r >> 4, e = 4 * ((r >> 3) & 1) + (r & 3), h = (r >> 2) & 1;
-#pragma unroll
-    for (int cc = 0; cc < COLS / 8; cc += 2) {
-        unsigned piece[3];
-        split3_pair(rv.x[cc], rv.x[cc + 1], piece);
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-            const int col = p0 + 8 * (cc + u), g = col >> 5, t = col & 31;
-#pragma unroll
-            for (int p = 0; p < 3; p++)
-                lds[((((g * 3 + p) * 2 + c) * 2 + h) * 32 + t) * 8 + e] = (unsigned short)(u ? piece[p] >> 16 : piece[p] & 0xffffu);
-        }
-    }
-}
-
-template <int FR, int COLS>
-__device__ __forceinline__ void wide_contract_bf16(const floatx16 (&acc)[FR], const uintx4 *lds, int lane,
-                                                   WideAcc<FR, COLS> &out) {
-    constexpr int kGroups = COLS / 32;
-    // partial products, lowest order first: (mid,mid) (hi,lo) (lo,hi) (hi,mid) (mid,hi) (hi,hi)
-    constexpr int kPieceA[6] = {1, 0, 2, 0, 1, 0}, kPieceB[6] = {1, 2, 0, 1, 0, 0};
-#pragma unroll
-    for (int c = 0; c < 2; c++) {
-        uintx4 a[FR][3];
-#pragma unroll
-        for (int q = 0; q < FR; q++) {
-#pragma unroll
-            for (int e2 = 0; e2 < 4; e2++) {
-                unsigned piece[3];
-                split3_pair(acc[q][8 * c + 2 * e2], acc[q][8 * c + 2 * e2 + 1], piece);
-#pragma unroll
-                for (int p = 0; p < 3; p++) a[q][p][e2] = piece[p];
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < kGroups; g++) {
-            uintx4 b[3];
-#pragma unroll
-            for (int p = 0; p < 3; p++) b[p] = lds[(((g * 3 + p) * 2 + c) * 2) * 32 + lane];   // half h, column t: lane = 32 h + t
-#pragma unroll
-            for (int pr = 0; pr < 6; pr++)
-#pragma unroll
-                for (int q = 0; q < FR; q++)
-                    out.g32[q][g] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[q][kPieceA[pr]]),
-                                                                            __builtin_bit_cast(bf16x8, b[kPieceB[pr]]),
-                                                                            out.g32[q][g], 0, 0, 0);
-        }
-    }
-}
-
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
 template <int KS, int FR, int KF, int COLS>
 __global__ void __launch_bounds__(64 * kSplitWideWaves, 2)
@@ -147,10 +65,7 @@ __global__ void __launch_bounds__(64 * kSplitWideWaves, 2)
                           const uintx4 *__restrict__ PB, int64_t na_blocks, int64_t nb_blocks, int64_t a_chunk_blocks,
                           float *__restrict__ partial, int64_t nb_pad, int tcols, bool y_fastest) {
     using G = WideGeo<COLS>;
-    // passes of 32 and 64 columns contract on the bf16 matrix cores, the others on the fp32 steps
-    constexpr bool kBf16 = split_wide_bf16_contraction(COLS, KS);
-    constexpr int kStageWords = kBf16 ? SplitWideBf16Geo<kBf16 ? COLS : 32>::kStageDw : G::kStage;
-    __shared__ __attribute__((aligned(16))) float stage[2][kStageWords];   // shared by the four waves
+    __shared__ __attribute__((aligned(16))) float stage[2][G::kStage];   // shared by the four waves
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
     const int tid = threadIdx.x;
@@ -184,8 +99,7 @@ __global__ void __launch_bounds__(64 * kSplitWideWaves, 2)
     if (a0 < a1) {
         load_split_wide<KS>(fa, PA, a0, lane);
         split_wide_fetch<COLS>(rv, vecp, vec_ld, tcols, a0, tid);
-        if constexpr (kBf16) split_wide_stage_bf16<COLS>(rv, (unsigned short *)stage[0], tid);
-        else split_wide_stage<COLS>(rv, stage[0], tid);
+        split_wide_stage<COLS>(rv, stage[0], tid);
     }
     wide_barrier();
     // One barrier per A block: a stage is written after the barrier that follows its last reader and read after the
@@ -221,13 +135,8 @@ __global__ void __launch_bounds__(64 * kSplitWideWaves, 2)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[q][r] = kernel_value<KF>(acc[q][r]);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (kBf16) {
-            wide_contract_bf16<FR, COLS>(acc, (const uintx4 *)lds, lane, out);
-            if (has1) split_wide_stage_bf16<COLS>(rv, (unsigned short *)stage[buf ^ 1], tid);
-        } else {
-            wide_contract<FR, COLS>(acc, lds, j, h, out);
-            if (has1) split_wide_stage<COLS>(rv, stage[buf ^ 1], tid);
-        }
+        wide_contract<FR, COLS>(acc, lds, j, h, out);
+        if (has1) split_wide_stage<COLS>(rv, stage[buf ^ 1], tid);
         wide_barrier();
         buf ^= 1;
     }

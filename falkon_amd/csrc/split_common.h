@@ -31,7 +31,6 @@ inline int64_t split_ksteps(int64_t d) { return (d + 2 + 15) / 16; }
 constexpr int64_t kSplitWideMaxD = kSplitMaxD;
 constexpr int kSplitWideMaxCols = 64;
 constexpr int kSplitWideBlocksPerWave = 2;
-constexpr bool split_wide_bf16_contraction(int cols, int ks) { return (cols == 32 || cols == 64) && ks <= 3; }
 constexpr int split_wide_form_cols(int tcols, int ks) {
     return tcols <= 8 ? 8 : tcols <= 16 ? 16 : tcols <= 32 ? 32 : tcols <= 40 ? 40 : tcols <= 48 && ks >= 3 ? 48 : 64;
 }

@@ -169,6 +169,31 @@ def test_accuracy_is_that_of_the_fp32_kernels(dev, scale):
     assert e_split <= 1.5 * e_plain + 2e-7, (e_split, e_plain)
 
 
+@pytest.mark.parametrize("d,t", [(28, 32), (28, 64), (40, 33), (9, 64), (46, 100)])
+def test_cancelling_columns_with_many_right_hand_sides(dev, d, t):
+    """Columns whose terms cancel two hundredfold (a nearly constant kernel matrix against right-hand sides that sum to
+    almost nothing), at the widths of the 32- and 64-column passes: the mode may not be further from the fp64 result
+    than the plain fp32 kernels are (the same bound as above, on the worst column), for K v and for K^T(K v)."""
+    g = np.random.default_rng(300 + d + t)
+    n, m = 3000, 2048
+    X = torch.from_numpy(g.standard_normal((n, d)).astype(np.float32))
+    C = torch.from_numpy(g.standard_normal((m, d)).astype(np.float32))
+    z = g.standard_normal((m, t))
+    v = torch.from_numpy((z - z.mean(0) * (1 - 1 / 200)).astype(np.float32))
+    sigma = torch.tensor([12.0 * np.sqrt(d)], dtype=torch.float64)             # K within a few percent of 1
+    K = brute.radial_brute(X, C, sigma, "gaussian")
+    exact_m = K @ v.double().numpy()
+    exact_d = K.T @ exact_m
+    cancel = np.abs(exact_m).sum(0) / (np.abs(K) @ np.abs(v.double().numpy())).sum(0)
+    assert cancel.max() < 0.05                                                   # the columns do cancel
+    Xg, Cg, vg = X.to(dev), C.to(dev), v.to(dev)
+    ks, kp = GaussianKernel(sigma, opt=SPLIT), GaussianKernel(sigma, opt=PLAIN)
+    e_split, e_plain = rel_err(ks.mmv(Xg, Cg, vg), exact_m), rel_err(kp.mmv(Xg, Cg, vg), exact_m)
+    assert e_split <= 1.5 * e_plain + 2e-7, ("mmv", e_split, e_plain)
+    e_split, e_plain = rel_err(ks.dmmv(Xg, Cg, vg, None), exact_d), rel_err(kp.dmmv(Xg, Cg, vg, None), exact_d)
+    assert e_split <= 1.5 * e_plain + 2e-7, ("dmmv", e_split, e_plain)
+
+
 def test_config2_and_config3_shapes_reduced(dev):
     for name, N, M in (("C2", 100_000, 5_000), ("C3", 200_000, 5_000)):
         X, C, sigma, v, w = inputs.make_config(name, N=N, M=M)
