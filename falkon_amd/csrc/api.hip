@@ -72,6 +72,9 @@ constexpr int64_t kWideChunkBlocks = 64;  // column chunks wider than 4 accumula
 // given) instead of the rules for large problems; kTinyChunkBlocks is the shortest chunk that is worth a workgroup's
 // prologue and its partial result, whose cost is counted as kWgOverheadPercent / 100 of a block step.
 constexpr int64_t kComputeUnits = 256;
+constexpr int64_t kResidentWgs = 2 * kComputeUnits;   // the register-resident kernels run two workgroups per compute unit
+constexpr int64_t kMinRounds = 10;
+constexpr int64_t kWgOverheadBlocks = 5;
 constexpr int64_t kUnderfilledWgs = 4 * kComputeUnits;
 constexpr int64_t kTinyChunkBlocks = 2;
 constexpr int64_t kWgOverheadPercent = 50;
@@ -98,9 +101,11 @@ static void plan_register_resident(Plan &p, int64_t na_blocks, int64_t nb_blocks
     if (max_splits < 1) max_splits = 1;
     if (splits > max_splits) splits = max_splits;
     p.col_chunk = col_chunk;
+    int64_t min_splits = 1;            // what the chunk caps below ask for
     if (t > 4 && p.col_chunk > 4 && elem_bytes == 4) {     // (fp64 sums need no such cap: C2's shape with 64 columns
         int64_t want = (na_blocks + kWideChunkBlocks - 1) / kWideChunkBlocks;   // would write 10 GB of partial sums)
         if (splits < want) splits = want;
+        if (min_splits < want) min_splits = want;
     }
     // a reduction chunk is streamed by every output tile that shares it: keep it within half of one XCD's
     // 4 MB L2 so that those re-reads hit L2 instead of HBM (only where there is more than one output tile)
@@ -114,9 +119,36 @@ static void plan_register_resident(Plan &p, int64_t na_blocks, int64_t nb_blocks
         const int64_t affordable = kL2PartialBytes / (per_split > 0 ? per_split : 1);
         if (want > affordable) want = affordable;
         if (splits < want) splits = want;
+        if (min_splits < want) min_splits = want;
     }
     if (splits > kMaxSplits) splits = kMaxSplits;
     if (splits < 1) splits = 1;
+    if (b_tiles * splits >= kUnderfilledWgs && na_blocks > 0 && b_tiles > 0) {
+        // Large problem: between the split count that gives kMinRounds rounds of resident workgroups and the one chosen so
+        // far, take the one with the shortest estimated run.  A workgroup costs its chunk plus a fixed overhead
+        // (dispatch, loading its resident blocks, its partial result: about kWgOverheadBlocks block steps), so fewer,
+        // longer workgroups are cheaper, as long as there are enough rounds for the workgroups to drift apart and
+        // the last, partly filled round is not nearly empty: that round is counted as 0.35 + 0.65 x of a full one
+        // when a fraction x of the slots is used.  Measured on config 2 (fp32): K v with 5 splits (9770 workgroups)
+        // -> 3 (5862): 9.46 -> 9.35 ms per launch; K^T u with 203 splits (8120) -> 128 (5120): 9.44 -> 9.40 ms, while
+        // 104 splits (4160 = 8.1 rounds) take 9.60 ms.  The lower bounds set above (chunk caps) are kept.
+        int64_t lo = (kMinRounds * kResidentWgs + b_tiles - 1) / b_tiles;
+        if (lo < 1) lo = 1;
+        if (lo < splits) {
+            if (min_splits > lo) lo = min_splits;
+            int64_t best = splits, best_cost = -1;
+            for (int64_t s = lo; s <= splits; s++) {
+                int64_t c = (na_blocks + s - 1) / s;
+                if (t == 1 && c > 1 && (c & 1)) c += 1;
+                const int64_t wgs = b_tiles * ((na_blocks + c - 1) / c);
+                const int64_t full = wgs / kResidentWgs, rem = wgs % kResidentWgs;
+                const int64_t rounds_milli = full * 1000 + (rem ? 350 + 650 * rem / kResidentWgs : 0);
+                const int64_t cost = rounds_milli * (c + kWgOverheadBlocks);
+                if (best_cost < 0 || cost < best_cost) { best = s; best_cost = cost; }
+            }
+            splits = best;
+        }
+    }
     if (b_tiles * splits < kUnderfilledWgs && na_blocks > 0 && b_tiles > 0) {
         // small problem: the split count with the shortest estimated makespan, at least the one chosen so far (the
         // chunk caps above still hold); ties go to fewer splits
