@@ -72,11 +72,24 @@ __device__ __forceinline__ void stage_rowvals(const RowVals<TT> &rv, float *lds,
     __builtin_amdgcn_wave_barrier();
 }
 
+// (the block's base address is wave-uniform, i.e. scalar arithmetic where the block index is a scalar, and the lane's
+// part a 32-bit offset: computed per lane in 64 bits the addresses of a two-block trip cost a dozen multi-cycle vector
+// instructions, which do not overlap with the MFMAs)
+// a wave-uniform 64-bit value as a pair of scalars
+__device__ __forceinline__ int64_t as_scalar(int64_t v) {
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 template <int DP>
 __device__ __forceinline__ void load_a(float (&a)[DP], const float *__restrict__ PA, int64_t ab, int j, int h) {
-    const float *p = PA + (ab * (2 * DP) + (int64_t)h * DP) * 32 + j;
+    // one block index per wave; the pointer keeps its global address space through the round trip
+    typedef const float __attribute__((address_space(1))) *global_floats;
+    const global_floats blk = (global_floats)as_scalar((int64_t)(PA + ab * (2 * DP * 32)));
+    const int off = h * (DP * 32) + j;
 #pragma unroll
-    for (int s = 0; s < DP; s++) a[s] = p[s * 32];
+    for (int s = 0; s < DP; s++) a[s] = blk[off + s * 32];
 }
 
 // FOLD: the accumulators start from the A block's half norms alone (the output side's half norm arrives through the
@@ -189,6 +202,8 @@ __device__ __forceinline__ void reduce_blocks(const float *__restrict__ PA, cons
     using RV = RowVals<TT>;
     float fa0[DP], fa1[DP];
     RV rv;
+    a0 = as_scalar(a0);      // the chunk's bounds are the same for the whole wave: block indices stay scalar
+    a1 = as_scalar(a1);
     if (a0 >= a1) return;
     int since_flush = 0;
     // One right-hand side and four resident blocks (the kernels of the single-column products at up to 32 features):
@@ -205,22 +220,28 @@ __device__ __forceinline__ void reduce_blocks(const float *__restrict__ PA, cons
         // The scheduling barriers keep the phases of a step apart in the generated code: the loads of the next block
         // are issued before the tile's arithmetic, and the staging of its row values, which has to wait for their
         // load, stays behind the tile (hoisted to the front it waits out a full memory latency with nothing in flight).
-        const int64_t last = a1 - 1;
-        fetch_rowvals<TT>(rv, src, a0);
-        load_a<DP>(fa0, PA, a0, j, h);
+        // Block indices count from the chunk's first block, in 32 bits: the loop's comparisons and the blocks' base
+        // addresses are then scalar instructions (a 64-bit less-than exists on the vector ALU only).
+        const float *const PAc = PA + a0 * (2 * DP * 32);
+        const float *srcc[RV::C];
+#pragma unroll
+        for (int c = 0; c < RV::C; c++) srcc[c] = src[c] + a0 * 32;
+        const int nblk = (int)(a1 - a0), last = nblk - 1;
+        fetch_rowvals<TT>(rv, srcc, 0);
+        load_a<DP>(fa0, PAc, 0, j, h);
         stage_rowvals<TT>(rv, lds0, lane);
-        for (int64_t ab = a0; ab < a1; ab += 2) {
-            const bool second = ab + 1 < a1;
-            const int64_t n1 = second ? ab + 1 : last;
-            fetch_rowvals<TT>(rv, src, n1);    // first: staged right after this tile step
-            load_a<DP>(fa1, PA, n1, j, h);
+        for (int ab = 0; ab < nblk; ab += 2) {
+            const bool second = ab + 1 < nblk;
+            const int n1 = second ? ab + 1 : last;
+            fetch_rowvals<TT>(rv, srcc, n1);    // first: staged right after this tile step
+            load_a<DP>(fa1, PAc, n1, j, h);
             __builtin_amdgcn_sched_barrier(0);
             tile_step<DP, FR, TT, NOADD, KF, RAW, true>(fa0, lds0, h, breg, hb, o1);
             __builtin_amdgcn_sched_barrier(0);
             stage_rowvals<TT>(rv, lds1, lane, second);
-            const int64_t n2 = ab + 2 < last ? ab + 2 : last;
-            fetch_rowvals<TT>(rv, src, n2);
-            load_a<DP>(fa0, PA, n2, j, h);
+            const int n2 = ab + 2 < last ? ab + 2 : last;
+            fetch_rowvals<TT>(rv, srcc, n2);
+            load_a<DP>(fa0, PAc, n2, j, h);
             __builtin_amdgcn_sched_barrier(0);
             tile_step<DP, FR, TT, NOADD, KF, RAW, true>(fa1, lds1, h, breg, hb, o1);
             __builtin_amdgcn_sched_barrier(0);
