@@ -97,6 +97,22 @@ __device__ __forceinline__ void xcd_remap_banded(unsigned &bx, unsigned &by) {
 }
 #endif
 
+#if defined(__HIPCC__)
+// A wave-uniform 64-bit value as a pair of scalars, and a wave-uniform global address as a scalar base: loads through
+// it take the form "scalar base + 32-bit lane offset", and the arithmetic that leads to the base is scalar too.  (Per-lane
+// 64-bit address arithmetic runs on the vector ALU, where it does not overlap with the MFMAs.)  The pointer keeps its
+// global address space through the round trip; a generic pointer would turn the loads into flat loads.
+__device__ __forceinline__ int64_t as_scalar(int64_t v) {
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+template <typename T>
+__device__ __forceinline__ const T __attribute__((address_space(1))) *scalar_base(const T *p) {
+    return (const T __attribute__((address_space(1))) *)as_scalar((int64_t)p);
+}
+#endif
+
 // error plumbing -------------------------------------------------------------
 int fail(int code, const char *fmt, ...);
 #define FLK_HIP(expr)                                                                      \

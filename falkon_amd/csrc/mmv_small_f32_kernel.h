@@ -75,18 +75,9 @@ __device__ __forceinline__ void stage_rowvals(const RowVals<TT> &rv, float *lds,
 // (the block's base address is wave-uniform, i.e. scalar arithmetic where the block index is a scalar, and the lane's
 // part a 32-bit offset: computed per lane in 64 bits the addresses of a two-block trip cost a dozen multi-cycle vector
 // instructions, which do not overlap with the MFMAs)
-// a wave-uniform 64-bit value as a pair of scalars
-__device__ __forceinline__ int64_t as_scalar(int64_t v) {
-    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
-    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)((uint64_t)v >> 32));
-    return (int64_t)(((uint64_t)hi << 32) | lo);
-}
-
 template <int DP>
 __device__ __forceinline__ void load_a(float (&a)[DP], const float *__restrict__ PA, int64_t ab, int j, int h) {
-    // one block index per wave; the pointer keeps its global address space through the round trip
-    typedef const float __attribute__((address_space(1))) *global_floats;
-    const global_floats blk = (global_floats)as_scalar((int64_t)(PA + ab * (2 * DP * 32)));
+    const auto blk = scalar_base(PA + ab * (2 * DP * 32));      // one block index per wave
     const int off = h * (DP * 32) + j;
 #pragma unroll
     for (int s = 0; s < DP; s++) a[s] = blk[off + s * 32];

@@ -34,13 +34,15 @@ template <int DP, int TT>
 __device__ __forceinline__ void load_afrag64(AFrag64<DP, TT> &f, const double *__restrict__ PA,
                                              const double *__restrict__ hA, const double *__restrict__ vecp,
                                              int64_t vec_ld, int64_t ab, int j, int q) {
-    const double *p = PA + (ab * (4 * DP) + (int64_t)q * DP) * 16 + j;
+    // scalar block bases, 32-bit lane offsets (flk_common.h: scalar_base)
+    const auto blk = scalar_base(PA + ab * (4 * DP * 16));
+    const int off = q * (DP * 16) + j;
 #pragma unroll
-    for (int s = 0; s < DP; s++) f.a[s] = p[s * 16];
-    const int64_t r0 = ab * 16 + 4 * q;
-    f.hn = *(const doublex4 *)(hA + r0);
+    for (int s = 0; s < DP; s++) f.a[s] = blk[off + s * 16];
+    typedef const doublex4 __attribute__((address_space(1))) *rows4;
+    f.hn = *(rows4)(scalar_base(hA + ab * 16) + 4 * q);
 #pragma unroll
-    for (int t = 0; t < TT; t++) f.vec[t] = *(const doublex4 *)(vecp + t * vec_ld + r0);
+    for (int t = 0; t < TT; t++) f.vec[t] = *(rows4)(scalar_base(vecp + t * vec_ld + ab * 16) + 4 * q);
 }
 
 // RAW (Gaussian only): the output rows' half norms stay out of the exponent (they multiply the finished sums), so the
@@ -79,14 +81,23 @@ __device__ __forceinline__ void reduce_blocks64(const double *__restrict__ PA, c
                                                 int j, int q, const double (&breg)[FR][DP], const double (&hb)[FR],
                                                 double (&o1)[FR][TT], double (&o2)[FR][TT], const double *exp_tab) {
     AFrag64<DP, TT> f0, f1;
-    if (a0 < a1) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, a0, j, q);
+    // the chunk's bounds are the same for the whole wave; block indices count from its first block, in 32 bits, so
+    // that the loop's comparisons and the blocks' base addresses are scalar instructions
+    a0 = as_scalar(a0);
+    a1 = as_scalar(a1);
+    if (a0 >= a1) return;
+    PA += a0 * (4 * DP * 16);
+    hA += a0 * 16;
+    vecp += a0 * 16;
+    const int nblk = (int)(a1 - a0);
+    load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, 0, j, q);
     int since_flush = 0;
-    for (int64_t ab = a0; ab < a1; ab += 2) {
-        const bool has1 = ab + 1 < a1;
+    for (int ab = 0; ab < nblk; ab += 2) {
+        const bool has1 = ab + 1 < nblk;
         if (has1) load_afrag64<DP, TT>(f1, PA, hA, vecp, vec_ld, ab + 1, j, q);
         tile_step64<DP, FR, TT, RAW>(f0, breg, hb, o1, exp_tab);
         if (has1) {
-            if (ab + 2 < a1) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, ab + 2, j, q);
+            if (ab + 2 < nblk) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, ab + 2, j, q);
             tile_step64<DP, FR, TT, RAW>(f1, breg, hb, o1, exp_tab);
         }
         since_flush += 2;
