@@ -292,7 +292,7 @@ static int pack_impl(int kf, const void *X, int64_t n, int64_t d, int64_t rs, in
     PackedView v = packed_view<T>(packed, n, d);
     // odd-d fp32 operands of the register-resident kernel carry 1.0 in their one padding feature
     const bool one_pad = sizeof(T) == 4 && f32_fold_applies(d);
-    return launch_pack<T, T>((const T *)X, n, d, rs, cs, (const T *)sigma, n_sigma, operand_scale(kf), (T *)v.data,
+    return launch_pack<T, T>((const T *)X, n, d, rs, cs, (const T *)sigma, n_sigma, operand_scale(kf, sizeof(T) == 8), (T *)v.data,
                              (T *)v.hnorm, v.dpad, v.nblk, one_pad, st);
 }
 
@@ -314,7 +314,7 @@ static int pack_pair_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int6
     const bool one_pad = sizeof(T) == 4 && f32_fold_applies(d);
     return launch_pack_pair<T>((const T *)X1, n, x1_rs, x1_cs, (T *)P1.data, (T *)P1.hnorm, P1.nblk, (const T *)X2, m,
                                x2_rs, x2_cs, (T *)P2.data, (T *)P2.hnorm, P2.nblk, d, (const T *)sigma, n_sigma,
-                               operand_scale(kf), P1.dpad, one_pad, (const T *)v, v_rs, v_cs, vp, t, zero_planes, st);
+                               operand_scale(kf, sizeof(T) == 8), P1.dpad, one_pad, (const T *)v, v_rs, v_cs, vp, t, zero_planes, st);
 }
 
 template <typename T>
@@ -444,11 +444,11 @@ static int fmm_impl(int kf, const void *X1, int64_t n, int64_t x1_rs, int64_t x1
     if (ws_bytes < need || ws == nullptr)
         return fail(FLK_ENOMEM, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
     PackedView P1 = packed_view<T>(ws, n, d), P2 = packed_view<T>((char *)ws + packed_bytes<T>(n, d), m, d);
-    if ((rc = launch_pack<TI, T>((const TI *)X1, n, d, x1_rs, x1_cs, (const TI *)sigma, n_sigma, operand_scale(kf),
+    if ((rc = launch_pack<TI, T>((const TI *)X1, n, d, x1_rs, x1_cs, (const TI *)sigma, n_sigma, operand_scale(kf, sizeof(T) == 8),
                                  (T *)P1.data,
                                  (T *)P1.hnorm, P1.dpad, P1.nblk, false, st)))
         return rc;
-    if ((rc = launch_pack<TI, T>((const TI *)X2, m, d, x2_rs, x2_cs, (const TI *)sigma, n_sigma, operand_scale(kf),
+    if ((rc = launch_pack<TI, T>((const TI *)X2, m, d, x2_rs, x2_cs, (const TI *)sigma, n_sigma, operand_scale(kf, sizeof(T) == 8),
                                  (T *)P2.data,
                                  (T *)P2.hnorm, P2.dpad, P2.nblk, false, st)))
         return rc;
@@ -572,7 +572,7 @@ static int pack_split_impl(int kf, const char *name, const void *X, int64_t n, i
     if (n_sigma != 1 && n_sigma != d)
         return fail(FLK_EINVAL, "The size of sigma (%lld) must match the number of features (%lld) or be 1",
                     (long long)n_sigma, (long long)d);
-    return launch_pack_split((const float *)X, n, d, rs, cs, (const float *)sigma, n_sigma, operand_scale(kf), packed, st);
+    return launch_pack_split((const float *)X, n, d, rs, cs, (const float *)sigma, n_sigma, operand_scale(kf, false), packed, st);
 }
 
 static size_t fmmv_split_ws_bytes(int64_t n, int64_t m, int64_t d, int64_t t) {

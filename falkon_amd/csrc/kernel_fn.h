@@ -6,7 +6,8 @@
 // (D = |x/sigma - c/sigma|, L = log2 e):
 //
 //   Gaussian   (falkon/kernels/distance_kernel.py:140-159): scale sqrt(L), e = -L D^2/2, K = exp2(e); the
-//              reference's clamp of the squared distance at 1e-20 is K <= 1;
+//              reference's clamp of the squared distance at 1e-20 is K <= 1; (in double precision the scale is
+//              sqrt(2048 L) and K = exp2(e / 2048), see kGaussExpBits;)
 //   Laplacian  (distance_kernel.py:182-205): scale sqrt(2) L, -e = (L D)^2 =: q^2, K = exp(-D) = exp2(-q);
 //   Matern 3/2 (distance_kernel.py:243-254): scale sqrt(6) L, q = L s with s = sqrt(3) D,
 //              K = (1 + s) exp(-s) = (1 + q/L) exp2(-q);
@@ -29,14 +30,22 @@ constexpr double kSqrt2 = 1.4142135623730951;
 constexpr double kSqrt3 = 1.7320508075688772;
 constexpr double kSqrt5 = 2.23606797749979;
 
-// factor on x / sigma when a matrix is packed for the kernel
-inline double operand_scale(int kf) {
+// The Gaussian's exponent in double precision is carried times 2^kGaussExpBits (the packed rows take the square root of
+// that factor, the half norms the factor itself, at no cost): the accumulator then holds E = 2048 e, whose integer and
+// fractional parts are what the table-based exponential needs (exp2_table_scaled), one conversion and one v_fract_f64
+// instead of the three additions that round e to a multiple of 1/2048.
+constexpr int kGaussExpBits = 11;
+constexpr double kGaussExpScale = 2048.0;
+constexpr double kSqrtGaussExpScale = 45.254833995939045;       // sqrt(2048)
+
+// factor on x / sigma when a matrix is packed for the kernel (packed_f64: the packed operand is double precision)
+inline double operand_scale(int kf, bool packed_f64) {
     switch (kf) {
         case FLK_LAPLACIAN:
         case FLK_LAPLACIAN_DU: return kLog2e * kSqrt2;
         case FLK_MATERN32:  return kSqrt3 * kLog2e * kSqrt2;
         case FLK_MATERN52:  return kSqrt5 * kLog2e * kSqrt2;
-        default:            return kSqrtLog2e;
+        default:            return packed_f64 ? kSqrtLog2e * kSqrtGaussExpScale : kSqrtLog2e;
     }
 }
 
@@ -126,13 +135,35 @@ __device__ __forceinline__ double exp2_table(double e, const double *tab) {
     return __builtin_ldexp(y, N >> kExpTableBits);
 }
 
-// How a kernel function evaluates 2^x in double precision: by polynomial, or from the table in LDS
+// 2^(E / 2048) for E <= 0 from the same table: N = ceil(E) (v_cvt_i32_f64 truncates towards zero and saturates, so no
+// clamp is needed: from -2^31 on the result is 0), x = E - N = -fract(-E) in (-1, 0], 2^(E/2048) = 2^(N >> 11) *
+// tab[N & 2047] * 2^(x/2048); the last factor is 1 + fx (a1 + fx (a2 + fx a3)) with fx = -x, the cubic through the
+// Chebyshev nodes of (2^y - 1) / y on [-2^-11, 0] (relative error 1.7e-17 before rounding, exactly 1 at x = 0).
+// Eight fp64 and three 32-bit instructions per value.  E must not be positive: ceil and fract would disagree there.
+template <bool ON_FMA = true>
+__device__ __forceinline__ double exp2_table_scaled(double E, const double *tab) {
+    const int N = (int)E;
+    const double fx = __builtin_amdgcn_fract(-E);
+    double p = fma(-0x1.c6a1c7b96fda5p-38, fx, 0x1.ebfbdfcbdb733p-25);
+    p = fma(p, fx, -0x1.62e42fefa38b4p-12);
+    p = fma(p, fx, 1.0);
+    const double entry = tab[N & (kExpTableSize - 1)];
+    double y;
+    if constexpr (ON_FMA) asm("v_fma_f64 %0, %1, %2, 0" : "=v"(y) : "v"(p), "v"(entry));
+    else y = p * entry;
+    return __builtin_ldexp(y, N >> kExpTableBits);
+}
+
+// How a kernel function evaluates 2^x in double precision: by polynomial, or from the table in LDS.  scaled(E) is
+// 2^(E / 2048) for E <= 0, the Gaussian's form.
 struct Exp2Poly {
     __device__ __forceinline__ double operator()(double e) const { return exp2_nonpositive(e); }
+    __device__ __forceinline__ double scaled(double E) const { return exp2_nonpositive(E * (1.0 / kGaussExpScale)); }
 };
 template <bool ON_FMA> struct Exp2Table {
     const double *tab;
     __device__ __forceinline__ double operator()(double e) const { return exp2_table<ON_FMA>(e, tab); }
+    __device__ __forceinline__ double scaled(double E) const { return exp2_table_scaled<ON_FMA>(E, tab); }
 };
 
 template <int KF> struct KernelFn;
@@ -142,8 +173,9 @@ template <> struct KernelFn<FLK_GAUSSIAN> {
     static __device__ __forceinline__ float value(float e) {
         return __builtin_amdgcn_fmed3f(__builtin_amdgcn_exp2f(e), 0.0f, 1.0f);
     }
+    // (double precision: the accumulator holds 2048 e, see kGaussExpBits)
     template <class E> static __device__ __forceinline__ double value(double e, E ex) {
-        return ex(fmin(e, 0.0));
+        return ex.scaled(fmin(e, 0.0));
     }
 };
 

@@ -20,6 +20,15 @@ namespace flk {
 
 typedef double doublex4 __attribute__((ext_vector_type(4)));
 
+// The Gaussian's half norms and exponents are carried times 2048 (kernel_fn.h, kGaussExpBits).  Where the output rows'
+// half norms are factored out of the sums (RAW), the exponent x.c + hA is bounded by -hB of the output row and can be
+// positive, which the exponential does not take: every wave shifts it down by the largest -hB of its resident rows,
+// rounded up to the next whole bit, so that it is negative, and multiplies the shift back into the finished sums.  The
+// rows' -hB may be up to kRawMaxBits bits: a term that matters for a row (within 2^-60 of its largest) is then no
+// smaller than 2^-(kRawMaxBits + 60), far inside the normal range.  (A constant shift would be simpler, but the
+// exponent would then always carry the rounding error of a number that size, 3e-14 of the kernel value at 450 bits.)
+constexpr double kRawMaxBits = 449.0;
+
 constexpr int kWavesPerWg64 = 4;
 constexpr int kFlushEvery64 = 16;
 
@@ -49,12 +58,17 @@ __device__ __forceinline__ void load_afrag64(AFrag64<DP, TT> &f, const double *_
 // accumulators start from the A block's half norms alone and the kernel value is the bare 2^e, not clamped at 1.
 template <int DP, int FR, int TT, bool RAW>
 __device__ __forceinline__ void tile_step64(const AFrag64<DP, TT> &f, const double (&breg)[FR][DP],
-                                            const double (&hb)[FR], double (&o1)[FR][TT], const double *exp_tab) {
+                                            const double (&hb)[FR], double (&o1)[FR][TT], const double *exp_tab,
+                                            double raw_shift) {
     doublex4 acc[FR];
+    // RAW: the exponent is shifted down by the wave's raw_shift (four subtractions per A block)
+    doublex4 hn_raw;
+#pragma unroll
+    for (int r = 0; r < 4; r++) hn_raw[r] = f.hn[r] - raw_shift;
 #pragma unroll
     for (int c = 0; c < FR; c++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) acc[c][r] = RAW ? f.hn[r] : f.hn[r] + hb[c];
+        for (int r = 0; r < 4; r++) acc[c][r] = RAW ? hn_raw[r] : f.hn[r] + hb[c];
 #pragma unroll
     for (int s = 0; s < DP; s++)
 #pragma unroll
@@ -67,8 +81,8 @@ __device__ __forceinline__ void tile_step64(const AFrag64<DP, TT> &f, const doub
             // LDS latency: those variants evaluate the polynomial; measured d = 28, T = 4: 16.2 ms against 18.8)
             double k;
             if constexpr (TT <= 2)
-                k = RAW ? exp2_table<(DP > 4)>(acc[c][r], exp_tab) : kernel_value<FLK_KF, (DP > 4)>(acc[c][r], exp_tab);
-            else k = RAW ? exp2_nonpositive(acc[c][r]) : kernel_value<FLK_KF>(acc[c][r]);
+                k = RAW ? exp2_table_scaled<(DP > 4)>(acc[c][r], exp_tab) : kernel_value<FLK_KF, (DP > 4)>(acc[c][r], exp_tab);
+            else k = RAW ? Exp2Poly{}.scaled(acc[c][r]) : kernel_value<FLK_KF>(acc[c][r]);
 #pragma unroll
             for (int t = 0; t < TT; t++) o1[c][t] = __builtin_fma(k, f.vec[t][r], o1[c][t]);
         }
@@ -79,7 +93,8 @@ template <int DP, int FR, int TT, bool RAW>
 __device__ __forceinline__ void reduce_blocks64(const double *__restrict__ PA, const double *__restrict__ hA,
                                                 const double *__restrict__ vecp, int64_t vec_ld, int64_t a0, int64_t a1,
                                                 int j, int q, const double (&breg)[FR][DP], const double (&hb)[FR],
-                                                double (&o1)[FR][TT], double (&o2)[FR][TT], const double *exp_tab) {
+                                                double (&o1)[FR][TT], double (&o2)[FR][TT], const double *exp_tab,
+                                                double raw_shift) {
     AFrag64<DP, TT> f0, f1;
     // the chunk's bounds are the same for the whole wave; block indices count from its first block, in 32 bits, so
     // that the loop's comparisons and the blocks' base addresses are scalar instructions
@@ -95,10 +110,10 @@ __device__ __forceinline__ void reduce_blocks64(const double *__restrict__ PA, c
     for (int ab = 0; ab < nblk; ab += 2) {
         const bool has1 = ab + 1 < nblk;
         if (has1) load_afrag64<DP, TT>(f1, PA, hA, vecp, vec_ld, ab + 1, j, q);
-        tile_step64<DP, FR, TT, RAW>(f0, breg, hb, o1, exp_tab);
+        tile_step64<DP, FR, TT, RAW>(f0, breg, hb, o1, exp_tab, raw_shift);
         if (has1) {
             if (ab + 2 < nblk) load_afrag64<DP, TT>(f0, PA, hA, vecp, vec_ld, ab + 2, j, q);
-            tile_step64<DP, FR, TT, RAW>(f1, breg, hb, o1, exp_tab);
+            tile_step64<DP, FR, TT, RAW>(f1, breg, hb, o1, exp_tab, raw_shift);
         }
         since_flush += 2;
         if (since_flush >= kFlushEvery64) {
@@ -154,24 +169,32 @@ __global__ void __launch_bounds__(256, 2)
         for (int t = 0; t < TT; t++) { o1[c][t] = 0.0; o2[c][t] = 0.0; }
 
     // Gaussian: 2^hB_j is taken out of the sums, out_j = 2^hB_j sum_i 2^(x_i.c_j + hA_i) vec_i, which saves an add and
-    // the clamp per kernel value, as long as 2^(-hB_j) is nowhere near the fp64 range; every wave checks its own
+    // the clamp per kernel value, as long as 2^(-hB_j) is nowhere near the fp64 range (kRawMaxBits); every wave checks its own
     // resident rows (rows with a non-finite half norm fail the check).  On that path a kernel value is not clamped
     // entry by entry: where two points coincide K is 1 to rounding instead of exactly 1.
     constexpr bool kCanFactorOut = KF == FLK_GAUSSIAN;
     bool factored = false;
+    double raw_shift = 0.0;
     if constexpr (kCanFactorOut) {
         bool small_norms = true;
+        double most = 0.0;             // largest -hB among the wave's resident rows, in units of 1/2048 bit
 #pragma unroll
-        for (int c = 0; c < FR; c++) small_norms = small_norms && hb[c] >= -900.0;
+        for (int c = 0; c < FR; c++) {
+            small_norms = small_norms && hb[c] >= -kRawMaxBits * kGaussExpScale;
+            most = fmax(most, -hb[c]);
+        }
         factored = __all(small_norms);
+        for (int off = 32; off > 0; off >>= 1) most = fmax(most, __shfl_xor(most, off, 64));
+        // a whole number of bits above it: both factors 2^(-shift/2048) and 2^(shift/2048) are then exact powers of two
+        raw_shift = (floor(most * (1.0 / kGaussExpScale)) + 1.0) * kGaussExpScale;
     }
     if (kCanFactorOut && factored)
-        reduce_blocks64<DP, FR, TT, true>(PA, hA, vecp, vec_ld, a0, a1, j, q, breg, hb, o1, o2, exp_tab);
+        reduce_blocks64<DP, FR, TT, true>(PA, hA, vecp, vec_ld, a0, a1, j, q, breg, hb, o1, o2, exp_tab, raw_shift);
     else
-        reduce_blocks64<DP, FR, TT, false>(PA, hA, vecp, vec_ld, a0, a1, j, q, breg, hb, o1, o2, exp_tab);
+        reduce_blocks64<DP, FR, TT, false>(PA, hA, vecp, vec_ld, a0, a1, j, q, breg, hb, o1, o2, exp_tab, 0.0);
 #pragma unroll
     for (int c = 0; c < FR; c++) {
-        const double out_scale = (kCanFactorOut && factored) ? exp2_nonpositive(hb[c]) : 1.0;
+        const double out_scale = (kCanFactorOut && factored) ? exp2_nonpositive((hb[c] + raw_shift) * (1.0 / kGaussExpScale)) : 1.0;
 #pragma unroll
         for (int t = 0; t < TT; t++) {
             double s = o2[c][t] + o1[c][t];

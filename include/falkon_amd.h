@@ -78,8 +78,8 @@ int flk_kernel_timing_read(double *total_ms, int64_t *launches);
 
 /* ---- packed operands ------------------------------------------------------
  * The kernels consume each data matrix in a "packed" form: rows are scaled by
- * a kernel-specific factor over sigma (sqrt(log2 e) for the Gaussian: a packed
- * operand is only valid for the kernel it was packed for), regrouped in blocks of 32 (f32) or 16 (f64) rows stored
+ * a kernel-specific factor over sigma (sqrt(log2 e) for the Gaussian in f32, sqrt(2048 log2 e) in f64: a packed
+ * operand is only valid for the kernel and the dtype it was packed for), regrouped in blocks of 32 (f32) or 16 (f64) rows stored
  * feature-major, zero padded, and followed by the vector -1/2*||row||^2.
  * This replaces the reference's per-block `mat / sigma` and `square_norm`
  * prologue of rbf_core (falkon/kernels/distance_kernel.py:148-154;

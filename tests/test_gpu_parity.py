@@ -617,6 +617,7 @@ def test_packed_entry_points(dev, dtype, n, m, d, t):
         _backend.raise_for_status(rc, "flk_gauss_pack")
         packed[name] = buf
     # layout: [block][feature][row] (fp64 rows permuted inside a block), then -1/2 |x~|^2, x~ = sqrt(log2 e) x / sigma
+    # (fp64: x~ = sqrt(2048 log2 e) x / sigma: the Gaussian's exponent is carried times 2048 in double precision)
     if d <= 64:
         dpad = (d + 1) // 2 * 2 if dtype == torch.float32 else (d + 3) // 4 * 4
     else:
@@ -624,7 +625,7 @@ def test_packed_entry_points(dev, dtype, n, m, d, t):
     nblk = (n + blk - 1) // blk
     flat = packed["X"].view(dtype)
     data = flat[:nblk * dpad * blk].view(nblk, dpad, blk)
-    scaled = (X.double() * np.sqrt(np.log2(np.e)) / sigma.double())
+    scaled = (X.double() * np.sqrt(np.log2(np.e) * (1.0 if dtype == torch.float32 else 2048.0)) / sigma.double())
     pos = torch.arange(blk) if dtype == torch.float32 else torch.tensor([4 * (r % 4) + r // 4 for r in range(blk)])
     rows = torch.arange(n)
     got_rows = data[rows // blk, :d, pos[rows % blk]]
