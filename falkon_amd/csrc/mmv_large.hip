@@ -74,6 +74,24 @@ __device__ __forceinline__ const T *stage_src(const T *__restrict__ P, int64_t b
     return P + (b * dpad + (s0 + s) * TR::KG + lg) * TR::BLK + jv * TR::VPL;
 }
 
+// The same address as a scalar base (block and chunk: the same for the 64 lanes of a wave) plus the lane's 32-bit offset
+// inside the chunk, which does not change from chunk to chunk or tile to tile.
+template <typename T, int KC>
+__device__ __forceinline__ int stage_lane_offset(int vi) {
+    typedef LTraits<T> TR;
+    constexpr int VPB = TR::BLK / TR::VPL;
+    const int jv = vi % VPB, lg = (vi / VPB) % TR::KG, s = (vi / (VPB * TR::KG)) % KC;
+    return (s * TR::KG + lg) * TR::BLK + jv * TR::VPL;
+}
+template <typename T, int KC>
+__device__ __forceinline__ auto stage_base(const T *__restrict__ P, int64_t blk0, int64_t nblk, int64_t dpad, int vi) {
+    typedef LTraits<T> TR;
+    constexpr int VPB = TR::BLK / TR::VPL;
+    int64_t b = blk0 + __builtin_amdgcn_readfirstlane(vi / (VPB * TR::KG * KC));
+    if (b >= nblk) b = nblk - 1;                 // past the end: any valid block (its rows get zero weight / are not stored)
+    return scalar_base(P + b * dpad * TR::BLK);
+}
+
 // KF (= FLK_KF) is a template parameter only to give every kernel function's instantiations their own symbols
 // O = void: the product (partial sums of K against vec).  O = an element type: the kernel matrix itself, entry
 // (a, b) stored as O at kout[a * kout_ld + b] (then TT = 1, vecp is not read and partial not written).
@@ -155,6 +173,17 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
             for (int r = 0; r < TR::ACCN; r++) out2[q][g][r] = T(0);
 
+    // where a thread's staged vectors come from: offsets inside a chunk (fixed), bases of the output tile's blocks (fixed)
+    int aoff[G::A_VPT], boff[G::B_VPT];
+    decltype(scalar_base(PB)) bbase[G::B_VPT];
+#pragma unroll
+    for (int c = 0; c < G::A_VPT; c++) aoff[c] = stage_lane_offset<T, KC>(tid + c * kLThreads);
+#pragma unroll
+    for (int c = 0; c < G::B_VPT; c++) {
+        boff[c] = stage_lane_offset<T, KC>(tid + c * kLThreads);
+        bbase[c] = stage_base<T, KC>(PB, bblk0, nb_blocks, dpad, tid + c * kLThreads);
+    }
+
     for (int64_t at = at0; at < at1; at++) {
         const int64_t ablk0 = at * G::NAB;
         acc_t acc[WA_FR][WB_FR];
@@ -167,14 +196,19 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 
         V16 ra[G::A_VPT], rb[G::B_VPT];
         constexpr bool kScalarBlk = sizeof(T) == 4 && TT >= 48;
+        // global addresses: a scalar base per staged block (the tile's blocks; the chunk adds a scalar offset) plus the
+        // lane's 32-bit offset inside a chunk
+        typedef const V16 __attribute__((address_space(1))) *global_v16;
+        decltype(scalar_base(PA)) abase[G::A_VPT];
+#pragma unroll
+        for (int c = 0; c < G::A_VPT; c++) abase[c] = stage_base<T, KC>(PA, ablk0, na_blocks, dpad, tid + c * kLThreads);
+        typedef const T __attribute__((address_space(1))) *global_t;
         auto fetch = [&](int64_t chunk) {
-            const int64_t s0 = chunk * KC;
+            const int64_t s0 = chunk * (KC * TR::KG * TR::BLK * (int64_t)sizeof(T));      // bytes
 #pragma unroll
-            for (int c = 0; c < G::A_VPT; c++)
-                ra[c] = *(const V16 *)stage_src<T, KC, kScalarBlk>(PA, ablk0, na_blocks, dpad, s0, tid + c * kLThreads);
+            for (int c = 0; c < G::A_VPT; c++) ra[c] = *(global_v16)((global_t)as_scalar((int64_t)abase[c] + s0) + aoff[c]);
 #pragma unroll
-            for (int c = 0; c < G::B_VPT; c++)
-                rb[c] = *(const V16 *)stage_src<T, KC, kScalarBlk>(PB, bblk0, nb_blocks, dpad, s0, tid + c * kLThreads);
+            for (int c = 0; c < G::B_VPT; c++) rb[c] = *(global_v16)((global_t)as_scalar((int64_t)bbase[c] + s0) + boff[c]);
         };
         auto commit = [&](int buf) {
 #pragma unroll
