@@ -239,6 +239,9 @@ __device__ __forceinline__ void reduce_blocks(const float *__restrict__ PA, cons
             stage_rowvals<TT>(rv, lds0, lane);
             since_flush += 2;
             if (TWO_LEVEL && since_flush >= kFlushEvery) {
+                // (the empty asm keeps this a branch taken every eighth trip: turned into selects it costs a dozen
+                // vector instructions in every trip)
+                asm volatile("" ::: "memory");
                 since_flush = 0;
 #pragma unroll
                 for (int q = 0; q < FR; q++)
