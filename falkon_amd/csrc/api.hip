@@ -85,6 +85,7 @@ struct Plan {
     int splits;            // grid.y
     int partials;          // partial results the finalize kernel sums (= splits x partials per split)
     int col_chunk;         // right-hand sides per pass
+    int a_tile_blocks = 0; // LDS-tiled kernel: reduction blocks per tile that chunk counts in
     int64_t dpad = 0;      // padded feature count of the operands (register-resident kernels)
 };
 
@@ -188,7 +189,8 @@ static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t d
                                dpad * Geo<T>::BLK * (int64_t)sizeof(T), Geo<T>::BLK, mmv_small_max_cols<T>(dpad, t), t,
                                (int64_t)sizeof(T));
     } else {
-        const int64_t a_tiles = (na_blocks + mmv_large_a_tile_blocks<T>() - 1) / mmv_large_a_tile_blocks<T>();
+        p.a_tile_blocks = mmv_large_a_tile_blocks<T>(t);
+        const int64_t a_tiles = (na_blocks + p.a_tile_blocks - 1) / p.a_tile_blocks;
         const int64_t b_tiles = (nb_blocks + mmv_large_b_tile_blocks<T>(t) - 1) / mmv_large_b_tile_blocks<T>(t);
         int64_t splits = (kTargetWgsLarge + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
         if (splits > a_tiles) splits = a_tiles;
@@ -265,7 +267,7 @@ static int mmv_packed_planar(int kf, const PackedView &A, const PackedView &B, c
             partials = 0;  // empty reduction: finalize sums nothing and writes the addend (or zero)
         } else {
             ScopedKernelTimer timer(st);
-            int rc = p.large ? launch_mmv_large<T>(kf, A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st)
+            int rc = p.large ? launch_mmv_large<T>(kf, A, B, vecp + t0 * A.npad, A.npad, tc, p.a_tile_blocks, p.chunk, p.splits, partial, st)
                              : launch_mmv_small<T>(kf, A, B, vecp + t0 * A.npad, A.npad, tc, p.chunk, p.splits, partial, st);
             if (rc != FLK_OK) return rc;
         }

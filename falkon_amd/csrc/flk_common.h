@@ -182,7 +182,7 @@ constexpr int64_t kColPad = 31;
 
 // LDS-tiled ("large d") product kernel: any padded feature count, up to mmv_large_max_cols columns per pass.
 // Writes splits * mmv_large_partials_per_split partial results.
-template <typename T> int mmv_large_a_tile_blocks();
+template <typename T> int mmv_large_a_tile_blocks(int64_t t);   // reduction blocks per tile with t columns in all
 template <typename T> int mmv_large_b_tile_blocks(int64_t t);   // output blocks per workgroup with t columns in all
 template <typename T> int mmv_large_partials_per_split();
 template <typename T> int mmv_large_max_cols(int64_t t);   // columns per pass when there are t in all
@@ -208,7 +208,8 @@ template <typename T> int mmv_large_max_cols(int64_t t);   // columns per pass w
                                          double *partial, hipStream_t st);                                        \
     template <typename T>                                                                                         \
     int launch_mmv_large_kf##KF(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld,          \
-                                int tcols, int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st);    \
+                                int tcols, int a_tile_blocks, int64_t a_tiles_per_chunk, int splits, T *partial,  \
+                                hipStream_t st);                                                                  \
     template <typename T, typename O>                                                                             \
     int launch_fmm_kf##KF(const PackedView &A, const PackedView &B, O *out, int64_t ld, hipStream_t st);          \
     template <typename T, typename O>                                                                             \
@@ -242,8 +243,9 @@ inline int launch_mmv_small(int kf, const PackedView &A, const PackedView &B, co
 }
 template <typename T>
 inline int launch_mmv_large(int kf, const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
-                            int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
-#define FLK_CALL(KF) launch_mmv_large_kf##KF<T>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st)
+                            int a_tile_blocks, int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
+#define FLK_CALL(KF) \
+    launch_mmv_large_kf##KF<T>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st)
     FLK_SWITCH_KF(kf, FLK_CALL)
 #undef FLK_CALL
 }

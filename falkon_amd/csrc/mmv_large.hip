@@ -275,7 +275,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
         // the one barrier of the chunk sits BEFORE the last step's MFMAs: by then every wave holds its last
         // operands in registers, so right after the barrier a wave issues the reads of the next chunk's
         // first step and covers their latency with the MFMAs it still has to issue.
-        static_assert(WA_FR == 4 && WB_FR == 2, "the step fence lists its operands explicitly");
+        static_assert((WA_FR == 4 || WA_FR == 8) && WB_FR == 2, "the step fence lists its operands explicitly");
         constexpr int kCommitStep = KC / 2;
         static_assert(KC % 2 == 0, "the two operand sets alternate by step and must line up across chunks");
         T av[2][WA_FR], bv[2][WB_FR];          // operand sets: step s uses set s%2 while set (s+1)%2 is being read
@@ -314,6 +314,10 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                 asm volatile("" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[1][0]), "+v"(acc[1][1]),
                                   "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[3][0]), "+v"(acc[3][1])
                              : "v"(la), "v"(lb) : "memory");
+                if constexpr (WA_FR == 8)
+                    asm volatile("" : "+v"(acc[4][0]), "+v"(acc[4][1]), "+v"(acc[5][0]), "+v"(acc[5][1]),
+                                      "+v"(acc[6][0]), "+v"(acc[6][1]), "+v"(acc[7][0]), "+v"(acc[7][1])
+                                 : "v"(la), "v"(lb) : "memory");
 #pragma unroll
                 for (int p = 0; p < WA_FR; p++)
 #pragma unroll
@@ -542,11 +546,14 @@ template <typename T> struct LCfg;
 // fp32: 4 waves (2 x 2), two workgroups per CU so that one workgroup's barrier and LDS latencies are covered
 // by the other; tile 256 (A) x 128 (B) rows.
 template <> struct LCfg<float>  { static constexpr int WVA = 2, WVB = 2, WA_FR = 4, WB_FR = 2, KC = 8; };
-// fp64: 8 waves (2 x 4), one workgroup per CU; tile 128 (A) x 128 (B) rows.  (Feature stages of four steps instead of
-// eight, which would leave room for the exponential's table in LDS, were measured over d = 65 .. 1000: 3 to 7 % faster
-// below 128 features, 2 to 3 % slower from 256 on with up to four columns, and the table itself gained nothing in this
-// kernel's epilogue, where eight waves read it at once; not kept.)
-template <> struct LCfg<double> { static constexpr int WVA = 2, WVB = 4, WA_FR = 4, WB_FR = 2, KC = 8; };
+// fp64: 8 waves (2 x 4), one workgroup per CU; tile 256 (A) x 128 (B) rows in feature stages of four steps: every wave
+// holds 8 x 2 accumulator blocks (128 registers), so that a byte staged through LDS feeds a third more MFMAs than on a
+// 128 x 128 tile in stages of eight steps, which the kernel used before (measured, dfmmv at N = 5e5, M = 1e4, d = 784, 10
+// columns: 245.5 -> 239.4 ms; one column 241.8 -> 238.3, 16 columns 247.0 -> 242.6; N = 5e5, M = 2e4, d = 100: 76.1 -> 73.2,
+// 10 columns 88.0 -> 83.4; N = 2.5e5, M = 2e4, d = 300: 97.5 -> 95.4).  (On the 128 x 128 tile, stages of four steps
+// instead of eight were 3 to 7 % faster below 128 features and 2 to 3 % slower from 256 on; the exponential's table in
+// LDS gained nothing in this kernel's epilogue, where eight waves read it at once.)
+template <> struct LCfg<double> { static constexpr int WVA = 2, WVB = 4, WA_FR = 8, WB_FR = 2, KC = 4; };
 
 // fp32 with 17 .. 32 columns: the row values of an A tile take 34 KB of LDS, two workgroups with the 48 KB of feature
 // stages each no longer fit a CU; 8 waves (2 x 4) on a 256 x 256 tile, one workgroup per CU.
@@ -557,7 +564,12 @@ struct LCfgWide64 { static constexpr int WVA = 2, WVB = 4, WA_FR = 4, WB_FR = 2,
 
 constexpr int kLargeMaxCols = 16;
 #if FLK_KF == FLK_GAUSSIAN   // the tile geometry is the same for every kernel function: defined once
-template <typename T> int mmv_large_a_tile_blocks() { return LCfg<T>::WVA * LCfg<T>::WA_FR; }
+// Reduction blocks per tile: every pass of a call walks the same tiles, so the count follows the call's columns in all
+// (fp64 beyond 16 columns: the 128-row tile of the many-column configuration, also for a last pass of few columns).
+template <typename T> int mmv_large_a_tile_blocks(int64_t t) {
+    if (sizeof(T) == 8 && t > kLargeMaxCols) return LCfgWide64::WVA * LCfgWide64::WA_FR;
+    return LCfg<T>::WVA * LCfg<T>::WA_FR;
+}
 template <typename T> int mmv_large_b_tile_blocks(int64_t t) {
     if (sizeof(T) == 4 && t > kLargeMaxCols) return LCfgWide32::WVB * LCfgWide32::WB_FR;
     return LCfg<T>::WVB * LCfg<T>::WB_FR;
@@ -568,8 +580,8 @@ template <typename T> int mmv_large_max_cols(int64_t t) {
 }
 template int mmv_large_max_cols<float>(int64_t);
 template int mmv_large_max_cols<double>(int64_t);
-template int mmv_large_a_tile_blocks<float>();
-template int mmv_large_a_tile_blocks<double>();
+template int mmv_large_a_tile_blocks<float>(int64_t);
+template int mmv_large_a_tile_blocks<double>(int64_t);
 template int mmv_large_b_tile_blocks<float>(int64_t);
 template int mmv_large_b_tile_blocks<double>(int64_t);
 template int mmv_large_partials_per_split<float>();
@@ -578,7 +590,10 @@ template int mmv_large_partials_per_split<double>();
 
 template <typename T, int TT, typename C = LCfg<T>>
 static int launch_large_tt(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld, int tcols,
-                           int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
+                           int a_tile_blocks, int64_t a_tiles_per_chunk, int splits, T *partial, hipStream_t st) {
+    if (a_tile_blocks != C::WVA * C::WA_FR)
+        return fail(FLK_EINVAL, "mmv_large: the launch plan counts tiles of %d blocks, the kernel's hold %d", a_tile_blocks,
+                    C::WVA * C::WA_FR);
     const int64_t nbb = C::WVB * C::WB_FR;
     dim3 grid((unsigned)((B.nblk + nbb - 1) / nbb), (unsigned)splits);
     // feature chunks that hold features of the data, and the MFMA steps of the last of them that do
@@ -631,36 +646,39 @@ template int FLK_CAT(launch_fmm_large_kf, FLK_KF)<double, float>(const PackedVie
 
 template <typename T>
 int FLK_CAT(launch_mmv_large_kf, FLK_KF)(const PackedView &A, const PackedView &B, const T *vecp, int64_t vec_ld,
-                                         int tcols, int64_t a_tiles_per_chunk, int splits, T *partial,
-                                         hipStream_t st) {
+                                         int tcols, int a_tile_blocks, int64_t a_tiles_per_chunk, int splits,
+                                         T *partial, hipStream_t st) {
     if (A.dpad != B.dpad) return fail(FLK_EINVAL, "mmv_large: operands packed with different feature counts");
     const int most = 4 * kLargeMaxCols;
     if (tcols < 1 || tcols > most) return fail(FLK_EINVAL, "mmv_large: column chunk %d not in 1..%d", tcols, most);
     if (tcols > kLargeMaxCols) {
         if constexpr (sizeof(T) == 4) {
             if (tcols > 3 * kLargeMaxCols)
-                return launch_large_tt<T, 64, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+                return launch_large_tt<T, 64, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
             if (tcols > 2 * kLargeMaxCols)       // 33 to 48 columns: a group of 32 and a group of 16
-                return launch_large_tt<T, 48, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
-            return launch_large_tt<T, 32, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+                return launch_large_tt<T, 48, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
+            return launch_large_tt<T, 32, LCfgWide32>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
         } else {
             if (tcols > 3 * kLargeMaxCols)
-                return launch_large_tt<T, 64, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+                return launch_large_tt<T, 64, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
             if (tcols > 2 * kLargeMaxCols)       // 33 to 48 columns: three groups of 16
-                return launch_large_tt<T, 48, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
-            return launch_large_tt<T, 32, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+                return launch_large_tt<T, 48, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
+            return launch_large_tt<T, 32, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
         }
     }
-    if (tcols == 1) return launch_large_tt<T, 1>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
-    if (tcols == 2) return launch_large_tt<T, 2>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
-    if (tcols <= 4) return launch_large_tt<T, 4>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
+    if constexpr (sizeof(T) == 8)       // a last pass of few columns behind passes of many: on their tiles
+        if (a_tile_blocks == LCfgWide64::WVA * LCfgWide64::WA_FR && a_tile_blocks != LCfg<T>::WVA * LCfg<T>::WA_FR)
+            return launch_large_tt<T, 32, LCfgWide64>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
+    if (tcols == 1) return launch_large_tt<T, 1>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
+    if (tcols == 2) return launch_large_tt<T, 2>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
+    if (tcols <= 4) return launch_large_tt<T, 4>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
     if constexpr (kLargeFmaCols<T> == 8)
-        if (tcols <= 8) return launch_large_tt<T, 8>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);
-    return launch_large_tt<T, 16>(A, B, vecp, vec_ld, tcols, a_tiles_per_chunk, splits, partial, st);   // MFMA epilogue
+        if (tcols <= 8) return launch_large_tt<T, 8>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);
+    return launch_large_tt<T, 16>(A, B, vecp, vec_ld, tcols, a_tile_blocks, a_tiles_per_chunk, splits, partial, st);   // MFMA epilogue
 }
 template int FLK_CAT(launch_mmv_large_kf, FLK_KF)<float>(const PackedView &, const PackedView &, const float *, int64_t,
-                                                         int, int64_t, int, float *, hipStream_t);
+                                                         int, int, int64_t, int, float *, hipStream_t);
 template int FLK_CAT(launch_mmv_large_kf, FLK_KF)<double>(const PackedView &, const PackedView &, const double *,
-                                                          int64_t, int, int64_t, int, double *, hipStream_t);
+                                                          int64_t, int, int, int64_t, int, double *, hipStream_t);
 
 }  // namespace flk
