@@ -201,7 +201,9 @@ int flk_cg_update(int mode, void *X, void *R, void *P, const void *Q, const void
  *      part below the diagonal blocks is read.
  *   dinv, dinv_t: inverses of the diagonal blocks L[k*block .. , k*block ..] and the transposes of those inverses,
  *      block k at + k*block*block elements, row-major with leading dimension `block` (a smaller last block keeps
- *      that leading dimension); the caller computes them once per factor.  block: a multiple of 4.
+ *      that leading dimension); the caller computes them once per factor.  The inverses are triangular, and the
+ *      kernels read a few entries on the other side of the diagonal (rows are processed four at a time): those
+ *      entries must be stored as zeros.  block: a multiple of 4.
  *   transposed == 0 solves L x = b, otherwise L^T x = b.
  *   b, x: t columns of m elements each, column c at + c*ldb, + c*ldx; work: flk_tri_solve_work_elems(m, t, block)
  *      elements of the data dtype (partial sums of the panel products); three distinct buffers.
