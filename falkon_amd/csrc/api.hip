@@ -72,7 +72,6 @@ constexpr int64_t kWideChunkBlocks = 64;  // column chunks wider than 4 accumula
 // given) instead of the rules for large problems; kTinyChunkBlocks is the shortest chunk that is worth a workgroup's
 // prologue and its partial result, whose cost is counted as kWgOverheadPercent / 100 of a block step.
 constexpr int64_t kComputeUnits = 256;
-constexpr int64_t kResidentWgs = 2 * kComputeUnits;   // the register-resident kernels run two workgroups per compute unit
 constexpr int64_t kMinRounds = 10;
 constexpr int64_t kWgOverheadBlocks = 5;
 constexpr int64_t kUnderfilledWgs = 4 * kComputeUnits;
@@ -93,9 +92,11 @@ constexpr int64_t kTargetWgsLarge = 16384;  // two 256-thread workgroups per CU:
 
 // Plan of a register-resident product kernel: per_wg output blocks per workgroup, a_block_bytes per packed
 // reduction block of blk rows, col_chunk right-hand sides per pass, results of elem_bytes per element.
+// wgs_per_cu: workgroups of the kernel that a compute unit holds at once.
 static void plan_register_resident(Plan &p, int64_t na_blocks, int64_t nb_blocks, int64_t per_wg, int64_t a_block_bytes,
-                                   int64_t blk, int col_chunk, int64_t t, int64_t elem_bytes) {
+                                   int64_t blk, int col_chunk, int64_t t, int64_t elem_bytes, int wgs_per_cu = 2) {
     p.large = false;
+    const int64_t kResidentWgs = wgs_per_cu * kComputeUnits;
     const int64_t b_tiles = (nb_blocks + per_wg - 1) / per_wg;
     int64_t splits = (kTargetWgs + b_tiles - 1) / (b_tiles > 0 ? b_tiles : 1);
     int64_t max_splits = na_blocks / kMinChunkBlocks;
@@ -183,11 +184,11 @@ template <typename T>
 static Plan make_plan(int64_t na_blocks, int64_t nb_blocks, int64_t d, int64_t dpad, int64_t t) {
     Plan p;
     p.dpad = dpad;
-    p.large = d > mmv_small_max_d<T>();
+    p.large = !mmv_small_serves<T>(d, t);
     if (!p.large) {
         plan_register_resident(p, na_blocks, nb_blocks, mmv_small_b_blocks_per_wg<T>(dpad, t),
                                dpad * Geo<T>::BLK * (int64_t)sizeof(T), Geo<T>::BLK, mmv_small_max_cols<T>(dpad, t), t,
-                               (int64_t)sizeof(T));
+                               (int64_t)sizeof(T), mmv_small_wgs_per_cu<T>(dpad, t));
     } else {
         p.a_tile_blocks = mmv_large_a_tile_blocks<T>(t);
         const int64_t a_tiles = (na_blocks + p.a_tile_blocks - 1) / p.a_tile_blocks;

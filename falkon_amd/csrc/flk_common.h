@@ -171,8 +171,12 @@ int launch_cg_update(int mode, T *X, T *R, T *P, const T *Q, const T *B, int64_t
 
 // Register-resident ("small d") product kernel; the queries do not depend on the kernel function.
 template <typename T> int64_t mmv_small_max_d();
+// Whether the register-resident kernels serve a product of d features with t right-hand sides in all (beyond
+// mmv_small_max_d: some single-column products, on operands padded for the LDS-tiled kernel).
+template <typename T> bool mmv_small_serves(int64_t d, int64_t t);
 // (t: right-hand sides of the call; the fp32 kernels switch to their 32-column variant beyond a few columns)
 template <typename T> int mmv_small_b_blocks_per_wg(int64_t dpad, int64_t t);
+template <typename T> int mmv_small_wgs_per_cu(int64_t dpad, int64_t t);      // workgroups of that kernel a CU holds at once
 template <typename T> int mmv_small_max_cols(int64_t dpad, int64_t t);   // right-hand sides per pass
 template <typename T> int mmv_small_width(int64_t dpad, int tc);         // planes the kernel serving tc columns reads
 

@@ -75,9 +75,13 @@ __device__ __forceinline__ void stage_rowvals(const RowVals<TT> &rv, float *lds,
 // (the block's base address is wave-uniform, i.e. scalar arithmetic where the block index is a scalar, and the lane's
 // part a 32-bit offset: computed per lane in 64 bits the addresses of a two-block trip cost a dozen multi-cycle vector
 // instructions, which do not overlap with the MFMAs)
+// Floats of a packed block of 32 rows whose features are consumed in DP steps: 2 DP features up to 64, and the
+// feature count padded for the LDS-tiled kernel (whole chunks of kLargeKChunk steps, zeros past the data) beyond.
+constexpr int block_floats(int dp) { return (dp <= 32 ? 2 * dp : (2 * dp + 2 * (int)kLargeKChunk - 1) / (2 * (int)kLargeKChunk) * (2 * (int)kLargeKChunk)) * 32; }
+
 template <int DP>
 __device__ __forceinline__ void load_a(float (&a)[DP], const float *__restrict__ PA, int64_t ab, int j, int h) {
-    const auto blk = scalar_base(PA + ab * (2 * DP * 32));      // one block index per wave
+    const auto blk = scalar_base(PA + ab * block_floats(DP));      // one block index per wave
     const int off = h * (DP * 32) + j;
 #pragma unroll
     for (int s = 0; s < DP; s++) a[s] = blk[off + s * 32];
@@ -213,7 +217,7 @@ __device__ __forceinline__ void reduce_blocks(const float *__restrict__ PA, cons
         // load, stays behind the tile (hoisted to the front it waits out a full memory latency with nothing in flight).
         // Block indices count from the chunk's first block, in 32 bits: the loop's comparisons and the blocks' base
         // addresses are then scalar instructions (a 64-bit less-than exists on the vector ALU only).
-        const float *const PAc = PA + a0 * (2 * DP * 32);
+        const float *const PAc = PA + a0 * block_floats(DP);
         const float *srcc[RV::C];
 #pragma unroll
         for (int c = 0; c < RV::C; c++) srcc[c] = src[c] + a0 * 32;
@@ -291,7 +295,9 @@ constexpr float kFactorOutMaxBits = 64.0f;
 // x.c + hA can be positive, so on that path a kernel value is not clamped entry by entry: where two points
 // coincide K is 1 to rounding (1 + 1e-6 at worst) instead of exactly 1.
 template <int DP, int FR, int TT, bool FOLD, int KF>
-__global__ void __launch_bounds__(256, 2)   // two waves per SIMD: at most 256 registers per lane
+// Two waves per SIMD (at most 256 registers per lane), except the single-column kernel with four resident blocks beyond
+// 32 features: its resident fragments alone take up to 128 registers, and it runs one wave per SIMD on up to 512.
+__global__ void __launch_bounds__(256, (DP > 16 && FR == 4) ? 1 : 2)
     mmv_small_f32_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
                          int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB, int64_t na_blocks,
                          int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial, int64_t nb_pad,

@@ -226,6 +226,7 @@ constexpr int fr64_for(int dp, int fr, int tt) {
 
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<double>() { return 4 * kMaxDp64Fr2; }
+template <> bool mmv_small_serves<double>(int64_t d, int64_t) { return d <= 4 * kMaxDp64Fr2; }
 // more than four right-hand sides: the 16-column kernel of mmv_small_f64_wide.hip, which reads 16 planes
 // (beyond 16 columns two groups of 16 share one evaluation of K: 17 columns that way take less time than a
 // 16-column pass and a one-column pass, at every feature count)
@@ -244,6 +245,7 @@ template <> int mmv_small_width<double>(int64_t dpad, int tc) {
     if (tc > kWideCols64) return 2 * kWideCols64;
     return tc > fma_cols64(dpad) ? kWideCols64 : tc;
 }
+template <> int mmv_small_wgs_per_cu<double>(int64_t, int64_t) { return 2; }
 template <> int mmv_small_b_blocks_per_wg<double>(int64_t dpad, int64_t t) {
     const int fr = (dpad / 4) <= kMaxDp64Fr4 ? 4 : 2;
     if (t >= 2 && t <= fma_cols64(dpad)) return kWavesPerWg64 * fr64_for((int)(dpad / 4), fr, (int)t);

@@ -42,6 +42,10 @@ def _rand(n, d, m, t, dtype, seed, scale=1.0):
     (600, 500, 28, 6),
     (500, 400, 31, 21),     # more columns than one pass holds
     (300, 300, 40, 9),      # d > 32: column chunks of four
+    (700, 1300, 40, 1),     # 33 .. 64 features, one column: four resident blocks per wave (fp32), two waves per SIMD
+    (333, 1111, 47, 1),     # ... an odd feature count, and 48 padded features: from there on one wave per SIMD
+    (450, 2049, 63, 1),
+    (450, 700, 50, 2),      # two columns keep two resident blocks
 ])
 def test_mmv_dmmv_vs_oracle(dev, dtype, n, m, d, t):
     X, C, v, w = _rand(n, d, m, t, dtype, seed=n * 7 + m)
@@ -92,7 +96,12 @@ def test_reference_fixture_fp64(dev, order, sig):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("n,m,d,t", [
     (100, 250, 110, 2),     # the reference's large-d shape (tests/test_kernels.py:594-601)
-    (300, 257, 65, 1),      # first d beyond the register-resident kernel
+    (300, 257, 65, 1),      # 65 .. 96 features, one column: the register-resident fp32 kernel on operands packed for the
+    (1500, 1030, 72, 1),    # LDS-tiled one (fp64 and more columns: the LDS-tiled kernel); an odd number of reduction blocks
+    (260, 3000, 81, 1),
+    (900, 520, 96, 1),
+    (900, 520, 97, 1),      # first d beyond it
+    (640, 333, 90, 2),
     (1000, 700, 200, 3),
     (513, 300, 784, 10),    # configuration 4's d and T
     (40, 1100, 131, 17),    # more columns than one pass holds, odd d
