@@ -31,6 +31,7 @@ template <> bool mmv_small_serves<float>(int64_t d, int64_t t) { return d <= 2 *
 template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad, int64_t t) {
     if (t > fma_cols(dpad))
         return kWavesPerWg * wide_blocks_per_wave((int)(dpad / 2), wide_form_cols((int)(t < kWideMaxColumns ? t : kWideMaxColumns)));
+    if (t == 1 && dpad / 2 > kMaxDpFr4OneColumn) return kWavesPerWg * 3;
     return kWavesPerWg * (((dpad / 2) <= kMaxDpFr4 || t == 1) ? 4 : 2);     // (one column: four blocks at every width)
 }
 // The single-column kernel with four resident blocks needs more than 256 registers per lane from 48 padded features on

@@ -205,7 +205,7 @@ __device__ __forceinline__ void reduce_blocks(const float *__restrict__ PA, cons
     // a branch-free loop body with its phases pinned.  Measured on N = 1e6, M = 2e4, dfmmv: d = 28 19.95 -> 19.32 ms,
     // d = 16 12.62 -> 12.29.  The other shapes keep the loop below (with two or four columns the pinned reads do
     // not fit the registers; with two resident blocks it measured slower: d = 64 46.8 -> 51.3 ms).
-    if constexpr (TT == 1 && FR == 4) {
+    if constexpr (TT == 1 && FR >= 3) {
         // Both tile steps of the body always run and every block's loads are issued unconditionally, one block ahead.
         // (With loads or a tile step under a condition the compiler sinks the loads to their use, and at each wait
         // has to assume that they may not have been issued, so it waits for the newest loads instead of the ones it
@@ -295,9 +295,10 @@ constexpr float kFactorOutMaxBits = 64.0f;
 // x.c + hA can be positive, so on that path a kernel value is not clamped entry by entry: where two points
 // coincide K is 1 to rounding (1 + 1e-6 at worst) instead of exactly 1.
 template <int DP, int FR, int TT, bool FOLD, int KF>
-// Two waves per SIMD (at most 256 registers per lane), except the single-column kernel with four resident blocks beyond
-// 32 features: its resident fragments alone take up to 128 registers, and it runs one wave per SIMD on up to 512.
-__global__ void __launch_bounds__(256, (DP > 16 && FR == 4) ? 1 : 2)
+// Two waves per SIMD (at most 256 registers per lane), except the single-column kernels with four (up to 96 features) or
+// three (up to 128) resident blocks beyond 32 features: their resident fragments alone take up to 192 registers, and they
+// run one wave per SIMD on up to 512.
+__global__ void __launch_bounds__(256, (DP > 16 && FR >= 3) ? 1 : 2)
     mmv_small_f32_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
                          int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB, int64_t na_blocks,
                          int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial, int64_t nb_pad,
@@ -309,7 +310,7 @@ __global__ void __launch_bounds__(256, (DP > 16 && FR == 4) ? 1 : 2)
     // (wider column chunks are out of registers with two loops; with two resident blocks per wave, beyond 32 features,
     // the kernel with both loops measured slower than the plain one: d = 64, one column, 46.8 ms per dfmmv at N = 1e6,
     // M = 2e4 against 42.9, d = 40 32.9 against 27.8)
-    constexpr bool kCanFactorOut = !FOLD && KF == FLK_GAUSSIAN && TT <= 2 && FR == 4;
+    constexpr bool kCanFactorOut = !FOLD && KF == FLK_GAUSSIAN && TT <= 2 && FR >= 3;
     __shared__ __attribute__((aligned(16))) float stage[kWavesPerWg][2][RV::N];
     unsigned bx, by;
     xcd_remap(bx, by, y_fastest);
