@@ -27,7 +27,7 @@ constexpr int kWideMaxColumns = 64;    // per pass of the wide kernel
 
 #if FLK_KF == FLK_GAUSSIAN   // the geometry does not depend on the kernel function: defined once
 template <> int64_t mmv_small_max_d<float>() { return 2 * kMaxDpFr2; }
-template <> bool mmv_small_serves<float>(int64_t d, int64_t t) { return d <= 2 * kMaxDpFr2 || (t == 1 && d <= 2 * kMaxDpOneColumn); }
+template <> bool mmv_small_serves<float>(int64_t d, int64_t t) { return d <= 2 * kMaxDpFr2 || (t >= 1 && t <= 4 && d <= 2 * kMaxDpOneColumn); }
 template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad, int64_t t) {
     if (t > fma_cols(dpad))
         return kWavesPerWg * wide_blocks_per_wave((int)(dpad / 2), wide_form_cols((int)(t < kWideMaxColumns ? t : kWideMaxColumns)));
@@ -37,7 +37,7 @@ template <> int mmv_small_b_blocks_per_wg<float>(int64_t dpad, int64_t t) {
 // The single-column kernel with four resident blocks needs more than 256 registers per lane from 48 padded features on
 // and then runs one wave per SIMD; every other form runs two.
 template <> int mmv_small_wgs_per_cu<float>(int64_t dpad, int64_t t) {
-    return (t == 1 && dpad / 2 >= kMinDpOneWave) ? 1 : 2;
+    return ((t == 1 && dpad / 2 >= kMinDpOneWave) || dpad / 2 > kMaxDpFr2) ? 1 : 2;
 }
 template <> int mmv_small_max_cols<float>(int64_t dpad, int64_t t) {
     return t > fma_cols(dpad) ? kWideMaxColumns : fma_cols(dpad);

@@ -298,7 +298,7 @@ template <int DP, int FR, int TT, bool FOLD, int KF>
 // Two waves per SIMD (at most 256 registers per lane), except the single-column kernels with four (up to 96 features) or
 // three (up to 128) resident blocks beyond 32 features: their resident fragments alone take up to 192 registers, and they
 // run one wave per SIMD on up to 512.
-__global__ void __launch_bounds__(256, (DP > 16 && FR >= 3) ? 1 : 2)
+__global__ void __launch_bounds__(256, (DP > 32 || (DP > 16 && FR >= 3)) ? 1 : 2)
     mmv_small_f32_kernel(const float *__restrict__ PA, const float *__restrict__ hA, const float *__restrict__ vecp,
                          int64_t vec_ld, const float *__restrict__ PB, const float *__restrict__ hB, int64_t na_blocks,
                          int64_t nb_blocks, int64_t a_chunk_blocks, float *__restrict__ partial, int64_t nb_pad,

@@ -40,7 +40,7 @@ def _data(n, m, d, t, dtype, seed):
     (200, 131, 28, 1), (513, 300, 9, 3), (257, 100, 64, 1),      # register-resident kernels, folded (d = 9) and plain
     (150, 260, 16, 4), (140, 200, 52, 4),      # column counts where the fp64 kernels differ by kernel function
     (300, 257, 65, 2), (129, 64, 200, 10), (64, 300, 784, 5),    # LDS-tiled kernel, both epilogues
-    (600, 1090, 44, 1), (500, 777, 89, 1), (400, 650, 121, 1),   # one column beyond 32 features (fp32): four resident blocks up to 96 features, three up to 128
+    (600, 1090, 44, 1), (500, 777, 89, 1), (400, 650, 121, 1), (350, 420, 77, 3),   # beyond 32 features (fp32): one column on four resident blocks up to 96 features, three up to 128; few columns on two
 ])
 def test_products_vs_oracle(dev, dtype, name, n, m, d, t):
     X, C, v, w = _data(n, m, d, t, dtype, seed=n + 3 * d)

@@ -105,7 +105,10 @@ def test_reference_fixture_fp64(dev, order, sig):
     (700, 1033, 113, 1),
     (520, 900, 128, 1),
     (520, 900, 129, 1),     # first d beyond the register-resident kernels
-    (640, 333, 90, 2),
+    (640, 333, 90, 2),      # ... two to four columns up to 128 features: two resident blocks per wave
+    (300, 1400, 70, 4),
+    (500, 300, 127, 3),
+    (500, 300, 128, 5),     # five columns beyond 64 features: the LDS-tiled kernel
     (1000, 700, 200, 3),
     (513, 300, 784, 10),    # configuration 4's d and T
     (40, 1100, 131, 17),    # more columns than one pass holds, odd d
