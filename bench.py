@@ -83,8 +83,8 @@ def measured_traffic(workload, dtype, cross_term="f32"):
 
 def product_kernel_name(d, T, dtype):
     """The kernel the library picks for d features and T right-hand sides (csrc/mmv_small_f32.hip, mmv_small_f64.hip)."""
-    if d > 64:
-        return "mmv_large_kernel"
+    if d > 64:      # fp32 with up to four columns: the register-resident kernel up to 128 features
+        return "mmv_small_f32_kernel" if dtype == "f32" and d <= 128 and T <= 4 else "mmv_large_kernel"
     if dtype == "f32":
         steps = (d + 1) // 2
         fma_cols = 6 if 8 < steps <= 16 else 4
@@ -566,6 +566,9 @@ def main():
                     help="C5 only: FalkonOptions(cg_capture_graph=True), the CG iterations replayed from HIP graphs")
     ap.add_argument("--rhs", type=int, default=0, metavar="T",
                     help="right-hand sides instead of the configuration's own number (not a headline workload)")
+    ap.add_argument("--features", type=int, default=0, metavar="D",
+                    help="feature count instead of the configuration's own (C2, C3 or C4 with --no-cpu-baseline; not a "
+                         "headline workload: the same matrices' shape at another d)")
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="only the timed steps of one workload (C2 unless --workload names another): neither the CPU "
                          "baseline, nor the side measurements, nor the other configurations (profiling runs)")
@@ -583,6 +586,12 @@ def main():
         args.steps = 2 if args.workload == "C5" else 50
     if args.warmup is None:
         args.warmup = 1 if args.workload == "C5" else 3
+    if args.features:
+        if args.workload not in WORKLOADS or not args.no_cpu_baseline or args.features < 1:
+            print("bench.py: --features needs --no-cpu-baseline and one of the workloads C2, C3, C4", file=sys.stderr)
+            sys.exit(2)
+        seed, N, _, M, T, has_w = WORKLOADS[args.workload]
+        WORKLOADS[args.workload] = (seed, N, args.features, M, T, has_w)
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only; --gpus must be 1 "
               "(sharding would split the rows of X and end with one M x T all-reduce; it is not built)",
@@ -646,7 +655,7 @@ def main():
             out = torch.empty(M if op == "dmmv" else N, T, dtype=tdt, device=dev)
             call = (lambda: kernel.dmmv(Xg, Cg, vg, wg, out=out)) if op == "dmmv" else (lambda: kernel.mmv(Xg, Cg, vg, out=out))
             meas = measure_products(lib, call, steps, warmup)
-            rec = product_record(workload, op, dtype, N, d, M, T, meas, kernel_name, split, traffic_ok=not rhs)
+            rec = product_record(workload, op, dtype, N, d, M, T, meas, kernel_name, split, traffic_ok=not rhs and not args.features)
             note(f"gpu {workload} {op} {dtype}: {rec['ms_per_step']:.3f} ms per step, roofline frac {rec['roofline']['frac']:.3f}")
             recs[(op, dtype)] = rec
             if args.no_cpu_baseline:
