@@ -3,6 +3,7 @@
 Test infrastructure only.  Everything is generated on the host with numpy's
 ``default_rng`` so the same arrays can be rebuilt anywhere from the seed.
 """
+import dataclasses
 from dataclasses import dataclass
 from typing import Optional
 
@@ -48,15 +49,19 @@ CONFIGS = {
 }
 
 
-def make_config(name: str, N: Optional[int] = None, M: Optional[int] = None, dtype: Optional[torch.dtype] = None):
+def make_config(name: str, N: Optional[int] = None, M: Optional[int] = None, dtype: Optional[torch.dtype] = None,
+                d: Optional[int] = None, T: Optional[int] = None):
     """Build (X, C, sigma, v, w) for a configuration, optionally at reduced N / M.
 
     Draw order X, idx, sigma, v, w from ``default_rng(seed)``; ``C = X[idx]`` with
     ``idx = rng.choice(N, M, replace=False)`` as falkon/center_selection.py:227-239.
     A reduced N draws a smaller X from the same generator (not a prefix of the
     full-size X); reduced-size runs are self-consistent, not slices of the full run.
+    ``d`` / ``T`` give the configuration's shape another feature count / number of right-hand sides.
     """
     cfg = CONFIGS[name]
+    if d is not None or T is not None:
+        cfg = dataclasses.replace(cfg, d=cfg.d if d is None else d, T=cfg.T if T is None else T)
     N = cfg.N if N is None else N
     M = cfg.M if M is None else M
     dtype = cfg.dtype if dtype is None else dtype

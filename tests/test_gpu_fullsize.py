@@ -30,8 +30,8 @@ def _columns_of_kt_u(X, C_sub, sigma, u, block=500_000):
     return acc
 
 
-def _full_size_checks(dev, name, dtype, n_rows=3000, n_centres=48, bf16x3=False):
-    X, C, sigma, v, w = inputs.make_config(name, dtype=dtype)
+def _full_size_checks(dev, name, dtype, n_rows=3000, n_centres=48, bf16x3=False, d=None, T=None):
+    X, C, sigma, v, w = inputs.make_config(name, dtype=dtype, d=d, T=T)
     opt = FalkonOptions(bf16x3_cross_term=bf16x3)
     N, M, T = X.shape[0], C.shape[0], v.shape[1]
     tol = TOL[dtype]
@@ -122,6 +122,13 @@ def test_config2_full_size_against_the_cpu_path(dev):
         assert e_gpu32 < e_cpu32 / 10                      # the GPU is the more accurate of the two fp32 results
         assert abs(e_pair - e_cpu32) < 0.1 * e_cpu32       # and their distance is the CPU path's own error
         assert e_pair < 10 * TOL[torch.float32]
+
+
+@pytest.mark.parametrize("d,t", [(40, 1), (64, 1), (96, 1), (128, 1), (100, 3)])
+def test_config2_shape_at_33_to_128_features(dev, d, t):
+    """Configuration 2's sizes with 40 to 128 features: the register-resident fp32 kernels with four, three (one column)
+    or two (three columns) resident blocks per wave, from 65 features on on operands packed for the LDS-tiled kernel."""
+    _full_size_checks(dev, "C2", torch.float32, n_rows=1500, n_centres=24, d=d, T=t)
 
 
 @pytest.mark.parametrize("bf16x3", [False, True], ids=["fp32-mfma", "bf16x3"])

@@ -353,6 +353,7 @@ def test_memory_budget_reuses_a_recent_driver_report(monkeypatch):
     monkeypatch.setattr(torch.cuda, "memory_reserved", lambda dev: 0)
     monkeypatch.setattr(torch.cuda, "memory_allocated", lambda dev: 0)
     utils._recent_free.clear()
+    monkeypatch.setattr(utils, "_FREE_MEMORY_TTL", 3600.0)      # (50 ms in the library: a loaded machine must not age the report here)
     dev = torch.device("cuda", 0)
     big = utils.usable_gpu_memory(dev, float("inf"), 0.9, enough=2**30)
     assert len(calls) == 1 and big == pytest.approx(0.9 * 80 * 2**30)
@@ -376,6 +377,7 @@ def test_out_of_memory_on_a_reused_report_is_planned_again(monkeypatch):
     utils = importlib.import_module("falkon_amd.mmv_ops.utils")
     calls, runs = [], []
     monkeypatch.setattr(torch.cuda, "mem_get_info", lambda dev: (calls.append(dev), (80 * 2**30, 288 * 2**30))[1])
+    monkeypatch.setattr(utils, "_FREE_MEMORY_TTL", 3600.0)      # the reuse below must not depend on how fast this machine is
     utils._recent_free.clear()
     utils._reused.clear()
     dev = torch.device("cuda", 0)
