@@ -131,6 +131,19 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     constexpr int kVecStride = kEpiCols + 1;
     constexpr int kRowBuf = kMfmaEpi ? G::A_ROWS * (1 + kVecStride) : (1 + TT) * G::A_ROWS;
     __shared__ __attribute__((aligned(32))) T ldsRow[kRowBuf];   // [hA | vec ...] of the A tile
+    // fp64 products: 2^x from the table in LDS (kernel_fn.h; 16 KB beside the stages and the row values).  The epilogue is
+    // a fixed cost per kernel value, so this pays where a tile has few feature chunks: N = 5e5, M = 2e4, dfmmv, one column,
+    // d = 65 54.4 -> 51.7 ms, 100 73.0 -> 70.5, 128 89.0 -> 86.1, 300 189.0 -> 188.0, 784 unchanged; 10 columns 1 to 3 %.
+    constexpr bool kExpTab = sizeof(T) == 8 && !kStore;
+    __shared__ double exp_tab[kExpTab ? kExpTableSize : 1];
+    if constexpr (kExpTab) {
+        exp2_table_fill(exp_tab, threadIdx.x, kLThreads);
+        __syncthreads();
+    }
+    auto kval = [&](T e) -> T {
+        if constexpr (kExpTab) return (T)kernel_value<FLK_KF, true>((double)e, exp_tab);
+        else return kernel_value<FLK_KF>(e);
+    };
 
     unsigned bx, by;
     // (Banding the contracting mode as well was measured on N = 5e5, M = 1e4, d = 784: bytes fetched per launch
@@ -376,7 +389,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
                 for (int q = 0; q < WB_FR; q++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) kv[q][e] = kernel_value<FLK_KF>(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
+                    for (int e = 0; e < 4; e++) kv[q][e] = kval(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
 #pragma unroll
                 for (int tg = 0; tg < NTG; tg++) {
                     const int t0 = 4 * tg;
@@ -415,7 +428,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
                     for (int q = 0; q < WB_FR; q++)
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            acc[p][q][4 * g + e] = kernel_value<FLK_KF>(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
+                            acc[p][q][4 * g + e] = kval(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
                 }
             }
             // out2[q][j-rows][t] += sum_i K[i][j] vec[i][t]: accumulator register s of a lane is exactly the MFMA
@@ -551,8 +564,7 @@ template <> struct LCfg<float>  { static constexpr int WVA = 2, WVB = 2, WA_FR =
 // 128 x 128 tile in stages of eight steps, which the kernel used before (measured, dfmmv at N = 5e5, M = 1e4, d = 784, 10
 // columns: 245.5 -> 239.4 ms; one column 241.8 -> 238.3, 16 columns 247.0 -> 242.6; N = 5e5, M = 2e4, d = 100: 76.1 -> 73.2,
 // 10 columns 88.0 -> 83.4; N = 2.5e5, M = 2e4, d = 300: 97.5 -> 95.4).  (On the 128 x 128 tile, stages of four steps
-// instead of eight were 3 to 7 % faster below 128 features and 2 to 3 % slower from 256 on; the exponential's table in
-// LDS gained nothing in this kernel's epilogue, where eight waves read it at once.)
+// instead of eight were 3 to 7 % faster below 128 features and 2 to 3 % slower from 256 on.)
 template <> struct LCfg<double> { static constexpr int WVA = 2, WVB = 4, WA_FR = 8, WB_FR = 2, KC = 4; };
 
 // fp32 with 17 .. 32 columns: the row values of an A tile take 34 KB of LDS, two workgroups with the 48 KB of feature
