@@ -117,6 +117,10 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
     // as [row][16 or 32 columns] at an odd stride.  Fewer columns: per-lane FMAs, vec staged planar.
     // fp32: the 32x32x2 step has room for 32 columns (lane % 32), fp64's 16x16x4 for 16.
     constexpr bool kMfmaEpi = TT > kLargeFmaCols<T>;
+    // fp64 with one column: the accumulators of a lane all belong to one output row j and start from hB_j, one
+    // addition per kernel value less in the epilogue (measured, dfmmv at N = 5e5, M = 2e4: d = 65 51.4 -> 50.1 ms,
+    // 128 86.0 -> 84.2, 784 472.1 -> 463.7; with four columns, with the MFMA epilogue and in fp32 it is a loss of up to 1 %)
+    constexpr bool kSeeded = !kStore && sizeof(T) == 8 && TT == 1;
     // More columns than one step holds: NC groups of columns ride on the same kernel values (one more contraction
     // per group, NC times the output accumulators).
     constexpr int kGroupCols = (sizeof(T) == 4 && TT > 16) ? 32 : 16;
@@ -205,7 +209,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
             for (int q = 0; q < WB_FR; q++)
 #pragma unroll
-                for (int r = 0; r < TR::ACCN; r++) acc[p][q][r] = T(0);
+                for (int r = 0; r < TR::ACCN; r++) acc[p][q][r] = kSeeded ? hb[q] : T(0);
 
         V16 ra[G::A_VPT], rb[G::B_VPT];
         constexpr bool kScalarBlk = sizeof(T) == 4 && TT >= 48;
@@ -389,7 +393,7 @@ __global__ void __launch_bounds__(64 * WVA * WVB, (WVA * WVB == 4 ? 2 : 1))   //
 #pragma unroll
                 for (int q = 0; q < WB_FR; q++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) kv[q][e] = kval(acc[p][q][4 * g + e] + (hn[e] + hb[q]));
+                    for (int e = 0; e < 4; e++) kv[q][e] = kval(acc[p][q][4 * g + e] + (kSeeded ? hn[e] : hn[e] + hb[q]));
 #pragma unroll
                 for (int tg = 0; tg < NTG; tg++) {
                     const int t0 = 4 * tg;
