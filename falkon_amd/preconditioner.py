@@ -25,7 +25,10 @@ from .options import FalkonOptions
 __all__ = ("FalkonPreconditioner", "LogisticPreconditioner")
 
 TRSV_BLOCK = 2048        # rows per diagonal block of the blocked triangular solves
-TRSV_MIN_SIZE = 4096     # smaller factors go to torch.linalg.solve_triangular directly
+TRSV_MIN_SIZE = 4096     # smaller factors on the host go to torch.linalg.solve_triangular directly
+# Device-resident factors take the blocked route from this size on: the library's triangular solve with one right-hand
+# side costs 0.18 ms at M = 1 000 and 1.0 ms at M = 4 000 on the GPU, the product with the inverted block 11 to 30 us.
+TRSV_MIN_SIZE_DEVICE = 64
 
 
 def _gram_of_lower_factor(L: torch.Tensor, block: Optional[int] = None) -> torch.Tensor:
@@ -90,9 +93,16 @@ class _BlockedTriangular:
         self.L = L
         M = L.shape[0]
         block = TRSV_BLOCK if block is None else block
-        min_size = TRSV_MIN_SIZE if min_size is None else min_size
-        self.bounds = [(k, min(k + block, M)) for k in range(0, M, block)] if M >= min_size else []
+        self._block, self._min_size = block, min_size
+        self._set_bounds()
         self._build()
+
+    def _set_bounds(self):
+        M = self.L.shape[0]
+        min_size = self._min_size
+        if min_size is None:
+            min_size = TRSV_MIN_SIZE_DEVICE if self.L.is_cuda else TRSV_MIN_SIZE
+        self.bounds = [(k, min(k + self._block, M)) for k in range(0, M, self._block)] if M >= min_size else []
 
     def _build(self):
         L = self.L
@@ -103,6 +113,8 @@ class _BlockedTriangular:
         if not self.bounds:
             return
         block = self.bounds[0][1] - self.bounds[0][0]
+        if len(self.bounds) == 1:
+            block = (block + 3) // 4 * 4             # a single block: any leading dimension serves; flk_tri_solve wants a multiple of 4
         # the inverted diagonal blocks, block k at [k] with leading dimension `block` (zero beyond a smaller last
         # block), and their transposes: the layout flk_tri_solve reads; the torch path uses views of the same memory
         self._stack = torch.zeros(len(self.bounds), block, block, dtype=L.dtype, device=L.device)
@@ -117,6 +129,7 @@ class _BlockedTriangular:
 
     def to(self, device):
         self.L = self.L.to(device)
+        self._set_bounds()
         self._build()
         return self
 

@@ -54,6 +54,28 @@ def test_blocked_solves_match_lapack(dev, dtype, order, m, block, t):
         assert float((got.double() - other.double()).norm() / want.norm()) < tol
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("m,t", [(64, 1), (130, 2), (1001, 1), (2000, 4), (2047, 3), (3000, 1)])
+def test_small_device_factors_take_the_blocked_route(dev, dtype, m, t):
+    """Factors below 4096 rows on the GPU (small models: the library's single-right-hand-side triangular solve costs 0.2 to
+    1 ms there) run the same blocked solve with the default sizes: one inverted block up to 2048 rows, whatever m is
+    modulo 4; on the host such factors keep the library routine."""
+    L = _factor(m, dtype, seed=m + t, order="C")
+    assert not _BlockedTriangular(L).bounds                         # host: library solve
+    tri = _BlockedTriangular(L.to(dev))
+    b = torch.randn(m, t, dtype=dtype, generator=torch.Generator().manual_seed(4)).to(dev)
+    assert tri.bounds and tri._native_applies(b)
+    moved = _BlockedTriangular(L).to(dev)                           # built on the host, then moved
+    assert moved.bounds and moved._native_applies(b)
+    L64, b64 = L.double().to(dev), b.double()
+    for transposed, solve, solve_moved in ((False, tri.solve, moved.solve), (True, tri.solve_t, moved.solve_t)):
+        got = solve(b)
+        op = L64.T if transposed else L64
+        res = float((op @ got.double() - b64).norm() / b64.norm())
+        assert res < (5e-6 if dtype == torch.float32 else 1e-13), (transposed, res)
+        assert torch.equal(got, solve_moved(b)) and torch.equal(got, solve(b))
+
+
 def test_raw_c_abi_call_and_argument_checks(dev):
     lib = _backend.load()
     m, block = 2048 + 512, 1024
