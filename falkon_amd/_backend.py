@@ -69,6 +69,8 @@ _SIGNATURES["flk_cg_update"] = (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_v
 _SIGNATURES["flk_tri_solve_work_elems"] = (c_int64, [c_int64, c_int64, c_int64])
 _SIGNATURES["flk_tri_solve"] = (c_int, [c_int, c_int, c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64,
                                         c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p])
+_SIGNATURES["flk_potrf_tile_rows"] = (c_int64, [c_int])
+_SIGNATURES["flk_potrf_tile"] = (c_int, [c_int, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p])
 NOALLOC_SCRATCH_BYTES = 64 << 20
 
 

@@ -24,7 +24,7 @@ PER_KERNEL_FN = ["mmv_small_f32.hip", "mmv_small_f32_fold.hip", "mmv_small_f32_w
 # together), so that the parallel build does not end on one of them running alone.
 SOURCES = [(src, kf) for src in PER_KERNEL_FN for kf in KERNEL_FNS]
 SOURCES.sort(key=lambda job: {"mmv_small_f32_wide.hip": 0, "mmv_small_f32.hip": 1, "mmv_small_f32_fold.hip": 2}.get(job[0], 3))
-SOURCES += [("api.hip", None), ("pack.hip", None), ("pack_split.hip", None), ("cg.hip", None), ("trsv.hip", None)]
+SOURCES += [("api.hip", None), ("pack.hip", None), ("pack_split.hip", None), ("cg.hip", None), ("trsv.hip", None), ("potrf.hip", None)]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

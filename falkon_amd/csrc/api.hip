@@ -942,6 +942,23 @@ int flk_tri_solve(int dtype, int transposed, const void *L, int64_t m, int64_t l
     return fail(FLK_EINVAL, "unknown dtype %d", dtype);
 }
 
+int64_t flk_potrf_tile_rows(int dtype) { return known_dtype(dtype, false) ? potrf_tile_rows(dtype) : 0; }
+
+int flk_potrf_tile(int dtype, void *A, int64_t n, int64_t lda, void *inv, int64_t ldinv, int *info, int64_t info_base,
+                   void *stream) {
+    g_err[0] = 0;
+    if (n < 0) return fail(FLK_EINVAL, "flk_potrf_tile: negative size");
+    if (n == 0) return FLK_OK;
+    if (!A || !inv || !info) return fail(FLK_EINVAL, "flk_potrf_tile: null pointer");
+    if (lda < n || ldinv < n) return fail(FLK_EINVAL, "flk_potrf_tile: leading dimension below n");
+    if (A == inv) return fail(FLK_EINVAL, "flk_potrf_tile: A and inv must be distinct buffers");
+    if (info_base < 0 || info_base + n > 0x7fffffff) return fail(FLK_EINVAL, "flk_potrf_tile: info_base out of range");
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == FLK_F32) return launch_potrf_tile<float>((float *)A, n, lda, (float *)inv, ldinv, info, (int)info_base, st);
+    if (dtype == FLK_F64) return launch_potrf_tile<double>((double *)A, n, lda, (double *)inv, ldinv, info, (int)info_base, st);
+    return fail(FLK_EINVAL, "unknown dtype %d", dtype);
+}
+
 size_t flk_gauss_fmm_workspace_bytes(int64_t n, int64_t m, int64_t d, int dtype, int compute_f64) {
     if (n < 0 || m < 0 || d < 1 || d > flk_max_d(dtype) || !known_dtype(dtype, true)) return 0;
     if (fmm_split_applies(d, dtype, compute_f64)) return split_packed_bytes(n, d) + split_packed_bytes(m, d);

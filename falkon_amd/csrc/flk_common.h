@@ -129,6 +129,10 @@ int fail(int code, const char *fmt, ...);
     } while (0)
 
 // Blocked triangular solve with a resident factor and the inverses of its diagonal blocks (trsv.hip)
+// Cholesky factor of one diagonal tile and the inverse of that factor (potrf.hip)
+int potrf_tile_rows(int dtype);
+template <typename T>
+int launch_potrf_tile(T *A, int64_t n, int64_t lda, T *inv, int64_t ldinv, int *info, int info_base, hipStream_t st);
 int64_t tri_solve_work_elems(int64_t m, int64_t t, int64_t block);
 template <typename T>
 int launch_tri_solve(const T *L, int64_t m, int64_t ld, int row_major, const T *dinv, const T *dinv_t, int64_t block,

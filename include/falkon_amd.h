@@ -216,6 +216,23 @@ int flk_tri_solve(int dtype, int transposed, const void *L, int64_t m, int64_t l
                   const void *dinv, const void *dinv_t, int64_t block,
                   const void *b, int64_t ldb, void *x, int64_t ldx, int64_t t, void *work, void *stream);
 
+/* ---- diagonal tiles of the preconditioner's Cholesky factorisations ---------------
+ * flk_potrf_tile serves the two factorisations of M x M matrices that build the preconditioner
+ * (falkon/preconditioner/flk_preconditioner.py:115,152: potrf_wrapper; falkon/preconditioner/pc_utils.py: the
+ * library potrf behind it).  A blocked factorisation spends nearly all its flop in matrix products, but its diagonal
+ * tiles are a chain of M dependent column steps; this entry point runs that chain for one tile inside one workgroup.
+ *   A: n x n, n <= flk_potrf_tile_rows(dtype), element (i, j) at A[i*lda + j]; the lower triangle is read and
+ *      overwritten with the Cholesky factor L (A = L L^T); the elements above the diagonal are left alone.
+ *   inv: n x n at inv[i*ldinv + j], a buffer distinct from A: receives L^-1 with zeros above the diagonal, so that the
+ *      triangular solve of the panel below the tile is the matrix product  panel <- panel * inv^T.
+ *   info: one int in device memory that the caller clears before the first tile.  A pivot that is not positive (or
+ *      is NaN) at row j stores info_base + j + 1 there unless a failure is already recorded; L and inv are NaN from
+ *      that row on.  The call does not synchronise and does not read info on the host. */
+int64_t flk_potrf_tile_rows(int dtype);
+
+int flk_potrf_tile(int dtype, void *A, int64_t n, int64_t lda, void *inv, int64_t ldinv, int *info, int64_t info_base,
+                   void *stream);
+
 /* ---- explicit kernel matrix -------------------------------------------------
  * flk_gauss_fmm replaces falkon.mmv_ops.fmm.fmm for the dense Gaussian case
  *   (falkon/mmv_ops/fmm.py:699-708 -> :298-388 block loop -> distance_kernel.py:140-159):
