@@ -15,6 +15,20 @@ constexpr int kPotrfThreads = 256;
 constexpr int kPotrfTile = 128;        // rows of a tile: 16 x 16 threads own 8 x 8 elements each
 constexpr int kPotrfOwn = kPotrfTile / 16;
 
+// Square root of a positive pivot and its reciprocal.  Single precision: the hardware's reciprocal square root as the
+// seed and one correction each (the library's sqrt and division cost some twenty dependent instructions per column
+// step, on the critical path of a chain of 128 steps); double precision: the library routines.
+__device__ __forceinline__ void pivot_root(float d, float &l, float &rl) {
+    const float y = __builtin_amdgcn_rsqf(d);
+    const float g = d * y;
+    l = __builtin_fmaf(__builtin_fmaf(-g, g, d), 0.5f * y, g);
+    rl = __builtin_fmaf(__builtin_fmaf(-l, y, 1.0f), y, y);
+}
+__device__ __forceinline__ void pivot_root(double d, double &l, double &rl) {
+    l = sqrt(d);
+    rl = 1.0 / l;
+}
+
 // A: n x n (n <= 128), element (i, j) at A[i * lda + j]; the lower triangle is read and overwritten with the factor,
 // the rest is left alone.  inv: n x n at inv[i * ldinv + j], the inverse of the factor with zeros above the diagonal.
 // info: left alone on success; a pivot that is not positive (or is NaN) at row j stores info_base + j + 1 there
@@ -61,26 +75,28 @@ __global__ void __launch_bounds__(kPotrfThreads) potrf_tile_kernel(T *__restrict
             const T d = cb[j];
             T l, rl;
             if (d > T(0)) {
-                l = sqrt(d);
-                rl = T(1) / l;
+                pivot_root(d, l, rl);
             } else {
                 if (tid == 0 && *info == 0) *info = info_base + j + 1;
                 l = rl = __builtin_nan("");
             }
+            // what this thread needs of column j and of row j of x, scaled by 1 / l_jj; only the slab that holds column
+            // j has rows and columns on both sides of it (zeros there switch the updates off)
             T lrow[Q], lcol[Q], xrow[Q];
 #pragma unroll
-            for (int a = jb; a < Q; a++) lrow[a] = ti + 16 * a > j ? cb[ti + 16 * a] * rl : T(0);      // l_ij for my rows
+            for (int a = jb; a < Q; a++) lrow[a] = cb[ti + 16 * a] * rl;                     // l_ij for my rows
 #pragma unroll
-            for (int b = jb; b < Q; b++) lcol[b] = tc + 16 * b > j ? cb[tc + 16 * b] * rl : T(0);      // l_cj for my columns
+            for (int b = jb; b < Q; b++) lcol[b] = cb[tc + 16 * b] * rl;                     // l_cj for my columns
 #pragma unroll
-            for (int b = 0; b <= jb; b++) xrow[b] = tc + 16 * b <= j ? rb[tc + 16 * b] * rl : T(0);    // x_jc, scaled
+            for (int b = 0; b <= jb; b++) xrow[b] = rb[tc + 16 * b] * rl;                    // x_jc, scaled
+            if (ti <= jj) lrow[jb] = T(0);
+            if (tc <= jj) lcol[jb] = T(0);
+            if (tc > jj) xrow[jb] = T(0);
             if (tc == jj) {
 #pragma unroll
-                for (int a = jb; a < Q; a++) {
-                    const int i = ti + 16 * a;
-                    if (i > j) r[a][jb] = lrow[a];
-                    else if (i == j) r[a][jb] = l;
-                }
+                for (int a = jb + 1; a < Q; a++) r[a][jb] = lrow[a];
+                if (ti > jj) r[jb][jb] = lrow[jb];
+                else if (ti == jj) r[jb][jb] = l;
             }
             if (ti == jj) {
 #pragma unroll
