@@ -54,6 +54,9 @@ CHOL_MIN_SIZE = 16384      # smaller matrices go to torch.linalg.cholesky direct
 # library routine takes 3 us per column whatever the size (0.63 ms at 256 rows, 12.8 ms at 4096).
 CHOL_TILE_MIN_SIZE = 256
 CHOL_RIGHT_LOOKING = True
+# Block columns of the right-looking device factorisation: every update is then a product of 2048 terms (M = 40 000:
+# 228 ms and L L^T 3.9e-6 from the matrix, against 234 ms and 6.1e-6 with 4096, 236 ms and 2.9e-6 with 1024).
+CHOL_BLOCK_DEVICE = 2048
 
 
 def _not_positive_definite(order: int):
@@ -107,8 +110,9 @@ def _cholesky_lower_(A: torch.Tensor, block: Optional[int] = None, min_size: Opt
     library routine if the matrix is not positive definite.
     """
     M = A.shape[0]
-    block = CHOL_BLOCK if block is None else block
     tiles = _tiles_apply(A) and min_size is None
+    if block is None:
+        block = CHOL_BLOCK_DEVICE if tiles and M > CHOL_BLOCK else CHOL_BLOCK     # up to 4096 rows: rank-128 updates only
     min_size = CHOL_MIN_SIZE if min_size is None else min_size
     info = torch.zeros(1, dtype=torch.int32, device=A.device) if tiles else None
     if tiles and M <= block:

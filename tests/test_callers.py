@@ -234,7 +234,8 @@ def test_config5_reduced_end_to_end(dev, monkeypatch):
     import falkon_amd.preconditioner as pcm
     monkeypatch.setattr(pcm, "TRSV_BLOCK", 256)
     monkeypatch.setattr(pcm, "TRSV_MIN_SIZE", 512)
-    monkeypatch.setattr(pcm, "CHOL_BLOCK", 512)              # and the blocked Cholesky (used from M = 16384 on)
+    monkeypatch.setattr(pcm, "CHOL_BLOCK", 512)              # and the blocked Cholesky (host matrices from M = 16384 on;
+    monkeypatch.setattr(pcm, "CHOL_BLOCK_DEVICE", 512)       # device matrices beyond one block column of 2048)
     monkeypatch.setattr(pcm, "CHOL_MIN_SIZE", 1024)
     model4 = Falkon(GaussianKernel(sigma), lam, M=M, maxiter=20, center_selection=FixedSelector(C))
     model4.fit(X.to(dev), Y.to(dev))

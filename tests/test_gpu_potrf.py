@@ -5,7 +5,6 @@ Reference behaviour: falkon/preconditioner/flk_preconditioner.py:115,152 (potrf_
 failure on a matrix that is not positive definite); falkon/tests/test_chol_prec.py:17-67 pins the factors through
 their products, as the reconstruction checks below do.
 """
-import ctypes
 
 import pytest
 import torch
@@ -100,7 +99,7 @@ def test_tile_rejects_bad_arguments():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-@pytest.mark.parametrize("m,block", [(256, None), (300, None), (1000, None), (1337, 512), (2048, 512), (4100, None)])
+@pytest.mark.parametrize("m,block", [(256, None), (300, None), (1000, None), (1337, 512), (2048, 512), (4100, None), (4500, 1024)])
 def test_blocked_factorisation_on_the_device(m, block, dtype):
     """_cholesky_lower_ on a device matrix: tiles inside the diagonal blocks, matrix products around them."""
     from falkon_amd.preconditioner import _cholesky_lower_, _tiles_apply
