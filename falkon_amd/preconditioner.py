@@ -53,7 +53,6 @@ CHOL_MIN_SIZE = 16384      # smaller matrices go to torch.linalg.cholesky direct
 # Device-resident row-major matrices from this size on factorise their diagonal blocks by tiles (``flk_potrf_tile``): the
 # library routine takes 3 us per column whatever the size (0.63 ms at 256 rows, 12.8 ms at 4096).
 CHOL_TILE_MIN_SIZE = 256
-CHOL_RIGHT_LOOKING = True
 # Block columns of the right-looking device factorisation: every update is then a product of 2048 terms (M = 40 000:
 # 228 ms and L L^T 3.9e-6 from the matrix, against 234 ms and 6.1e-6 with 4096, 236 ms and 2.9e-6 with 1024).
 CHOL_BLOCK_DEVICE = 2048
@@ -100,14 +99,14 @@ def _cholesky_by_tiles_(B: torch.Tensor, info: torch.Tensor, first_row: int) -> 
 
 def _cholesky_lower_(A: torch.Tensor, block: Optional[int] = None, min_size: Optional[int] = None) -> torch.Tensor:
     """Lower Cholesky factor of the symmetric positive definite ``A`` (only its lower triangle is read; ``A`` may be
-    overwritten).
+    overwritten).  Raises ``torch.linalg.LinAlgError`` like the library routine if the matrix is not positive definite.
 
-    Large matrices are factorised in place, left-looking by block columns: one large matrix product per
-    panel (``A[k:, k] -= L[k:, :k] L[k, :k]^T``), the diagonal block on its own, one triangular solve for the rest
-    of the panel.  Nearly all of the M^3/3 flop run in the matrix products; at M = 50 000 this takes about half the
-    time of the library routine on the whole matrix.  The diagonal blocks of a device matrix are factorised by tiles
-    (``_cholesky_by_tiles_``), those of a host matrix by the library.  Raises ``torch.linalg.LinAlgError`` like the
-    library routine if the matrix is not positive definite.
+    Device matrices (row-major, from 256 rows on) are factorised in place, right-looking by block columns: the
+    diagonal block by tiles (``_cholesky_by_tiles_``), the rows below it through the library's triangular solve, then
+    one product per block column of the rest of the lower block triangle, so that nearly all of the M^3/3 flop run in
+    large matrix products and no entry meets a sum of more than 2048 products at once (up to 4096 rows: one block,
+    rank-128 updates only).  Large host matrices take the same steps with the library's factorisation of the diagonal
+    blocks; small host matrices and column-major device matrices go to the library routine whole.
     """
     M = A.shape[0]
     tiles = _tiles_apply(A) and min_size is None
@@ -119,23 +118,12 @@ def _cholesky_lower_(A: torch.Tensor, block: Optional[int] = None, min_size: Opt
         _cholesky_by_tiles_(A, info, 0)
     elif M < min_size and not tiles or M <= block:
         return torch.linalg.cholesky(A)
-    elif tiles and CHOL_RIGHT_LOOKING:
-        # right-looking by block columns: the diagonal block by tiles, the rows below it through the library's
-        # triangular solve, then one product per block column of the rest (its lower block triangle only)
-        for k0 in range(0, M, block):
-            k1 = min(k0 + block, M)
-            _cholesky_by_tiles_(A[k0:k1, k0:k1], info, k0)
-            if k1 < M:
-                Lkk = A[k0:k1, k0:k1].tril()
-                A[k1:, k0:k1] = torch.linalg.solve_triangular(Lkk.T, A[k1:, k0:k1], upper=True, left=False)
-                for c0 in range(k1, M, block):
-                    c1 = min(c0 + block, M)
-                    A[c0:, c0:c1].addmm_(A[c0:, k0:k1], A[c0:c1, k0:k1].T, alpha=-1.0)
     else:
+        # right-looking by block columns: the diagonal block (by tiles on the device, by the library on the host), the
+        # rows below it through the library's triangular solve, then one product per block column of the rest (its
+        # lower block triangle only)
         for k0 in range(0, M, block):
             k1 = min(k0 + block, M)
-            if k0 > 0:
-                A[k0:, k0:k1].addmm_(A[k0:, :k0], A[k0:k1, :k0].T, alpha=-1.0)
             if tiles:
                 _cholesky_by_tiles_(A[k0:k1, k0:k1], info, k0)
                 Lkk = A[k0:k1, k0:k1].tril()
@@ -144,6 +132,9 @@ def _cholesky_lower_(A: torch.Tensor, block: Optional[int] = None, min_size: Opt
                 A[k0:k1, k0:k1] = Lkk
             if k1 < M:
                 A[k1:, k0:k1] = torch.linalg.solve_triangular(Lkk.T, A[k1:, k0:k1], upper=True, left=False)
+                for c0 in range(k1, M, block):
+                    c1 = min(c0 + block, M)
+                    A[c0:, c0:c1].addmm_(A[c0:, k0:k1], A[c0:c1, k0:k1].T, alpha=-1.0)
     if tiles:
         failed = int(info.item())
         if failed:
