@@ -31,20 +31,30 @@ TRSV_MIN_SIZE = 4096     # smaller factors on the host go to torch.linalg.solve_
 TRSV_MIN_SIZE_DEVICE = 64
 
 
-def _gram_of_lower_factor(L: torch.Tensor, block: Optional[int] = None) -> torch.Tensor:
+GRAM_TERMS = 2048        # products summed at once in T T^T
+
+
+def _gram_of_lower_factor(L: torch.Tensor, block: Optional[int] = None, terms: Optional[int] = None) -> torch.Tensor:
     """``L^T L`` for a lower-triangular ``L``, valid in the lower triangle (and the diagonal blocks); the
     blocks above the diagonal are left zero.  Enough for a Cholesky factorisation, which reads one triangle.
 
     Row block i of the product only involves rows i0.. of L (the rows above are zero in those columns) and
     only its columns up to the diagonal block are needed: M^3/3 flop instead of the 2 M^3 of a full product,
     the saving the reference gets from its LAUUM kernel (falkon/preconditioner/flk_preconditioner.py:133-138).
+    The sum over the rows of L is taken ``terms`` rows at a time and added up block by block: one product over all
+    M rows rounds a sum of tens of thousands of products in single precision at once (M = 40 000: entries of
+    size 900 came out 6.8e-3 from the double-precision product, which is 1.7e-7 after the division by M, next to
+    a penalty of 1e-6), in pieces of 2048 it is 1.9e-4, for 6 % more time.
     """
     M = L.shape[0]
     block = TRSV_BLOCK if block is None else block
+    terms = GRAM_TERMS if terms is None else terms
     G = torch.zeros_like(L)
     for i0 in range(0, M, block):
         i1 = min(i0 + block, M)
-        torch.mm(L[i0:, i0:i1].T, L[i0:, :i1], out=G[i0:i1, :i1])
+        for k0 in range(i0, M, terms):
+            k1 = min(k0 + terms, M)
+            G[i0:i1, :i1].addmm_(L[k0:k1, i0:i1].T, L[k0:k1, :i1])
     return G
 
 
