@@ -467,6 +467,8 @@ def run_c5(args, lib, defer_cpu=False):
     flop_per_launch = N * M * (2 * d + 4 + 2)
     kern_avg = kern_ms / max(launches, 1)
     achieved = flop_per_launch / (kern_avg * 1e-3) / 1e12
+    # (the counters were taken at the full size only)
+    c5_traffic, c5_traffic_src = measured_traffic("C5", "f32") if (N, M) == (2_000_000, 50_000) and not split else (None, None)
     res = {
         "metric": "dfmmv kernel-entries/sec (N*M*T/s) fp32 inside Falkon.fit, 1 MI355X",
         "value": N * M * n_dmmv / cg, "unit": "kernel entries/s", "n_gpus": 1, "steps": args.steps,
@@ -480,7 +482,8 @@ def run_c5(args, lib, defer_cpu=False):
         "cg_graph": bool(args.cg_graph), "product_kernel_s_per_fit": kern_ms * 1e-3 / max(args.steps, 1),
         "cg_s_over_product_kernel_s": cg / (kern_ms * 1e-3 / max(args.steps, 1)) if kern_ms > 0 else None,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / FP32_PEAK_TFLOPS, "traffic": None, "kernel": "mmv_small_f32_kernel",
+                     "frac": achieved / FP32_PEAK_TFLOPS, "traffic": c5_traffic, "traffic_source": c5_traffic_src,
+                     "kernel": "mmv_small_f32_kernel",
                      "launches_per_step": launches / max(args.steps, 1), "avg_launch_ms": kern_avg,
                      "flop_per_launch": flop_per_launch},
     }
