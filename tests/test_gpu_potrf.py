@@ -139,3 +139,32 @@ def test_blocked_factorisation_of_a_kernel_matrix_and_failure():
     from falkon_amd.preconditioner import _tiles_apply
     assert not _tiles_apply(K.T.contiguous().T)
     torch.testing.assert_close(_cholesky_lower_(K.T.contiguous().T.clone()), lib_factor, rtol=1e-4, atol=1e-5)
+
+
+def test_factorisation_at_config5_size_reconstructs_the_kernel_matrix():
+    """M = 50 000 centres in 28 dimensions (config 5's preconditioner): the factor of K + eps * M * I reproduces sampled
+    rows of the matrix, in double precision, to a few hundred units in the last place of its entries (the sums
+    behind an entry are taken 2048 products at a time), and T T^T formed from it agrees with the double-precision
+    product of the same factor on sampled rows."""
+    from falkon_amd import GaussianKernel
+    from falkon_amd.preconditioner import _cholesky_lower_, _gram_of_lower_factor
+    dev = torch.device("cuda:0")
+    M = 50_000
+    g = torch.Generator().manual_seed(1005)
+    C = torch.randn(M, 28, generator=g).to(dev)
+    K = GaussianKernel(3.8)(C, C)
+    K.diagonal().add_(1e-5 * M)
+    rows = torch.tensor([0, 1, 127, 128, 2047, 2048, 4095, 4096, 25_000, 49_871, M - 1], device=dev)
+    want = K[rows].double()
+    L = _cholesky_lower_(K)                                    # in place: K's storage now holds the factor
+    assert bool((L.diagonal() > 0).all())
+    got = torch.zeros_like(want)
+    for k0 in range(0, M, 5000):                               # (L L^T)[rows] in double precision, 5000 columns of L at a time
+        got += L[rows, k0:k0 + 5000].double() @ L[:, k0:k0 + 5000].double().T
+    assert (got - want).abs().max().item() <= 2e-5 * want.abs().max().item()
+    G = _gram_of_lower_factor(L)
+    cols = slice(0, 2048)
+    want_g = L[:, rows].double().T @ L[:, cols].double()       # (L^T L)[rows, :2048]; valid where column <= row
+    mask = torch.arange(2048, device=dev)[None, :] <= rows[:, None]
+    diff = ((G[rows, cols].double() - want_g) * mask).abs().max().item()
+    assert diff <= 2e-6 * want_g.abs().max().item(), (diff, want_g.abs().max().item())
