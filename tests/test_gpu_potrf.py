@@ -168,3 +168,22 @@ def test_factorisation_at_config5_size_reconstructs_the_kernel_matrix():
     mask = torch.arange(2048, device=dev)[None, :] <= rows[:, None]
     diff = ((G[rows, cols].double() - want_g) * mask).abs().max().item()
     assert diff <= 2e-6 * want_g.abs().max().item(), (diff, want_g.abs().max().item())
+
+
+@pytest.mark.parametrize("m,d,sigma", [(383, 1, 4.52), (1000, 1, 1.89), (4097, 3, 2.36), (6145, 1, 2.29)])
+def test_double_precision_on_nearly_singular_kernel_matrices(m, d, sigma):
+    """Kernel matrices of low-dimensional data with the double-precision jitter of 1e-13 M (condition number beyond
+    1e14): the products with inverted tiles take a step of refinement there, and L L^T stays as close to the
+    matrix as the library's factor leaves it (without the step: 1e-12 against 1e-14)."""
+    from falkon_amd import GaussianKernel
+    from falkon_amd.preconditioner import _cholesky_lower_
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(m)
+    C = torch.randn(m, d, generator=g, dtype=torch.float64).to(dev)
+    K = GaussianKernel(sigma)(C, C)
+    K.diagonal().add_(1e-13 * m)
+    lib_factor = torch.linalg.cholesky(K)
+    L = _cholesky_lower_(K.clone())
+    err = ((L @ L.T) - K).abs().max().item()
+    err_lib = ((lib_factor @ lib_factor.T) - K).abs().max().item()
+    assert err <= max(8 * err_lib, 1e-13), (err, err_lib)
