@@ -118,3 +118,77 @@ def test_fixed_seed_shape_sweep(dev):
         print(f"[sweep {it}] {name} {dtype} n={n} m={m} d={d} t={t} seed={seed} Fx={fx} Fv={fv} w={use_w}", flush=True)
         X, C, v, w = _case(n, m, d, t, dtype, seed)
         _check(dev, name, X, C, v, w if use_w else None, sigma, fx, fv)
+
+
+def _laid_out(t, mode):
+    """t in one of four layouts: C order, F order, a column band of a wider row-major matrix (row stride beyond the
+    columns), a row band of a taller column-major matrix (column stride beyond the rows)."""
+    if mode == 0 or t.shape[1] == 0:
+        return t.contiguous()
+    if mode == 1:
+        return t.T.contiguous().T
+    if mode == 2:
+        big = torch.zeros(t.shape[0], t.shape[1] + 3, dtype=t.dtype, device=t.device)
+        big[:, 1:1 + t.shape[1]] = t
+        return big[:, 1:1 + t.shape[1]]
+    big = torch.zeros(t.shape[1], t.shape[0] + 5, dtype=t.dtype, device=t.device)
+    big[:, 2:2 + t.shape[0]] = t.T
+    return big[:, 2:2 + t.shape[0]].T
+
+
+def test_fixed_seed_sweep_of_call_variants(dev):
+    """200 calls drawn from a fixed seed that vary what the host side has to get right: each operand in host or
+    device memory (host rows are streamed), in four memory layouts, isotropic or per-dimension lengthscales, a given
+    ``out`` (C or F order, on the side the reference would allocate it) or none, w or none, an empty X1, and memory
+    budgets down to 8 MB (row blocks; a budget that is too small must raise MemoryError).  Results against the fp64
+    CPU path, measured on the scale of the summed terms."""
+    from falkon_amd import FalkonOptions
+    rng = np.random.default_rng(20240601)
+    for it in range(200):
+        dtype = torch.float32 if rng.random() < 0.5 else torch.float64
+        d = int(rng.choice([1, 3, 9, 28, 33, 64, 65, 100, 300]))
+        t = int(rng.choice([1, 2, 3, 5, 10, 17, 40, 70]))
+        n, m = int(rng.integers(1, 6000)), int(rng.integers(1, 2500))
+        if rng.random() < 0.05:
+            n = 0
+        if rng.random() < 0.05:
+            m = int(rng.integers(1, 20))
+        seed = int(rng.integers(1 << 30))
+        per_dim = bool(rng.random() < 0.4)
+        scale = 0.6 * np.sqrt(d) + 0.4
+        sigma = torch.tensor(rng.uniform(0.5, 2.0, d) * scale, dtype=torch.float64) if per_dim else float(scale)
+        name = NAMES[int(rng.integers(4))]
+        budget = float(rng.choice([np.inf, np.inf, 64e6, 8e6]))
+        host = [bool(rng.random() < 0.25) for _ in range(4)]
+        lay = [int(rng.integers(4)) for _ in range(4)]
+        use_w, use_out = bool(rng.random() < 0.7), bool(rng.random() < 0.5)
+        out_lay = [int(rng.integers(2)), int(rng.integers(2))]
+        print(f"[variants {it}] {name} {dtype} n={n} m={m} d={d} t={t} seed={seed} per_dim={per_dim} budget={budget:g} "
+              f"host={host} layouts={lay} w={use_w} out={use_out}", flush=True)
+        X, C, v, w = _case(n, m, d, t, dtype, seed)
+        Xa, Ca, va, wa = (_laid_out(a if h else a.to(dev), l) for a, h, l in zip((X, C, v, w), host, lay))
+        kernel = _kernel(name, sigma)
+        opt = FalkonOptions(max_gpu_mem=budget)
+        try:
+            where = "cpu" if any(host[:3]) else dev
+            om = _laid_out(torch.full((n, t), 7.0, dtype=dtype, device=where), out_lay[0]) if use_out else None
+            got_m = kernel.mmv(Xa, Ca, va, out=om, opt=opt)
+            where = "cpu" if any(host[:3]) or (use_w and host[3]) else dev
+            od = _laid_out(torch.full((m, t), 7.0, dtype=dtype, device=where), out_lay[1]) if use_out else None
+            got_d = kernel.dmmv(Xa, Ca, va, wa if use_w else None, out=od, opt=opt)
+        except MemoryError:
+            assert budget <= 8e6, "only the 8 MB budget may be too small for these sizes"
+            continue
+        if use_out:
+            assert got_m.data_ptr() == om.data_ptr() and got_d.data_ptr() == od.data_ptr()
+        assert got_m.shape == (n, t) and got_d.shape == (m, t)
+        if n == 0:
+            assert bool((got_d == 0).all())
+            continue
+        Xd, Cd, vd, wd = X.double(), C.double(), v.double(), (w.double() if use_w else None)
+        ref_m = mmv_ref.fmmv_ref(Xd, Cd, vd, sigma, kernel_name=name)
+        ref_d = mmv_ref.fdmmv_ref(Xd, Cd, vd, wd, sigma, kernel_name=name)
+        abs_m = mmv_ref.fmmv_ref(Xd, Cd, vd.abs(), sigma, kernel_name=name)
+        abs_d = mmv_ref.fdmmv_ref(Xd, Cd, vd.abs(), None if wd is None else wd.abs(), sigma, kernel_name=name)
+        tol = 3e-6 if dtype == torch.float32 else 1e-12
+        assert scaled_err(got_m, ref_m, abs_m) < tol and scaled_err(got_d, ref_d, abs_d) < tol
