@@ -464,6 +464,20 @@ def run_c5(args, lib, defer_cpu=False):
         del model, pred
     fit, pre, prd = float(np.mean(fit_s)), float(np.mean(pre_s)), float(np.mean(pred_s))
     cg = fit - pre
+    # the same preconditioner with the diagonal blocks of its factorisations left to the library routine
+    # (FalkonOptions(pc_tile_factorisation=False)), built twice, the second build timed
+    from falkon_amd.preconditioner import FalkonPreconditioner
+    opt_lib = FalkonOptions(bf16x3_cross_term=split, pc_tile_factorisation=False)
+    pre_lib = None
+    for _ in range(2):
+        pc = FalkonPreconditioner(lam, GaussianKernel(sigma, opt=opt_lib), opt_lib)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        pc.init(Xg[:M])
+        torch.cuda.synchronize()
+        pre_lib = time.perf_counter() - t0
+        del pc
+    note(f"  C5 preconditioner with the library's factorisation of the diagonal blocks: {pre_lib:.2f} s")
     flop_per_launch = N * M * (2 * d + 4 + 2)
     kern_avg = kern_ms / max(launches, 1)
     achieved = flop_per_launch / (kern_avg * 1e-3) / 1e12
@@ -479,6 +493,9 @@ def run_c5(args, lib, defer_cpu=False):
                                f"penalty=1e-6, {iters} CG iterations ({n_dmmv} dfmmv + 1 fmmv), test rows {Nts}, "
                                f"fp32{' with the bf16x3 cross term' if split else ''}, data resident in HBM"},
         "fit_s": fit, "preconditioner_s": pre, "cg_s": cg, "predict_s": prd, "test_mse": mse, "test_error_rate": err,
+        "preconditioner": "K(C,C) by this library, two blocked Cholesky factorisations and T T^T on library GEMMs, "
+                          "their diagonal tiles by flk_potrf_tile",
+        "preconditioner_s_with_library_factorisation_of_diagonal_blocks": pre_lib,
         "cg_graph": bool(args.cg_graph), "product_kernel_s_per_fit": kern_ms * 1e-3 / max(args.steps, 1),
         "cg_s_over_product_kernel_s": cg / (kern_ms * 1e-3 / max(args.steps, 1)) if kern_ms > 0 else None,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",

@@ -75,6 +75,9 @@ class PreconditionerOptions:
     pc_epsilon_32: float = 1e-5                       # jitter (times M) on the diagonal of K(C,C) in fp32
     pc_epsilon_64: float = 1e-13                      # ... in fp64
     cpu_preconditioner: bool = False                  # carried, unused
+    # False: the diagonal blocks of the two Cholesky factorisations go to the library routine (torch.linalg.cholesky)
+    # instead of this library's tile kernel (flk_potrf_tile); everything else stays as it is
+    pc_tile_factorisation: bool = True
 
     def pc_epsilon(self, dtype):
         return _by_precision(dtype, self.pc_epsilon_32, self.pc_epsilon_64)

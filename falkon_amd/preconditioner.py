@@ -117,7 +117,8 @@ def _cholesky_by_tiles_(B: torch.Tensor, info: torch.Tensor, first_row: int) -> 
                 B[j1:, j1:].addmm_(panel, panel.T, alpha=-1.0)
 
 
-def _cholesky_lower_(A: torch.Tensor, block: Optional[int] = None, min_size: Optional[int] = None) -> torch.Tensor:
+def _cholesky_lower_(A: torch.Tensor, block: Optional[int] = None, min_size: Optional[int] = None,
+                     use_tiles: bool = True) -> torch.Tensor:
     """Lower Cholesky factor of the symmetric positive definite ``A`` (only its lower triangle is read; ``A`` may be
     overwritten).  Raises ``torch.linalg.LinAlgError`` like the library routine if the matrix is not positive definite.
 
@@ -129,7 +130,7 @@ def _cholesky_lower_(A: torch.Tensor, block: Optional[int] = None, min_size: Opt
     blocks; small host matrices and column-major device matrices go to the library routine whole.
     """
     M = A.shape[0]
-    tiles = _tiles_apply(A) and min_size is None
+    tiles = use_tiles and _tiles_apply(A) and min_size is None
     if block is None:
         block = CHOL_BLOCK_DEVICE if tiles and M > CHOL_BLOCK else CHOL_BLOCK     # up to 4096 rows: rank-128 updates only
     min_size = CHOL_MIN_SIZE if min_size is None else min_size
@@ -325,7 +326,7 @@ class FalkonPreconditioner:
             C = self.kernel(X, X, opt=self.params)                     # fp64-computed when no_single_kernel
             eps = self.params.pc_epsilon(C.dtype)
             C.diagonal().add_(eps * M)
-            LT = _cholesky_lower_(C)
+            LT = _cholesky_lower_(C, use_tiles=self.params.pc_tile_factorisation)
             del C
             if weight_vec is None:
                 G = _gram_of_lower_factor(LT)                           # T T^T, lower triangle only
@@ -334,7 +335,7 @@ class FalkonPreconditioner:
                 G = _gram_of_lower_factor(LT * root)
             G.mul_(1.0 / M)
             G.diagonal().add_(self._lambda)
-            self.LA = _cholesky_lower_(G)
+            self.LA = _cholesky_lower_(G, use_tiles=self.params.pc_tile_factorisation)
             self.LT = LT
             self._T, self._A = _BlockedTriangular(self.LT), _BlockedTriangular(self.LA)
 
@@ -392,13 +393,13 @@ class LogisticPreconditioner(FalkonPreconditioner):
             if self.LT is None:                                         # first step only
                 C = self.kernel(X, X, opt=self.params)
                 C.diagonal().add_(self.params.pc_epsilon(C.dtype) * M)
-                self.LT = _cholesky_lower_(C)
+                self.LT = _cholesky_lower_(C, use_tiles=self.params.pc_tile_factorisation)
                 self._T = _BlockedTriangular(self.LT)
             at_centres = self.LT @ alpha.to(self.LT.dtype)              # T^T beta
             root = self.loss.ddf(Y.to(self.LT.dtype), at_centres).reshape(-1, 1).sqrt()
             G = _gram_of_lower_factor(self.LT * root)                   # T W T^T, lower triangle
             G.mul_(1.0 / N)                                             # 1/N here, not 1/M (logistic_preconditioner.py:146)
             G.diagonal().add_(penalty)
-            self.LA = _cholesky_lower_(G)
+            self.LA = _cholesky_lower_(G, use_tiles=self.params.pc_tile_factorisation)
             self._A = _BlockedTriangular(self.LA)
             self._lambda = penalty
