@@ -187,3 +187,29 @@ def test_double_precision_on_nearly_singular_kernel_matrices(m, d, sigma):
     err = ((L @ L.T) - K).abs().max().item()
     err_lib = ((lib_factor @ lib_factor.T) - K).abs().max().item()
     assert err <= max(8 * err_lib, 1e-13), (err, err_lib)
+
+
+def test_option_keeps_the_library_factorisation():
+    """FalkonOptions(pc_tile_factorisation=False): the preconditioner's factors come from the library routine and agree
+    with the default's to single-precision rounding on a well-conditioned problem."""
+    from falkon_amd import FalkonOptions, GaussianKernel
+    from falkon_amd.preconditioner import FalkonPreconditioner
+    import falkon_amd.preconditioner as pcm
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(11)
+    C = torch.randn(1500, 10, generator=g).to(dev)
+    factors = {}
+    for tiles in (True, False):
+        opt = FalkonOptions(pc_tile_factorisation=tiles)
+        calls = []
+        real = pcm._cholesky_by_tiles_
+        pcm._cholesky_by_tiles_ = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+        try:
+            pc = FalkonPreconditioner(1e-3, GaussianKernel(3.0, opt=opt), opt)
+            pc.init(C)
+        finally:
+            pcm._cholesky_by_tiles_ = real
+        assert bool(calls) == tiles
+        factors[tiles] = (pc.LT.clone(), pc.LA.clone())
+    for a, b in zip(factors[True], factors[False]):
+        assert (a - b).abs().max().item() <= 2e-4 * b.abs().max().item()
