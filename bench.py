@@ -469,7 +469,7 @@ def run_c5(args, lib, defer_cpu=False):
     from falkon_amd.preconditioner import FalkonPreconditioner
     opt_lib = FalkonOptions(bf16x3_cross_term=split, pc_tile_factorisation=False)
     pre_lib = None
-    for _ in range(2):
+    for _ in range(0 if args.no_cpu_baseline else 2):      # (a baseline leg: skipped with the CPU legs)
         pc = FalkonPreconditioner(lam, GaussianKernel(sigma, opt=opt_lib), opt_lib)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -477,7 +477,8 @@ def run_c5(args, lib, defer_cpu=False):
         torch.cuda.synchronize()
         pre_lib = time.perf_counter() - t0
         del pc
-    note(f"  C5 preconditioner with the library's factorisation of the diagonal blocks: {pre_lib:.2f} s")
+    if pre_lib is not None:
+        note(f"  C5 preconditioner with the library's factorisation of the diagonal blocks: {pre_lib:.2f} s")
     flop_per_launch = N * M * (2 * d + 4 + 2)
     kern_avg = kern_ms / max(launches, 1)
     achieved = flop_per_launch / (kern_avg * 1e-3) / 1e12
