@@ -20,7 +20,7 @@ from ..options import BaseOptions
 from ..utils.helpers import sizeof_dtype
 from .utils import check_contiguity, create_output_mat, retry_with_fresh_memory_report, usable_gpu_memory
 
-__all__ = ("fmmv", "fdmmv", "gauss_fmmv_native", "gauss_fdmmv_native")
+__all__ = ("fmmv", "fdmmv", "gauss_fmmv_native", "gauss_fdmmv_native", "PackedProducts")
 
 _DTYPE_CODE = {torch.float32: _backend.FLK_F32, torch.float64: _backend.FLK_F64}
 
@@ -383,6 +383,108 @@ def _fdmmv_explicit(X1, X2, v, w, out, sigma_dev, kernel_fn: int, dev, opt: Base
     if outd is not out:
         out.copy_(outd)
     return True
+
+
+class PackedProducts:
+    """``K(X1, X2)`` with both matrices packed once, for callers that multiply by the same kernel matrix many times
+    (a conjugate-gradient solve: falkon/optim/conjgrad.py:262-285 calls ``dmmv`` on the same X and centres in every
+    iteration).  The one-shot products pack their operands on every call (for a million rows of 28 features 64 us,
+    5 % of a product with a thousand centres); here ``flk_kernel_pack`` runs once and every product is
+    ``flk_kernel_mmv_packed`` on the packed copies, which gives bit for bit what ``fmmv`` / ``fdmmv`` give.
+
+    ``create`` returns None where this does not apply (operands not both on one GPU, a gradient required, the bf16x3
+    mode, or packed copies and workspace that do not fit the memory budget next to the data): the caller then keeps
+    to ``kernel.mmv`` / ``kernel.dmmv``."""
+
+    def __init__(self, X1, X2, kernel_fn, code, sigma_dev, p1, p2):
+        self.n, self.d = X1.shape
+        self.m = X2.shape[0]
+        self.dtype, self.device = X1.dtype, X1.device
+        self.kernel_fn, self.code, self.sigma_dev = kernel_fn, code, sigma_dev
+        self.p1, self.p2 = p1, p2
+        self._ws = None
+
+    @classmethod
+    def create(cls, X1: torch.Tensor, X2: torch.Tensor, kernel, opt: Optional[BaseOptions] = None,
+               columns: int = 1) -> Optional["PackedProducts"]:
+        opt = opt if opt is not None else BaseOptions()
+        if not (X1.is_cuda and X2.is_cuda and X1.device == X2.device and X1.dim() == 2 and X2.dim() == 2):
+            return None
+        if X1.dtype not in _DTYPE_CODE or X1.dtype != X2.dtype or X1.shape[1] != X2.shape[1] or opt.use_cpu:
+            return None
+        if X1.requires_grad or X2.requires_grad or any(p.requires_grad for p in kernel.diff_params.values()):
+            return None
+        code = _arith_code(X1.dtype, opt)
+        if code != _DTYPE_CODE[X1.dtype] or X1.shape[0] == 0 or X2.shape[0] == 0:
+            return None
+        try:
+            kernel_fn = _kernel_fn(kernel)
+            check_contiguity((X1, "X1"), (X2, "X2"))
+        except (NotImplementedError, ValueError):
+            return None
+        lib = _backend.load()
+        (n, d), m = X1.shape, X2.shape[0]
+        if d > lib.flk_max_d(code):
+            return None
+        b1, b2 = lib.flk_gauss_packed_bytes(n, d, code), lib.flk_gauss_packed_bytes(m, d, code)
+        ws = max(lib.flk_gauss_mmv_packed_workspace_bytes(m, n, d, columns, code),
+                 lib.flk_gauss_mmv_packed_workspace_bytes(n, m, d, columns, code))
+        sz = sizeof_dtype(X1.dtype)
+        need = b1 + b2 + ws + (n + m) * columns * sz
+        if need > usable_gpu_memory(X1.device, opt.max_gpu_mem, opt.memory_slack, enough=need):
+            return None
+        with torch.inference_mode():
+            sigma_dev = kernel._sigma_on(X1.device, X1.dtype, cached=False)
+            packed = []
+            with _current(X1.device):
+                stream = _stream_handle(X1.device)
+                for A, nbytes in ((X1, b1), (X2, b2)):
+                    buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=X1.device)
+                    rc = lib.flk_kernel_pack(kernel_fn, A.data_ptr(), A.shape[0], d, A.stride(0), A.stride(1),
+                                             sigma_dev.data_ptr(), sigma_dev.numel(), code, buf.data_ptr(), nbytes, stream)
+                    _backend.raise_for_status(rc, "flk_kernel_pack")
+                    packed.append(buf)
+            made = cls(X1, X2, kernel_fn, code, sigma_dev, packed[0], packed[1])
+            made._ws = torch.empty(max(ws, 1), dtype=torch.uint8, device=X1.device)     # (no allocation under a graph capture)
+        return made
+
+    def _product(self, pa, na, pb, nb, vec, addend, out):
+        lib = _backend.load()
+        t = vec.shape[1]
+        ws_bytes = lib.flk_gauss_mmv_packed_workspace_bytes(na, nb, self.d, t, self.code)
+        if self._ws is None or self._ws.numel() < ws_bytes:
+            self._ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=self.device)
+        add = (addend.data_ptr(), addend.stride(0), addend.stride(1)) if addend is not None else (None, 0, 0)
+        with _current(self.device):
+            rc = lib.flk_kernel_mmv_packed(self.kernel_fn, pa.data_ptr(), na, pb.data_ptr(), nb, self.d, vec.data_ptr(),
+                                           vec.stride(0), vec.stride(1), t, *add, out.data_ptr(), out.stride(0),
+                                           out.stride(1), self.code, self._ws.data_ptr(), ws_bytes,
+                                           _stream_handle(self.device))
+        _backend.raise_for_status(rc, "flk_kernel_mmv_packed")
+        return out
+
+    def _check(self, name, t, rows):
+        if t.dim() != 2 or t.shape[0] != rows or t.dtype != self.dtype or t.device != self.device:
+            raise ValueError(f"{name} must be a {rows}-row matrix of {self.dtype} on {self.device}")
+        check_contiguity((t, name))
+
+    def mmv(self, v: torch.Tensor, w: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``K(X1, X2) @ v (+ w)``, N x T."""
+        self._check("v", v, self.m)
+        if w is not None:
+            self._check("w", w, self.n)
+        out = torch.empty((self.n, v.shape[1]), dtype=self.dtype, device=self.device) if out is None else out
+        return self._product(self.p2, self.m, self.p1, self.n, v, w, out)
+
+    def mmv_t(self, u: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``K(X1, X2)^T @ u``, M x T."""
+        self._check("u", u, self.n)
+        out = torch.empty((self.m, u.shape[1]), dtype=self.dtype, device=self.device) if out is None else out
+        return self._product(self.p1, self.n, self.p2, self.m, u, None, out)
+
+    def dmmv(self, v: torch.Tensor, w: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``K^T (K v + w)``, M x T."""
+        return self.mmv_t(self.mmv(v, w), out)
 
 
 def fmmv(X1: torch.Tensor, X2: torch.Tensor, v: torch.Tensor, kernel, out: Optional[torch.Tensor] = None,

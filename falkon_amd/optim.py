@@ -212,6 +212,7 @@ class FalkonConjugateGradient:
         are then library GEMMs on it instead of kernel evaluations."""
         self.kernel, self.preconditioner, self.params, self.weight_fn = kernel, preconditioner, opt, weight_fn
         self.stored_knm = stored_knm
+        self._packed = None          # X and the centres packed once for the solve (PackedProducts), where that applies
         cg_fields = ("cg_epsilon_32", "cg_epsilon_64", "cg_tolerance", "cg_full_gradient_every",
                      "cg_differential_convergence", "cg_capture_graph")
         self.optimizer = ConjugateGradient(ConjugateGradientOptions(**{f: getattr(opt, f) for f in cg_fields}))
@@ -223,6 +224,8 @@ class FalkonConjugateGradient:
         inner = pc.invA(sol)
         if self.stored_knm is not None:
             gram = self.stored_knm.T @ (self.stored_knm @ pc.invT(inner))
+        elif self._packed is not None:
+            gram = self._packed.dmmv(pc.invT(inner))                              # the same product on operands packed once
         else:
             gram = self.kernel.dmmv(X, M, pc.invT(inner), None, opt=self.params)  # K_nm^T K_nm (.): the hot call
         return pc.invAt(pc.invTt(gram / n) + penalty * inner)
@@ -233,6 +236,8 @@ class FalkonConjugateGradient:
         inner = pc.invA(sol)
         if self.stored_knm is not None:
             gram = self.stored_knm.T @ (self.stored_knm @ pc.invT(inner)).mul_(y_weights)
+        elif self._packed is not None:
+            gram = self._packed.mmv_t(self._packed.mmv(pc.invT(inner)).mul_(y_weights))
         else:
             weighted = self.kernel.mmv(X, M, pc.invT(inner), None, opt=self.params).mul_(y_weights)
             gram = self.kernel.mmv(M, X, weighted, None, opt=self.params)
@@ -257,6 +262,20 @@ class FalkonConjugateGradient:
         else:
             operator = functools.partial(self.falkon_mmv, penalty=_lambda, X=X, M=M, n=n)
         self.optimizer.capture_ok = bool(X.is_cuda and M.is_cuda and Y.is_cuda)
-        kty = self.stored_knm.T @ y_over_n if self.stored_knm is not None else self.kernel.mmv(M, X, y_over_n, opt=self.params)
-        rhs = self.preconditioner.apply_t(kty)                                                # B^T K_nm^T (W) y / n
-        return self.optimizer.solve(initial_solution, rhs, operator, max_iter, callback)
+        self._packed = None
+        if self.stored_knm is None and getattr(self.params, "cg_pack_once", True) and Y.is_cuda:
+            from .mmv_ops.fmmv import PackedProducts
+            self._packed = PackedProducts.create(X, M, self.kernel, self.params, columns=Y.shape[1])
+            if self._packed is not None and (Y.device != X.device or Y.dtype != X.dtype):
+                self._packed = None
+        try:
+            if self.stored_knm is not None:
+                kty = self.stored_knm.T @ y_over_n
+            elif self._packed is not None:
+                kty = self._packed.mmv_t(y_over_n)
+            else:
+                kty = self.kernel.mmv(M, X, y_over_n, opt=self.params)
+            rhs = self.preconditioner.apply_t(kty)                                            # B^T K_nm^T (W) y / n
+            return self.optimizer.solve(initial_solution, rhs, operator, max_iter, callback)
+        finally:
+            self._packed = None                                                               # frees the packed copies

@@ -65,6 +65,8 @@ class ConjugateGradientOptions:
     cg_differential_convergence: bool = False         # a converged column is frozen while the others go on
     cg_capture_graph: bool = False                    # not in the reference: GPU solves capture each kind of iteration
                                                       # (operator + update) into a HIP graph once and replay it
+    cg_pack_once: bool = True                         # not in the reference: a GPU fit packs X and the centres once for
+                                                      # the whole solve instead of once per product (same results)
 
     def cg_epsilon(self, dtype):
         return _by_precision(dtype, self.cg_epsilon_32, self.cg_epsilon_64)

@@ -506,3 +506,22 @@ def test_reference_precomputed_kernel_fit(dev, incore):
     # (penalty 1e-6, ten iterations: the coefficients feel the different summation order of the two routes)
     a, b = flk.alpha_.cpu().numpy(), plain.alpha_.cpu().numpy()
     np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-6 * np.abs(b).max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("weighted", [False, True])
+def test_fit_with_operands_packed_once_is_the_same_fit(dev, weighted):
+    """``cg_pack_once`` (the default: X and the centres packed once for the solve) changes no result: the coefficients of
+    a GPU fit are bit for bit those of a fit whose every product packs its operands itself; also with a weight function."""
+    X, Y, _, _ = _config5(20_000, 10)
+    Xg, Yg = X.to(dev), Y.to(dev)
+    C = X[:700].clone()
+    weight_fn = (lambda Y, X, idx: torch.where(Y > 0, 2.0, 1.0).to(Y.dtype)) if weighted else None
+    fits = []
+    for once in (True, False):
+        opt = FalkonOptions(cg_pack_once=once)
+        model = Falkon(GaussianKernel(3.8, opt=opt), 1e-6, M=700, maxiter=10, options=opt, weight_fn=weight_fn,
+                       center_selection=FixedSelector(C.to(dev), idx_centers=torch.arange(700)))
+        model.fit(Xg, Yg)
+        fits.append(model.alpha_.clone())
+    assert torch.equal(fits[0], fits[1])

@@ -758,3 +758,38 @@ def test_odd_reduction_blocks_single_column_and_coincident_points(dev, d, blocks
     got = k.mmv(Xg, Cg, vi.to(dev)).cpu()
     ref = mmv_ref.fmmv_ref(X, C, vi, sigma)
     assert torch.isinf(ref).all() and torch.equal(torch.isinf(got), torch.isinf(ref)) and not torch.isnan(got).any()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("name,n,m,d,t", [("gaussian", 3000, 700, 28, 1), ("gaussian", 1500, 333, 9, 3), ("laplacian", 900, 257, 40, 2),
+                                           ("2.5-matern", 700, 300, 100, 5), ("gaussian", 640, 129, 300, 1), ("1.5-matern", 33, 1, 3, 70)])
+def test_products_on_operands_packed_once(dev, dtype, name, n, m, d, t):
+    """``PackedProducts`` (X and the centres packed once, what a GPU fit's solver uses for its products) gives bit for
+    bit what ``mmv`` / ``dmmv`` give, for strided operands and per-dimension lengthscales too, and does not apply where
+    the one-shot calls have work it does not do (host operands, gradients, the bf16x3 mode, a tiny memory budget)."""
+    from falkon_amd import FalkonOptions, LaplacianKernel, MaternKernel
+    from falkon_amd.mmv_ops.fmmv import PackedProducts
+    X, C, v, w = (a.to(dev) for a in _rand(n, d, m, t, dtype, seed=n + d + t))
+    sigma = torch.linspace(1.5, 3.0, d, dtype=torch.float64) * (d ** 0.5) / 3
+    k = {"gaussian": lambda: GaussianKernel(sigma), "laplacian": lambda: LaplacianKernel(sigma),
+         "1.5-matern": lambda: MaternKernel(sigma, 1.5), "2.5-matern": lambda: MaternKernel(sigma, 2.5)}[name]()
+    Xf = X.T.contiguous().T                                      # an F-ordered X, a v with a row stride
+    vs = torch.zeros(m, t + 2, dtype=dtype, device=dev)[:, 1:1 + t]
+    vs.copy_(v)
+    pp = PackedProducts.create(Xf, C, k, columns=t)
+    assert pp is not None
+    assert torch.equal(pp.mmv(vs), k.mmv(X, C, v))
+    assert torch.equal(pp.mmv(v, w), k.mmv(X, C, v) + w) or rel_err(pp.mmv(v, w), k.mmv(X, C, v) + w) < TOL[dtype]
+    u = torch.randn(n, t, dtype=dtype, device=dev)
+    assert torch.equal(pp.mmv_t(u), k.mmv(C, X, u))
+    assert torch.equal(pp.dmmv(v, w), k.dmmv(X, C, v, w))
+    assert torch.equal(pp.dmmv(v), k.dmmv(X, C, v, None))
+    out = torch.empty(m, t, dtype=dtype, device=dev)
+    assert pp.dmmv(v, w, out=out) is out and torch.equal(out, k.dmmv(X, C, v, w))
+    with pytest.raises(ValueError):
+        pp.mmv(v[:-1] if m > 1 else v.to(torch.float64 if dtype == torch.float32 else torch.float32))
+    assert PackedProducts.create(X.cpu(), C, k) is None
+    assert PackedProducts.create(X.clone().requires_grad_(True), C, k) is None
+    assert PackedProducts.create(X, C, k, FalkonOptions(bf16x3_cross_term=True)) is None or dtype == torch.float64
+    assert PackedProducts.create(X, C, k, FalkonOptions(max_gpu_mem=1000.0)) is None
