@@ -251,20 +251,23 @@ __global__ void __launch_bounds__(256) finalize_kernel(const T *__restrict__ par
 }
 
 // The same for many partial results of few outputs (the K^T u side of a product with few centres: hundreds of splits
-// of a thousand rows): 64 outputs per workgroup, each wave sums a quarter of the partial results (a contiguous
-// range, in order) and the four sums are added in order, so the result does not depend on timing.
+// of a thousand rows): 64 outputs per workgroup, each of its NW waves sums its share of the partial results (a
+// contiguous range, in order) and the NW sums are added in order, so the result does not depend on timing.  Four waves up
+// to kFinalizeWideMin partial results, sixteen beyond (a thousand outputs are sixteen workgroups: with 1737 partial
+// results each, four waves per workgroup took 23 us, a quarter of them spent by each wave in one dependent chain).
 constexpr int kFinalizeSplitMin = 16;
-template <typename T>
-__global__ void __launch_bounds__(256) finalize_split_kernel(const T *__restrict__ partial, int splits, int64_t tt,
-                                                             int64_t nb, int64_t nb_pad, const T *__restrict__ addend,
-                                                             int64_t add_rs, int64_t add_cs, T *__restrict__ out,
-                                                             int64_t out_rs, int64_t out_cs, bool zero_pad,
-                                                             const T *__restrict__ row_half_norm) {
-    __shared__ double red[4][64];
+constexpr int kFinalizeWideMin = 256;
+template <typename T, int NW>
+__global__ void __launch_bounds__(64 * NW) finalize_split_kernel(const T *__restrict__ partial, int splits, int64_t tt,
+                                                                 int64_t nb, int64_t nb_pad, const T *__restrict__ addend,
+                                                                 int64_t add_rs, int64_t add_cs, T *__restrict__ out,
+                                                                 int64_t out_rs, int64_t out_cs, bool zero_pad,
+                                                                 const T *__restrict__ row_half_norm) {
+    __shared__ double red[NW][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t b = (int64_t)blockIdx.x * 64 + lane;
     const int64_t t = blockIdx.y;
-    const int per = (splits + 3) / 4;
+    const int per = (splits + NW - 1) / NW;
     const int sp0 = wave * per < splits ? wave * per : splits;
     const int sp1 = sp0 + per < splits ? sp0 + per : splits;
     red[wave][lane] = b < nb ? sum_partials(partial + t * nb_pad + b, tt * nb_pad, sp0, sp1) : 0.0;
@@ -274,7 +277,9 @@ __global__ void __launch_bounds__(256) finalize_split_kernel(const T *__restrict
         if (zero_pad) out[b * out_rs + t * out_cs] = T(0);
         return;
     }
-    double s = ((red[0][lane] + red[1][lane]) + red[2][lane]) + red[3][lane];
+    double s = red[0][lane];
+#pragma unroll
+    for (int w = 1; w < NW; w++) s += red[w][lane];
     if (addend) s += (double)addend[b * add_rs + t * add_cs];
     T res = (T)s;
     if (row_half_norm && !finite_value(row_half_norm[b])) res = quiet_nan<T>();
@@ -286,8 +291,12 @@ int launch_finalize(const T *partial, int splits, int64_t t, int64_t nb, int64_t
                     int64_t add_rs, int64_t add_cs, T *out, int64_t out_rs, int64_t out_cs, bool zero_pad,
                     const T *row_half_norm, hipStream_t st) {
     if (nb_pad == 0 || t == 0) return FLK_OK;
-    if (splits >= kFinalizeSplitMin)
-        hipLaunchKernelGGL(finalize_split_kernel<T>, dim3((unsigned)((nb_pad + 63) / 64), (unsigned)t), dim3(256), 0, st,
+    if (splits >= kFinalizeWideMin)
+        hipLaunchKernelGGL((finalize_split_kernel<T, 16>), dim3((unsigned)((nb_pad + 63) / 64), (unsigned)t), dim3(1024), 0, st,
+                           partial, splits, t, nb, nb_pad, addend, add_rs, add_cs, out, out_rs, out_cs, zero_pad,
+                           row_half_norm);
+    else if (splits >= kFinalizeSplitMin)
+        hipLaunchKernelGGL((finalize_split_kernel<T, 4>), dim3((unsigned)((nb_pad + 63) / 64), (unsigned)t), dim3(256), 0, st,
                            partial, splits, t, nb, nb_pad, addend, add_rs, add_cs, out, out_rs, out_cs, zero_pad,
                            row_half_norm);
     else
